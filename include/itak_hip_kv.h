@@ -1,0 +1,290 @@
+/*
+ * itak_hip_kv: MI355X (gfx950) KV cache and attention backend, C ABI.
+ *
+ * One itak_pool owns the device-resident KV storage of up to max_slots independent
+ * sequences. A slot is one sequence's cache: the device twin of one
+ * attention::KvCache (crates/attention/src/cache.rs:308-834) and, through the
+ * itak_compute_* calls, of one cpu_compute::CpuCompute
+ * (crates/cpu-compute/src/cpu.rs:246-339). A Rust backend crate binds these
+ * symbols and implements muse_glimmer::Compute::attention
+ * (crates/muse-glimmer/src/compute.rs:82), the inherent cache_checkpoint /
+ * cache_rewind / cache_release / reset calls and itak_spec::TargetDriver
+ * (crates/itak-spec/src/driver.rs:42-99) on top of them.
+ *
+ * Conventions
+ *   - Every call returns an itak_status. 0 is success; 1..14 are the variants of
+ *     attention::AttentionError in declaration order
+ *     (crates/attention/src/error.rs:9-127); 15 is a cpu-compute StepFailed
+ *     refusal; the rest are this library's own.
+ *   - Nothing aborts or throws across the boundary. After a failure,
+ *     itak_last_error() returns the message (AttentionError's Display text for
+ *     codes 1..14) and itak_last_error_info() the variant's fields.
+ *   - "host" pointers are ordinary process memory; "device" pointers are HIP
+ *     device memory on the pool's device. Calls taking host pointers return
+ *     after the result is in host memory. Calls taking device pointers only
+ *     enqueue work on the pool's stream (itak_pool_set_stream).
+ *   - Rows are [kv_heads][head_dim] flat, queries and outputs
+ *     [query][q_heads][head_dim] flat, exactly as in the reference
+ *     (cache.rs:11-15, attention.rs:94-103).
+ *   - A pool is not thread-safe; use it from one thread at a time, as one
+ *     CpuCompute is (cpu.rs:246-253).
+ */
+#ifndef ITAK_HIP_KV_H
+#define ITAK_HIP_KV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int32_t itak_status;
+
+enum {
+    ITAK_OK = 0,
+    ITAK_ZERO_DIMENSION = 1,
+    ITAK_INVALID_WINDOW = 2,
+    ITAK_SIZE_OVERFLOW = 3,
+    ITAK_SHAPE_MISMATCH = 4,
+    ITAK_INVALID_LAYER = 5,
+    ITAK_OUT_OF_ORDER_POSITION = 6,
+    ITAK_NON_DIVISIBLE_HEADS = 7,
+    ITAK_NO_VISIBLE_KEYS = 8,
+    ITAK_CHECKPOINT_BUSY = 9,
+    ITAK_STALE_CHECKPOINT = 10,
+    ITAK_CHECKPOINT_TOO_DEEP = 11,
+    ITAK_CHECKPOINT_RANGE_EXCEEDED = 12,
+    ITAK_BULK_RESTORE_NOT_FRESH = 13,
+    ITAK_REWIND_OUT_OF_RANGE = 14,
+    ITAK_STEP_FAILED = 15,      /* GlimmerError::StepFailed (muse-glimmer/src/error.rs:69-76) */
+    ITAK_HIP_ERROR = 16,        /* a HIP runtime call failed; message carries hipGetErrorString */
+    ITAK_INVALID_ARGUMENT = 17, /* null pointer, unknown slot, unknown enum value */
+    ITAK_NO_FREE_SLOT = 18,     /* every slot of the pool is in use */
+    ITAK_CAPACITY_EXCEEDED = 19,/* a slot would outgrow the pool's per-slot row capacity */
+    ITAK_UNSUPPORTED = 20       /* a shape or layer kind this build has no kernel for */
+};
+
+/* Storage / source element types. */
+enum { ITAK_ELEM_F32 = 0, ITAK_ELEM_F16 = 1 };
+
+/* Layer kinds (attention::LayerKind, cache.rs:36-48). */
+enum { ITAK_LAYER_GLOBAL = 0, ITAK_LAYER_WINDOWED = 1 };
+
+/* itak_pool_config.flags */
+enum {
+    /* Zero the rows a truncate / rewind drops, so the raw device bytes (not only the
+       visible rows) equal those of a cache that never held them. */
+    ITAK_POOL_SCRUB_ON_TRUNCATE = 1u
+};
+
+typedef struct itak_pool itak_pool;
+
+typedef struct itak_pool_config {
+    uint32_t layer_count;
+    const uint8_t *layer_kinds; /* [layer_count] ITAK_LAYER_*; NULL = all global */
+    const uint64_t *windows;    /* [layer_count], read for windowed layers; may be NULL */
+    uint64_t num_kv_heads;
+    uint64_t head_dim;
+    uint32_t elem;          /* ITAK_ELEM_F32 (reference storage) or ITAK_ELEM_F16 */
+    uint32_t max_slots;     /* sequences the pool can hold at once */
+    uint64_t capacity_rows; /* positions one slot can hold per global layer */
+    int32_t device;         /* HIP device ordinal */
+    uint32_t flags;         /* ITAK_POOL_* */
+} itak_pool_config;
+
+/* The fields of the last refusal, in the order the Rust variant declares them
+   (what, then the integers: e.g. ShapeMismatch = what, a=expected, b=actual). */
+typedef struct itak_error_info {
+    int32_t code;
+    char what[96];
+    uint64_t a, b, c, d;
+} itak_error_info;
+
+/* attention::Checkpoint (cache.rs:229-273). Per-layer bases: itak_kv_checkpoint_bases. */
+typedef struct itak_checkpoint {
+    uint64_t cache_id;
+    uint64_t serial;
+    uint64_t max_round_tokens;
+    uint64_t saved_bytes;
+} itak_checkpoint;
+
+/* attention::LayerStats (cache.rs:88-98). */
+typedef struct itak_layer_stats {
+    uint64_t layer;
+    uint32_t kind;
+    uint32_t reserved;
+    uint64_t window;
+    uint64_t appended;
+    uint64_t stored;
+} itak_layer_stats;
+
+/* One sequence's share of a batched device step. */
+typedef struct itak_batch_item {
+    uint32_t slot;
+    uint32_t rows; /* new positions this slot appends and queries in this step */
+} itak_batch_item;
+
+/* One layer of a prefix snapshot held in host or device memory
+   (itak_kv::LayerSnapshot, crates/itak-kv/src/snapshot.rs:144-151). */
+typedef struct itak_snapshot_layer {
+    uint64_t first_position;
+    uint64_t rows;
+    const void *keys;   /* [rows][kv_heads][head_dim], oldest first */
+    const void *values; /* same shape */
+} itak_snapshot_layer;
+
+/* ---- library ------------------------------------------------------------------ */
+
+/* ABI version of this header; bumps on any incompatible change. */
+uint32_t itak_abi_version(void);
+
+/* Message of the last failure on this pool (or, with NULL, of the last failed
+   itak_pool_create on this thread). Valid until the next call on the same pool. */
+const char *itak_last_error(const itak_pool *pool);
+itak_status itak_last_error_info(const itak_pool *pool, itak_error_info *out);
+
+/* ---- pool and slots ------------------------------------------------------------- */
+
+/* Allocates and zero-fills the device KV storage: KvCache::new for every slot
+   (cache.rs:327-371; same zero-dimension / window / overflow refusals). */
+itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out);
+void itak_pool_destroy(itak_pool *pool);
+
+/* Stream every later call on this pool enqueues on (a hipStream_t; NULL = the
+   null stream). The pool never creates streams of its own. */
+itak_status itak_pool_set_stream(itak_pool *pool, void *hip_stream);
+itak_status itak_pool_synchronize(itak_pool *pool);
+/* Bytes of device memory the pool holds for KV rows. */
+uint64_t itak_pool_device_bytes(const itak_pool *pool);
+
+/* A slot is one sequence's cache. acquire = a fresh KvCache; reset = CpuCompute::reset
+   (cpu.rs:264-268): drop everything, positions restart at 0, outstanding checkpoint
+   handles go stale. */
+itak_status itak_slot_acquire(itak_pool *pool, uint32_t *slot);
+itak_status itak_slot_release(itak_pool *pool, uint32_t slot);
+itak_status itak_slot_reset(itak_pool *pool, uint32_t slot);
+
+/* ---- KvCache, per slot (crates/attention/src/cache.rs) ---------------------------- */
+
+uint64_t itak_kv_layer_count(const itak_pool *pool);  /* cache.rs:374-376 */
+uint64_t itak_kv_num_kv_heads(const itak_pool *pool); /* cache.rs:379-381 */
+uint64_t itak_kv_head_dim(const itak_pool *pool);     /* cache.rs:384-386 */
+/* KvCache::layer_kind (cache.rs:403-405). */
+itak_status itak_kv_layer_kind(itak_pool *pool, uint64_t layer, uint32_t *kind, uint64_t *window);
+/* KvCache::stored_len (cache.rs:408-410). */
+itak_status itak_kv_stored_len(itak_pool *pool, uint32_t slot, uint64_t layer, uint64_t *out);
+/* KvCache::next_position (cache.rs:413-415). */
+itak_status itak_kv_next_position(itak_pool *pool, uint32_t slot, uint64_t layer, uint64_t *out);
+/* KvCache::append (cache.rs:423-474): one position's K and V rows, host f32.
+   f16 pools store round-to-nearest-even halves (spec:
+   crates/wgpu-compute/src/kernels/k1_q4k_gemv.rs:285-329). */
+itak_status itak_kv_append(itak_pool *pool, uint32_t slot, uint64_t layer, const float *k,
+                           uint64_t k_len, const float *v, uint64_t v_len, uint64_t position);
+/* KvCache::restore_bulk (cache.rs:513-577): install rows for positions
+   first_position.. into a fresh layer. keys/values may be pinned host memory
+   (read in place by the gather kernel), ordinary host memory (staged) or device
+   memory; *_len count elements of src_elem type. An f32 source into an f16 pool is
+   converted exactly as append converts; an f16 source needs an f16 pool. */
+itak_status itak_kv_restore_bulk(itak_pool *pool, uint32_t slot, uint64_t layer,
+                                 uint64_t first_position, const void *keys, uint64_t keys_len,
+                                 const void *values, uint64_t values_len, uint32_t src_elem);
+/* KvSnapshot::restore (crates/itak-kv/src/snapshot.rs:321-334) for a whole snapshot:
+   validates every layer against token_count first (snapshot.rs:187-236), then
+   gathers all layers into the fresh slot. */
+itak_status itak_kv_restore_snapshot(itak_pool *pool, uint32_t slot, uint64_t token_count,
+                                     const itak_snapshot_layer *layers, uint64_t layer_count,
+                                     uint32_t src_elem);
+/* KvCache::stats (cache.rs:588-599); out holds layer_count entries. */
+itak_status itak_kv_stats(itak_pool *pool, uint32_t slot, itak_layer_stats *out);
+/* CacheView::{position_at,key,value} (cache.rs:878-903) for `rows` visible entries
+   starting at visible index `first`: raw storage elements (f32 or f16 bits) in
+   [row][kv_head][head_dim] order, plus each row's absolute position. Host outputs;
+   any of the three may be NULL. */
+itak_status itak_kv_read_rows(itak_pool *pool, uint32_t slot, uint64_t layer, uint64_t first,
+                              uint64_t rows, void *keys_out, void *values_out,
+                              uint64_t *positions_out);
+/* Every storage row of one slot and layer, capacity_rows long, visible or not
+   (what the scrub guarantee is checked on). Host outputs. */
+itak_status itak_kv_read_raw(itak_pool *pool, uint32_t slot, uint64_t layer, void *keys_out,
+                             void *values_out);
+/* KvCache::checkpoint_active / checkpoint / rewind_to / release (cache.rs:601-833). */
+itak_status itak_kv_checkpoint_active(itak_pool *pool, uint32_t slot, int32_t *out);
+itak_status itak_kv_checkpoint(itak_pool *pool, uint32_t slot, uint64_t max_round_tokens,
+                               itak_checkpoint *out);
+/* Checkpoint::bases (cache.rs:253-255); out holds layer_count entries. */
+itak_status itak_kv_checkpoint_bases(itak_pool *pool, uint32_t slot, const itak_checkpoint *cp,
+                                     uint64_t *out);
+itak_status itak_kv_rewind_to(itak_pool *pool, uint32_t slot, const itak_checkpoint *cp,
+                              uint64_t target);
+itak_status itak_kv_release(itak_pool *pool, uint32_t slot, const itak_checkpoint *cp);
+/* Batched truncation on speculative rejection: slot i drops every position
+   >= new_lengths[i] on all layers (the global-layer arm of KvCache::rewind_to,
+   cache.rs:788-791,814, without a checkpoint object). Refuses a length ahead of any
+   layer (RewindOutOfRange) or a slot with a live checkpoint (CheckpointBusy). */
+itak_status itak_kv_truncate(itak_pool *pool, const uint32_t *slots, const uint64_t *new_lengths,
+                             uint32_t count);
+
+/* ---- attention over one slot, host pointers ---------------------------------------- */
+
+/* attention::gqa_attention (crates/attention/src/attention.rs:104-215) over the slot's
+   view of `layer`. scale = NaN selects 1/sqrt(head_dim) (attention.rs:35-37).
+   softcap > 0 caps each scaled score as cap*tanh(s/cap) before the softmax
+   (formula: crates/torch-math/src/logits.rs:26-37); 0 disables it. */
+itak_status itak_gqa_attention(itak_pool *pool, uint32_t slot, uint64_t layer, const float *q,
+                               uint64_t q_len, uint64_t num_queries, uint64_t num_q_heads,
+                               const uint64_t *query_positions, uint64_t positions_len,
+                               float scale, float softcap, float *out);
+
+/* ---- CpuCompute, per slot (crates/cpu-compute/src/cpu.rs) --------------------------- */
+
+/* Compute::attention on a global (NoPE) layer (cpu.rs:506-655): checks whole rows,
+   cross-checks cache_position against the slot's position for `layer`, then for
+   each row appends its K/V and attends at its own position. q is
+   [rows][q_heads*head_dim], k and v [rows][kv_heads*head_dim]; out has q_len
+   elements. The slot is never advanced past what was appended: a failed call
+   leaves it ahead of the caller's position and the next call refuses until
+   itak_slot_reset, as the reference does. */
+itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t layer, const float *q,
+                                   uint64_t q_len, const float *k, uint64_t k_len, const float *v,
+                                   uint64_t v_len, uint64_t num_q_heads, uint64_t cache_position,
+                                   float softcap, float *out);
+/* CpuCompute::cache_checkpoint / cache_rewind / cache_release (cpu.rs:270-339): the
+   KvCache calls plus the "no KV state exists yet" refusals before a first forward. */
+itak_status itak_compute_cache_checkpoint(itak_pool *pool, uint32_t slot,
+                                          uint64_t max_round_tokens, itak_checkpoint *out);
+itak_status itak_compute_cache_rewind(itak_pool *pool, uint32_t slot, const itak_checkpoint *cp,
+                                      uint64_t target);
+itak_status itak_compute_cache_release(itak_pool *pool, uint32_t slot, const itak_checkpoint *cp);
+
+/* ---- batched device-resident step --------------------------------------------------- */
+
+/* The body of Compute::attention (cpu.rs:586-646) for several slots at once with all
+   tensors already on the device: item i appends items[i].rows new K/V rows at its
+   slot's next position for `layer`, then query row r of that item attends at
+   position base+r (the causal mask makes append-all-then-attend equal the
+   reference's row-at-a-time order on a global layer). q_dev is
+   [sum rows][q_heads*head_dim], k_dev and v_dev [sum rows][kv_heads*head_dim],
+   out_dev like q_dev, items in order. rows = 1 is decode, a few rows a speculative
+   verify block, many rows a prefill chunk. Enqueues on the pool's stream and
+   returns without waiting. No counterpart in the reference, whose slots are
+   separate threads (crates/itak-engine/src/engine.rs:336-383). */
+itak_status itak_attention_step_device(itak_pool *pool, uint64_t layer,
+                                       const itak_batch_item *items, uint32_t item_count,
+                                       const float *q_dev, const float *k_dev, const float *v_dev,
+                                       float *out_dev, uint64_t num_q_heads, float scale,
+                                       float softcap);
+/* The append half alone (K5 APPEND_SHADER's job,
+   crates/wgpu-compute/src/kernels/k5_rope_kv.rs:90-123), device tensors. */
+itak_status itak_kv_append_device(itak_pool *pool, uint64_t layer, const itak_batch_item *items,
+                                  uint32_t item_count, const float *k_dev, const float *v_dev);
+
+/* f32 -> f16 bits on the device with the cache's conversion (for tests of the
+   rounding rule over arbitrary inputs). Device pointers, pool's stream. */
+itak_status itak_convert_f32_to_f16_device(itak_pool *pool, const float *src_dev,
+                                           uint16_t *dst_dev, uint64_t count);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,30 @@
+"""MI355X (gfx950) KV-cache and attention backend: Python front end of the C ABI.
+
+The names mirror the reference's Rust API for this path (attention::KvCache,
+attention::gqa_attention, cpu_compute::CpuCompute, muse_glimmer::{AttentionRequest,
+PositionCache}); every operation runs in the HIP library, nothing falls back to the CPU.
+"""
+from .hip_compute import (  # noqa: F401
+    AttentionError,
+    AttentionParams,
+    AttentionRequest,
+    CacheView,
+    Checkpoint,
+    GlimmerConfig,
+    HipCompute,
+    KvCache,
+    KvPool,
+    LayerKind,
+    LayerStats,
+    PositionCache,
+    StepFailed,
+    gqa_attention,
+    kv_head_for_query_head,
+)
+from . import _native  # noqa: F401
+
+__all__ = [
+    "AttentionError", "AttentionParams", "AttentionRequest", "CacheView", "Checkpoint",
+    "GlimmerConfig", "HipCompute", "KvCache", "KvPool", "LayerKind", "LayerStats",
+    "PositionCache", "StepFailed", "gqa_attention", "kv_head_for_query_head",
+]

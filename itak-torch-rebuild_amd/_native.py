@@ -1,0 +1,131 @@
+"""ctypes binding of libitak_hip_kv.so (the C ABI declared in include/itak_hip_kv.h).
+
+There is no fallback: if the library is missing or does not export a declared symbol,
+import fails with an error that says how to build it.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libitak_hip_kv.so")
+
+OK = 0
+STATUS_NAMES = {
+    1: "ZeroDimension", 2: "InvalidWindow", 3: "SizeOverflow", 4: "ShapeMismatch",
+    5: "InvalidLayer", 6: "OutOfOrderPosition", 7: "NonDivisibleHeads", 8: "NoVisibleKeys",
+    9: "CheckpointBusy", 10: "StaleCheckpoint", 11: "CheckpointTooDeep",
+    12: "CheckpointRangeExceeded", 13: "BulkRestoreNotFresh", 14: "RewindOutOfRange",
+    15: "StepFailed", 16: "HipError", 17: "InvalidArgument", 18: "NoFreeSlot",
+    19: "CapacityExceeded", 20: "Unsupported",
+}
+ELEM_F32, ELEM_F16 = 0, 1
+LAYER_GLOBAL, LAYER_WINDOWED = 0, 1
+POOL_SCRUB_ON_TRUNCATE = 1
+
+
+class PoolConfig(C.Structure):
+    _fields_ = [
+        ("layer_count", C.c_uint32),
+        ("layer_kinds", C.c_void_p),
+        ("windows", C.c_void_p),
+        ("num_kv_heads", C.c_uint64),
+        ("head_dim", C.c_uint64),
+        ("elem", C.c_uint32),
+        ("max_slots", C.c_uint32),
+        ("capacity_rows", C.c_uint64),
+        ("device", C.c_int32),
+        ("flags", C.c_uint32),
+    ]
+
+
+class ErrorInfo(C.Structure):
+    _fields_ = [("code", C.c_int32), ("what", C.c_char * 96), ("a", C.c_uint64),
+                ("b", C.c_uint64), ("c", C.c_uint64), ("d", C.c_uint64)]
+
+
+class CheckpointRaw(C.Structure):
+    _fields_ = [("cache_id", C.c_uint64), ("serial", C.c_uint64),
+                ("max_round_tokens", C.c_uint64), ("saved_bytes", C.c_uint64)]
+
+
+class LayerStatsRaw(C.Structure):
+    _fields_ = [("layer", C.c_uint64), ("kind", C.c_uint32), ("reserved", C.c_uint32),
+                ("window", C.c_uint64), ("appended", C.c_uint64), ("stored", C.c_uint64)]
+
+
+class BatchItem(C.Structure):
+    _fields_ = [("slot", C.c_uint32), ("rows", C.c_uint32)]
+
+
+class SnapshotLayer(C.Structure):
+    _fields_ = [("first_position", C.c_uint64), ("rows", C.c_uint64), ("keys", C.c_void_p),
+                ("values", C.c_void_p)]
+
+
+_P = C.c_void_p
+_u32, _u64, _f32, _i32 = C.c_uint32, C.c_uint64, C.c_float, C.c_int32
+
+# name -> (restype, argtypes): every symbol include/itak_hip_kv.h declares.
+PROTOTYPES = {
+    "itak_abi_version": (_u32, []),
+    "itak_last_error": (C.c_char_p, [_P]),
+    "itak_last_error_info": (_i32, [_P, C.POINTER(ErrorInfo)]),
+    "itak_pool_create": (_i32, [C.POINTER(PoolConfig), C.POINTER(_P)]),
+    "itak_pool_destroy": (None, [_P]),
+    "itak_pool_set_stream": (_i32, [_P, _P]),
+    "itak_pool_synchronize": (_i32, [_P]),
+    "itak_pool_device_bytes": (_u64, [_P]),
+    "itak_slot_acquire": (_i32, [_P, C.POINTER(_u32)]),
+    "itak_slot_release": (_i32, [_P, _u32]),
+    "itak_slot_reset": (_i32, [_P, _u32]),
+    "itak_kv_layer_count": (_u64, [_P]),
+    "itak_kv_num_kv_heads": (_u64, [_P]),
+    "itak_kv_head_dim": (_u64, [_P]),
+    "itak_kv_layer_kind": (_i32, [_P, _u64, C.POINTER(_u32), C.POINTER(_u64)]),
+    "itak_kv_stored_len": (_i32, [_P, _u32, _u64, C.POINTER(_u64)]),
+    "itak_kv_next_position": (_i32, [_P, _u32, _u64, C.POINTER(_u64)]),
+    "itak_kv_append": (_i32, [_P, _u32, _u64, _P, _u64, _P, _u64, _u64]),
+    "itak_kv_restore_bulk": (_i32, [_P, _u32, _u64, _u64, _P, _u64, _P, _u64, _u32]),
+    "itak_kv_restore_snapshot": (_i32, [_P, _u32, _u64, C.POINTER(SnapshotLayer), _u64, _u32]),
+    "itak_kv_stats": (_i32, [_P, _u32, C.POINTER(LayerStatsRaw)]),
+    "itak_kv_read_rows": (_i32, [_P, _u32, _u64, _u64, _u64, _P, _P, _P]),
+    "itak_kv_read_raw": (_i32, [_P, _u32, _u64, _P, _P]),
+    "itak_kv_checkpoint_active": (_i32, [_P, _u32, C.POINTER(_i32)]),
+    "itak_kv_checkpoint": (_i32, [_P, _u32, _u64, C.POINTER(CheckpointRaw)]),
+    "itak_kv_checkpoint_bases": (_i32, [_P, _u32, C.POINTER(CheckpointRaw), _P]),
+    "itak_kv_rewind_to": (_i32, [_P, _u32, C.POINTER(CheckpointRaw), _u64]),
+    "itak_kv_release": (_i32, [_P, _u32, C.POINTER(CheckpointRaw)]),
+    "itak_kv_truncate": (_i32, [_P, _P, _P, _u32]),
+    "itak_gqa_attention": (_i32, [_P, _u32, _u64, _P, _u64, _u64, _u64, _P, _u64, _f32, _f32, _P]),
+    "itak_compute_attention": (_i32, [_P, _u32, _u64, _P, _u64, _P, _u64, _P, _u64, _u64, _u64,
+                                      _f32, _P]),
+    "itak_compute_cache_checkpoint": (_i32, [_P, _u32, _u64, C.POINTER(CheckpointRaw)]),
+    "itak_compute_cache_rewind": (_i32, [_P, _u32, C.POINTER(CheckpointRaw), _u64]),
+    "itak_compute_cache_release": (_i32, [_P, _u32, C.POINTER(CheckpointRaw)]),
+    "itak_attention_step_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P, _P, _P,
+                                          _u64, _f32, _f32]),
+    "itak_kv_append_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P]),
+    "itak_convert_f32_to_f16_device": (_i32, [_P, _P, _P, _u64]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the library and bind every declared symbol; raises if anything is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python {os.path.join(HERE, 'build.py')}` "
+            "(hipcc --offload-arch=gfx950). There is no CPU fallback.")
+    lib = C.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in PROTOTYPES.items():
+        fn = getattr(lib, name)  # AttributeError names the missing symbol
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib

@@ -1,0 +1,133 @@
+// Shared declarations between the host logic (pool.hip) and the kernel files.
+// Nothing here is part of the public ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace itak {
+
+// Device layout of the KV pool, in elements of the storage type. One "plane" is the
+// rows of one (layer, slot, side, kv_head): capacity x head_dim elements, contiguous,
+// so a workgroup that streams one KV head reads one unbroken run of memory.
+//   element(layer, slot, side, head, row, d) =
+//     layer*layer_stride + slot*slot_stride + side*side_stride + head*head_stride + row*head_dim + d
+// side 0 = keys, 1 = values.
+struct PoolGeom {
+    uint32_t kv_heads;
+    uint32_t head_dim;
+    uint32_t capacity;  // rows per plane
+    uint32_t max_slots;
+    uint64_t head_stride;   // capacity * head_dim
+    uint64_t side_stride;   // kv_heads * head_stride
+    uint64_t slot_stride;   // 2 * side_stride
+    uint64_t layer_stride;  // max_slots * slot_stride
+};
+
+constexpr int kMaxBatchItems = 64;
+
+// ---- append ---------------------------------------------------------------------
+struct AppendItem {
+    uint32_t slot;
+    uint32_t rows;
+    uint32_t pos0;      // storage row of the item's first new row
+    uint32_t src_row0;  // row offset of the item inside k_src / v_src
+};
+struct AppendBatch {
+    uint32_t n;
+    uint32_t total_rows;
+    AppendItem item[kMaxBatchItems];
+};
+hipError_t launch_append(void *layer_base, int elem_f16, const PoolGeom &g, const AppendBatch &b,
+                         const float *k_src, const float *v_src, hipStream_t stream);
+
+// ---- zero fill of dropped rows (truncate scrub, slot reset) ------------------------
+struct ZeroItem {
+    uint32_t slot;
+    uint32_t row_from;
+    uint32_t row_to;  // exclusive
+    uint32_t pad;
+};
+struct ZeroBatch {
+    uint32_t n;
+    uint32_t max_rows;
+    ZeroItem item[kMaxBatchItems];
+};
+hipError_t launch_zero_rows(void *pool_base, int elem_f16, const PoolGeom &g, uint32_t layer_from,
+                            uint32_t layer_to, const ZeroBatch &b, hipStream_t stream);
+
+// ---- snapshot restore (gather from [row][kv_head][d] sources into the planes) --------
+constexpr int kMaxRestoreLayers = 64;
+struct RestoreLayer {
+    const void *keys;
+    const void *values;
+    uint32_t layer;
+    uint32_t rows;
+    uint32_t first_row;  // destination storage row of source row 0
+    uint32_t pad;
+};
+struct RestoreBatch {
+    uint32_t n;
+    uint32_t max_rows;
+    uint32_t slot;
+    uint32_t pad;
+    RestoreLayer layer[kMaxRestoreLayers];
+};
+hipError_t launch_restore(void *pool_base, int dst_f16, int src_f16, const PoolGeom &g,
+                          const RestoreBatch &b, hipStream_t stream);
+
+// ---- row readback: planes -> [row][kv_head][d] ---------------------------------------
+hipError_t launch_read_rows(const void *layer_base, int elem_f16, const PoolGeom &g, uint32_t slot,
+                            uint32_t first_row, uint32_t rows, void *keys_out, void *values_out,
+                            hipStream_t stream);
+
+hipError_t launch_convert_f16(const float *src, uint16_t *dst, uint64_t count, hipStream_t stream);
+
+// ---- attention ----------------------------------------------------------------------
+// One item = one slot's query rows against that slot's rows of one layer. Query row r
+// sits at position pos0 + r unless q_pos is given. A workgroup owns (item, row block,
+// kv head, split of the key range) and writes either the final output (splits == 1) or
+// a partial (m, l, acc[head_dim]) per query vector that the last workgroup to finish
+// for that (item, row block, kv head) merges.
+struct AttnItem {
+    uint32_t slot;
+    uint32_t rows;
+    uint32_t pos0;
+    uint32_t q_row0;        // first row of the item in q / out
+    uint32_t kv_len;        // stored rows visible to the item's last query row (exclusive end)
+    uint32_t splits;
+    uint32_t keys_per_split;
+    uint32_t block0;        // first workgroup index of the item
+    uint32_t ws0;           // first partial index of the item
+    uint32_t cnt0;          // first arrival counter of the item
+};
+struct AttnBatch {
+    uint32_t n;
+    uint32_t total_blocks;
+    uint32_t rows_per_block;
+    uint32_t pad;
+    AttnItem item[kMaxBatchItems];
+};
+struct AttnParams {
+    const void *layer_base;
+    PoolGeom g;
+    const float *q;
+    float *out;
+    const uint32_t *q_pos;  // optional explicit positions, [sum rows]
+    float *ws;              // partials: (head_dim + 2) floats each
+    uint32_t *counters;     // arrival counters, zero between launches
+    uint32_t q_heads;
+    uint32_t group;         // q_heads / kv_heads
+    float scale;
+    float softcap;
+};
+
+// Generic VALU path: f32 or f16 storage, any head_dim <= 256, group <= 64.
+hipError_t launch_attn_generic(int elem_f16, const AttnParams &p, const AttnBatch &b,
+                               hipStream_t stream);
+// Query rows one workgroup of the generic kernel carries (0 = shape not supported).
+uint32_t attn_generic_rows_per_block(uint32_t group, uint32_t head_dim);
+// Keys per tile of the generic kernel for a head_dim.
+uint32_t attn_generic_tile(uint32_t head_dim);
+
+}  // namespace itak

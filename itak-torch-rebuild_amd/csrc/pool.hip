@@ -1,0 +1,1178 @@
+// Host side of the C ABI: the pool, its slots, the per-slot bookkeeping that mirrors
+// attention::KvCache (crates/attention/src/cache.rs) and cpu_compute::CpuCompute
+// (crates/cpu-compute/src/cpu.rs), and the launch logic for the kernels in this directory.
+// All validation happens here, in the reference's order, before anything is enqueued.
+#include "../../include/itak_hip_kv.h"
+#include "internal.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+using namespace itak;
+
+namespace {
+
+struct LiveCheckpoint {
+    bool live = false;
+    uint64_t serial = 0;
+    uint64_t max_round_tokens = 0;
+    std::vector<uint64_t> bases;
+};
+
+struct Slot {
+    bool in_use = false;
+    bool built = false;  // CpuCompute's KvState exists (cpu.rs:560-564)
+    uint64_t cache_id = 0;
+    uint64_t next_serial = 0;
+    std::vector<uint64_t> appended;  // per layer: positions appended == next position
+    LiveCheckpoint cp;
+};
+
+struct ErrorState {
+    std::string message;
+    itak_error_info info{};
+};
+
+thread_local ErrorState g_create_error;
+uint64_t g_next_cache_id = 1;  // cache.rs:32
+
+}  // namespace
+
+struct itak_pool {
+    itak_pool_config cfg{};
+    PoolGeom g{};
+    int elem_f16 = 0;
+    uint32_t elem_bytes = 4;
+    uint64_t row = 0;  // kv_heads * head_dim
+    unsigned char *base = nullptr;
+    uint64_t bytes = 0;
+    hipStream_t stream = nullptr;
+    std::vector<Slot> slots;
+    // Device scratch, grown on demand and reused: staging for host-pointer calls,
+    // split partials and arrival counters.
+    unsigned char *stage = nullptr;
+    uint64_t stage_bytes = 0;
+    float *ws = nullptr;
+    uint64_t ws_floats = 0;
+    uint32_t *counters = nullptr;
+    uint64_t n_counters = 0;
+    mutable ErrorState err;
+};
+
+namespace {
+
+// ------------------------------------------------------------------------------ errors
+
+itak_status set_error(ErrorState &e, int32_t code, const char *what, uint64_t a, uint64_t b,
+                      uint64_t c, uint64_t d, const char *fmt, ...) {
+    e.info = itak_error_info{};
+    e.info.code = code;
+    if (what) snprintf(e.info.what, sizeof(e.info.what), "%s", what);
+    e.info.a = a;
+    e.info.b = b;
+    e.info.c = c;
+    e.info.d = d;
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    e.message = buf;
+    return code;
+}
+
+#define ULL(x) static_cast<unsigned long long>(x)
+
+// The Display texts of AttentionError (crates/attention/src/error.rs:129-214).
+itak_status zero_dimension(ErrorState &e, const char *what) {
+    return set_error(e, ITAK_ZERO_DIMENSION, what, 0, 0, 0, 0, "%s must be positive, got 0", what);
+}
+itak_status invalid_window(ErrorState &e, uint64_t window) {
+    return set_error(e, ITAK_INVALID_WINDOW, nullptr, window, 0, 0, 0,
+                     "sliding window must be positive, got %llu", ULL(window));
+}
+itak_status size_overflow(ErrorState &e, const char *what) {
+    return set_error(e, ITAK_SIZE_OVERFLOW, what, 0, 0, 0, 0, "%s: element count overflows usize",
+                     what);
+}
+itak_status shape_mismatch(ErrorState &e, const char *what, uint64_t expected, uint64_t actual) {
+    return set_error(e, ITAK_SHAPE_MISMATCH, what, expected, actual, 0, 0,
+                     "%s: got %llu, expected %llu", what, ULL(actual), ULL(expected));
+}
+itak_status invalid_layer(ErrorState &e, uint64_t layer, uint64_t layer_count) {
+    return set_error(e, ITAK_INVALID_LAYER, nullptr, layer, layer_count, 0, 0,
+                     "layer %llu out of range, cache has %llu layers", ULL(layer),
+                     ULL(layer_count));
+}
+itak_status out_of_order(ErrorState &e, uint64_t layer, uint64_t expected, uint64_t actual) {
+    return set_error(e, ITAK_OUT_OF_ORDER_POSITION, nullptr, layer, expected, actual, 0,
+                     "layer %llu appends must be in order: expected position %llu, got %llu",
+                     ULL(layer), ULL(expected), ULL(actual));
+}
+itak_status non_divisible(ErrorState &e, uint64_t q_heads, uint64_t kv_heads) {
+    return set_error(e, ITAK_NON_DIVISIBLE_HEADS, nullptr, q_heads, kv_heads, 0, 0,
+                     "%llu query heads do not divide evenly across %llu KV heads", ULL(q_heads),
+                     ULL(kv_heads));
+}
+itak_status no_visible_keys(ErrorState &e, uint64_t position) {
+    return set_error(e, ITAK_NO_VISIBLE_KEYS, nullptr, position, 0, 0, 0,
+                     "query at position %llu has no visible keys", ULL(position));
+}
+itak_status checkpoint_busy(ErrorState &e) {
+    return set_error(e, ITAK_CHECKPOINT_BUSY, nullptr, 0, 0, 0, 0,
+                     "a checkpoint is already outstanding on this cache; release it before "
+                     "taking another");
+}
+itak_status stale_checkpoint(ErrorState &e, uint64_t serial) {
+    return set_error(e, ITAK_STALE_CHECKPOINT, nullptr, serial, 0, 0, 0,
+                     "checkpoint %llu is not this cache's live checkpoint (already released or "
+                     "foreign)",
+                     ULL(serial));
+}
+itak_status range_exceeded(ErrorState &e, uint64_t layer, uint64_t position, uint64_t limit) {
+    return set_error(e, ITAK_CHECKPOINT_RANGE_EXCEEDED, nullptr, layer, position, limit, 0,
+                     "layer %llu append at position %llu is outside the live checkpoint's saved "
+                     "range (first unsaved position %llu); refusing so a later rewind cannot meet "
+                     "a slot it cannot restore",
+                     ULL(layer), ULL(position), ULL(limit));
+}
+itak_status not_fresh(ErrorState &e, uint64_t layer, uint64_t appended) {
+    return set_error(e, ITAK_BULK_RESTORE_NOT_FRESH, nullptr, layer, appended, 0, 0,
+                     "layer %llu already holds %llu appended positions; bulk restore installs "
+                     "into a fresh layer only",
+                     ULL(layer), ULL(appended));
+}
+itak_status rewind_range(ErrorState &e, uint64_t layer, uint64_t base, uint64_t appended,
+                         uint64_t target) {
+    return set_error(e, ITAK_REWIND_OUT_OF_RANGE, nullptr, layer, base, appended, target,
+                     "rewind target %llu is outside layer %llu's checkpoint range [%llu, %llu]",
+                     ULL(target), ULL(layer), ULL(base), ULL(appended));
+}
+itak_status hip_error(ErrorState &e, hipError_t code, const char *doing) {
+    return set_error(e, ITAK_HIP_ERROR, doing, uint64_t(code), 0, 0, 0, "%s: HIP error %d (%s)",
+                     doing, int(code), hipGetErrorString(code));
+}
+itak_status invalid_argument(ErrorState &e, const char *what) {
+    return set_error(e, ITAK_INVALID_ARGUMENT, what, 0, 0, 0, 0, "invalid argument: %s", what);
+}
+itak_status capacity_exceeded(ErrorState &e, uint64_t layer, uint64_t need, uint64_t capacity) {
+    return set_error(e, ITAK_CAPACITY_EXCEEDED, nullptr, layer, need, capacity, 0,
+                     "layer %llu would hold %llu positions but the pool's slots hold %llu",
+                     ULL(layer), ULL(need), ULL(capacity));
+}
+itak_status unsupported(ErrorState &e, const char *what) {
+    return set_error(e, ITAK_UNSUPPORTED, what, 0, 0, 0, 0, "unsupported: %s", what);
+}
+
+#define HIP_TRY(pool, call, doing)                                   \
+    do {                                                             \
+        hipError_t _e = (call);                                      \
+        if (_e != hipSuccess) return hip_error((pool)->err, _e, doing); \
+    } while (0)
+
+// ------------------------------------------------------------------------------ helpers
+
+Slot *find_slot(itak_pool *pool, uint32_t slot) {
+    if (slot >= pool->slots.size() || !pool->slots[slot].in_use) return nullptr;
+    return &pool->slots[slot];
+}
+
+void *layer_base(itak_pool *pool, uint64_t layer) {
+    return pool->base + layer * pool->g.layer_stride * pool->elem_bytes;
+}
+
+itak_status ensure_stage(itak_pool *pool, uint64_t bytes) {
+    if (bytes <= pool->stage_bytes) return ITAK_OK;
+    HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize before growing staging");
+    if (pool->stage) HIP_TRY(pool, hipFree(pool->stage), "free staging");
+    pool->stage = nullptr;
+    pool->stage_bytes = 0;
+    uint64_t want = std::max<uint64_t>(bytes + bytes / 2, 1u << 20);
+    HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&pool->stage), want), "allocate staging");
+    pool->stage_bytes = want;
+    return ITAK_OK;
+}
+
+itak_status ensure_workspace(itak_pool *pool, uint64_t floats, uint64_t counters) {
+    if (floats > pool->ws_floats) {
+        HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize before growing workspace");
+        if (pool->ws) HIP_TRY(pool, hipFree(pool->ws), "free workspace");
+        pool->ws = nullptr;
+        pool->ws_floats = 0;
+        uint64_t want = std::max<uint64_t>(floats + floats / 2, 1u << 18);
+        HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&pool->ws), want * sizeof(float)),
+                "allocate split workspace");
+        pool->ws_floats = want;
+    }
+    if (counters > pool->n_counters) {
+        HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize before growing counters");
+        if (pool->counters) HIP_TRY(pool, hipFree(pool->counters), "free counters");
+        pool->counters = nullptr;
+        pool->n_counters = 0;
+        uint64_t want = std::max<uint64_t>(counters * 2, 4096);
+        HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&pool->counters), want * 4),
+                "allocate arrival counters");
+        // Counters are zero between launches: the merging workgroup resets its own.
+        HIP_TRY(pool, hipMemsetAsync(pool->counters, 0, want * 4, pool->stream),
+                "zero arrival counters");
+        pool->n_counters = want;
+    }
+    return ITAK_OK;
+}
+
+uint64_t align_up(uint64_t x, uint64_t a) { return (x + a - 1) / a * a; }
+
+// One item's query rows against its slot; fills the split plan.
+struct PlanInput {
+    uint32_t slot;
+    uint32_t rows;
+    uint32_t pos0;
+    uint32_t kv_len;
+};
+
+// Builds the work list for the generic kernel and launches it. q/out are device pointers.
+itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, uint32_t n,
+                          const float *q_dev, float *out_dev, const uint32_t *q_pos_dev,
+                          uint64_t q_heads, float scale, float softcap) {
+    const uint32_t group = uint32_t(q_heads / pool->g.kv_heads);
+    const uint32_t rpb = attn_generic_rows_per_block(group, pool->g.head_dim);
+    if (rpb == 0) return unsupported(pool->err, "head_dim above 256 or GQA group too wide");
+    const uint32_t tile = attn_generic_tile(pool->g.head_dim);
+    constexpr uint64_t kTargetBlocks = 1024;  // about four workgroups per CU
+
+    uint32_t q_row0 = 0;
+    for (uint32_t first = 0; first < n; first += kMaxBatchItems) {
+        const uint32_t count = std::min<uint32_t>(kMaxBatchItems, n - first);
+        AttnBatch b{};
+        b.n = count;
+        b.rows_per_block = rpb;
+        uint64_t key_work = 0;
+        for (uint32_t i = 0; i < count; ++i) {
+            const PlanInput &pi = in[first + i];
+            const uint64_t qblocks = (pi.rows + rpb - 1) / rpb;
+            key_work += qblocks * pool->g.kv_heads * pi.kv_len;
+        }
+        uint64_t kps = align_up(std::max<uint64_t>((key_work + kTargetBlocks - 1) / kTargetBlocks,
+                                                   tile),
+                                tile);
+        uint32_t block0 = 0, ws0 = 0, cnt0 = 0;
+        for (uint32_t i = 0; i < count; ++i) {
+            const PlanInput &pi = in[first + i];
+            AttnItem &it = b.item[i];
+            it.slot = pi.slot;
+            it.rows = pi.rows;
+            it.pos0 = pi.pos0;
+            it.q_row0 = q_row0;
+            it.kv_len = pi.kv_len;
+            it.keys_per_split = uint32_t(kps);
+            it.splits = uint32_t((pi.kv_len + kps - 1) / kps);
+            if (it.splits == 0) it.splits = 1;
+            const uint32_t qblocks = (pi.rows + rpb - 1) / rpb;
+            it.block0 = block0;
+            it.ws0 = ws0;
+            it.cnt0 = cnt0;
+            block0 += qblocks * pool->g.kv_heads * it.splits;
+            if (it.splits > 1) ws0 += pi.rows * uint32_t(q_heads) * it.splits;
+            cnt0 += qblocks * pool->g.kv_heads;
+            q_row0 += pi.rows;
+        }
+        b.total_blocks = block0;
+        itak_status st =
+            ensure_workspace(pool, uint64_t(ws0) * (pool->g.head_dim + 2), cnt0);
+        if (st != ITAK_OK) return st;
+        AttnParams p{};
+        p.layer_base = layer_base(pool, layer);
+        p.g = pool->g;
+        p.q = q_dev;
+        p.out = out_dev;
+        p.q_pos = q_pos_dev;
+        p.ws = pool->ws;
+        p.counters = pool->counters;
+        p.q_heads = uint32_t(q_heads);
+        p.group = group;
+        p.scale = scale;
+        p.softcap = softcap;
+        HIP_TRY(pool, launch_attn_generic(pool->elem_f16, p, b, pool->stream),
+                "launch attention");
+    }
+    return ITAK_OK;
+}
+
+float default_scale(uint64_t head_dim) {  // attention.rs:35-37
+    return 1.0f / std::sqrt(static_cast<float>(head_dim));
+}
+
+// Appends `rows` rows per item from device sources; the caller has validated everything.
+itak_status run_append(itak_pool *pool, uint64_t layer, const itak_batch_item *items, uint32_t n,
+                       const float *k_dev, const float *v_dev) {
+    uint32_t src_row = 0;
+    for (uint32_t first = 0; first < n; first += kMaxBatchItems) {
+        const uint32_t count = std::min<uint32_t>(kMaxBatchItems, n - first);
+        AppendBatch b{};
+        b.n = count;
+        const uint32_t chunk_row0 = src_row;
+        for (uint32_t i = 0; i < count; ++i) {
+            const itak_batch_item &bi = items[first + i];
+            b.item[i].slot = bi.slot;
+            b.item[i].rows = bi.rows;
+            b.item[i].pos0 = uint32_t(pool->slots[bi.slot].appended[layer]);
+            b.item[i].src_row0 = src_row - chunk_row0;
+            src_row += bi.rows;
+        }
+        b.total_rows = src_row - chunk_row0;
+        HIP_TRY(pool,
+                launch_append(layer_base(pool, layer), pool->elem_f16, pool->g, b,
+                              k_dev + uint64_t(chunk_row0) * pool->row,
+                              v_dev + uint64_t(chunk_row0) * pool->row, pool->stream),
+                "launch append");
+    }
+    for (uint32_t i = 0; i < n; ++i) pool->slots[items[i].slot].appended[layer] += items[i].rows;
+    return ITAK_OK;
+}
+
+// The append preconditions of KvCache::append (cache.rs:445-471) for `rows` consecutive
+// positions starting at the layer's next one; returns how many rows may be appended
+// before a refusal (rows if none) and leaves that refusal in the error state.
+itak_status check_append_rows(itak_pool *pool, Slot &s, uint64_t layer, uint64_t rows,
+                              uint64_t *ok_rows) {
+    uint64_t ok = rows;
+    itak_status st = ITAK_OK;
+    const uint64_t start = s.appended[layer];
+    if (s.cp.live) {
+        const uint64_t limit = s.cp.bases[layer] + s.cp.max_round_tokens;
+        if (start + rows > limit) {
+            ok = limit > start ? limit - start : 0;
+            st = range_exceeded(pool->err, layer, start + ok, limit);
+        }
+    }
+    if (start + ok > pool->g.capacity) {
+        ok = pool->g.capacity > start ? pool->g.capacity - start : 0;
+        st = capacity_exceeded(pool->err, layer, start + ok + 1, pool->g.capacity);
+    }
+    *ok_rows = ok;
+    return st;
+}
+
+itak_status scrub_rows(itak_pool *pool, const ZeroBatch &zb) {
+    HIP_TRY(pool,
+            launch_zero_rows(pool->base, pool->elem_f16, pool->g, 0, pool->cfg.layer_count, zb,
+                             pool->stream),
+            "launch row scrub");
+    return ITAK_OK;
+}
+
+// Pointer kinds for restore sources. For memory the device can read in place, `usable`
+// is the address a kernel should dereference.
+enum class PtrKind { Device, PinnedHost, PlainHost };
+PtrKind classify(const void *p, const void **usable) {
+    *usable = p;
+    hipPointerAttribute_t attr{};
+    hipError_t e = hipPointerGetAttributes(&attr, p);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();  // an unknown pointer is ordinary host memory, not a failure
+        return PtrKind::PlainHost;
+    }
+    if (attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged)
+        return PtrKind::Device;
+    if (attr.type == hipMemoryTypeHost) {
+        if (attr.devicePointer) *usable = attr.devicePointer;
+        return PtrKind::PinnedHost;
+    }
+    return PtrKind::PlainHost;
+}
+
+}  // namespace
+
+// ======================================================================== public ABI
+
+extern "C" {
+
+uint32_t itak_abi_version(void) { return 1; }
+
+const char *itak_last_error(const itak_pool *pool) {
+    return pool ? pool->err.message.c_str() : g_create_error.message.c_str();
+}
+
+itak_status itak_last_error_info(const itak_pool *pool, itak_error_info *out) {
+    if (!out) return ITAK_INVALID_ARGUMENT;
+    *out = pool ? pool->err.info : g_create_error.info;
+    return ITAK_OK;
+}
+
+itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out) {
+    ErrorState &e = g_create_error;
+    if (!out) return invalid_argument(e, "out is null");
+    *out = nullptr;
+    if (!config) return invalid_argument(e, "config is null");
+    // KvCache::new (cache.rs:327-351) and LayerCache::new (cache.rs:125-141).
+    if (config->layer_count == 0) return zero_dimension(e, "layer pattern");
+    if (config->num_kv_heads == 0) return zero_dimension(e, "num_kv_heads");
+    if (config->head_dim == 0) return zero_dimension(e, "head_dim");
+    bool any_windowed = false;
+    for (uint32_t i = 0; i < config->layer_count; ++i) {
+        if (config->layer_kinds && config->layer_kinds[i] == ITAK_LAYER_WINDOWED) {
+            any_windowed = true;
+            const uint64_t w = config->windows ? config->windows[i] : 0;
+            if (w == 0) return invalid_window(e, 0);
+        } else if (config->layer_kinds && config->layer_kinds[i] != ITAK_LAYER_GLOBAL) {
+            return invalid_argument(e, "unknown layer kind");
+        }
+    }
+    uint64_t row = 0;
+    if (__builtin_mul_overflow(config->num_kv_heads, config->head_dim, &row))
+        return size_overflow(e, "kv row length");
+    if (any_windowed) {
+        for (uint32_t i = 0; i < config->layer_count; ++i) {
+            if (config->layer_kinds[i] != ITAK_LAYER_WINDOWED) continue;
+            uint64_t slots = 0;
+            if (__builtin_mul_overflow(config->windows[i], row, &slots))
+                return size_overflow(e, "windowed layer storage");
+        }
+        return unsupported(e, "windowed (ring) layers have no device storage in this build");
+    }
+    if (config->elem != ITAK_ELEM_F32 && config->elem != ITAK_ELEM_F16)
+        return invalid_argument(e, "elem is neither ITAK_ELEM_F32 nor ITAK_ELEM_F16");
+    if (config->max_slots == 0) return zero_dimension(e, "max_slots");
+    if (config->capacity_rows == 0) return zero_dimension(e, "capacity_rows");
+    if (config->capacity_rows > (1ull << 30) || config->head_dim > (1u << 16) ||
+        config->num_kv_heads > (1u << 16))
+        return size_overflow(e, "global layer storage");
+    const uint64_t elem_bytes = config->elem == ITAK_ELEM_F16 ? 2 : 4;
+    uint64_t head_stride, side_stride, slot_stride, layer_stride, total, bytes;
+    if (__builtin_mul_overflow(config->capacity_rows, config->head_dim, &head_stride) ||
+        __builtin_mul_overflow(head_stride, config->num_kv_heads, &side_stride) ||
+        __builtin_mul_overflow(side_stride, uint64_t(2), &slot_stride) ||
+        __builtin_mul_overflow(slot_stride, uint64_t(config->max_slots), &layer_stride) ||
+        __builtin_mul_overflow(layer_stride, uint64_t(config->layer_count), &total) ||
+        __builtin_mul_overflow(total, elem_bytes, &bytes))
+        return size_overflow(e, "global layer storage");
+
+    hipError_t he = hipSetDevice(config->device);
+    if (he != hipSuccess) return hip_error(e, he, "select device");
+    itak_pool *pool = new itak_pool();
+    pool->cfg = *config;
+    pool->cfg.layer_kinds = nullptr;  // all global; the caller's arrays are not retained
+    pool->cfg.windows = nullptr;
+    pool->elem_f16 = config->elem == ITAK_ELEM_F16;
+    pool->elem_bytes = uint32_t(elem_bytes);
+    pool->row = row;
+    pool->g.kv_heads = uint32_t(config->num_kv_heads);
+    pool->g.head_dim = uint32_t(config->head_dim);
+    pool->g.capacity = uint32_t(config->capacity_rows);
+    pool->g.max_slots = config->max_slots;
+    pool->g.head_stride = head_stride;
+    pool->g.side_stride = side_stride;
+    pool->g.slot_stride = slot_stride;
+    pool->g.layer_stride = layer_stride;
+    pool->bytes = bytes;
+    he = hipMalloc(reinterpret_cast<void **>(&pool->base), bytes);
+    if (he != hipSuccess) {
+        delete pool;
+        return hip_error(e, he, "allocate KV pool");
+    }
+    // Fresh storage is all zero bytes, as the reference's ring storage is
+    // (cache.rs:139) and as the scrub guarantee needs.
+    he = hipMemset(pool->base, 0, bytes);
+    if (he != hipSuccess) {
+        (void)hipFree(pool->base);
+        delete pool;
+        return hip_error(e, he, "zero KV pool");
+    }
+    pool->slots.resize(config->max_slots);
+    *out = pool;
+    return ITAK_OK;
+}
+
+void itak_pool_destroy(itak_pool *pool) {
+    if (!pool) return;
+    (void)hipStreamSynchronize(pool->stream);
+    if (pool->base) (void)hipFree(pool->base);
+    if (pool->stage) (void)hipFree(pool->stage);
+    if (pool->ws) (void)hipFree(pool->ws);
+    if (pool->counters) (void)hipFree(pool->counters);
+    delete pool;
+}
+
+itak_status itak_pool_set_stream(itak_pool *pool, void *hip_stream) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize the previous stream");
+    pool->stream = static_cast<hipStream_t>(hip_stream);
+    return ITAK_OK;
+}
+
+itak_status itak_pool_synchronize(itak_pool *pool) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize");
+    return ITAK_OK;
+}
+
+uint64_t itak_pool_device_bytes(const itak_pool *pool) { return pool ? pool->bytes : 0; }
+
+itak_status itak_slot_acquire(itak_pool *pool, uint32_t *slot) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (!slot) return invalid_argument(pool->err, "slot is null");
+    for (uint32_t i = 0; i < pool->slots.size(); ++i) {
+        Slot &s = pool->slots[i];
+        if (s.in_use) continue;
+        s = Slot{};
+        s.in_use = true;
+        s.cache_id = g_next_cache_id++;
+        s.appended.assign(pool->cfg.layer_count, 0);
+        *slot = i;
+        return ITAK_OK;
+    }
+    return set_error(pool->err, ITAK_NO_FREE_SLOT, nullptr, pool->slots.size(), 0, 0, 0,
+                     "all %llu slots of the pool are in use", ULL(pool->slots.size()));
+}
+
+itak_status itak_slot_reset(itak_pool *pool, uint32_t slot) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    uint64_t max_rows = 0;
+    for (uint64_t a : s->appended) max_rows = std::max(max_rows, a);
+    if (max_rows > 0) {
+        ZeroBatch zb{};
+        zb.n = 1;
+        zb.max_rows = uint32_t(max_rows);
+        zb.item[0] = ZeroItem{slot, 0, uint32_t(max_rows), 0};
+        itak_status st = scrub_rows(pool, zb);
+        if (st != ITAK_OK) return st;
+    }
+    std::fill(s->appended.begin(), s->appended.end(), 0);
+    s->built = false;
+    s->cp = LiveCheckpoint{};
+    s->next_serial = 0;
+    s->cache_id = g_next_cache_id++;  // outstanding handles go stale (cache.rs:721-728)
+    return ITAK_OK;
+}
+
+itak_status itak_slot_release(itak_pool *pool, uint32_t slot) {
+    itak_status st = itak_slot_reset(pool, slot);
+    if (st != ITAK_OK) return st;
+    pool->slots[slot].in_use = false;
+    return ITAK_OK;
+}
+
+uint64_t itak_kv_layer_count(const itak_pool *pool) { return pool ? pool->cfg.layer_count : 0; }
+uint64_t itak_kv_num_kv_heads(const itak_pool *pool) { return pool ? pool->g.kv_heads : 0; }
+uint64_t itak_kv_head_dim(const itak_pool *pool) { return pool ? pool->g.head_dim : 0; }
+
+itak_status itak_kv_layer_kind(itak_pool *pool, uint64_t layer, uint32_t *kind, uint64_t *window) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
+    if (kind) *kind = ITAK_LAYER_GLOBAL;
+    if (window) *window = 0;
+    return ITAK_OK;
+}
+
+itak_status itak_kv_stored_len(itak_pool *pool, uint32_t slot, uint64_t layer, uint64_t *out) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
+    *out = s->appended[layer];  // global layer: stored == appended (cache.rs:154-159)
+    return ITAK_OK;
+}
+
+itak_status itak_kv_next_position(itak_pool *pool, uint32_t slot, uint64_t layer, uint64_t *out) {
+    return itak_kv_stored_len(pool, slot, layer, out);
+}
+
+itak_status itak_kv_append(itak_pool *pool, uint32_t slot, uint64_t layer, const float *k,
+                           uint64_t k_len, const float *v, uint64_t v_len, uint64_t position) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    // cache.rs:430-471, in order.
+    if (k_len != pool->row) return shape_mismatch(pool->err, "k", pool->row, k_len);
+    if (v_len != pool->row) return shape_mismatch(pool->err, "v", pool->row, v_len);
+    if (s->cp.live && layer < pool->cfg.layer_count) {
+        const uint64_t limit = s->cp.bases[layer] + s->cp.max_round_tokens;
+        if (position >= limit) return range_exceeded(pool->err, layer, position, limit);
+    }
+    if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
+    if (position != s->appended[layer])
+        return out_of_order(pool->err, layer, s->appended[layer], position);
+    if (position >= pool->g.capacity)
+        return capacity_exceeded(pool->err, layer, position + 1, pool->g.capacity);
+    if (!k || !v) return invalid_argument(pool->err, "k or v is null");
+    const uint64_t bytes = pool->row * sizeof(float);
+    itak_status st = ensure_stage(pool, 2 * bytes);
+    if (st != ITAK_OK) return st;
+    float *kd = reinterpret_cast<float *>(pool->stage);
+    float *vd = kd + pool->row;
+    HIP_TRY(pool, hipMemcpyAsync(kd, k, bytes, hipMemcpyHostToDevice, pool->stream), "upload k");
+    HIP_TRY(pool, hipMemcpyAsync(vd, v, bytes, hipMemcpyHostToDevice, pool->stream), "upload v");
+    itak_batch_item item{slot, 1};
+    st = run_append(pool, layer, &item, 1, kd, vd);
+    if (st != ITAK_OK) return st;
+    HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after append");
+    return ITAK_OK;
+}
+
+itak_status itak_kv_append_device(itak_pool *pool, uint64_t layer, const itak_batch_item *items,
+                                  uint32_t item_count, const float *k_dev, const float *v_dev) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
+    if (item_count && (!items || !k_dev || !v_dev))
+        return invalid_argument(pool->err, "items, k_dev or v_dev is null");
+    std::vector<uint8_t> seen(pool->slots.size(), 0);
+    for (uint32_t i = 0; i < item_count; ++i) {
+        Slot *s = find_slot(pool, items[i].slot);
+        if (!s) return invalid_argument(pool->err, "slot is not in use");
+        if (seen[items[i].slot]++) return invalid_argument(pool->err, "slot listed twice in one step");
+        uint64_t ok = 0;
+        itak_status st = check_append_rows(pool, *s, layer, items[i].rows, &ok);
+        if (st != ITAK_OK) return st;
+    }
+    return run_append(pool, layer, items, item_count, k_dev, v_dev);
+}
+
+static itak_status restore_layers(itak_pool *pool, uint32_t slot, Slot &s,
+                                  const itak_snapshot_layer *layers, const uint64_t *layer_ids,
+                                  uint64_t count, uint32_t src_elem) {
+    if (src_elem != ITAK_ELEM_F32 && src_elem != ITAK_ELEM_F16)
+        return invalid_argument(pool->err, "src_elem is neither ITAK_ELEM_F32 nor ITAK_ELEM_F16");
+    if (src_elem == ITAK_ELEM_F16 && !pool->elem_f16)
+        return unsupported(pool->err, "an f16 snapshot restores only into an f16 pool");
+    const uint64_t src_bytes_per_elem = src_elem == ITAK_ELEM_F16 ? 2 : 4;
+    // Sources the device cannot read in place are staged through one temporary buffer.
+    uint64_t stage_need = 0;
+    for (uint64_t i = 0; i < count; ++i) {
+        if (layers[i].rows == 0) continue;
+        const uint64_t bytes = layers[i].rows * pool->row * src_bytes_per_elem;
+        const void *unused;
+        if (classify(layers[i].keys, &unused) == PtrKind::PlainHost) stage_need += align_up(bytes, 256);
+        if (classify(layers[i].values, &unused) == PtrKind::PlainHost) stage_need += align_up(bytes, 256);
+    }
+    unsigned char *temp = nullptr;
+    if (stage_need) HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&temp), stage_need), "allocate restore staging");
+    uint64_t temp_off = 0;
+    itak_status st = ITAK_OK;
+    for (uint64_t first = 0; first < count && st == ITAK_OK; first += kMaxRestoreLayers) {
+        const uint64_t n = std::min<uint64_t>(kMaxRestoreLayers, count - first);
+        RestoreBatch b{};
+        b.slot = slot;
+        for (uint64_t i = 0; i < n; ++i) {
+            const itak_snapshot_layer &L = layers[first + i];
+            if (L.rows == 0) continue;
+            const uint64_t bytes = L.rows * pool->row * src_bytes_per_elem;
+            const void *src[2] = {L.keys, L.values};
+            for (int side = 0; side < 2; ++side) {
+                const void *usable;
+                if (classify(src[side], &usable) != PtrKind::PlainHost) {
+                    src[side] = usable;
+                    continue;
+                }
+                hipError_t he = hipMemcpyAsync(temp + temp_off, src[side], bytes,
+                                               hipMemcpyHostToDevice, pool->stream);
+                if (he != hipSuccess) {
+                    st = hip_error(pool->err, he, "stage snapshot rows");
+                    break;
+                }
+                src[side] = temp + temp_off;
+                temp_off += align_up(bytes, 256);
+            }
+            if (st != ITAK_OK) break;
+            RestoreLayer &R = b.layer[b.n++];
+            R.keys = src[0];
+            R.values = src[1];
+            R.layer = uint32_t(layer_ids ? layer_ids[first + i] : first + i);
+            R.rows = uint32_t(L.rows);
+            R.first_row = uint32_t(L.first_position);  // global layer: slot_of(p) == p
+            b.max_rows = std::max(b.max_rows, R.rows);
+        }
+        if (st != ITAK_OK) break;
+        hipError_t he = launch_restore(pool->base, pool->elem_f16, src_elem == ITAK_ELEM_F16,
+                                       pool->g, b, pool->stream);
+        if (he != hipSuccess) st = hip_error(pool->err, he, "launch restore gather");
+    }
+    hipError_t he = hipStreamSynchronize(pool->stream);
+    if (st == ITAK_OK && he != hipSuccess) st = hip_error(pool->err, he, "synchronize after restore");
+    if (temp) (void)hipFree(temp);
+    if (st != ITAK_OK) return st;
+    for (uint64_t i = 0; i < count; ++i) {
+        const uint64_t layer = layer_ids ? layer_ids[i] : i;
+        s.appended[layer] = layers[i].first_position + layers[i].rows;  // cache.rs:568
+    }
+    return ITAK_OK;
+}
+
+itak_status itak_kv_restore_bulk(itak_pool *pool, uint32_t slot, uint64_t layer,
+                                 uint64_t first_position, const void *keys, uint64_t keys_len,
+                                 const void *values, uint64_t values_len, uint32_t src_elem) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    // cache.rs:520-546, in order.
+    if (keys_len != values_len || keys_len % pool->row != 0)
+        return shape_mismatch(pool->err, "bulk restore rows", values_len, keys_len);
+    const uint64_t rows = keys_len / pool->row;
+    if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
+    if (s->appended[layer] != 0) return not_fresh(pool->err, layer, s->appended[layer]);
+    if (first_position != 0)
+        return shape_mismatch(pool->err, "bulk restore first position (global layer)", 0,
+                              first_position);
+    if (rows > pool->g.capacity) return capacity_exceeded(pool->err, layer, rows, pool->g.capacity);
+    if (rows && (!keys || !values)) return invalid_argument(pool->err, "keys or values is null");
+    itak_snapshot_layer L{first_position, rows, keys, values};
+    return restore_layers(pool, slot, *s, &L, &layer, 1, src_elem);
+}
+
+itak_status itak_kv_restore_snapshot(itak_pool *pool, uint32_t slot, uint64_t token_count,
+                                     const itak_snapshot_layer *layers, uint64_t layer_count,
+                                     uint32_t src_elem) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    if (!layers) return invalid_argument(pool->err, "layers is null");
+    // KvSnapshot::validate (snapshot.rs:187-236) for an all-global geometry.
+    if (layer_count != pool->cfg.layer_count)
+        return set_error(pool->err, ITAK_STEP_FAILED, "restore_snapshot", layer_count,
+                         pool->cfg.layer_count, 0, 0,
+                         "snapshot carries %llu layer blocks but its geometry has %llu layers",
+                         ULL(layer_count), ULL(pool->cfg.layer_count));
+    for (uint64_t i = 0; i < layer_count; ++i) {
+        if (layers[i].first_position != 0)
+            return set_error(pool->err, ITAK_STEP_FAILED, "restore_snapshot", i,
+                             layers[i].first_position, 0, 0,
+                             "layer %llu: first stored position is %llu but 0 follows from token "
+                             "count %llu and kind Global",
+                             ULL(i), ULL(layers[i].first_position), ULL(token_count));
+        if (layers[i].rows != token_count)
+            return set_error(pool->err, ITAK_STEP_FAILED, "restore_snapshot", i, layers[i].rows,
+                             token_count, 0,
+                             "layer %llu: holds %llu rows but %llu rows were expected", ULL(i),
+                             ULL(layers[i].rows), ULL(token_count));
+        if (token_count && (!layers[i].keys || !layers[i].values))
+            return invalid_argument(pool->err, "a layer's keys or values is null");
+    }
+    // KvSnapshot::restore builds a fresh cache (snapshot.rs:321-334): every layer must be
+    // fresh here, checked for all layers before any is touched.
+    for (uint64_t i = 0; i < layer_count; ++i)
+        if (s->appended[i] != 0) return not_fresh(pool->err, i, s->appended[i]);
+    if (token_count > pool->g.capacity)
+        return capacity_exceeded(pool->err, 0, token_count, pool->g.capacity);
+    return restore_layers(pool, slot, *s, layers, nullptr, layer_count, src_elem);
+}
+
+itak_status itak_kv_stats(itak_pool *pool, uint32_t slot, itak_layer_stats *out) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    if (!out) return invalid_argument(pool->err, "out is null");
+    for (uint32_t i = 0; i < pool->cfg.layer_count; ++i) {
+        out[i] = itak_layer_stats{i, ITAK_LAYER_GLOBAL, 0, 0, s->appended[i], s->appended[i]};
+    }
+    return ITAK_OK;
+}
+
+static itak_status read_rows_common(itak_pool *pool, uint32_t slot, uint64_t layer, uint64_t first,
+                                    uint64_t rows, void *keys_out, void *values_out) {
+    if (rows == 0 || (!keys_out && !values_out)) return ITAK_OK;
+    const uint64_t bytes = rows * pool->row * pool->elem_bytes;
+    itak_status st = ensure_stage(pool, 2 * align_up(bytes, 256));
+    if (st != ITAK_OK) return st;
+    void *kd = keys_out ? pool->stage : nullptr;
+    void *vd = values_out ? pool->stage + align_up(bytes, 256) : nullptr;
+    HIP_TRY(pool,
+            launch_read_rows(layer_base(pool, layer), pool->elem_f16, pool->g, slot,
+                             uint32_t(first), uint32_t(rows), kd, vd, pool->stream),
+            "launch row readback");
+    if (keys_out)
+        HIP_TRY(pool, hipMemcpyAsync(keys_out, kd, bytes, hipMemcpyDeviceToHost, pool->stream),
+                "download keys");
+    if (values_out)
+        HIP_TRY(pool, hipMemcpyAsync(values_out, vd, bytes, hipMemcpyDeviceToHost, pool->stream),
+                "download values");
+    HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after readback");
+    return ITAK_OK;
+}
+
+itak_status itak_kv_read_rows(itak_pool *pool, uint32_t slot, uint64_t layer, uint64_t first,
+                              uint64_t rows, void *keys_out, void *values_out,
+                              uint64_t *positions_out) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
+    const uint64_t stored = s->appended[layer];
+    if (first > stored || rows > stored - first)
+        return shape_mismatch(pool->err, "visible rows", stored, first + rows);
+    if (positions_out)
+        for (uint64_t i = 0; i < rows; ++i) positions_out[i] = first + i;  // cache.rs:878-883
+    return read_rows_common(pool, slot, layer, first, rows, keys_out, values_out);
+}
+
+itak_status itak_kv_read_raw(itak_pool *pool, uint32_t slot, uint64_t layer, void *keys_out,
+                             void *values_out) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
+    return read_rows_common(pool, slot, layer, 0, pool->g.capacity, keys_out, values_out);
+}
+
+itak_status itak_kv_checkpoint_active(itak_pool *pool, uint32_t slot, int32_t *out) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    *out = s->cp.live ? 1 : 0;
+    return ITAK_OK;
+}
+
+itak_status itak_kv_checkpoint(itak_pool *pool, uint32_t slot, uint64_t max_round_tokens,
+                               itak_checkpoint *out) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    if (!out) return invalid_argument(pool->err, "out is null");
+    // cache.rs:635-651; with no windowed layer there is no CheckpointTooDeep bound.
+    if (s->cp.live) return checkpoint_busy(pool->err);
+    if (max_round_tokens == 0) return zero_dimension(pool->err, "max_round_tokens");
+    s->next_serial += 1;
+    s->cp.live = true;
+    s->cp.serial = s->next_serial;
+    s->cp.max_round_tokens = max_round_tokens;
+    s->cp.bases = s->appended;
+    out->cache_id = s->cache_id;
+    out->serial = s->cp.serial;
+    out->max_round_tokens = max_round_tokens;
+    out->saved_bytes = 0;  // global layers save no rows: rewind is truncation (cache.rs:675-677)
+    return ITAK_OK;
+}
+
+static itak_status live_data(itak_pool *pool, Slot &s, const itak_checkpoint *cp) {
+    if (!cp) return invalid_argument(pool->err, "checkpoint is null");
+    if (s.cp.live && s.cp.serial == cp->serial && cp->cache_id == s.cache_id) return ITAK_OK;
+    return stale_checkpoint(pool->err, cp->serial);  // cache.rs:721-728
+}
+
+itak_status itak_kv_checkpoint_bases(itak_pool *pool, uint32_t slot, const itak_checkpoint *cp,
+                                     uint64_t *out) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    itak_status st = live_data(pool, *s, cp);
+    if (st != ITAK_OK) return st;
+    std::copy(s->cp.bases.begin(), s->cp.bases.end(), out);
+    return ITAK_OK;
+}
+
+// Drops positions >= target on every layer of the slot (the caller validated the range).
+static itak_status truncate_slots(itak_pool *pool, const uint32_t *slots, const uint64_t *targets,
+                                  uint32_t count) {
+    if (pool->cfg.flags & ITAK_POOL_SCRUB_ON_TRUNCATE) {
+        for (uint32_t first = 0; first < count; first += kMaxBatchItems) {
+            const uint32_t n = std::min<uint32_t>(kMaxBatchItems, count - first);
+            ZeroBatch zb{};
+            for (uint32_t i = 0; i < n; ++i) {
+                const Slot &s = pool->slots[slots[first + i]];
+                uint64_t max_len = 0;
+                for (uint64_t a : s.appended) max_len = std::max(max_len, a);
+                if (max_len <= targets[first + i]) continue;
+                zb.item[zb.n++] = ZeroItem{slots[first + i], uint32_t(targets[first + i]),
+                                           uint32_t(max_len), 0};
+                zb.max_rows = std::max<uint32_t>(zb.max_rows, uint32_t(max_len - targets[first + i]));
+            }
+            itak_status st = scrub_rows(pool, zb);
+            if (st != ITAK_OK) return st;
+        }
+    }
+    for (uint32_t i = 0; i < count; ++i) {
+        Slot &s = pool->slots[slots[i]];
+        for (uint64_t &a : s.appended) a = std::min(a, targets[i]);  // cache.rs:788-791,814
+    }
+    return ITAK_OK;
+}
+
+itak_status itak_kv_rewind_to(itak_pool *pool, uint32_t slot, const itak_checkpoint *cp,
+                              uint64_t target) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    itak_status st = live_data(pool, *s, cp);
+    if (st != ITAK_OK) return st;
+    // Validate every layer before touching any (cache.rs:772-783).
+    for (uint64_t li = 0; li < s->appended.size(); ++li) {
+        const uint64_t base = s->cp.bases[li];
+        if (target < base || target > s->appended[li])
+            return rewind_range(pool->err, li, base, s->appended[li], target);
+    }
+    return truncate_slots(pool, &slot, &target, 1);
+}
+
+itak_status itak_kv_release(itak_pool *pool, uint32_t slot, const itak_checkpoint *cp) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    itak_status st = live_data(pool, *s, cp);
+    if (st != ITAK_OK) return st;
+    s->cp.live = false;  // cache.rs:824-833
+    return ITAK_OK;
+}
+
+itak_status itak_kv_truncate(itak_pool *pool, const uint32_t *slots, const uint64_t *new_lengths,
+                             uint32_t count) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (count && (!slots || !new_lengths))
+        return invalid_argument(pool->err, "slots or new_lengths is null");
+    for (uint32_t i = 0; i < count; ++i) {
+        Slot *s = find_slot(pool, slots[i]);
+        if (!s) return invalid_argument(pool->err, "slot is not in use");
+        if (s->cp.live) return checkpoint_busy(pool->err);
+        for (uint64_t li = 0; li < s->appended.size(); ++li)
+            if (new_lengths[i] > s->appended[li])
+                return rewind_range(pool->err, li, 0, s->appended[li], new_lengths[i]);
+    }
+    return truncate_slots(pool, slots, new_lengths, count);
+}
+
+itak_status itak_gqa_attention(itak_pool *pool, uint32_t slot, uint64_t layer, const float *q,
+                               uint64_t q_len, uint64_t num_queries, uint64_t num_q_heads,
+                               const uint64_t *query_positions, uint64_t positions_len,
+                               float scale, float softcap, float *out) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
+    // attention.rs:115-146, in order.
+    if (positions_len != num_queries)
+        return shape_mismatch(pool->err, "query_positions", num_queries, positions_len);
+    const uint64_t expected_q = num_queries * num_q_heads * pool->g.head_dim;
+    if (q_len != expected_q) return shape_mismatch(pool->err, "q", expected_q, q_len);
+    if (num_queries == 0) return ITAK_OK;
+    if (num_q_heads == 0) return zero_dimension(pool->err, "num_q_heads");
+    if (num_q_heads % pool->g.kv_heads != 0)
+        return non_divisible(pool->err, num_q_heads, pool->g.kv_heads);
+    if (!q || !out || !query_positions)
+        return invalid_argument(pool->err, "q, out or query_positions is null");
+    const uint64_t stored = s->appended[layer];
+    // A global layer's view holds positions 0..stored: a query sees at least position 0
+    // unless the view is empty (attention.rs:160-173).
+    if (stored == 0) return no_visible_keys(pool->err, query_positions[0]);
+    if (std::isnan(scale)) scale = default_scale(pool->g.head_dim);
+
+    bool consecutive = true;
+    for (uint64_t i = 1; i < num_queries; ++i)
+        consecutive = consecutive && query_positions[i] == query_positions[0] + i;
+    const uint64_t q_bytes = q_len * sizeof(float);
+    const uint64_t pos_bytes = align_up(num_queries * sizeof(uint32_t), 256);
+    itak_status st = ensure_stage(pool, 2 * align_up(q_bytes, 256) + pos_bytes);
+    if (st != ITAK_OK) return st;
+    float *qd = reinterpret_cast<float *>(pool->stage);
+    float *od = reinterpret_cast<float *>(pool->stage + align_up(q_bytes, 256));
+    uint32_t *pd = reinterpret_cast<uint32_t *>(pool->stage + 2 * align_up(q_bytes, 256));
+    HIP_TRY(pool, hipMemcpyAsync(qd, q, q_bytes, hipMemcpyHostToDevice, pool->stream), "upload q");
+    std::vector<uint32_t> pos32;
+    if (!consecutive) {
+        pos32.resize(num_queries);
+        for (uint64_t i = 0; i < num_queries; ++i)
+            pos32[i] = uint32_t(std::min<uint64_t>(query_positions[i], 0xffffffffu));
+        HIP_TRY(pool,
+                hipMemcpyAsync(pd, pos32.data(), num_queries * 4, hipMemcpyHostToDevice,
+                               pool->stream),
+                "upload query positions");
+    }
+    PlanInput pi{slot, uint32_t(num_queries),
+                 uint32_t(std::min<uint64_t>(query_positions[0], 0xffffffffu - num_queries)),
+                 uint32_t(stored)};
+    st = run_attention(pool, layer, &pi, 1, qd, od, consecutive ? nullptr : pd, num_q_heads, scale,
+                       softcap);
+    if (st != ITAK_OK) return st;
+    HIP_TRY(pool, hipMemcpyAsync(out, od, q_bytes, hipMemcpyDeviceToHost, pool->stream),
+            "download attention output");
+    HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after attention");
+    return ITAK_OK;
+}
+
+// Validates one batched step and returns the per-item plan (positions before the append).
+static itak_status plan_step(itak_pool *pool, uint64_t layer, const itak_batch_item *items,
+                             uint32_t item_count, uint64_t num_q_heads,
+                             std::vector<PlanInput> &plan) {
+    if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
+    if (num_q_heads == 0) return zero_dimension(pool->err, "num_q_heads");
+    if (num_q_heads % pool->g.kv_heads != 0)
+        return non_divisible(pool->err, num_q_heads, pool->g.kv_heads);
+    std::vector<uint8_t> seen(pool->slots.size(), 0);
+    plan.clear();
+    for (uint32_t i = 0; i < item_count; ++i) {
+        Slot *s = find_slot(pool, items[i].slot);
+        if (!s) return invalid_argument(pool->err, "slot is not in use");
+        if (seen[items[i].slot]++) return invalid_argument(pool->err, "slot listed twice in one step");
+        uint64_t ok = 0;
+        itak_status st = check_append_rows(pool, *s, layer, items[i].rows, &ok);
+        if (st != ITAK_OK) return st;
+        const uint64_t base = s->appended[layer];
+        plan.push_back(PlanInput{items[i].slot, items[i].rows, uint32_t(base),
+                                 uint32_t(base + items[i].rows)});
+    }
+    return ITAK_OK;
+}
+
+itak_status itak_attention_step_device(itak_pool *pool, uint64_t layer,
+                                       const itak_batch_item *items, uint32_t item_count,
+                                       const float *q_dev, const float *k_dev, const float *v_dev,
+                                       float *out_dev, uint64_t num_q_heads, float scale,
+                                       float softcap) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (item_count == 0) return ITAK_OK;
+    if (!items || !q_dev || !k_dev || !v_dev || !out_dev)
+        return invalid_argument(pool->err, "items or a device tensor is null");
+    std::vector<PlanInput> plan;
+    itak_status st = plan_step(pool, layer, items, item_count, num_q_heads, plan);
+    if (st != ITAK_OK) return st;
+    if (std::isnan(scale)) scale = default_scale(pool->g.head_dim);
+    st = run_append(pool, layer, items, item_count, k_dev, v_dev);
+    if (st != ITAK_OK) return st;
+    // Rows of zero-row items contribute nothing.
+    std::vector<PlanInput> active;
+    for (const PlanInput &p : plan)
+        if (p.rows) active.push_back(p);
+    // run_attention numbers q rows by walking the items in order, so zero-row items may
+    // simply be dropped.
+    return run_attention(pool, layer, active.data(), uint32_t(active.size()), q_dev, out_dev,
+                         nullptr, num_q_heads, scale, softcap);
+}
+
+itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t layer, const float *q,
+                                   uint64_t q_len, const float *k, uint64_t k_len, const float *v,
+                                   uint64_t v_len, uint64_t num_q_heads, uint64_t cache_position,
+                                   float softcap, float *out) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    const char *step = "attention";
+    // cpu.rs:529-556: whole rows, matching K/V row counts.
+    const uint64_t q_width = num_q_heads * pool->g.head_dim;
+    if (q_width == 0 || q_len % q_width != 0)
+        return set_error(pool->err, ITAK_STEP_FAILED, step, q_len, q_width, 0, 0,
+                         "query projection holds %llu elements, not a whole number of "
+                         "%llu-wide rows",
+                         ULL(q_len), ULL(q_width));
+    const uint64_t rows = q_len / q_width;
+    if (k_len != rows * pool->row || v_len != rows * pool->row)
+        return set_error(pool->err, ITAK_STEP_FAILED, step, k_len, v_len, rows * pool->row, 0,
+                         "key/value projections hold %llu/%llu elements for %llu rows, expected "
+                         "%llu/%llu",
+                         ULL(k_len), ULL(v_len), ULL(rows), ULL(rows * pool->row),
+                         ULL(rows * pool->row));
+    if (layer >= pool->cfg.layer_count) {
+        invalid_layer(pool->err, layer, pool->cfg.layer_count);
+        pool->err.info.code = ITAK_STEP_FAILED;  // forwarded as StepFailed text (cpu.rs:565-568)
+        return ITAK_STEP_FAILED;
+    }
+    s->built = true;  // KvState::build on first use (cpu.rs:560-564)
+    const uint64_t appended = s->appended[layer];
+    if (appended != cache_position)  // cpu.rs:569-581
+        return set_error(pool->err, ITAK_STEP_FAILED, step, layer, appended, cache_position, 0,
+                         "KV state for layer %llu is at position %llu but the sequence cache is "
+                         "at position %llu: the two disagree, so attending would read the wrong "
+                         "history. Pair one Cache with one compute slot per sequence, or reset "
+                         "the slot when a sequence is abandoned (a forward that failed midway "
+                         "leaves the KV state ahead of the cache and also needs a reset)",
+                         ULL(layer), ULL(appended), ULL(cache_position));
+    if (rows == 0) return ITAK_OK;
+    if (num_q_heads % pool->g.kv_heads != 0) {
+        non_divisible(pool->err, num_q_heads, pool->g.kv_heads);
+        pool->err.info.code = ITAK_STEP_FAILED;
+        return ITAK_STEP_FAILED;
+    }
+    if (!q || !k || !v || !out) return invalid_argument(pool->err, "q, k, v or out is null");
+
+    // Row-at-a-time appends stop at the first refusal (cpu.rs:623-631): rows before it are
+    // in the cache when the call fails, exactly as in the reference.
+    uint64_t ok_rows = rows;
+    itak_status refusal = check_append_rows(pool, *s, layer, rows, &ok_rows);
+    ErrorState saved = pool->err;
+
+    const uint64_t q_bytes = align_up(q_len * sizeof(float), 256);
+    const uint64_t kv_bytes = align_up(k_len * sizeof(float), 256);
+    itak_status st = ensure_stage(pool, 2 * q_bytes + 2 * kv_bytes);
+    if (st != ITAK_OK) return st;
+    float *qd = reinterpret_cast<float *>(pool->stage);
+    float *od = reinterpret_cast<float *>(pool->stage + q_bytes);
+    float *kd = reinterpret_cast<float *>(pool->stage + 2 * q_bytes);
+    float *vd = reinterpret_cast<float *>(pool->stage + 2 * q_bytes + kv_bytes);
+    HIP_TRY(pool, hipMemcpyAsync(kd, k, k_len * 4, hipMemcpyHostToDevice, pool->stream), "upload k");
+    HIP_TRY(pool, hipMemcpyAsync(vd, v, v_len * 4, hipMemcpyHostToDevice, pool->stream), "upload v");
+    itak_batch_item item{slot, uint32_t(ok_rows)};
+    st = run_append(pool, layer, &item, 1, kd, vd);
+    if (st != ITAK_OK) return st;
+    if (refusal != ITAK_OK) {
+        HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after append");
+        pool->err = saved;
+        pool->err.info.code = ITAK_STEP_FAILED;
+        return ITAK_STEP_FAILED;
+    }
+    HIP_TRY(pool, hipMemcpyAsync(qd, q, q_len * 4, hipMemcpyHostToDevice, pool->stream), "upload q");
+    PlanInput pi{slot, uint32_t(rows), uint32_t(appended), uint32_t(appended + rows)};
+    st = run_attention(pool, layer, &pi, 1, qd, od, nullptr, num_q_heads,
+                       default_scale(pool->g.head_dim), softcap);  // AttentionParams::new(), cpu.rs:584
+    if (st != ITAK_OK) return st;
+    HIP_TRY(pool, hipMemcpyAsync(out, od, q_len * 4, hipMemcpyDeviceToHost, pool->stream),
+            "download attention output");
+    HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after attention");
+    return ITAK_OK;
+}
+
+static itak_status no_kv_state(itak_pool *pool, const char *step, const char *detail) {
+    return set_error(pool->err, ITAK_STEP_FAILED, step, 0, 0, 0, 0, "%s", detail);
+}
+
+static itak_status as_step_failed(itak_pool *pool, itak_status st) {
+    if (st == ITAK_OK) return st;
+    pool->err.info.code = ITAK_STEP_FAILED;  // map_err(step_failed(...)) in cpu.rs:292-294
+    return ITAK_STEP_FAILED;
+}
+
+itak_status itak_compute_cache_checkpoint(itak_pool *pool, uint32_t slot,
+                                          uint64_t max_round_tokens, itak_checkpoint *out) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    if (!s->built)  // cpu.rs:284-290
+        return no_kv_state(pool, "cache_checkpoint",
+                           "no KV state exists yet: a speculative round checkpoints after a first "
+                           "forward has built the cache (the spec's prefill), not before");
+    return as_step_failed(pool, itak_kv_checkpoint(pool, slot, max_round_tokens, out));
+}
+
+itak_status itak_compute_cache_rewind(itak_pool *pool, uint32_t slot, const itak_checkpoint *cp,
+                                      uint64_t target) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    if (!s->built)  // cpu.rs:311-317
+        return no_kv_state(pool, "cache_rewind",
+                           "no KV state exists: the sequence was reset after the checkpoint was "
+                           "taken");
+    return as_step_failed(pool, itak_kv_rewind_to(pool, slot, cp, target));
+}
+
+itak_status itak_compute_cache_release(itak_pool *pool, uint32_t slot, const itak_checkpoint *cp) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    if (!s->built)  // cpu.rs:327-333
+        return no_kv_state(pool, "cache_release",
+                           "no KV state exists: the sequence was reset after the checkpoint was "
+                           "taken");
+    return as_step_failed(pool, itak_kv_release(pool, slot, cp));
+}
+
+itak_status itak_convert_f32_to_f16_device(itak_pool *pool, const float *src_dev,
+                                           uint16_t *dst_dev, uint64_t count) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (count && (!src_dev || !dst_dev)) return invalid_argument(pool->err, "src or dst is null");
+    HIP_TRY(pool, launch_convert_f16(src_dev, dst_dev, count, pool->stream), "launch conversion");
+    return ITAK_OK;
+}
+
+}  // extern "C"

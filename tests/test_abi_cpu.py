@@ -1,0 +1,112 @@
+"""CPU-only checks of the C ABI: the library loads, exports exactly what the header
+declares, and refuses bad construction arguments by name without touching a GPU."""
+import ctypes as C
+import subprocess
+
+import pytest
+
+from helpers import declared_symbols, pkg
+
+
+def test_library_exports_every_declared_symbol():
+    N = pkg()._native
+    lib = N.load()
+    declared = declared_symbols()
+    assert len(declared) >= 30
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+    assert sorted(N.PROTOTYPES) == declared, "binding table and header disagree"
+    out = subprocess.check_output(["nm", "-D", "--defined-only", N.LIB_PATH], text=True)
+    exported = sorted(l.split()[-1] for l in out.splitlines() if " T itak_" in l)
+    assert exported == declared
+    assert lib.itak_abi_version() == 1
+
+
+def test_library_does_not_link_the_oracle():
+    N = pkg()._native
+    out = subprocess.check_output(["ldd", N.LIB_PATH], text=True)
+    assert "oracle" not in out
+    syms = subprocess.check_output(["nm", "-D", N.LIB_PATH], text=True)
+    assert "orc_" not in syms
+
+
+def _create(**kw):
+    N = pkg()._native
+    lib = N.load()
+    cfg = N.PoolConfig()
+    cfg.layer_count = kw.get("layers", 1)
+    cfg.num_kv_heads = kw.get("kv_heads", 2)
+    cfg.head_dim = kw.get("head_dim", 128)
+    cfg.elem = kw.get("elem", N.ELEM_F32)
+    cfg.max_slots = kw.get("max_slots", 1)
+    cfg.capacity_rows = kw.get("capacity", 16)
+    kinds = kw.get("kinds")
+    windows = kw.get("windows")
+    keep = []
+    if kinds is not None:
+        arr = (C.c_uint8 * len(kinds))(*kinds)
+        keep.append(arr)
+        cfg.layer_kinds = C.cast(arr, C.c_void_p)
+    if windows is not None:
+        arr = (C.c_uint64 * len(windows))(*windows)
+        keep.append(arr)
+        cfg.windows = C.cast(arr, C.c_void_p)
+    handle = C.c_void_p()
+    status = lib.itak_pool_create(C.byref(cfg), C.byref(handle))
+    info = N.ErrorInfo()
+    lib.itak_last_error_info(None, C.byref(info))
+    return status, info, (lib.itak_last_error(None) or b"").decode(), handle
+
+
+def test_construction_refusals_need_no_gpu():
+    # The refusals of KvCache::new (crates/attention/tests/cache_tests.rs:133-183).
+    status, info, msg, _ = _create(layers=0)
+    assert (status, info.what) == (1, b"layer pattern")
+    assert msg == "layer pattern must be positive, got 0"
+    status, info, _, _ = _create(kv_heads=0)
+    assert (status, info.what) == (1, b"num_kv_heads")
+    status, info, _, _ = _create(head_dim=0)
+    assert (status, info.what) == (1, b"head_dim")
+    status, info, msg, _ = _create(kinds=[1], windows=[0])
+    assert status == 2 and msg == "sliding window must be positive, got 0"
+    status, info, _, _ = _create(kinds=[1], windows=[2**64 - 1])
+    assert (status, info.what) == (3, b"windowed layer storage")
+    status, info, _, _ = _create(kv_heads=2**64 - 1, head_dim=2)
+    assert (status, info.what) == (3, b"kv row length")
+    # Ring layers have no device storage yet: refused by name, not half-built.
+    status, info, msg, _ = _create(kinds=[1], windows=[4])
+    assert status == 20 and "windowed" in msg
+    status, _, msg, _ = _create(elem=7)
+    assert status == 17
+
+
+def test_python_front_end_raises_named_errors_without_a_gpu():
+    P = pkg()
+    with pytest.raises(P.AttentionError) as e:
+        P.KvPool([], 2, 128)
+    assert e.value == P.AttentionError("ZeroDimension", what="layer pattern")
+    with pytest.raises(P.AttentionError) as e:
+        P.LayerKind.windowed(0)
+    assert e.value == P.AttentionError("InvalidWindow", window=0)
+    with pytest.raises(P.AttentionError) as e:
+        P.kv_head_for_query_head(0, 3, 2)
+    assert e.value == P.AttentionError("NonDivisibleHeads", num_q_heads=3, num_kv_heads=2)
+    for h in range(32):
+        assert P.kv_head_for_query_head(h, 32, 2) == (0 if h < 16 else 1)
+    assert abs(float(P.AttentionParams.new().scale_for(128)) - 0.08838835) < 1e-7
+    cache = P.PositionCache()
+    cache.advance(5)
+    cache.rewind_to(3)
+    assert cache.position() == 3
+
+
+def test_product_sources_never_reference_the_oracle():
+    import os
+
+    root = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                        "itak-torch-rebuild_amd")
+    for dirpath, _, files in os.walk(root):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "import oracle" not in text and "itak_oracle" not in text, f

@@ -1,0 +1,271 @@
+"""GQA attention on the GPU through the C ABI: the reference's attention cases
+(crates/attention/tests/attention_tests.rs) and the Compute::attention contract
+(crates/cpu-compute/src/cpu.rs:506-655, tests/forward_tests.rs), checked against the oracle.
+
+Tolerances: f32 KV outputs within 1e-5 of the oracle relative to the largest output
+magnitude; f16 KV outputs within 2e-3 max-abs of the oracle run over the same f16-rounded
+cache."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import max_abs, normal, pkg, rel_err
+
+pytestmark = pytest.mark.gpu
+
+F32_REL = 1e-5
+F16_ABS = 2e-3
+
+
+def P():
+    return pkg()
+
+
+def E(variant, **f):
+    return P().AttentionError(variant, **f)
+
+
+def both(kv_heads, head_dim, rows, elem="f32", layers=1, capacity=None):
+    """The same rows appended to a GPU cache and to the oracle."""
+    cap = capacity or max(16, len(rows) + 8)
+    g = P().KvCache.new([P().LayerKind.Global] * layers, kv_heads, head_dim, elem=elem,
+                        capacity_rows=cap)
+    c = oracle.KvCache.new([oracle.LayerKind.Global] * layers, kv_heads, head_dim,
+                           store_f16=(elem == "f16"))
+    if len(rows):
+        k = np.stack([np.asarray(r[0], dtype=np.float32).reshape(-1) for r in rows])
+        v = np.stack([np.asarray(r[1], dtype=np.float32).reshape(-1) for r in rows])
+        for layer in range(layers):
+            g.restore_bulk(layer, 0, k, v)
+            c.restore_bulk(layer, 0, k, v)
+    return g, c
+
+
+def close(a, b, tol):
+    return abs(float(a) - b) <= tol
+
+
+def test_global_layer_sees_everything():
+    # attention_tests.rs:47-61.
+    g, _ = both(1, 1, [([1.0], [1000.0]), ([1.0], [3.0]), ([1.0], [5.0])])
+    out = P().gqa_attention([1.0], 1, 1, [2], g.view(0), P().AttentionParams.new())
+    assert close(out[0], 336.0, 1e-3), out[0]
+
+
+def test_causal_mask_blocks_future_positions():
+    # attention_tests.rs:63-85.
+    g, _ = both(1, 1, [([0.0], [1.0]), ([10.0], [100.0]), ([10.0], [1000.0])])
+    out = P().gqa_attention([1.0, 1.0], 2, 1, [0, 1], g.view(0), P().AttentionParams.new())
+    assert close(out[0], 1.0, 1e-6), out[0]
+    assert 99.9 < out[1] < 100.0, out[1]
+
+
+def test_gqa_head_sharing_glimmer_shape_32_to_2():
+    # attention_tests.rs:87-114.
+    g, _ = both(2, 2, [([1.0, 0.0, 1.0, 0.0], [10.0, 0.0, 20.0, 0.0])])
+    out = P().gqa_attention([1.0, 0.0] * 32, 1, 32, [0], g.view(0), P().AttentionParams.new())
+    for h in range(32):
+        assert close(out[h * 2], 10.0 if h < 16 else 20.0, 1e-6), (h, out[h * 2])
+        assert close(out[h * 2 + 1], 0.0, 1e-6)
+
+
+def test_gqa_head_sharing_smaller_ratio_4_to_2():
+    # attention_tests.rs:116-140.
+    g, _ = both(2, 1, [([1.0, 1.0], [7.0, 9.0])])
+    out = P().gqa_attention([1.0] * 4, 1, 4, [0], g.view(0), P().AttentionParams.new())
+    for h, expected in [(0, 7.0), (1, 7.0), (2, 9.0), (3, 9.0)]:
+        assert close(out[h], expected, 1e-6), (h, out[h])
+
+
+def test_attention_validation_is_named_errors_not_faults():
+    # attention_tests.rs:152-212.
+    empty = P().KvCache.new([P().LayerKind.Global], 2, 2)
+    with pytest.raises(P().AttentionError) as e:
+        P().gqa_attention([1.0, 0.0, 1.0, 0.0], 1, 2, [0], empty.view(0))
+    assert e.value == E("NoVisibleKeys", position=0)
+    g, _ = both(2, 2, [([1.0, 0.0, 1.0, 0.0], [1.0, 0.0, 1.0, 0.0])])
+    view = g.view(0)
+    with pytest.raises(P().AttentionError) as e:
+        P().gqa_attention([1.0] * 6, 1, 3, [0], view)
+    assert e.value == E("NonDivisibleHeads", num_q_heads=3, num_kv_heads=2)
+    with pytest.raises(P().AttentionError) as e:
+        P().gqa_attention([1.0], 1, 2, [0], view)
+    assert e.value == E("ShapeMismatch", what="q", expected=4, actual=1)
+    with pytest.raises(P().AttentionError) as e:
+        P().gqa_attention([1.0] * 4, 2, 2, [0], view)
+    assert e.value == E("ShapeMismatch", what="query_positions", expected=2, actual=1)
+    assert P().gqa_attention([], 0, 2, [], view).size == 0
+
+
+def test_scale_is_a_parameter_and_softcap_follows_the_formula():
+    d = 16
+    k1, k2 = np.zeros(d, dtype=np.float32), np.zeros(d, dtype=np.float32)
+    k2[0] = np.log(3.0) * 4.0
+    q = np.zeros(d, dtype=np.float32)
+    q[0] = 1.0
+    g, c = both(1, d, [(k1, np.full(d, 0.0)), (k2, np.full(d, 4.0))])
+    A = P().AttentionParams
+    assert close(P().gqa_attention(q, 1, 1, [1], g.view(0), A.new())[0], 3.0, 1e-5)
+    assert close(P().gqa_attention(q, 1, 1, [1], g.view(0), A.with_scale(0.5))[0], 3.6, 1e-5)
+    # Softcap: scores (0, 2 ln 3) at scale 0.5 become cap*tanh(s/cap).
+    cap = 1.5
+    got = P().gqa_attention(q, 1, 1, [1], g.view(0), A(scale=0.5, softcap=cap))[0]
+    want = oracle.gqa_attention(q, 1, 1, [1], c.view(0),
+                                oracle.AttentionParams(scale=0.5, softcap=cap))[0]
+    assert close(got, want, 1e-5)
+    assert close(got, 4.0 * np.exp(cap * np.tanh(2 * np.log(3.0) / cap))
+                 / (1 + np.exp(cap * np.tanh(2 * np.log(3.0) / cap))), 1e-5)
+
+
+@pytest.mark.parametrize("elem", ["f32", "f16"])
+@pytest.mark.parametrize("n,qh,kvh,d,nq,softcap", [
+    (513, 32, 4, 64, 1, 0.0),     # the CPU-runnable decode shape
+    (300, 32, 4, 128, 1, 0.0),
+    (300, 32, 4, 128, 7, 30.0),   # verify-block shape with softcap
+    (77, 8, 8, 32, 3, 0.0),       # MHA
+    (130, 6, 2, 20, 5, 0.0),      # head_dim % 4 == 0 but not a power of two
+    (45, 4, 2, 3, 2, 0.0),        # scalar path
+    (1000, 16, 1, 256, 2, 0.0),   # MQA, largest head_dim
+    (9, 2, 1, 1, 9, 0.0),
+])
+def test_matches_the_oracle_on_seeded_shapes(elem, n, qh, kvh, d, nq, softcap):
+    rng = np.random.default_rng(n * 7 + d)
+    keys = normal(rng, n, kvh * d)
+    vals = normal(rng, n, kvh * d)
+    g, c = both(kvh, d, list(zip(keys, vals)), elem=elem)
+    q = normal(rng, nq, qh * d)
+    positions = list(range(n - nq, n))
+    params = dict(softcap=softcap)
+    got = P().gqa_attention(q, nq, qh, positions, g.view(0), P().AttentionParams(**params))
+    want = oracle.gqa_attention(q, nq, qh, positions, c.view(0), oracle.AttentionParams(**params))
+    if elem == "f32":
+        assert rel_err(got, want) <= F32_REL
+    else:
+        assert max_abs(got, want) <= F16_ABS
+    # Arbitrary (non-consecutive, repeated, future) positions take the explicit-position path.
+    positions = [n - 1, 0, n // 2, n + 5][:nq] + [n // 3] * max(0, nq - 4)
+    got = P().gqa_attention(q, nq, qh, positions, g.view(0), P().AttentionParams(**params))
+    want = oracle.gqa_attention(q, nq, qh, positions, c.view(0), oracle.AttentionParams(**params))
+    assert (rel_err(got, want) <= F32_REL) if elem == "f32" else (max_abs(got, want) <= F16_ABS)
+
+
+def glimmer_cfg(layers=2, q_heads=8, kv_heads=2, d=16):
+    return P().GlimmerConfig(layers=[P().LayerKind.Global] * layers, q_heads=q_heads,
+                             kv_heads=kv_heads, key_length=d, value_length=d)
+
+
+def test_compute_attention_is_append_then_attend_per_row():
+    # cpu.rs:586-646; incremental decode equals one-shot prefill (forward_tests.rs:641-719).
+    rng = np.random.default_rng(17)
+    cfg = glimmer_cfg()
+    G = P().LayerKind.Global
+    rows = 11
+    q = normal(rng, 2, rows, cfg.q_width())
+    k = normal(rng, 2, rows, cfg.k_width())
+    v = normal(rng, 2, rows, cfg.v_width())
+    one_shot = P().HipCompute.new(elem="f32", capacity_rows=32)
+    stepwise = P().HipCompute.new(elem="f32", capacity_rows=32)
+    cache_a, cache_b = P().PositionCache(), P().PositionCache()
+    ref = oracle.KvCache.new([oracle.LayerKind.Global] * 2, cfg.kv_heads, cfg.key_length)
+    outs = []
+    for layer in range(2):
+        outs.append(one_shot.attention(
+            P().AttentionRequest(q[layer], k[layer], v[layer], layer, G, cfg), cache_a))
+        want = oracle.attention_step(ref, layer, q[layer], k[layer], v[layer], cfg.q_heads, 0)
+        assert rel_err(outs[layer], want) <= F32_REL
+    cache_a.advance(rows)
+    for i in range(rows):
+        for layer in range(2):
+            o = stepwise.attention(
+                P().AttentionRequest(q[layer, i], k[layer, i], v[layer, i], layer, G, cfg), cache_b)
+            assert rel_err(o, outs[layer].reshape(rows, -1)[i]) <= 2 * F32_REL
+        cache_b.advance(1)
+    a, b = one_shot.kv_cache(), stepwise.kv_cache()
+    for layer in range(2):
+        ak, av = a.read_raw(layer)
+        bk, bv = b.read_raw(layer)
+        assert ak.tobytes() == bk.tobytes() and av.tobytes() == bv.tobytes()
+
+
+def test_compute_attention_refusals_follow_the_reference():
+    rng = np.random.default_rng(4)
+    cfg = glimmer_cfg()
+    G = P().LayerKind.Global
+    hc = P().HipCompute.new(elem="f32", capacity_rows=16)
+    cache = P().PositionCache()
+    with pytest.raises(P().StepFailed) as e:
+        hc.cache_checkpoint(3)
+    assert e.value.step == "cache_checkpoint" and "no KV state exists yet" in e.value.detail
+    q, k, v = normal(rng, cfg.q_width()), normal(rng, cfg.k_width()), normal(rng, cfg.v_width())
+    with pytest.raises(P().StepFailed) as e:
+        hc.attention(P().AttentionRequest(q[:-1], k, v, 0, G, cfg), cache)
+    assert "not a whole number" in e.value.detail
+    with pytest.raises(P().StepFailed) as e:
+        hc.attention(P().AttentionRequest(q, k[:-1], v, 0, G, cfg), cache)
+    assert "key/value projections hold" in e.value.detail
+    with pytest.raises(P().StepFailed) as e:
+        hc.attention(P().AttentionRequest(q, k, v, 0, P().LayerKind.SlidingWindow, cfg), cache)
+    assert "does not match the config's kind" in e.value.detail
+    hc.attention(P().AttentionRequest(q, k, v, 0, G, cfg), cache)
+    # The model did not advance the position cache: the next call must refuse
+    # (forward_tests.rs:1153-1181), and keep refusing until reset.
+    with pytest.raises(P().StepFailed) as e:
+        hc.attention(P().AttentionRequest(q, k, v, 0, G, cfg), cache)
+    assert "is at position 1 but the sequence cache is at position 0" in e.value.detail
+    other = glimmer_cfg(kv_heads=4)
+    with pytest.raises(P().StepFailed) as e:
+        hc.attention(P().AttentionRequest(q, np.tile(k, 2), np.tile(v, 2), 0, G, other), cache)
+    assert "different shape" in e.value.detail
+    hc.reset()
+    hc.attention(P().AttentionRequest(q, k, v, 0, G, cfg), cache)
+
+
+def test_speculative_round_trip_rewind_restores_the_exact_continuation():
+    # itak-spec round order (session.rs:616-831): checkpoint -> verify block -> rewind ->
+    # release, and forward_tests.rs:1097-1151: the continuation after a rewind equals the
+    # continuation of a backend that never speculated.
+    rng = np.random.default_rng(23)
+    cfg = glimmer_cfg(layers=2, q_heads=8, kv_heads=2, d=32)
+    G = P().LayerKind.Global
+    prompt, block, accepted = 20, 7, 2
+    total = prompt + block + 4
+    q = normal(rng, 2, total, cfg.q_width())
+    k = normal(rng, 2, total, cfg.k_width())
+    v = normal(rng, 2, total, cfg.v_width())
+
+    def forward(hc, cache, lo, hi, qq=q, kk=k, vv=v):
+        outs = [hc.attention(P().AttentionRequest(qq[l, lo:hi], kk[l, lo:hi], vv[l, lo:hi], l, G,
+                                                  cfg), cache) for l in range(2)]
+        cache.advance(hi - lo)
+        return outs
+
+    spec, plain = P().HipCompute.new(elem="f16", capacity_rows=64), \
+        P().HipCompute.new(elem="f16", capacity_rows=64)
+    cs, cp_ = P().PositionCache(), P().PositionCache()
+    forward(spec, cs, 0, prompt)
+    forward(plain, cp_, 0, prompt)
+    handle = spec.cache_checkpoint(block)
+    assert handle.base(0) == prompt and handle.saved_bytes() == 0
+    # Verify block with draft rows that will be rejected (different K/V than the truth).
+    kk, vv = k.copy(), v.copy()
+    kk[:, prompt + 1 + accepted:prompt + block] += 3.0
+    vv[:, prompt + 1 + accepted:prompt + block] -= 2.0
+    forward(spec, cs, prompt, prompt + block, kk=kk, vv=vv)
+    with pytest.raises(P().StepFailed) as e:  # one row past the round bound
+        spec.attention(P().AttentionRequest(q[0, 0], k[0, 0], v[0, 0], 0, G, cfg), cs)
+    assert "outside the live checkpoint's saved range" in e.value.detail
+    keep = prompt + 1 + accepted
+    spec.cache_rewind(handle, keep)
+    cs.rewind_to(keep)
+    spec.cache_release(handle)
+    forward(plain, cp_, prompt, keep)
+    a = forward(spec, cs, keep, total)
+    b = forward(plain, cp_, keep, total)
+    for l in range(2):
+        assert a[l].tobytes() == b[l].tobytes()
+        sk, sv = spec.kv_cache().read_raw(l)
+        pk, pv = plain.kv_cache().read_raw(l)
+        assert sk.tobytes() == pk.tobytes() and sv.tobytes() == pv.tobytes()
+    with pytest.raises(P().StepFailed) as e:
+        spec.cache_release(handle)
+    assert "not this cache's live checkpoint" in e.value.detail
