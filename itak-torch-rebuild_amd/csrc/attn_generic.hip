@@ -360,15 +360,17 @@ hipError_t launch_attn_generic(int elem_f16, const AttnParams &p, const AttnBatc
             if (end > total_partials) total_partials = end;
         }
     }
+// Dynamic LDS above 64 KiB has to be granted per kernel before the first launch that
+// needs it; the grant is raised whenever a launch needs more than any earlier one.
 #define ITAK_LAUNCH(T, V)                                                                        \
     do {                                                                                         \
-        static bool configured = false;                                                         \
-        if (!configured) {                                                                       \
+        static size_t granted = 64 * 1024;                                                       \
+        if (lds > granted) {                                                                     \
             hipError_t e = hipFuncSetAttribute(                                                  \
                 reinterpret_cast<const void *>(&attn_generic_kernel<T, V>),                      \
-                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                         \
+                hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));                           \
             if (e != hipSuccess) return e;                                                       \
-            configured = true;                                                                   \
+            granted = lds;                                                                       \
         }                                                                                        \
         attn_generic_kernel<T, V><<<b.total_blocks, kThreads, lds, stream>>>(p, b, total_partials); \
     } while (0)

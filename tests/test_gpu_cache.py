@@ -93,7 +93,7 @@ def test_append_is_bit_exact_against_the_oracle(elem, kv_heads, head_dim):
     scale = np.float32(10.0) ** rng.integers(-8, 6, size=(n, 1)).astype(np.float32)
     k = normal(rng, n, kv_heads * head_dim) * scale
     v = normal(rng, n, kv_heads * head_dim) * scale
-    k[3, 0], v[3, 1] = np.inf, -np.inf
+    k[3, 0], v[3, -1] = np.inf, -np.inf
     k[4, 0] = np.nan
     k[5, :] = 65520.0          # rounds to infinity in f16
     v[5, :] = 5.9604645e-08    # 2^-24: the smallest subnormal half

@@ -123,8 +123,9 @@ def test_config3_ragged_continuous_batching_decode():
         # A shuffled slot order: the slot table, not the position in the batch, addresses KV.
         order = rng.permutation(slots)
         items = [(caches[s], 1) for s in order]
-        pool.attention_step_device(layer, items, qd.data_ptr(), new_k[order].contiguous().data_ptr(),
-                                   new_v[order].contiguous().data_ptr(), out.data_ptr(), Q_HEADS)
+        ord_k, ord_v = new_k[order].contiguous(), new_v[order].contiguous()
+        pool.attention_step_device(layer, items, qd.data_ptr(), ord_k.data_ptr(),
+                                   ord_v.data_ptr(), out.data_ptr(), Q_HEADS)
         torch.cuda.synchronize()
         got = out.cpu().numpy()
         for i, s in enumerate(order):
