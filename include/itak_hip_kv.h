@@ -152,7 +152,10 @@ itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out);
 void itak_pool_destroy(itak_pool *pool);
 
 /* Stream every later call on this pool enqueues on (a hipStream_t; NULL = the
-   null stream). The pool never creates streams of its own. */
+   null stream). The pool never creates streams of its own and does not wait for the
+   previous stream: ordering between the two is the caller's to arrange. The stream
+   may be one that is being captured into a HIP graph, provided the pool's scratch
+   buffers are already large enough (run the same step once uncaptured first). */
 itak_status itak_pool_set_stream(itak_pool *pool, void *hip_stream);
 itak_status itak_pool_synchronize(itak_pool *pool);
 /* Bytes of device memory the pool holds for KV rows. */
@@ -274,6 +277,12 @@ itak_status itak_attention_step_device(itak_pool *pool, uint64_t layer,
                                        const float *q_dev, const float *k_dev, const float *v_dev,
                                        float *out_dev, uint64_t num_q_heads, float scale,
                                        float softcap);
+/* The attention half alone: query row r of item i attends at position
+   len_i - rows_i + r, i.e. over rows the slot already holds (gqa_attention over the
+   slot's view, attention.rs:104-215, with the last rows_i positions as queries). */
+itak_status itak_attention_device(itak_pool *pool, uint64_t layer, const itak_batch_item *items,
+                                  uint32_t item_count, const float *q_dev, float *out_dev,
+                                  uint64_t num_q_heads, float scale, float softcap);
 /* The append half alone (K5 APPEND_SHADER's job,
    crates/wgpu-compute/src/kernels/k5_rope_kv.rs:90-123), device tensors. */
 itak_status itak_kv_append_device(itak_pool *pool, uint64_t layer, const itak_batch_item *items,

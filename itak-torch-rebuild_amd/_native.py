@@ -106,6 +106,8 @@ PROTOTYPES = {
     "itak_compute_cache_release": (_i32, [_P, _u32, C.POINTER(CheckpointRaw)]),
     "itak_attention_step_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P, _P, _P,
                                           _u64, _f32, _f32]),
+    "itak_attention_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P, _u64, _f32,
+                                     _f32]),
     "itak_kv_append_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P]),
     "itak_convert_f32_to_f16_device": (_i32, [_P, _P, _P, _u64]),
 }

@@ -129,7 +129,7 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p, At
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     kv[e] = to_f32(kplane[off + e]);
-                    vv[e] = to_f32(vplane[off + e]);
+                    vv[e] = to_f32(vplane[v_offset(p.g, t0 + kj, c + e)]);
                 }
             } else {
 #pragma unroll

@@ -10,19 +10,34 @@ namespace itak {
 // Device layout of the KV pool, in elements of the storage type. One "plane" is the
 // rows of one (layer, slot, side, kv_head): capacity x head_dim elements, contiguous,
 // so a workgroup that streams one KV head reads one unbroken run of memory.
-//   element(layer, slot, side, head, row, d) =
-//     layer*layer_stride + slot*slot_stride + side*side_stride + head*head_stride + row*head_dim + d
-// side 0 = keys, 1 = values.
+//   plane(layer, slot, side, head) =
+//     layer*layer_stride + slot*slot_stride + side*side_stride + head*head_stride
+// side 0 = keys, 1 = values. Key planes are row-major: row*head_dim + d. Value planes are
+// row-major too unless v_block != 0: then they are stored in blocks of v_block (= 32) rows,
+// each block transposed, element (row, d) at
+//     (row / 32) * 32 * head_dim + d * 32 + row % 32
+// so that the 8 consecutive rows an MFMA lane needs for one channel are 16 contiguous
+// bytes and a wavefront's operand load covers 1 KiB of contiguous memory.
 struct PoolGeom {
     uint32_t kv_heads;
     uint32_t head_dim;
-    uint32_t capacity;  // rows per plane
+    uint32_t capacity;  // rows per plane (a multiple of 32 when v_block != 0)
     uint32_t max_slots;
+    uint32_t v_block;   // 0 or 32
+    uint32_t pad;
     uint64_t head_stride;   // capacity * head_dim
     uint64_t side_stride;   // kv_heads * head_stride
     uint64_t slot_stride;   // 2 * side_stride
     uint64_t layer_stride;  // max_slots * slot_stride
 };
+
+constexpr uint32_t kVBlock = 32;
+
+// Element offset of (row, d) inside a value plane.
+__host__ __device__ inline uint64_t v_offset(const PoolGeom &g, uint32_t row, uint32_t d) {
+    if (g.v_block == 0) return uint64_t(row) * g.head_dim + d;
+    return uint64_t(row / kVBlock) * (kVBlock * g.head_dim) + uint64_t(d) * kVBlock + row % kVBlock;
+}
 
 constexpr int kMaxBatchItems = 64;
 

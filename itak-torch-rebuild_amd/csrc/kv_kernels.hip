@@ -1,10 +1,9 @@
 // KV row movement kernels for gfx950: append (f32 -> f16 RNE or f32 copy), zero fill of
 // dropped rows, snapshot gather-restore and row readback. All of them are pure byte
-// movement bound by HBM (or, for a pinned-host source, by the host link): every thread
-// moves one 16-byte source vector and the grid covers the rows exactly.
+// movement bound by HBM (or, for a pinned-host source, by the host link). Sources and
+// the reference's own cache use [row][kv_head][d]; the pool stores one plane per KV head,
+// and value planes of f16 pools in 32-row transposed blocks (see PoolGeom).
 #include "internal.h"
-
-#include <hip/hip_fp16.h>
 
 namespace itak {
 
@@ -31,61 +30,50 @@ __device__ __forceinline__ void store4(uint16_t *dst, const float4 &v) {
     packed.y = uint32_t(f32_to_f16_bits(v.z)) | (uint32_t(f32_to_f16_bits(v.w)) << 16);
     *reinterpret_cast<uint2 *>(dst) = packed;
 }
+__device__ __forceinline__ void store1(float *dst, float v) { *dst = v; }
+__device__ __forceinline__ void store1(uint16_t *dst, float v) { *dst = f32_to_f16_bits(v); }
+__device__ __forceinline__ void store1(uint16_t *dst, uint16_t v) { *dst = v; }
 
 // ---------------------------------------------------------------------------- append
-// Thread = one (row, side, kv head, 4-element chunk). head_dim % 4 == 0 takes the vector
-// path; other head dims go through the scalar kernel below.
-template <typename T>
-__global__ __launch_bounds__(256) void kv_append_vec4(T *__restrict__ layer_base, PoolGeom g,
-                                                      AppendBatch b,
-                                                      const float *__restrict__ k_src,
-                                                      const float *__restrict__ v_src) {
-    const uint32_t chunks = g.head_dim >> 2;
+// Thread = one (row, side, kv head, VEC-element chunk) of the new rows. Key planes and
+// row-major value planes take one vector store; blocked value planes take VEC 2-byte
+// stores 64 bytes apart (an append moves a few KiB, so their width does not matter).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void kv_append_kernel(T *__restrict__ layer_base, PoolGeom g,
+                                                        AppendBatch b,
+                                                        const float *__restrict__ k_src,
+                                                        const float *__restrict__ v_src) {
+    const uint32_t chunks = g.head_dim / VEC;
     const uint64_t per_row = 2ull * g.kv_heads * chunks;
     const uint64_t idx = blockIdx.x * 256ull + threadIdx.x;
     if (idx >= per_row * b.total_rows) return;
-    uint32_t row = uint32_t(idx / per_row);
+    const uint32_t row = uint32_t(idx / per_row);
     uint32_t rem = uint32_t(idx % per_row);
     const uint32_t side = rem / (g.kv_heads * chunks);
     rem -= side * g.kv_heads * chunks;
     const uint32_t head = rem / chunks;
-    const uint32_t d = (rem % chunks) << 2;
+    const uint32_t d = (rem % chunks) * VEC;
     uint32_t it = 0;
     while (it + 1 < b.n && row >= b.item[it + 1].src_row0) ++it;
     const AppendItem item = b.item[it];
-    const uint32_t local = row - item.src_row0;
+    const uint32_t dst_row = item.pos0 + (row - item.src_row0);
     const float *src = (side ? v_src : k_src) + (uint64_t(row) * g.kv_heads + head) * g.head_dim + d;
-    const float4 v = *reinterpret_cast<const float4 *>(src);
-    T *dst = layer_base + item.slot * g.slot_stride + side * g.side_stride +
-             head * g.head_stride + uint64_t(item.pos0 + local) * g.head_dim + d;
-    store4(dst, v);
-}
-
-__device__ __forceinline__ void store1(float *dst, float v) { *dst = v; }
-__device__ __forceinline__ void store1(uint16_t *dst, float v) { *dst = f32_to_f16_bits(v); }
-
-template <typename T>
-__global__ __launch_bounds__(256) void kv_append_scalar(T *__restrict__ layer_base, PoolGeom g,
-                                                        AppendBatch b,
-                                                        const float *__restrict__ k_src,
-                                                        const float *__restrict__ v_src) {
-    const uint64_t per_row = 2ull * g.kv_heads * g.head_dim;
-    const uint64_t idx = blockIdx.x * 256ull + threadIdx.x;
-    if (idx >= per_row * b.total_rows) return;
-    uint32_t row = uint32_t(idx / per_row);
-    uint32_t rem = uint32_t(idx % per_row);
-    const uint32_t side = rem / (g.kv_heads * g.head_dim);
-    rem -= side * g.kv_heads * g.head_dim;
-    const uint32_t head = rem / g.head_dim;
-    const uint32_t d = rem % g.head_dim;
-    uint32_t it = 0;
-    while (it + 1 < b.n && row >= b.item[it + 1].src_row0) ++it;
-    const AppendItem item = b.item[it];
-    const uint32_t local = row - item.src_row0;
-    const float *src = (side ? v_src : k_src) + (uint64_t(row) * g.kv_heads + head) * g.head_dim + d;
-    T *dst = layer_base + item.slot * g.slot_stride + side * g.side_stride +
-             head * g.head_stride + uint64_t(item.pos0 + local) * g.head_dim + d;
-    store1(dst, *src);
+    T *plane = layer_base + item.slot * g.slot_stride + side * g.side_stride + head * g.head_stride;
+    if constexpr (VEC == 4) {
+        const float4 v = *reinterpret_cast<const float4 *>(src);
+        if (side == 0 || g.v_block == 0) {
+            store4(plane + uint64_t(dst_row) * g.head_dim + d, v);
+        } else {
+            T *dst = plane + v_offset(g, dst_row, d);
+            store1(dst, v.x);
+            store1(dst + kVBlock, v.y);
+            store1(dst + 2 * kVBlock, v.z);
+            store1(dst + 3 * kVBlock, v.w);
+        }
+    } else {
+        const uint64_t off = (side == 0) ? uint64_t(dst_row) * g.head_dim + d : v_offset(g, dst_row, d);
+        store1(plane + off, *src);
+    }
 }
 
 hipError_t launch_append(void *layer_base, int elem_f16, const PoolGeom &g, const AppendBatch &b,
@@ -99,62 +87,64 @@ hipError_t launch_append(void *layer_base, int elem_f16, const PoolGeom &g, cons
     if (elem_f16) {
         auto *base = static_cast<uint16_t *>(layer_base);
         if (vec)
-            kv_append_vec4<uint16_t><<<blocks, 256, 0, stream>>>(base, g, b, k_src, v_src);
+            kv_append_kernel<uint16_t, 4><<<blocks, 256, 0, stream>>>(base, g, b, k_src, v_src);
         else
-            kv_append_scalar<uint16_t><<<blocks, 256, 0, stream>>>(base, g, b, k_src, v_src);
+            kv_append_kernel<uint16_t, 1><<<blocks, 256, 0, stream>>>(base, g, b, k_src, v_src);
     } else {
         auto *base = static_cast<float *>(layer_base);
         if (vec)
-            kv_append_vec4<float><<<blocks, 256, 0, stream>>>(base, g, b, k_src, v_src);
+            kv_append_kernel<float, 4><<<blocks, 256, 0, stream>>>(base, g, b, k_src, v_src);
         else
-            kv_append_scalar<float><<<blocks, 256, 0, stream>>>(base, g, b, k_src, v_src);
+            kv_append_kernel<float, 1><<<blocks, 256, 0, stream>>>(base, g, b, k_src, v_src);
     }
     return hipGetLastError();
 }
 
 // ------------------------------------------------------------------------- zero rows
-// grid = (blocks over the widest item's bytes, item, layer*2*kv_heads planes).
-__global__ __launch_bounds__(256) void kv_zero_rows(unsigned char *__restrict__ pool_base,
-                                                    uint32_t elem_bytes, PoolGeom g,
+// grid = (blocks over the widest item's elements, item, layer * 2 * kv_heads planes).
+template <typename T>
+__global__ __launch_bounds__(256) void kv_zero_rows(T *__restrict__ pool_base, PoolGeom g,
                                                     uint32_t layer_from, ZeroBatch b) {
     const ZeroItem item = b.item[blockIdx.y];
     if (item.row_to <= item.row_from) return;
     const uint32_t planes_per_layer = 2 * g.kv_heads;
     const uint32_t layer = layer_from + blockIdx.z / planes_per_layer;
-    const uint32_t plane = blockIdx.z % planes_per_layer;  // side*kv_heads + head
-    const uint64_t row_bytes = uint64_t(g.head_dim) * elem_bytes;
-    const uint64_t bytes = uint64_t(item.row_to - item.row_from) * row_bytes;
-    unsigned char *dst = pool_base +
-                         (layer * g.layer_stride + item.slot * g.slot_stride +
-                          plane * g.head_stride + uint64_t(item.row_from) * g.head_dim) *
-                             elem_bytes;
-    // Row starts are multiples of head_dim*elem_bytes; use 4-byte words when that allows.
-    if ((row_bytes & 3) == 0) {
-        const uint64_t words = bytes >> 2;
-        for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < words; i += gridDim.x * 256ull)
-            reinterpret_cast<uint32_t *>(dst)[i] = 0u;
-    } else {
-        for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < bytes; i += gridDim.x * 256ull)
-            dst[i] = 0;
+    const uint32_t plane_id = blockIdx.z % planes_per_layer;  // side * kv_heads + head
+    const uint32_t side = plane_id / g.kv_heads;
+    T *plane = pool_base + layer * g.layer_stride + item.slot * g.slot_stride +
+               plane_id * g.head_stride;
+    const uint64_t total = uint64_t(item.row_to - item.row_from) * g.head_dim;
+    const bool blocked = side == 1 && g.v_block != 0;
+    for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < total; i += gridDim.x * 256ull) {
+        if (blocked) {
+            // Consecutive threads walk the rows of one channel: contiguous inside a block.
+            const uint32_t rows = item.row_to - item.row_from;
+            const uint32_t d = uint32_t(i / rows);
+            const uint32_t row = item.row_from + uint32_t(i % rows);
+            plane[v_offset(g, row, d)] = T(0);
+        } else {
+            plane[uint64_t(item.row_from) * g.head_dim + i] = T(0);
+        }
     }
 }
 
 hipError_t launch_zero_rows(void *pool_base, int elem_f16, const PoolGeom &g, uint32_t layer_from,
                             uint32_t layer_to, const ZeroBatch &b, hipStream_t stream) {
     if (b.n == 0 || b.max_rows == 0 || layer_to <= layer_from) return hipSuccess;
-    const uint32_t elem_bytes = elem_f16 ? 2 : 4;
-    const uint64_t words = (uint64_t(b.max_rows) * g.head_dim * elem_bytes + 3) / 4;
-    uint32_t bx = uint32_t((words + 255) / 256);
+    const uint64_t elems = uint64_t(b.max_rows) * g.head_dim;
+    uint32_t bx = uint32_t((elems + 255) / 256);
     if (bx > 1024) bx = 1024;
-    if (bx == 0) bx = 1;
     const uint32_t planes_per_layer = 2 * g.kv_heads;
     // gridDim.z is limited to 65535: walk the layers in slices that fit.
     const uint32_t layers_per_launch = 65535 / planes_per_layer ? 65535 / planes_per_layer : 1;
     for (uint32_t l = layer_from; l < layer_to; l += layers_per_launch) {
         const uint32_t n = (layer_to - l < layers_per_launch) ? layer_to - l : layers_per_launch;
         dim3 grid(bx, b.n, n * planes_per_layer);
-        kv_zero_rows<<<grid, 256, 0, stream>>>(static_cast<unsigned char *>(pool_base), elem_bytes,
-                                               g, l, b);
+        if (elem_f16)
+            kv_zero_rows<uint16_t><<<grid, 256, 0, stream>>>(static_cast<uint16_t *>(pool_base), g,
+                                                             l, b);
+        else
+            kv_zero_rows<float><<<grid, 256, 0, stream>>>(static_cast<float *>(pool_base), g, l, b);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -162,52 +152,89 @@ hipError_t launch_zero_rows(void *pool_base, int elem_f16, const PoolGeom &g, ui
 }
 
 // ---------------------------------------------------------------------------- restore
-// Gather: source rows are [row][kv_head][d] (the snapshot's and the reference cache's
-// layout), destination planes are per KV head. grid = (blocks over rows*kv_heads*chunks,
-// side, layer entry). Sources may live in pinned host memory: each thread issues one
-// 16-byte read, so a wave covers 1 KiB of contiguous source per instruction.
-template <typename D>
-__global__ __launch_bounds__(256) void kv_restore_from_f32(D *__restrict__ pool_base, PoolGeom g,
-                                                           RestoreBatch b) {
+// Gather from [row][kv_head][d] sources (possibly pinned host memory, read in place) into
+// the planes. Row-major planes: thread = one 16-byte source vector, a wave covers 1 KiB
+// of contiguous source. grid = (blocks, side, layer entry).
+template <typename S, typename D>
+__global__ __launch_bounds__(256) void kv_restore_rows(D *__restrict__ pool_base, PoolGeom g,
+                                                       RestoreBatch b, uint32_t sides_from) {
+    constexpr int VEC = 16 / sizeof(S);
     const RestoreLayer L = b.layer[blockIdx.z];
-    const uint32_t side = blockIdx.y;
-    const uint32_t chunks = g.head_dim >> 2;
+    const uint32_t side = sides_from + blockIdx.y;
+    const uint32_t chunks = g.head_dim / VEC;
     const uint64_t total = uint64_t(L.rows) * g.kv_heads * chunks;
-    const float *src = static_cast<const float *>(side ? L.values : L.keys);
-    D *dst_layer = pool_base + L.layer * g.layer_stride + b.slot * g.slot_stride +
-                   side * g.side_stride;
+    const S *src = static_cast<const S *>(side ? L.values : L.keys);
+    D *dst_side = pool_base + L.layer * g.layer_stride + b.slot * g.slot_stride +
+                  side * g.side_stride;
     for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < total; i += gridDim.x * 256ull) {
         const uint32_t row = uint32_t(i / (g.kv_heads * chunks));
         const uint32_t rem = uint32_t(i % (g.kv_heads * chunks));
         const uint32_t head = rem / chunks;
-        const uint32_t d = (rem % chunks) << 2;
-        const float4 v = *reinterpret_cast<const float4 *>(src + i * 4);
-        store4(dst_layer + head * g.head_stride + uint64_t(L.first_row + row) * g.head_dim + d, v);
+        const uint32_t d = (rem % chunks) * VEC;
+        D *dst = dst_side + head * g.head_stride + uint64_t(L.first_row + row) * g.head_dim + d;
+        if constexpr (sizeof(S) == 4) {
+            store4(dst, *reinterpret_cast<const float4 *>(src + i * VEC));
+        } else {
+            *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(src + i * VEC);
+        }
     }
 }
 
-// f16 source into an f16 pool: raw 16-byte copies (8 halves), bit-exact by construction.
-__global__ __launch_bounds__(256) void kv_restore_from_f16(uint16_t *__restrict__ pool_base,
-                                                           PoolGeom g, RestoreBatch b) {
+// Blocked value planes: one workgroup moves one (32-row block, kv head): coalesced reads of
+// the 32 source rows into LDS (converted), then each thread writes 8 consecutive rows of
+// one channel as one 16-byte store, so both sides of the transpose are full-width.
+// Requires first_row % 32 == 0. grid = (row blocks, kv_heads, layer entry).
+template <typename S>
+__global__ __launch_bounds__(256) void kv_restore_v_blocked(uint16_t *__restrict__ pool_base,
+                                                            PoolGeom g, RestoreBatch b) {
+    extern __shared__ uint16_t tile[];  // [32][head_dim + 8]
     const RestoreLayer L = b.layer[blockIdx.z];
-    const uint32_t side = blockIdx.y;
-    const uint32_t chunks = g.head_dim >> 3;
-    const uint64_t total = uint64_t(L.rows) * g.kv_heads * chunks;
-    const uint16_t *src = static_cast<const uint16_t *>(side ? L.values : L.keys);
-    uint16_t *dst_layer = pool_base + L.layer * g.layer_stride + b.slot * g.slot_stride +
-                          side * g.side_stride;
-    for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < total; i += gridDim.x * 256ull) {
-        const uint32_t row = uint32_t(i / (g.kv_heads * chunks));
-        const uint32_t rem = uint32_t(i % (g.kv_heads * chunks));
-        const uint32_t head = rem / chunks;
-        const uint32_t d = (rem % chunks) << 3;
-        const uint4 v = *reinterpret_cast<const uint4 *>(src + i * 8);
-        *reinterpret_cast<uint4 *>(dst_layer + head * g.head_stride +
-                                   uint64_t(L.first_row + row) * g.head_dim + d) = v;
+    const uint32_t head = blockIdx.y;
+    const uint32_t D = g.head_dim;
+    const uint32_t stride = D + 8;
+    const S *src = static_cast<const S *>(L.values);
+    uint16_t *plane = pool_base + L.layer * g.layer_stride + b.slot * g.slot_stride +
+                      g.side_stride + head * g.head_stride;
+    const uint32_t nblocks = (L.rows + kVBlock - 1) / kVBlock;
+    for (uint32_t blk = blockIdx.x; blk < nblocks; blk += gridDim.x) {
+        const uint32_t row0 = blk * kVBlock;
+        constexpr int VEC = 16 / sizeof(S);
+        const uint32_t chunks = D / VEC;
+        for (uint32_t i = threadIdx.x; i < kVBlock * chunks; i += 256) {
+            const uint32_t r = i / chunks, c = (i % chunks) * VEC;
+            uint16_t *t = tile + r * stride + c;
+            if (row0 + r < L.rows) {
+                const S *s = src + (uint64_t(row0 + r) * g.kv_heads + head) * D + c;
+                if constexpr (sizeof(S) == 4) {
+                    store4(t, *reinterpret_cast<const float4 *>(s));
+                } else {
+                    *reinterpret_cast<uint4 *>(t) = *reinterpret_cast<const uint4 *>(s);
+                }
+            } else {
+                // Rows past the snapshot stay zero, as a fresh layer holds them.
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) t[e] = 0;
+            }
+        }
+        __syncthreads();
+        uint16_t *dst_blk = plane + uint64_t(L.first_row / kVBlock + blk) * (kVBlock * D);
+        for (uint32_t i = threadIdx.x; i < D * (kVBlock / 8); i += 256) {
+            const uint32_t d = i / (kVBlock / 8), r8 = (i % (kVBlock / 8)) * 8;
+            uint16_t v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = tile[(r8 + e) * stride + d];
+            uint4 packed;
+            packed.x = v[0] | (uint32_t(v[1]) << 16);
+            packed.y = v[2] | (uint32_t(v[3]) << 16);
+            packed.z = v[4] | (uint32_t(v[5]) << 16);
+            packed.w = v[6] | (uint32_t(v[7]) << 16);
+            *reinterpret_cast<uint4 *>(dst_blk + d * kVBlock + r8) = packed;
+        }
+        __syncthreads();
     }
 }
 
-// Scalar fallback for head dims the vector paths cannot take.
+// Element-wise fallback for head dims or alignments the vector paths cannot take.
 template <typename S, typename D>
 __global__ __launch_bounds__(256) void kv_restore_scalar(D *__restrict__ pool_base, PoolGeom g,
                                                          RestoreBatch b) {
@@ -215,56 +242,72 @@ __global__ __launch_bounds__(256) void kv_restore_scalar(D *__restrict__ pool_ba
     const uint32_t side = blockIdx.y;
     const uint64_t total = uint64_t(L.rows) * g.kv_heads * g.head_dim;
     const S *src = static_cast<const S *>(side ? L.values : L.keys);
-    D *dst_layer = pool_base + L.layer * g.layer_stride + b.slot * g.slot_stride +
-                   side * g.side_stride;
+    D *dst_side = pool_base + L.layer * g.layer_stride + b.slot * g.slot_stride +
+                  side * g.side_stride;
     for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < total; i += gridDim.x * 256ull) {
         const uint32_t row = uint32_t(i / (g.kv_heads * g.head_dim));
         const uint32_t rem = uint32_t(i % (g.kv_heads * g.head_dim));
         const uint32_t head = rem / g.head_dim;
         const uint32_t d = rem % g.head_dim;
-        D *dst = dst_layer + head * g.head_stride + uint64_t(L.first_row + row) * g.head_dim + d;
-        if constexpr (sizeof(S) == sizeof(D)) {
-            *dst = src[i];
-        } else {
-            store1(dst, src[i]);
-        }
+        const uint64_t off = side == 0 ? uint64_t(L.first_row + row) * g.head_dim + d
+                                       : v_offset(g, L.first_row + row, d);
+        store1(dst_side + head * g.head_stride + off, src[i]);
     }
 }
 
 hipError_t launch_restore(void *pool_base, int dst_f16, int src_f16, const PoolGeom &g,
                           const RestoreBatch &b, hipStream_t stream) {
     if (b.n == 0 || b.max_rows == 0) return hipSuccess;
-    bool aligned = true;
+    bool aligned = true, block_aligned = true;
     for (uint32_t i = 0; i < b.n; ++i) {
         aligned = aligned && (reinterpret_cast<uintptr_t>(b.layer[i].keys) % 16 == 0) &&
                   (reinterpret_cast<uintptr_t>(b.layer[i].values) % 16 == 0);
+        block_aligned = block_aligned && (b.layer[i].first_row % kVBlock == 0);
     }
     const uint32_t vec = src_f16 ? 8 : 4;
     const bool use_vec = aligned && (g.head_dim % vec == 0);
-    const uint64_t per_layer =
-        uint64_t(b.max_rows) * g.kv_heads * (use_vec ? g.head_dim / vec : g.head_dim);
+    if (!use_vec || (g.v_block != 0 && !block_aligned)) {
+        const uint64_t per_layer = uint64_t(b.max_rows) * g.kv_heads * g.head_dim;
+        uint32_t bx = uint32_t((per_layer + 255) / 256);
+        if (bx > 2048) bx = 2048;
+        dim3 grid(bx, 2, b.n);
+        if (src_f16)
+            kv_restore_scalar<uint16_t, uint16_t><<<grid, 256, 0, stream>>>(
+                static_cast<uint16_t *>(pool_base), g, b);
+        else if (dst_f16)
+            kv_restore_scalar<float, uint16_t><<<grid, 256, 0, stream>>>(
+                static_cast<uint16_t *>(pool_base), g, b);
+        else
+            kv_restore_scalar<float, float><<<grid, 256, 0, stream>>>(
+                static_cast<float *>(pool_base), g, b);
+        return hipGetLastError();
+    }
+    const uint64_t per_layer = uint64_t(b.max_rows) * g.kv_heads * (g.head_dim / vec);
     uint32_t bx = uint32_t((per_layer + 255) / 256);
     if (bx > 2048) bx = 2048;
-    dim3 grid(bx, 2, b.n);
-    if (src_f16) {
-        auto *base = static_cast<uint16_t *>(pool_base);
-        if (use_vec)
-            kv_restore_from_f16<<<grid, 256, 0, stream>>>(base, g, b);
-        else
-            kv_restore_scalar<uint16_t, uint16_t><<<grid, 256, 0, stream>>>(base, g, b);
-    } else if (dst_f16) {
-        auto *base = static_cast<uint16_t *>(pool_base);
-        if (use_vec)
-            kv_restore_from_f32<uint16_t><<<grid, 256, 0, stream>>>(base, g, b);
-        else
-            kv_restore_scalar<float, uint16_t><<<grid, 256, 0, stream>>>(base, g, b);
-    } else {
-        auto *base = static_cast<float *>(pool_base);
-        if (use_vec)
-            kv_restore_from_f32<float><<<grid, 256, 0, stream>>>(base, g, b);
-        else
-            kv_restore_scalar<float, float><<<grid, 256, 0, stream>>>(base, g, b);
-    }
+    const uint32_t row_sides = g.v_block != 0 ? 1 : 2;  // keys only when values are blocked
+    dim3 grid(bx, row_sides, b.n);
+    if (src_f16)
+        kv_restore_rows<uint16_t, uint16_t><<<grid, 256, 0, stream>>>(
+            static_cast<uint16_t *>(pool_base), g, b, 0);
+    else if (dst_f16)
+        kv_restore_rows<float, uint16_t><<<grid, 256, 0, stream>>>(
+            static_cast<uint16_t *>(pool_base), g, b, 0);
+    else
+        kv_restore_rows<float, float><<<grid, 256, 0, stream>>>(static_cast<float *>(pool_base), g,
+                                                               b, 0);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || g.v_block == 0) return e;
+    uint32_t nblocks = (b.max_rows + kVBlock - 1) / kVBlock;
+    if (nblocks > 1024) nblocks = 1024;
+    dim3 vgrid(nblocks, g.kv_heads, b.n);
+    const size_t lds = size_t(kVBlock) * (g.head_dim + 8) * sizeof(uint16_t);
+    if (src_f16)
+        kv_restore_v_blocked<uint16_t><<<vgrid, 256, lds, stream>>>(
+            static_cast<uint16_t *>(pool_base), g, b);
+    else
+        kv_restore_v_blocked<float><<<vgrid, 256, lds, stream>>>(
+            static_cast<uint16_t *>(pool_base), g, b);
     return hipGetLastError();
 }
 
@@ -286,7 +329,9 @@ __global__ __launch_bounds__(256) void kv_read_rows(const T *__restrict__ layer_
         const uint32_t rem = uint32_t(i % (g.kv_heads * g.head_dim));
         const uint32_t head = rem / g.head_dim;
         const uint32_t d = rem % g.head_dim;
-        out[i] = src_side[head * g.head_stride + uint64_t(first_row + row) * g.head_dim + d];
+        const uint64_t off = side == 0 ? uint64_t(first_row + row) * g.head_dim + d
+                                       : v_offset(g, first_row + row, d);
+        out[i] = src_side[head * g.head_stride + off];
     }
 }
 

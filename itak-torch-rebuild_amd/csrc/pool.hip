@@ -48,7 +48,8 @@ struct itak_pool {
     PoolGeom g{};
     int elem_f16 = 0;
     uint32_t elem_bytes = 4;
-    uint64_t row = 0;  // kv_heads * head_dim
+    uint64_t row = 0;         // kv_heads * head_dim
+    uint64_t rows_limit = 0;  // positions a slot may hold (the configured capacity)
     unsigned char *base = nullptr;
     uint64_t bytes = 0;
     hipStream_t stream = nullptr;
@@ -350,9 +351,9 @@ itak_status check_append_rows(itak_pool *pool, Slot &s, uint64_t layer, uint64_t
             st = range_exceeded(pool->err, layer, start + ok, limit);
         }
     }
-    if (start + ok > pool->g.capacity) {
-        ok = pool->g.capacity > start ? pool->g.capacity - start : 0;
-        st = capacity_exceeded(pool->err, layer, start + ok + 1, pool->g.capacity);
+    if (start + ok > pool->rows_limit) {
+        ok = pool->rows_limit > start ? pool->rows_limit - start : 0;
+        st = capacity_exceeded(pool->err, layer, start + ok + 1, pool->rows_limit);
     }
     *ok_rows = ok;
     return st;
@@ -443,8 +444,13 @@ itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out) {
         config->num_kv_heads > (1u << 16))
         return size_overflow(e, "global layer storage");
     const uint64_t elem_bytes = config->elem == ITAK_ELEM_F16 ? 2 : 4;
+    // f16 pools whose head_dim suits the MFMA kernels keep value planes in transposed
+    // 32-row blocks; their planes are padded to whole blocks.
+    const bool v_blocked = config->elem == ITAK_ELEM_F16 && config->head_dim % 16 == 0;
+    const uint64_t plane_rows =
+        v_blocked ? align_up(config->capacity_rows, kVBlock) : config->capacity_rows;
     uint64_t head_stride, side_stride, slot_stride, layer_stride, total, bytes;
-    if (__builtin_mul_overflow(config->capacity_rows, config->head_dim, &head_stride) ||
+    if (__builtin_mul_overflow(plane_rows, config->head_dim, &head_stride) ||
         __builtin_mul_overflow(head_stride, config->num_kv_heads, &side_stride) ||
         __builtin_mul_overflow(side_stride, uint64_t(2), &slot_stride) ||
         __builtin_mul_overflow(slot_stride, uint64_t(config->max_slots), &layer_stride) ||
@@ -463,8 +469,10 @@ itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out) {
     pool->row = row;
     pool->g.kv_heads = uint32_t(config->num_kv_heads);
     pool->g.head_dim = uint32_t(config->head_dim);
-    pool->g.capacity = uint32_t(config->capacity_rows);
+    pool->g.capacity = uint32_t(plane_rows);
     pool->g.max_slots = config->max_slots;
+    pool->g.v_block = v_blocked ? kVBlock : 0;
+    pool->rows_limit = config->capacity_rows;
     pool->g.head_stride = head_stride;
     pool->g.side_stride = side_stride;
     pool->g.slot_stride = slot_stride;
@@ -500,7 +508,6 @@ void itak_pool_destroy(itak_pool *pool) {
 
 itak_status itak_pool_set_stream(itak_pool *pool, void *hip_stream) {
     if (!pool) return ITAK_INVALID_ARGUMENT;
-    HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize the previous stream");
     pool->stream = static_cast<hipStream_t>(hip_stream);
     return ITAK_OK;
 }
@@ -599,8 +606,8 @@ itak_status itak_kv_append(itak_pool *pool, uint32_t slot, uint64_t layer, const
     if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
     if (position != s->appended[layer])
         return out_of_order(pool->err, layer, s->appended[layer], position);
-    if (position >= pool->g.capacity)
-        return capacity_exceeded(pool->err, layer, position + 1, pool->g.capacity);
+    if (position >= pool->rows_limit)
+        return capacity_exceeded(pool->err, layer, position + 1, pool->rows_limit);
     if (!k || !v) return invalid_argument(pool->err, "k or v is null");
     const uint64_t bytes = pool->row * sizeof(float);
     itak_status st = ensure_stage(pool, 2 * bytes);
@@ -719,7 +726,7 @@ itak_status itak_kv_restore_bulk(itak_pool *pool, uint32_t slot, uint64_t layer,
     if (first_position != 0)
         return shape_mismatch(pool->err, "bulk restore first position (global layer)", 0,
                               first_position);
-    if (rows > pool->g.capacity) return capacity_exceeded(pool->err, layer, rows, pool->g.capacity);
+    if (rows > pool->rows_limit) return capacity_exceeded(pool->err, layer, rows, pool->rows_limit);
     if (rows && (!keys || !values)) return invalid_argument(pool->err, "keys or values is null");
     itak_snapshot_layer L{first_position, rows, keys, values};
     return restore_layers(pool, slot, *s, &L, &layer, 1, src_elem);
@@ -757,8 +764,8 @@ itak_status itak_kv_restore_snapshot(itak_pool *pool, uint32_t slot, uint64_t to
     // fresh here, checked for all layers before any is touched.
     for (uint64_t i = 0; i < layer_count; ++i)
         if (s->appended[i] != 0) return not_fresh(pool->err, i, s->appended[i]);
-    if (token_count > pool->g.capacity)
-        return capacity_exceeded(pool->err, 0, token_count, pool->g.capacity);
+    if (token_count > pool->rows_limit)
+        return capacity_exceeded(pool->err, 0, token_count, pool->rows_limit);
     return restore_layers(pool, slot, *s, layers, nullptr, layer_count, src_elem);
 }
 
@@ -816,7 +823,7 @@ itak_status itak_kv_read_raw(itak_pool *pool, uint32_t slot, uint64_t layer, voi
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
     if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
-    return read_rows_common(pool, slot, layer, 0, pool->g.capacity, keys_out, values_out);
+    return read_rows_common(pool, slot, layer, 0, pool->rows_limit, keys_out, values_out);
 }
 
 itak_status itak_kv_checkpoint_active(itak_pool *pool, uint32_t slot, int32_t *out) {
@@ -1039,6 +1046,34 @@ itak_status itak_attention_step_device(itak_pool *pool, uint64_t layer,
     // simply be dropped.
     return run_attention(pool, layer, active.data(), uint32_t(active.size()), q_dev, out_dev,
                          nullptr, num_q_heads, scale, softcap);
+}
+
+itak_status itak_attention_device(itak_pool *pool, uint64_t layer, const itak_batch_item *items,
+                                  uint32_t item_count, const float *q_dev, float *out_dev,
+                                  uint64_t num_q_heads, float scale, float softcap) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (item_count == 0) return ITAK_OK;
+    if (!items || !q_dev || !out_dev)
+        return invalid_argument(pool->err, "items or a device tensor is null");
+    if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
+    if (num_q_heads == 0) return zero_dimension(pool->err, "num_q_heads");
+    if (num_q_heads % pool->g.kv_heads != 0)
+        return non_divisible(pool->err, num_q_heads, pool->g.kv_heads);
+    std::vector<PlanInput> plan;
+    for (uint32_t i = 0; i < item_count; ++i) {
+        Slot *s = find_slot(pool, items[i].slot);
+        if (!s) return invalid_argument(pool->err, "slot is not in use");
+        const uint64_t len = s->appended[layer];
+        if (items[i].rows == 0) continue;
+        if (len == 0) return no_visible_keys(pool->err, 0);
+        if (items[i].rows > len)
+            return shape_mismatch(pool->err, "query rows", len, items[i].rows);
+        plan.push_back(PlanInput{items[i].slot, items[i].rows, uint32_t(len - items[i].rows),
+                                 uint32_t(len)});
+    }
+    if (std::isnan(scale)) scale = default_scale(pool->g.head_dim);
+    return run_attention(pool, layer, plan.data(), uint32_t(plan.size()), q_dev, out_dev, nullptr,
+                         num_q_heads, scale, softcap);
 }
 
 itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t layer, const float *q,

@@ -254,6 +254,14 @@ class KvPool:
             self._h, layer, raw, n, q_ptr, k_ptr, v_ptr, out_ptr, num_q_heads,
             math.nan if scale is None else scale, softcap))
 
+    def attention_device(self, layer: int, items, q_ptr: int, out_ptr: int, num_q_heads: int,
+                         scale: Optional[float] = None, softcap: float = 0.0) -> None:
+        """Attend with each item's last `rows` stored positions as the queries' positions."""
+        raw, n = self._items(items)
+        _check(self._h, self._lib.itak_attention_device(
+            self._h, layer, raw, n, q_ptr, out_ptr, num_q_heads,
+            math.nan if scale is None else scale, softcap))
+
     def append_device(self, layer: int, items, k_ptr: int, v_ptr: int) -> None:
         raw, n = self._items(items)
         _check(self._h, self._lib.itak_kv_append_device(self._h, layer, raw, n, k_ptr, v_ptr))
