@@ -1,6 +1,6 @@
 // Generic GQA attention for gfx950: f32 or f16 KV storage, any head_dim <= 256, any
 // GQA group that fits the block, explicit or implied query positions, optional logit
-// softcap, split over the key range with the merge done by the last workgroup to arrive.
+// softcap, split over the key range (partials are merged by attn_combine_kernel).
 // It is the path every shape can take (and the only f32-storage path); the tuned f16
 // kernels elsewhere in this directory cover the shapes the engine actually serves.
 //
@@ -58,7 +58,6 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p, At
     float *m_s = Ss + kMaxR * TILE;       // [kMaxR]
     float *l_s = m_s + kMaxR;
     float *a_s = l_s + kMaxR;
-    __shared__ uint32_t ticket_s;
 
     const uint32_t tid = threadIdx.x;
 
@@ -274,51 +273,6 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p, At
             }
         }
     }
-    // Publish, then count arrivals; the last workgroup of this (item, row block, kv head)
-    // merges. Agent-scope fences make the partials visible across XCDs (each XCD has its
-    // own L2).
-    __threadfence();
-    __syncthreads();
-    uint32_t *counter = p.counters + item.cnt0 + qblock * p.g.kv_heads + kv_head;
-    if (tid == 0) {
-        ticket_s = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (ticket_s != item.splits - 1) return;
-    __threadfence();
-    if (tid == 0) {
-        __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    if (!pv_active) return;
-#pragma unroll 1
-    for (int i = 0; i < kMaxI; ++i) {
-        const uint32_t r = rbase + sh.rgroups * i;
-        if (r >= R) break;
-        const uint32_t row = row_begin + r / p.group;
-        const uint32_t head = kv_head * p.group + r % p.group;
-        const uint64_t ps0 = item.ws0 + (uint64_t(row) * p.q_heads + head) * item.splits;
-        float mx = -INFINITY;
-        for (uint32_t s = 0; s < item.splits; ++s) {
-            mx = fmaxf(mx, ws_ml[(ps0 + s) * 2]);
-        }
-        float lsum = 0.0f;
-        float o[VEC];
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) o[e] = 0.0f;
-        for (uint32_t s = 0; s < item.splits; ++s) {
-            const float ms = ws_ml[(ps0 + s) * 2];
-            const float ls = ws_ml[(ps0 + s) * 2 + 1];
-            const float w = (ms == -INFINITY) ? 0.0f : expf(ms - mx);
-            lsum += ls * w;
-            const float *a = ws_acc + (ps0 + s) * D + dc * VEC;
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) o[e] = fmaf(a[e], w, o[e]);
-        }
-        const float inv = 1.0f / lsum;
-        float *dst = p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * D + dc * VEC;
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) dst[e] = o[e] * inv;
-    }
 }
 
 size_t lds_bytes(uint32_t d, int vec) {
@@ -348,18 +302,11 @@ uint32_t attn_generic_rows_per_block(uint32_t group, uint32_t head_dim) {
 uint32_t attn_generic_tile(uint32_t head_dim) { return head_dim <= 128 ? 64 : 32; }
 
 hipError_t launch_attn_generic(int elem_f16, const AttnParams &p, const AttnBatch &b,
-                               hipStream_t stream) {
+                               uint32_t total_partials, hipStream_t stream) {
     if (b.total_blocks == 0) return hipSuccess;
     const uint32_t d = p.g.head_dim;
     const int vec = d % 4 == 0 ? 4 : 1;
     const size_t lds = lds_bytes(d, vec);
-    uint32_t total_partials = 0;
-    for (uint32_t i = 0; i < b.n; ++i) {
-        if (b.item[i].splits > 1) {
-            const uint32_t end = b.item[i].ws0 + b.item[i].rows * p.q_heads * b.item[i].splits;
-            if (end > total_partials) total_partials = end;
-        }
-    }
 // Dynamic LDS above 64 KiB has to be granted per kernel before the first launch that
 // needs it; the grant is raised whenever a launch needs more than any earlier one.
 #define ITAK_LAUNCH(T, V)                                                                        \

@@ -1,0 +1,439 @@
+// GQA flash-decode for gfx950, f16 KV, head_dim 128: split over the context, K and V
+// consumed straight from their planes as MFMA operands.
+//
+// One workgroup owns (item, kv head, split = a run of 32-key blocks). Each wavefront walks
+// its own blocks with a private online softmax and never synchronises inside the loop;
+// the wavefronts merge once through LDS at the end. Per 32-key block and per tile of 16
+// query vectors (a query vector = one query row of one Q head of the group):
+//
+//   S^T = K . Q^T   v_mfma_f32_16x16x32_f16, A = 16 key rows x 32 channels from the key
+//                   plane (16 bytes per lane), B = Q^T converted to f16 once per kernel.
+//   softmax         the lane that holds query vector j holds 8 consecutive keys of it, so
+//                   max/sum need two cross-lane steps; m, l and the rescale factor live in
+//                   the lane's own column.
+//   O^T += V^T . P^T  A = 16 channels x 32 keys from the blocked value plane (16 contiguous
+//                   bytes per lane, 1 KiB contiguous per wavefront load), B = P in the
+//                   registers the scores were produced in.
+//
+// All query heads of the KV group (and all rows of a speculative block) are columns of the
+// same MFMA, so K and V are read from HBM once per group. Scores, softmax state and
+// accumulators are f32; P and Q enter the MFMA as f16.
+//
+// Semantics: gqa_attention in crates/attention/src/attention.rs:104-215 on a global layer
+// (key kp visible to a query at position p iff kp <= p), with the optional softcap
+// cap*tanh(s/cap) of crates/torch-math/src/logits.rs:26-37 applied to the scaled scores.
+#include "internal.h"
+
+#include <math.h>
+
+namespace itak {
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kD = 128;          // head_dim this kernel is written for
+constexpr int kBlockKeys = 32;   // keys per block (= value plane block)
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// cap * tanh(x / cap) * log2(e), via exp2; x is a scaled score in natural units.
+__device__ __forceinline__ float softcap_log2(float x, float cap, float inv_cap) {
+    const float y = x * inv_cap;
+    // tanh(y) = 1 - 2 / (exp(2y) + 1); exp2 saturates to inf/0 at the tails, giving +-1.
+    const float e = fast_exp2(y * (2.0f * kLog2e));
+    const float t = 1.0f - 2.0f / (e + 1.0f);
+    return cap * kLog2e * t;
+}
+
+template <int NQ>
+struct WaveState {
+    float m[NQ];         // running max of this lane's query-vector column (log2 domain)
+    float l[NQ];         // this lane's share of the running denominator
+    floatx4 o[NQ][8];    // O^T accumulators: channel dt*16 + g*4 + r, query vector column
+};
+
+struct BlockOperands {
+    half8 k[2][4];  // [key half t][channel step s]
+    half8 v[8];     // [channel tile dt]
+};
+
+__device__ __forceinline__ void load_block(BlockOperands &b, const uint16_t *kplane,
+                                           const uint16_t *vplane, uint32_t kb, uint32_t g,
+                                           uint32_t i) {
+    // Key rows of MFMA tile t are interleaved so that the lane group g ends up holding
+    // scores of the 8 consecutive keys g*8 .. g*8+7: row i of tile t is key
+    // (i/4)*8 + t*4 + i%4 of the block.
+    const uint32_t key0 = kb * kBlockKeys + (i >> 2) * 8 + (i & 3);
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const uint16_t *row = kplane + uint64_t(key0 + t * 4) * kD + g * 8;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) b.k[t][s] = *reinterpret_cast<const half8 *>(row + s * 32);
+    }
+    const uint16_t *vb = vplane + uint64_t(kb) * (kBlockKeys * kD) + i * kBlockKeys + g * 8;
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt)
+        b.v[dt] = *reinterpret_cast<const half8 *>(vb + dt * 16 * kBlockKeys);
+}
+
+template <int NQ>
+__device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &b,
+                                              const half8 (&qb)[NQ][4], uint32_t kb, uint32_t g,
+                                              uint32_t jl, uint32_t pos0, uint32_t group,
+                                              uint32_t kv_len, float softcap, float inv_cap) {
+    const uint32_t key_base = kb * kBlockKeys + g * 8;  // first of this lane's 8 keys
+    const bool tail = (kb + 1) * kBlockKeys > kv_len;
+    if (tail) {
+        // Rows past the stored length may hold stale data: keep them out of P.V even as 0*x.
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (key_base + e >= kv_len) b.v[dt][e] = _Float16(0.0f);
+    }
+    const bool need_mask = (kb + 1) * kBlockKeys > pos0 + 1;
+#pragma unroll
+    for (int qt = 0; qt < NQ; ++qt) {
+        floatx4 s[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            s[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b.k[t][k], qb[qt][k], s[t], 0, 0, 0);
+        }
+        float sc[8];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sc[t * 4 + r] = s[t][r];
+        if (softcap > 0.0f) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sc[e] = softcap_log2(sc[e], softcap, inv_cap);
+        }
+        if (need_mask) {
+            const uint32_t pos = pos0 + (qt * 16 + jl) / group;  // this column's query position
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (key_base + e > pos) sc[e] = -INFINITY;
+        }
+        float mx = sc[0];
+#pragma unroll
+        for (int e = 1; e < 8; ++e) mx = fmaxf(mx, sc[e]);
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(st.m[qt], mx);
+        const bool dead = m_new == -INFINITY;  // nothing visible to this column so far
+        const float alpha = dead ? 1.0f : fast_exp2(st.m[qt] - m_new);
+        float p[8];
+        float sum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            p[e] = dead ? 0.0f : fast_exp2(sc[e] - m_new);
+            sum += p[e];
+        }
+        st.m[qt] = m_new;
+        st.l[qt] = st.l[qt] * alpha + sum;
+        half8 pb;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pb[e] = static_cast<_Float16>(p[e]);
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) {
+            st.o[qt][dt] *= alpha;
+            st.o[qt][dt] =
+                __builtin_amdgcn_mfma_f32_16x16x32_f16(b.v[dt], pb, st.o[qt][dt], 0, 0, 0);
+        }
+    }
+}
+
+template <int NQ, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams p, AttnBatch b,
+                                                                     uint32_t total_partials) {
+    extern __shared__ float lds[];
+    float *sm_m = lds;                          // [WAVES][NQ*16]
+    float *sm_l = sm_m + WAVES * NQ * 16;       // [WAVES][NQ*16]
+    float *sm_o = sm_l + WAVES * NQ * 16;       // [WAVES][NQ][8][64][4]
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = tid >> 6, lane = tid & 63;
+    const uint32_t g = lane >> 4, jl = lane & 15;
+
+    uint32_t it = 0;
+    while (it + 1 < b.n && blockIdx.x >= b.item[it + 1].block0) ++it;
+    const AttnItem item = b.item[it];
+    const uint32_t local = blockIdx.x - item.block0;
+    const uint32_t split = local % item.splits;
+    const uint32_t kv_head = local / item.splits;
+    const uint32_t group = p.group;
+    const uint32_t nvec = item.rows * group;
+
+    const uint16_t *kplane = static_cast<const uint16_t *>(p.layer_base) +
+                             item.slot * p.g.slot_stride + kv_head * p.g.head_stride;
+    const uint16_t *vplane = kplane + p.g.side_stride;
+
+    const uint32_t nblocks = (item.kv_len + kBlockKeys - 1) / kBlockKeys;
+    const uint32_t blocks_per_split = item.keys_per_split / kBlockKeys;
+    const uint32_t kb_begin = split * blocks_per_split;
+    const uint32_t kb_end = min(nblocks, kb_begin + blocks_per_split);
+
+    // Start the first block's loads before anything else: this kernel is latency bound.
+    BlockOperands buf_a, buf_b;
+    uint32_t kb = kb_begin + wave;
+    if (kb < kb_end) load_block(buf_a, kplane, vplane, kb, g, jl);
+
+    // ---- Q^T as the B operand: lane (g, jl) holds channels s*32 + g*8 .. +8 of vector jl.
+    const float softcap = p.softcap;
+    const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
+    const float qscale = softcap > 0.0f ? p.scale : p.scale * kLog2e;
+    half8 qb[NQ][4];
+#pragma unroll
+    for (int qt = 0; qt < NQ; ++qt) {
+        const uint32_t j = qt * 16 + jl;
+        if (j < nvec) {
+            const uint32_t row = j / group, head = kv_head * group + j % group;
+            const float *qp = p.q + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + g * 8;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const float4 a = *reinterpret_cast<const float4 *>(qp + s * 32);
+                const float4 c = *reinterpret_cast<const float4 *>(qp + s * 32 + 4);
+                qb[qt][s] = half8{static_cast<_Float16>(a.x * qscale), static_cast<_Float16>(a.y * qscale),
+                                  static_cast<_Float16>(a.z * qscale), static_cast<_Float16>(a.w * qscale),
+                                  static_cast<_Float16>(c.x * qscale), static_cast<_Float16>(c.y * qscale),
+                                  static_cast<_Float16>(c.z * qscale), static_cast<_Float16>(c.w * qscale)};
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) qb[qt][s] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+    }
+
+    WaveState<NQ> st;
+#pragma unroll
+    for (int qt = 0; qt < NQ; ++qt) {
+        st.m[qt] = -INFINITY;
+        st.l[qt] = 0.0f;
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) st.o[qt][dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    // ---- this wavefront's blocks, two register sets so the next block's loads fly while
+    // the current one is multiplied.
+    if (kb < kb_end) {
+        for (;;) {
+            const uint32_t kb2 = kb + WAVES;
+            const bool has2 = kb2 < kb_end;
+            if (has2) load_block(buf_b, kplane, vplane, kb2, g, jl);
+            process_block<NQ>(st, buf_a, qb, kb, g, jl, item.pos0, group, item.kv_len, softcap,
+                              inv_cap);
+            if (!has2) break;
+            const uint32_t kb3 = kb2 + WAVES;
+            const bool has3 = kb3 < kb_end;
+            if (has3) load_block(buf_a, kplane, vplane, kb3, g, jl);
+            process_block<NQ>(st, buf_b, qb, kb2, g, jl, item.pos0, group, item.kv_len, softcap,
+                              inv_cap);
+            if (!has3) break;
+            kb = kb3;
+        }
+    }
+
+    // ---- merge the wavefronts through LDS ------------------------------------------------
+#pragma unroll
+    for (int qt = 0; qt < NQ; ++qt) {
+        float l = st.l[qt];
+        l += __shfl_xor(l, 16);
+        l += __shfl_xor(l, 32);
+        if (g == 0) {
+            sm_m[wave * NQ * 16 + qt * 16 + jl] = st.m[qt];
+            sm_l[wave * NQ * 16 + qt * 16 + jl] = l;
+        }
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt)
+            *reinterpret_cast<floatx4 *>(sm_o + (((wave * NQ + qt) * 8 + dt) * 64 + lane) * 4) =
+                st.o[qt][dt];
+    }
+    __syncthreads();
+
+    float *ws_acc = p.ws;
+    float *ws_ml = p.ws + uint64_t(total_partials) * kD;
+    constexpr int kDtPerWave = 8 / WAVES;  // channel tiles each wavefront finishes
+#pragma unroll
+    for (int qt = 0; qt < NQ; ++qt) {
+        const uint32_t j = qt * 16 + jl;
+        float mw[WAVES], M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            mw[w] = sm_m[w * NQ * 16 + qt * 16 + jl];
+            M = fmaxf(M, mw[w]);
+        }
+        float L = 0.0f, wgt[WAVES];
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            wgt[w] = (mw[w] == -INFINITY) ? 0.0f : fast_exp2(mw[w] - M);
+            L += sm_l[w * NQ * 16 + qt * 16 + jl] * wgt[w];
+        }
+        if (j >= nvec) continue;
+        const uint32_t row = j / group, head = kv_head * group + j % group;
+        const uint64_t ps = item.ws0 + (uint64_t(row) * p.q_heads + head) * item.splits + split;
+#pragma unroll
+        for (int x = 0; x < kDtPerWave; ++x) {
+            const int dt = wave * kDtPerWave + x;
+            floatx4 acc{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w)
+                acc += *reinterpret_cast<const floatx4 *>(
+                           sm_o + (((w * NQ + qt) * 8 + dt) * 64 + lane) * 4) *
+                       wgt[w];
+            const uint32_t d = dt * 16 + g * 4;
+            if (item.splits == 1) {
+                const float inv = 1.0f / L;
+                acc *= inv;
+                *reinterpret_cast<floatx4 *>(
+                    p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + d) = acc;
+            } else {
+                *reinterpret_cast<floatx4 *>(ws_acc + ps * kD + d) = acc;
+            }
+        }
+        if (item.splits > 1 && wave == 0 && g == 0) {
+            ws_ml[ps * 2] = M;
+            ws_ml[ps * 2 + 1] = L;
+        }
+    }
+}
+
+}  // namespace
+
+bool attn_splitk_f16_supports(const PoolGeom &g, uint32_t group, uint32_t max_rows) {
+    return g.v_block == kVBlock && g.head_dim == kD && group >= 1 && max_rows >= 1 &&
+           max_rows * group <= 64;
+}
+
+// Fills splits / keys_per_split / block0 / ws0 for a batch (the caller has set slot, rows,
+// pos0, q_row0, kv_len) and returns the number of partials the launch will write.
+uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads) {
+    uint64_t blocks = 0;
+    for (uint32_t i = 0; i < b.n; ++i)
+        blocks += uint64_t(g.kv_heads) * ((b.item[i].kv_len + kBlockKeys - 1) / kBlockKeys);
+    const uint32_t waves = 4;
+    // About four workgroups per CU keeps every SIMD fed; short contexts get one block per
+    // wavefront, the least work a workgroup can usefully have.
+    constexpr uint64_t kTargetGroups = 1024;
+    uint64_t bps = (blocks + kTargetGroups - 1) / kTargetGroups;
+    bps = (bps + waves - 1) / waves * waves;
+    if (bps < waves) bps = waves;
+    uint32_t block0 = 0, ws0 = 0;
+    for (uint32_t i = 0; i < b.n; ++i) {
+        AttnItem &it = b.item[i];
+        const uint32_t nblocks = (it.kv_len + kBlockKeys - 1) / kBlockKeys;
+        it.keys_per_split = uint32_t(bps) * kBlockKeys;
+        it.splits = uint32_t((nblocks + bps - 1) / bps);
+        if (it.splits == 0) it.splits = 1;
+        it.block0 = block0;
+        it.ws0 = ws0;
+        block0 += g.kv_heads * it.splits;
+        if (it.splits > 1) ws0 += it.rows * q_heads * it.splits;
+    }
+    b.total_blocks = block0;
+    b.rows_per_block = 0;
+    return ws0;
+}
+
+hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                                  uint32_t max_rows, hipStream_t stream) {
+    if (b.total_blocks == 0) return hipSuccess;
+    const uint32_t nvec = max_rows * p.group;
+    constexpr int W = 4;
+#define ITAK_LAUNCH(NQ)                                                                          \
+    do {                                                                                         \
+        const size_t lds = (size_t(2) * W * NQ * 16 + size_t(W) * NQ * 8 * 64 * 4) * 4;           \
+        static size_t granted = 64 * 1024;                                                       \
+        if (lds > granted) {                                                                     \
+            hipError_t e = hipFuncSetAttribute(                                                  \
+                reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W>),                  \
+                hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));                           \
+            if (e != hipSuccess) return e;                                                       \
+            granted = lds;                                                                       \
+        }                                                                                        \
+        attn_splitk_f16_kernel<NQ, W><<<b.total_blocks, W * 64, lds, stream>>>(p, b,              \
+                                                                               total_partials); \
+    } while (0)
+    if (nvec <= 16)
+        ITAK_LAUNCH(1);
+    else if (nvec <= 32)
+        ITAK_LAUNCH(2);
+    else
+        ITAK_LAUNCH(4);
+#undef ITAK_LAUNCH
+    return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------ combine
+// Merges the split partials of one (query row, Q head): weights exp(m_s - M), output
+// sum_s w_s * acc_s / sum_s w_s * l_s. One 128-thread workgroup per (row, head); thread =
+// channel. grid = all (row, head) pairs of the batch, items whose splits == 1 exit at once.
+__global__ __launch_bounds__(128) void attn_combine_kernel(AttnParams p, AttnBatch b,
+                                                           uint32_t total_partials, int base2) {
+    __shared__ float w_s[1024];
+    __shared__ float red[4];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t D = p.g.head_dim;
+    // blockIdx.x -> (item, row, head): items are laid out by q_row0.
+    const uint32_t pair = blockIdx.x;
+    const uint32_t grow = pair / p.q_heads, head = pair % p.q_heads;
+    uint32_t it = 0;
+    while (it + 1 < b.n && grow >= b.item[it + 1].q_row0 - b.item[0].q_row0) ++it;
+    const AttnItem item = b.item[it];
+    if (item.splits == 1) return;
+    const uint32_t row = grow - (item.q_row0 - b.item[0].q_row0);
+    const uint64_t ps0 = item.ws0 + (uint64_t(row) * p.q_heads + head) * item.splits;
+    const float *ws_acc = p.ws;
+    const float *ws_ml = p.ws + uint64_t(total_partials) * D;
+
+    float mx = -INFINITY;
+    for (uint32_t s = tid; s < item.splits; s += 128) mx = fmaxf(mx, ws_ml[(ps0 + s) * 2]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    const float M = fmaxf(red[0], red[1]);
+    float lsum = 0.0f;
+    for (uint32_t s = tid; s < item.splits; s += 128) {
+        const float ms = ws_ml[(ps0 + s) * 2];
+        const float w = (ms == -INFINITY) ? 0.0f : (base2 ? exp2f(ms - M) : expf(ms - M));
+        w_s[s] = w;
+        lsum += w * ws_ml[(ps0 + s) * 2 + 1];
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) lsum += __shfl_xor(lsum, o);
+    if ((tid & 63) == 0) red[2 + (tid >> 6)] = lsum;
+    __syncthreads();
+    const float inv = 1.0f / (red[2] + red[3]);
+    for (uint32_t d = tid; d < D; d += 128) {
+        const float *a = ws_acc + ps0 * D + d;
+        float acc = 0.0f;
+        uint32_t s = 0;
+        for (; s + 8 <= item.splits; s += 8) {
+            float x[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) x[u] = a[uint64_t(s + u) * D];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc = fmaf(x[u], w_s[s + u], acc);
+        }
+        for (; s < item.splits; ++s) acc = fmaf(a[uint64_t(s) * D], w_s[s], acc);
+        p.out[(uint64_t(item.q_row0 + row) * p.q_heads + head) * D + d] = acc * inv;
+    }
+}
+
+hipError_t launch_attn_combine(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                               uint32_t total_rows, int base2, hipStream_t stream) {
+    bool any = false;
+    for (uint32_t i = 0; i < b.n; ++i) any = any || b.item[i].splits > 1;
+    if (!any || total_rows == 0) return hipSuccess;
+    attn_combine_kernel<<<total_rows * p.q_heads, 128, 0, stream>>>(p, b, total_partials, base2);
+    return hipGetLastError();
+}
+
+}  // namespace itak

@@ -102,8 +102,10 @@ hipError_t launch_convert_f16(const float *src, uint16_t *dst, uint64_t count, h
 // One item = one slot's query rows against that slot's rows of one layer. Query row r
 // sits at position pos0 + r unless q_pos is given. A workgroup owns (item, row block,
 // kv head, split of the key range) and writes either the final output (splits == 1) or
-// a partial (m, l, acc[head_dim]) per query vector that the last workgroup to finish
-// for that (item, row block, kv head) merges.
+// a partial (m, l, acc[head_dim]) per query vector; a second, small launch merges the
+// partials of each (row, Q head). Partials live in `ws`: first total_partials*head_dim
+// accumulators, then total_partials (m, l) pairs; the partial of (row, head, split) of
+// an item is ws0 + (row*q_heads + head)*splits + split.
 struct AttnItem {
     uint32_t slot;
     uint32_t rows;
@@ -114,7 +116,7 @@ struct AttnItem {
     uint32_t keys_per_split;
     uint32_t block0;        // first workgroup index of the item
     uint32_t ws0;           // first partial index of the item
-    uint32_t cnt0;          // first arrival counter of the item
+    uint32_t pad;
 };
 struct AttnBatch {
     uint32_t n;
@@ -130,19 +132,29 @@ struct AttnParams {
     float *out;
     const uint32_t *q_pos;  // optional explicit positions, [sum rows]
     float *ws;              // partials: (head_dim + 2) floats each
-    uint32_t *counters;     // arrival counters, zero between launches
     uint32_t q_heads;
     uint32_t group;         // q_heads / kv_heads
     float scale;
     float softcap;
 };
 
-// Generic VALU path: f32 or f16 storage, any head_dim <= 256, group <= 64.
+// Generic VALU path: f32 or f16 storage, any head_dim <= 256, group <= 64. Partials are in
+// natural-log domain (combine with base2 = 0).
 hipError_t launch_attn_generic(int elem_f16, const AttnParams &p, const AttnBatch &b,
-                               hipStream_t stream);
+                               uint32_t total_partials, hipStream_t stream);
 // Query rows one workgroup of the generic kernel carries (0 = shape not supported).
 uint32_t attn_generic_rows_per_block(uint32_t group, uint32_t head_dim);
 // Keys per tile of the generic kernel for a head_dim.
 uint32_t attn_generic_tile(uint32_t head_dim);
+
+// MFMA split-K path: f16 pools with blocked value planes, head_dim 128, rows*group <= 64.
+// Partials are in log2 domain (combine with base2 = 1).
+bool attn_splitk_f16_supports(const PoolGeom &g, uint32_t group, uint32_t max_rows);
+uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads);
+hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                                  uint32_t max_rows, hipStream_t stream);
+// Merge of split partials; total_rows = query rows of the batch.
+hipError_t launch_attn_combine(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                               uint32_t total_rows, int base2, hipStream_t stream);
 
 }  // namespace itak

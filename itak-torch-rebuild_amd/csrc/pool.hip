@@ -54,14 +54,12 @@ struct itak_pool {
     uint64_t bytes = 0;
     hipStream_t stream = nullptr;
     std::vector<Slot> slots;
-    // Device scratch, grown on demand and reused: staging for host-pointer calls,
-    // split partials and arrival counters.
+    // Device scratch, grown on demand and reused: staging for host-pointer calls and
+    // split partials.
     unsigned char *stage = nullptr;
     uint64_t stage_bytes = 0;
     float *ws = nullptr;
     uint64_t ws_floats = 0;
-    uint32_t *counters = nullptr;
-    uint64_t n_counters = 0;
     mutable ErrorState err;
 };
 
@@ -199,7 +197,7 @@ itak_status ensure_stage(itak_pool *pool, uint64_t bytes) {
     return ITAK_OK;
 }
 
-itak_status ensure_workspace(itak_pool *pool, uint64_t floats, uint64_t counters) {
+itak_status ensure_workspace(itak_pool *pool, uint64_t floats) {
     if (floats > pool->ws_floats) {
         HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize before growing workspace");
         if (pool->ws) HIP_TRY(pool, hipFree(pool->ws), "free workspace");
@@ -209,19 +207,6 @@ itak_status ensure_workspace(itak_pool *pool, uint64_t floats, uint64_t counters
         HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&pool->ws), want * sizeof(float)),
                 "allocate split workspace");
         pool->ws_floats = want;
-    }
-    if (counters > pool->n_counters) {
-        HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize before growing counters");
-        if (pool->counters) HIP_TRY(pool, hipFree(pool->counters), "free counters");
-        pool->counters = nullptr;
-        pool->n_counters = 0;
-        uint64_t want = std::max<uint64_t>(counters * 2, 4096);
-        HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&pool->counters), want * 4),
-                "allocate arrival counters");
-        // Counters are zero between launches: the merging workgroup resets its own.
-        HIP_TRY(pool, hipMemsetAsync(pool->counters, 0, want * 4, pool->stream),
-                "zero arrival counters");
-        pool->n_counters = want;
     }
     return ITAK_OK;
 }
@@ -236,13 +221,21 @@ struct PlanInput {
     uint32_t kv_len;
 };
 
-// Builds the work list for the generic kernel and launches it. q/out are device pointers.
+// Builds the work list and launches the attention kernels. q/out are device pointers.
+// f16 pools at head_dim 128 with up to 64 query vectors per KV head (decode and
+// speculative blocks) take the MFMA split-K kernel; everything else the generic kernel.
+// Either way a second small launch merges the split partials.
 itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, uint32_t n,
                           const float *q_dev, float *out_dev, const uint32_t *q_pos_dev,
                           uint64_t q_heads, float scale, float softcap) {
     const uint32_t group = uint32_t(q_heads / pool->g.kv_heads);
-    const uint32_t rpb = attn_generic_rows_per_block(group, pool->g.head_dim);
-    if (rpb == 0) return unsupported(pool->err, "head_dim above 256 or GQA group too wide");
+    uint32_t max_rows = 0;
+    for (uint32_t i = 0; i < n; ++i) max_rows = std::max(max_rows, in[i].rows);
+    const bool mfma = pool->elem_f16 && q_pos_dev == nullptr &&
+                      attn_splitk_f16_supports(pool->g, group, max_rows);
+    const uint32_t rpb = mfma ? 0 : attn_generic_rows_per_block(group, pool->g.head_dim);
+    if (!mfma && rpb == 0)
+        return unsupported(pool->err, "head_dim above 256 or GQA group too wide");
     const uint32_t tile = attn_generic_tile(pool->g.head_dim);
     constexpr uint64_t kTargetBlocks = 1024;  // about four workgroups per CU
 
@@ -251,17 +244,7 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         const uint32_t count = std::min<uint32_t>(kMaxBatchItems, n - first);
         AttnBatch b{};
         b.n = count;
-        b.rows_per_block = rpb;
-        uint64_t key_work = 0;
-        for (uint32_t i = 0; i < count; ++i) {
-            const PlanInput &pi = in[first + i];
-            const uint64_t qblocks = (pi.rows + rpb - 1) / rpb;
-            key_work += qblocks * pool->g.kv_heads * pi.kv_len;
-        }
-        uint64_t kps = align_up(std::max<uint64_t>((key_work + kTargetBlocks - 1) / kTargetBlocks,
-                                                   tile),
-                                tile);
-        uint32_t block0 = 0, ws0 = 0, cnt0 = 0;
+        uint32_t total_rows = 0;
         for (uint32_t i = 0; i < count; ++i) {
             const PlanInput &pi = in[first + i];
             AttnItem &it = b.item[i];
@@ -270,21 +253,40 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
             it.pos0 = pi.pos0;
             it.q_row0 = q_row0;
             it.kv_len = pi.kv_len;
-            it.keys_per_split = uint32_t(kps);
-            it.splits = uint32_t((pi.kv_len + kps - 1) / kps);
-            if (it.splits == 0) it.splits = 1;
-            const uint32_t qblocks = (pi.rows + rpb - 1) / rpb;
-            it.block0 = block0;
-            it.ws0 = ws0;
-            it.cnt0 = cnt0;
-            block0 += qblocks * pool->g.kv_heads * it.splits;
-            if (it.splits > 1) ws0 += pi.rows * uint32_t(q_heads) * it.splits;
-            cnt0 += qblocks * pool->g.kv_heads;
             q_row0 += pi.rows;
+            total_rows += pi.rows;
         }
-        b.total_blocks = block0;
-        itak_status st =
-            ensure_workspace(pool, uint64_t(ws0) * (pool->g.head_dim + 2), cnt0);
+        uint32_t partials = 0;
+        if (mfma) {
+            partials = attn_splitk_f16_plan(pool->g, b, uint32_t(q_heads));
+        } else {
+            b.rows_per_block = rpb;
+            uint64_t key_work = 0;
+            for (uint32_t i = 0; i < count; ++i) {
+                const uint64_t qblocks = (b.item[i].rows + rpb - 1) / rpb;
+                key_work += qblocks * pool->g.kv_heads * b.item[i].kv_len;
+            }
+            const uint64_t kps = align_up(
+                std::max<uint64_t>((key_work + kTargetBlocks - 1) / kTargetBlocks, tile), tile);
+            uint32_t block0 = 0;
+            for (uint32_t i = 0; i < count; ++i) {
+                AttnItem &it = b.item[i];
+                it.keys_per_split = uint32_t(kps);
+                it.splits = uint32_t((it.kv_len + kps - 1) / kps);
+                if (it.splits == 0) it.splits = 1;
+                if (it.splits > 1024) {  // the merge kernel holds at most 1024 weights
+                    it.keys_per_split = uint32_t(align_up((it.kv_len + 1023) / 1024, tile));
+                    it.splits = (it.kv_len + it.keys_per_split - 1) / it.keys_per_split;
+                }
+                const uint32_t qblocks = (it.rows + rpb - 1) / rpb;
+                it.block0 = block0;
+                it.ws0 = partials;
+                block0 += qblocks * pool->g.kv_heads * it.splits;
+                if (it.splits > 1) partials += it.rows * uint32_t(q_heads) * it.splits;
+            }
+            b.total_blocks = block0;
+        }
+        itak_status st = ensure_workspace(pool, uint64_t(partials) * (pool->g.head_dim + 2));
         if (st != ITAK_OK) return st;
         AttnParams p{};
         p.layer_base = layer_base(pool, layer);
@@ -293,13 +295,19 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         p.out = out_dev;
         p.q_pos = q_pos_dev;
         p.ws = pool->ws;
-        p.counters = pool->counters;
         p.q_heads = uint32_t(q_heads);
         p.group = group;
         p.scale = scale;
         p.softcap = softcap;
-        HIP_TRY(pool, launch_attn_generic(pool->elem_f16, p, b, pool->stream),
-                "launch attention");
+        if (mfma) {
+            HIP_TRY(pool, launch_attn_splitk_f16(p, b, partials, max_rows, pool->stream),
+                    "launch split-K attention");
+        } else {
+            HIP_TRY(pool, launch_attn_generic(pool->elem_f16, p, b, partials, pool->stream),
+                    "launch attention");
+        }
+        HIP_TRY(pool, launch_attn_combine(p, b, partials, total_rows, mfma ? 1 : 0, pool->stream),
+                "launch split merge");
     }
     return ITAK_OK;
 }
@@ -502,7 +510,6 @@ void itak_pool_destroy(itak_pool *pool) {
     if (pool->base) (void)hipFree(pool->base);
     if (pool->stage) (void)hipFree(pool->stage);
     if (pool->ws) (void)hipFree(pool->ws);
-    if (pool->counters) (void)hipFree(pool->counters);
     delete pool;
 }
 
