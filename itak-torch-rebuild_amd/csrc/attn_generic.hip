@@ -45,8 +45,8 @@ __device__ __forceinline__ Shape make_shape(uint32_t d) {
     return s;
 }
 
-template <typename T, int VEC>
-__global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p, AttnBatch b,
+template <typename T, int VEC, int N>
+__global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p, AttnBatchT<N> b,
                                                                 uint32_t total_partials) {
     extern __shared__ float lds[];
     const Shape sh = make_shape<VEC>(p.g.head_dim);
@@ -62,9 +62,7 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p, At
     const uint32_t tid = threadIdx.x;
 
     // ---- which work item is this workgroup? -------------------------------------
-    uint32_t it = 0;
-    while (it + 1 < b.n && blockIdx.x >= b.item[it + 1].block0) ++it;
-    const AttnItem item = b.item[it];
+    const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
     const uint32_t local = blockIdx.x - item.block0;
     const uint32_t split = local % item.splits;
     const uint32_t rest = local / item.splits;
@@ -124,10 +122,10 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p, At
             const uint32_t kj = i / sh.ncol, c = (i % sh.ncol) * VEC;
             float kv[VEC], vv[VEC];
             if (kj < tn) {
-                const uint64_t off = uint64_t(t0 + kj) * D + c;
+                const uint64_t koff = k_offset(p.g, t0 + kj, c);  // VEC channels share a piece
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
-                    kv[e] = to_f32(kplane[off + e]);
+                    kv[e] = to_f32(kplane[koff + e]);
                     vv[e] = to_f32(vplane[v_offset(p.g, t0 + kj, c + e)]);
                 }
             } else {
@@ -314,24 +312,30 @@ hipError_t launch_attn_generic(int elem_f16, const AttnParams &p, const AttnBatc
         static size_t granted = 64 * 1024;                                                       \
         if (lds > granted) {                                                                     \
             hipError_t e = hipFuncSetAttribute(                                                  \
-                reinterpret_cast<const void *>(&attn_generic_kernel<T, V>),                      \
+                reinterpret_cast<const void *>(&attn_generic_kernel<T, V, N>),                   \
                 hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));                           \
             if (e != hipSuccess) return e;                                                       \
             granted = lds;                                                                       \
         }                                                                                        \
-        attn_generic_kernel<T, V><<<b.total_blocks, kThreads, lds, stream>>>(p, b, total_partials); \
+        attn_generic_kernel<T, V, N><<<b.total_blocks, kThreads, lds, stream>>>(                 \
+            p, AttnBatchT<N>(b), total_partials);                                                \
     } while (0)
-    if (elem_f16) {
-        if (vec == 4)
-            ITAK_LAUNCH(uint16_t, 4);
-        else
-            ITAK_LAUNCH(uint16_t, 1);
-    } else {
-        if (vec == 4)
-            ITAK_LAUNCH(float, 4);
-        else
-            ITAK_LAUNCH(float, 1);
-    }
+#define ITAK_LAUNCH_TV()                 \
+    do {                                 \
+        if (elem_f16) {                  \
+            if (vec == 4)                \
+                ITAK_LAUNCH(uint16_t, 4);\
+            else                         \
+                ITAK_LAUNCH(uint16_t, 1);\
+        } else {                         \
+            if (vec == 4)                \
+                ITAK_LAUNCH(float, 4);   \
+            else                         \
+                ITAK_LAUNCH(float, 1);   \
+        }                                \
+    } while (0)
+    ITAK_DISPATCH_BATCH(b.n, ITAK_LAUNCH_TV());
+#undef ITAK_LAUNCH_TV
 #undef ITAK_LAUNCH
     return hipGetLastError();
 }

@@ -36,6 +36,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kD = 128;          // head_dim this kernel is written for
 constexpr int kBlockKeys = 32;   // keys per block (= value plane block)
+constexpr int kQStride = kD + 8; // LDS row stride of the staged queries (halves)
 constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -66,23 +67,84 @@ __device__ __forceinline__ void load_block(BlockOperands &b, const uint16_t *kpl
                                            uint32_t i) {
     // Key rows of MFMA tile t are interleaved so that the lane group g ends up holding
     // scores of the 8 consecutive keys g*8 .. g*8+7: row i of tile t is key
-    // (i/4)*8 + t*4 + i%4 of the block.
-    const uint32_t key0 = kb * kBlockKeys + (i >> 2) * 8 + (i & 3);
+    // (i/4)*8 + t*4 + i%4 of the block. The blocked key plane stores the 16-byte piece
+    // (tile t, channel chunk c, row i) at ((t*16 + c)*16 + i)*8, so the 64 lanes of the load
+    // for (t, s) (chunks s*4 .. s*4+3, rows 0..15) read 1 KiB of contiguous memory.
+    const uint16_t *kb_base = kplane + uint64_t(kb) * (kBlockKeys * kD) + (g * 16 + i) * 8;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        const uint16_t *row = kplane + uint64_t(key0 + t * 4) * kD + g * 8;
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int s = 0; s < 4; ++s) b.k[t][s] = *reinterpret_cast<const half8 *>(row + s * 32);
-    }
+        for (int s = 0; s < 4; ++s)
+            b.k[t][s] = *reinterpret_cast<const half8 *>(kb_base + ((t * 16 + s * 4) * 16) * 8);
     const uint16_t *vb = vplane + uint64_t(kb) * (kBlockKeys * kD) + i * kBlockKeys + g * 8;
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt)
         b.v[dt] = *reinterpret_cast<const half8 *>(vb + dt * 16 * kBlockKeys);
 }
 
+// Fused append for a block that contains new positions [pos0, kv_len): the operands the
+// wavefront holds for those keys are replaced by the converted source rows (bit-identical
+// to what the cache will hold), and the wavefront stores the rows into the planes. No other
+// wavefront reads these positions, so nothing depends on the stores within the launch.
+__device__ __forceinline__ half8 convert8(const float *src) {
+    const float4 a = *reinterpret_cast<const float4 *>(src);
+    const float4 c = *reinterpret_cast<const float4 *>(src + 4);
+    const uint16_t h[8] = {f32_to_f16_bits(a.x), f32_to_f16_bits(a.y), f32_to_f16_bits(a.z),
+                           f32_to_f16_bits(a.w), f32_to_f16_bits(c.x), f32_to_f16_bits(c.y),
+                           f32_to_f16_bits(c.z), f32_to_f16_bits(c.w)};
+    half8 out;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = __builtin_bit_cast(_Float16, h[e]);
+    return out;
+}
+
+__device__ __forceinline__ void patch_and_store_new_rows(BlockOperands &b, uint16_t *kplane,
+                                                         uint16_t *vplane, const float *k_new,
+                                                         const float *v_new, uint32_t row_width,
+                                                         uint32_t kb, uint32_t g, uint32_t i,
+                                                         uint32_t lane, uint32_t pos0,
+                                                         uint32_t kv_len) {
+    // k_new / v_new already point at this item's first new row and this KV head.
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const uint32_t key = kb * kBlockKeys + (i >> 2) * 8 + t * 4 + (i & 3);
+        if (key >= pos0 && key < kv_len) {
+            const float *src = k_new + uint64_t(key - pos0) * row_width + g * 8;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) b.k[t][s] = convert8(src + s * 32);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const uint32_t key = kb * kBlockKeys + g * 8 + e;
+        if (key >= pos0 && key < kv_len) {
+            const float *src = v_new + uint64_t(key - pos0) * row_width + i;
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt)
+                b.v[dt][e] = __builtin_bit_cast(_Float16, f32_to_f16_bits(src[dt * 16]));
+        }
+    }
+    // Store: lane owns channels 2*lane and 2*lane + 1 of every new row in this block.
+    const uint32_t first = max(pos0, kb * kBlockKeys);
+    const uint32_t last = min(kv_len, (kb + 1) * kBlockKeys);
+    for (uint32_t key = first; key < last; ++key) {
+        const float2 kk = *reinterpret_cast<const float2 *>(k_new + uint64_t(key - pos0) * row_width + lane * 2);
+        const float2 vv = *reinterpret_cast<const float2 *>(v_new + uint64_t(key - pos0) * row_width + lane * 2);
+        const uint32_t packed = uint32_t(f32_to_f16_bits(kk.x)) | (uint32_t(f32_to_f16_bits(kk.y)) << 16);
+        const uint32_t kin = key % kBlockKeys;
+        const uint32_t kt = (kin >> 2) & 1, ki = (kin >> 3) * 4 + (kin & 3);
+        *reinterpret_cast<uint32_t *>(kplane + uint64_t(key / kBlockKeys) * (kBlockKeys * kD) +
+                                      ((kt * 16 + (lane >> 2)) * 16 + ki) * 8 + (lane & 3) * 2) = packed;
+        uint16_t *vd = vplane + uint64_t(key / kBlockKeys) * (kBlockKeys * kD) +
+                       (lane * 2) * kBlockKeys + key % kBlockKeys;
+        vd[0] = f32_to_f16_bits(vv.x);
+        vd[kBlockKeys] = f32_to_f16_bits(vv.y);
+    }
+}
+
 template <int NQ>
 __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &b,
-                                              const half8 (&qb)[NQ][4], uint32_t kb, uint32_t g,
+                                              const _Float16 *sm_q, uint32_t kb, uint32_t g,
                                               uint32_t jl, uint32_t pos0, uint32_t group,
                                               uint32_t kv_len, float softcap, float inv_cap) {
     const uint32_t key_base = kb * kBlockKeys + g * 8;  // first of this lane's 8 keys
@@ -98,13 +160,19 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
     const bool need_mask = (kb + 1) * kBlockKeys > pos0 + 1;
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
+        // Q^T operand of this tile: lane (g, jl) holds channels k*32 + g*8 .. +8 of vector jl.
+        half8 qb[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            qb[k] = *reinterpret_cast<const half8 *>(sm_q + (qt * 16 + jl) * kQStride + k * 32 +
+                                                     g * 8);
         floatx4 s[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             s[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int k = 0; k < 4; ++k)
-                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b.k[t][k], qb[qt][k], s[t], 0, 0, 0);
+                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b.k[t][k], qb[k], s[t], 0, 0, 0);
         }
         float sc[8];
 #pragma unroll
@@ -150,30 +218,33 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
     }
 }
 
-template <int NQ, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams p, AttnBatch b,
+template <int NQ, int WAVES, int N>
+__global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams p, AttnBatchT<N> b,
                                                                      uint32_t total_partials) {
     extern __shared__ float lds[];
     float *sm_m = lds;                          // [WAVES][NQ*16]
     float *sm_l = sm_m + WAVES * NQ * 16;       // [WAVES][NQ*16]
     float *sm_o = sm_l + WAVES * NQ * 16;       // [WAVES][NQ][8][64][4]
+    _Float16 *sm_q = reinterpret_cast<_Float16 *>(sm_o + WAVES * NQ * 8 * 64 * 4);  // [NQ*16][kQStride]
 
     const uint32_t tid = threadIdx.x;
     const uint32_t wave = tid >> 6, lane = tid & 63;
     const uint32_t g = lane >> 4, jl = lane & 15;
 
-    uint32_t it = 0;
-    while (it + 1 < b.n && blockIdx.x >= b.item[it + 1].block0) ++it;
-    const AttnItem item = b.item[it];
+    const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
     const uint32_t local = blockIdx.x - item.block0;
     const uint32_t split = local % item.splits;
     const uint32_t kv_head = local / item.splits;
     const uint32_t group = p.group;
     const uint32_t nvec = item.rows * group;
 
-    const uint16_t *kplane = static_cast<const uint16_t *>(p.layer_base) +
-                             item.slot * p.g.slot_stride + kv_head * p.g.head_stride;
-    const uint16_t *vplane = kplane + p.g.side_stride;
+    uint16_t *kplane = static_cast<uint16_t *>(const_cast<void *>(p.layer_base)) +
+                       item.slot * p.g.slot_stride + kv_head * p.g.head_stride;
+    uint16_t *vplane = kplane + p.g.side_stride;
+    const uint32_t row_width = p.g.kv_heads * kD;
+    const bool fused = p.k_new != nullptr;
+    const float *k_new = fused ? p.k_new + uint64_t(item.q_row0) * row_width + kv_head * kD : nullptr;
+    const float *v_new = fused ? p.v_new + uint64_t(item.q_row0) * row_width + kv_head * kD : nullptr;
 
     const uint32_t nblocks = (item.kv_len + kBlockKeys - 1) / kBlockKeys;
     const uint32_t blocks_per_split = item.keys_per_split / kBlockKeys;
@@ -181,36 +252,45 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
     const uint32_t kb_end = min(nblocks, kb_begin + blocks_per_split);
 
     // Start the first block's loads before anything else: this kernel is latency bound.
-    BlockOperands buf_a, buf_b;
+    BlockOperands buf_a;
+    [[maybe_unused]] BlockOperands buf_b;
     uint32_t kb = kb_begin + wave;
     if (kb < kb_end) load_block(buf_a, kplane, vplane, kb, g, jl);
 
     // ---- Q^T as the B operand: lane (g, jl) holds channels s*32 + g*8 .. +8 of vector jl.
+    // The workgroup reads its query vectors once, coalesced, scales and converts them to
+    // f16 into LDS; each wavefront reads its operand registers from there per block.
     const float softcap = p.softcap;
     const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
     const float qscale = softcap > 0.0f ? p.scale : p.scale * kLog2e;
-    half8 qb[NQ][4];
-#pragma unroll
-    for (int qt = 0; qt < NQ; ++qt) {
-        const uint32_t j = qt * 16 + jl;
+    for (uint32_t f = tid; f < NQ * 16 * (kD / 4); f += WAVES * 64) {
+        const uint32_t j = f / (kD / 4), c4 = (f % (kD / 4)) * 4;
+        half4 h{0, 0, 0, 0};
         if (j < nvec) {
             const uint32_t row = j / group, head = kv_head * group + j % group;
-            const float *qp = p.q + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + g * 8;
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const float4 a = *reinterpret_cast<const float4 *>(qp + s * 32);
-                const float4 c = *reinterpret_cast<const float4 *>(qp + s * 32 + 4);
-                qb[qt][s] = half8{static_cast<_Float16>(a.x * qscale), static_cast<_Float16>(a.y * qscale),
-                                  static_cast<_Float16>(a.z * qscale), static_cast<_Float16>(a.w * qscale),
-                                  static_cast<_Float16>(c.x * qscale), static_cast<_Float16>(c.y * qscale),
-                                  static_cast<_Float16>(c.z * qscale), static_cast<_Float16>(c.w * qscale)};
-            }
-        } else {
-#pragma unroll
-            for (int s = 0; s < 4; ++s) qb[qt][s] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+            const float4 a = *reinterpret_cast<const float4 *>(
+                p.q + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + c4);
+            h = half4{static_cast<_Float16>(a.x * qscale), static_cast<_Float16>(a.y * qscale),
+                      static_cast<_Float16>(a.z * qscale), static_cast<_Float16>(a.w * qscale)};
         }
+        *reinterpret_cast<half4 *>(sm_q + j * kQStride + c4) = h;
     }
+    __syncthreads();
 
+    if (p.dbg == 1) {  // loads only
+        float acc = 0.0f;
+        if (kb < kb_end) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int s = 0; s < 4; ++s) acc += float(buf_a.k[t][s][0]);
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) acc += float(buf_a.v[dt][0]);
+        }
+        acc += float(sm_q[jl]);
+        if (acc == 1234.5f) p.out[0] = acc;
+        return;
+    }
     WaveState<NQ> st;
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
@@ -220,26 +300,50 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
         for (int dt = 0; dt < 8; ++dt) st.o[qt][dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
-    // ---- this wavefront's blocks, two register sets so the next block's loads fly while
-    // the current one is multiplied.
-    if (kb < kb_end) {
-        for (;;) {
-            const uint32_t kb2 = kb + WAVES;
-            const bool has2 = kb2 < kb_end;
-            if (has2) load_block(buf_b, kplane, vplane, kb2, g, jl);
-            process_block<NQ>(st, buf_a, qb, kb, g, jl, item.pos0, group, item.kv_len, softcap,
+    // ---- this wavefront's blocks. Up to 32 query vectors there are registers for two
+    // operand sets, so the next block's loads fly while the current one is multiplied; with
+    // 64 vectors the accumulators take that room and the other wavefronts hide the latency.
+    if constexpr (NQ <= 2) {
+        if (kb < kb_end) {
+            for (;;) {
+                const uint32_t kb2 = kb + WAVES;
+                const bool has2 = kb2 < kb_end;
+                if (has2) load_block(buf_b, kplane, vplane, kb2, g, jl);
+                if (fused && (kb + 1) * kBlockKeys > item.pos0)
+                    patch_and_store_new_rows(buf_a, kplane, vplane, k_new, v_new, row_width, kb, g,
+                                             jl, lane, item.pos0, item.kv_len);
+                process_block<NQ>(st, buf_a, sm_q, kb, g, jl, item.pos0, group, item.kv_len,
+                                  softcap, inv_cap);
+                if (!has2) break;
+                const uint32_t kb3 = kb2 + WAVES;
+                const bool has3 = kb3 < kb_end;
+                if (has3) load_block(buf_a, kplane, vplane, kb3, g, jl);
+                if (fused && (kb2 + 1) * kBlockKeys > item.pos0)
+                    patch_and_store_new_rows(buf_b, kplane, vplane, k_new, v_new, row_width, kb2, g,
+                                             jl, lane, item.pos0, item.kv_len);
+                process_block<NQ>(st, buf_b, sm_q, kb2, g, jl, item.pos0, group, item.kv_len,
+                                  softcap, inv_cap);
+                if (!has3) break;
+                kb = kb3;
+            }
+        }
+    } else {
+        while (kb < kb_end) {
+            if (fused && (kb + 1) * kBlockKeys > item.pos0)
+                patch_and_store_new_rows(buf_a, kplane, vplane, k_new, v_new, row_width, kb, g, jl,
+                                         lane, item.pos0, item.kv_len);
+            process_block<NQ>(st, buf_a, sm_q, kb, g, jl, item.pos0, group, item.kv_len, softcap,
                               inv_cap);
-            if (!has2) break;
-            const uint32_t kb3 = kb2 + WAVES;
-            const bool has3 = kb3 < kb_end;
-            if (has3) load_block(buf_a, kplane, vplane, kb3, g, jl);
-            process_block<NQ>(st, buf_b, qb, kb2, g, jl, item.pos0, group, item.kv_len, softcap,
-                              inv_cap);
-            if (!has3) break;
-            kb = kb3;
+            kb += WAVES;
+            if (kb < kb_end) load_block(buf_a, kplane, vplane, kb, g, jl);
         }
     }
 
+    if (p.dbg == 2) {  // no merge, no writes
+        float acc = st.m[0] + st.l[0] + st.o[0][0][0] + st.o[0][7][3];
+        if (acc == 1234.5f) p.out[0] = acc;
+        return;
+    }
     // ---- merge the wavefronts through LDS ------------------------------------------------
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
@@ -348,82 +452,150 @@ hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint3
     constexpr int W = 4;
 #define ITAK_LAUNCH(NQ)                                                                          \
     do {                                                                                         \
-        const size_t lds = (size_t(2) * W * NQ * 16 + size_t(W) * NQ * 8 * 64 * 4) * 4;           \
+        const size_t lds = (size_t(2) * W * NQ * 16 + size_t(W) * NQ * 8 * 64 * 4) * 4 +          \
+                           size_t(NQ) * 16 * kQStride * 2;                                       \
         static size_t granted = 64 * 1024;                                                       \
         if (lds > granted) {                                                                     \
             hipError_t e = hipFuncSetAttribute(                                                  \
-                reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W>),                  \
+                reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, N>),               \
                 hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));                           \
             if (e != hipSuccess) return e;                                                       \
             granted = lds;                                                                       \
         }                                                                                        \
-        attn_splitk_f16_kernel<NQ, W><<<b.total_blocks, W * 64, lds, stream>>>(p, b,              \
-                                                                               total_partials); \
+        attn_splitk_f16_kernel<NQ, W, N><<<b.total_blocks, W * 64, lds, stream>>>(               \
+            p, AttnBatchT<N>(b), total_partials);                                                \
     } while (0)
-    if (nvec <= 16)
-        ITAK_LAUNCH(1);
-    else if (nvec <= 32)
-        ITAK_LAUNCH(2);
-    else
-        ITAK_LAUNCH(4);
+#define ITAK_LAUNCH_NQ()             \
+    do {                             \
+        if (nvec <= 16)              \
+            ITAK_LAUNCH(1);          \
+        else if (nvec <= 32)         \
+            ITAK_LAUNCH(2);          \
+        else                         \
+            ITAK_LAUNCH(4);          \
+    } while (0)
+    ITAK_DISPATCH_BATCH(b.n, ITAK_LAUNCH_NQ());
+#undef ITAK_LAUNCH_NQ
 #undef ITAK_LAUNCH
     return hipGetLastError();
 }
 
 // ------------------------------------------------------------------------------ combine
-// Merges the split partials of one (query row, Q head): weights exp(m_s - M), output
-// sum_s w_s * acc_s / sum_s w_s * l_s. One 128-thread workgroup per (row, head); thread =
-// channel. grid = all (row, head) pairs of the batch, items whose splits == 1 exit at once.
-__global__ __launch_bounds__(128) void attn_combine_kernel(AttnParams p, AttnBatch b,
-                                                           uint32_t total_partials, int base2) {
+// Merges the split partials of one (query row, Q head): weights w_s = exp(m_s - M), output
+// sum_s w_s * acc_s / sum_s w_s * l_s. One 256-thread workgroup per (row, head): thread =
+// (4 channels, one of 8 split lanes). Every thread issues all its accumulator loads before
+// the weights are known, so the merge costs one memory round trip, not one per split.
+// grid = all (row, head) pairs of the batch; items whose splits == 1 exit at once.
+constexpr int kCombineThreads = 256;
+constexpr int kCombineMaxLoads = 8;  // accumulator loads in flight per thread and pass
+
+template <int N>
+__global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(AttnParams p,
+                                                                       AttnBatchT<N> b,
+                                                                       uint32_t total_partials,
+                                                                       int base2) {
     __shared__ float w_s[1024];
-    __shared__ float red[4];
+    __shared__ float red[8];
+    __shared__ float4 part[kCombineThreads];
     const uint32_t tid = threadIdx.x;
     const uint32_t D = p.g.head_dim;
-    // blockIdx.x -> (item, row, head): items are laid out by q_row0.
     const uint32_t pair = blockIdx.x;
     const uint32_t grow = pair / p.q_heads, head = pair % p.q_heads;
-    uint32_t it = 0;
-    while (it + 1 < b.n && grow >= b.item[it + 1].q_row0 - b.item[0].q_row0) ++it;
-    const AttnItem item = b.item[it];
+    const AttnItem item = b.item[b.find_by_row(grow)];
     if (item.splits == 1) return;
-    const uint32_t row = grow - (item.q_row0 - b.item[0].q_row0);
+    const uint32_t row = grow - (item.q_row0 - b.base_row);
     const uint64_t ps0 = item.ws0 + (uint64_t(row) * p.q_heads + head) * item.splits;
-    const float *ws_acc = p.ws;
-    const float *ws_ml = p.ws + uint64_t(total_partials) * D;
+    const float *ws_acc = p.ws + ps0 * D;
+    const float *ws_ml = p.ws + uint64_t(total_partials) * D + ps0 * 2;
+    const uint32_t S = item.splits;
 
+    // Thread layout for the accumulators: chunk c of 4 channels, split lane sl.
+    const uint32_t chunks = (D + 3) / 4;                       // 32 for head_dim 128
+    const uint32_t lanes = kCombineThreads / chunks ? kCombineThreads / chunks : 1;
+    const uint32_t c = tid % chunks, sl = tid / chunks;
+    const bool vec_ok = (D % 4 == 0) && sl < lanes;
+
+    // First pass of accumulator loads goes out before anything waits on m/l.
+    float4 x[kCombineMaxLoads];
+    if (vec_ok) {
+#pragma unroll
+        for (int u = 0; u < kCombineMaxLoads; ++u) {
+            const uint32_t s = sl + u * lanes;
+            x[u] = s < S ? *reinterpret_cast<const float4 *>(ws_acc + uint64_t(s) * D + c * 4)
+                         : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
     float mx = -INFINITY;
-    for (uint32_t s = tid; s < item.splits; s += 128) mx = fmaxf(mx, ws_ml[(ps0 + s) * 2]);
+    for (uint32_t s = tid; s < S; s += kCombineThreads) mx = fmaxf(mx, ws_ml[s * 2]);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
     if ((tid & 63) == 0) red[tid >> 6] = mx;
     __syncthreads();
-    const float M = fmaxf(red[0], red[1]);
+    const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     float lsum = 0.0f;
-    for (uint32_t s = tid; s < item.splits; s += 128) {
-        const float ms = ws_ml[(ps0 + s) * 2];
+    for (uint32_t s = tid; s < S; s += kCombineThreads) {
+        const float ms = ws_ml[s * 2];
         const float w = (ms == -INFINITY) ? 0.0f : (base2 ? exp2f(ms - M) : expf(ms - M));
         w_s[s] = w;
-        lsum += w * ws_ml[(ps0 + s) * 2 + 1];
+        lsum += w * ws_ml[s * 2 + 1];
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) lsum += __shfl_xor(lsum, o);
-    if ((tid & 63) == 0) red[2 + (tid >> 6)] = lsum;
+    if ((tid & 63) == 0) red[4 + (tid >> 6)] = lsum;
     __syncthreads();
-    const float inv = 1.0f / (red[2] + red[3]);
-    for (uint32_t d = tid; d < D; d += 128) {
-        const float *a = ws_acc + ps0 * D + d;
-        float acc = 0.0f;
-        uint32_t s = 0;
-        for (; s + 8 <= item.splits; s += 8) {
-            float x[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) x[u] = a[uint64_t(s + u) * D];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) acc = fmaf(x[u], w_s[s + u], acc);
+    const float inv = 1.0f / (red[4] + red[5] + red[6] + red[7]);
+    float *dst = p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * D;
+
+    if (D % 4 != 0) {  // scalar path for odd head dims
+        for (uint32_t d = tid; d < D; d += kCombineThreads) {
+            float acc = 0.0f;
+            for (uint32_t s = 0; s < S; ++s) acc = fmaf(ws_acc[uint64_t(s) * D + d], w_s[s], acc);
+            dst[d] = acc * inv;
         }
-        for (; s < item.splits; ++s) acc = fmaf(a[uint64_t(s) * D], w_s[s], acc);
-        p.out[(uint64_t(item.q_row0 + row) * p.q_heads + head) * D + d] = acc * inv;
+        return;
+    }
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (vec_ok) {
+#pragma unroll
+        for (int u = 0; u < kCombineMaxLoads; ++u) {
+            const uint32_t s = sl + u * lanes;
+            const float w = s < S ? w_s[s] : 0.0f;
+            acc.x = fmaf(x[u].x, w, acc.x);
+            acc.y = fmaf(x[u].y, w, acc.y);
+            acc.z = fmaf(x[u].z, w, acc.z);
+            acc.w = fmaf(x[u].w, w, acc.w);
+        }
+        for (uint32_t s0 = kCombineMaxLoads * lanes; s0 < S; s0 += kCombineMaxLoads * lanes) {
+#pragma unroll
+            for (int u = 0; u < kCombineMaxLoads; ++u) {
+                const uint32_t s = s0 + sl + u * lanes;
+                x[u] = s < S ? *reinterpret_cast<const float4 *>(ws_acc + uint64_t(s) * D + c * 4)
+                             : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int u = 0; u < kCombineMaxLoads; ++u) {
+                const uint32_t s = s0 + sl + u * lanes;
+                const float w = s < S ? w_s[s] : 0.0f;
+                acc.x = fmaf(x[u].x, w, acc.x);
+                acc.y = fmaf(x[u].y, w, acc.y);
+                acc.z = fmaf(x[u].z, w, acc.z);
+                acc.w = fmaf(x[u].w, w, acc.w);
+            }
+        }
+    }
+    part[tid] = acc;
+    __syncthreads();
+    if (tid < chunks) {
+        float4 sum = part[tid];
+        for (uint32_t l = 1; l < lanes; ++l) {
+            const float4 y = part[tid + l * chunks];
+            sum.x += y.x;
+            sum.y += y.y;
+            sum.z += y.z;
+            sum.w += y.w;
+        }
+        *reinterpret_cast<float4 *>(dst + tid * 4) =
+            make_float4(sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv);
     }
 }
 
@@ -432,7 +604,9 @@ hipError_t launch_attn_combine(const AttnParams &p, const AttnBatch &b, uint32_t
     bool any = false;
     for (uint32_t i = 0; i < b.n; ++i) any = any || b.item[i].splits > 1;
     if (!any || total_rows == 0) return hipSuccess;
-    attn_combine_kernel<<<total_rows * p.q_heads, 128, 0, stream>>>(p, b, total_partials, base2);
+    ITAK_DISPATCH_BATCH(b.n, (attn_combine_kernel<N><<<total_rows * p.q_heads, kCombineThreads, 0,
+                                                      stream>>>(p, AttnBatchT<N>(b), total_partials,
+                                                                base2)));
     return hipGetLastError();
 }
 

@@ -12,12 +12,18 @@ namespace itak {
 // so a workgroup that streams one KV head reads one unbroken run of memory.
 //   plane(layer, slot, side, head) =
 //     layer*layer_stride + slot*slot_stride + side*side_stride + head*head_stride
-// side 0 = keys, 1 = values. Key planes are row-major: row*head_dim + d. Value planes are
-// row-major too unless v_block != 0: then they are stored in blocks of v_block (= 32) rows,
-// each block transposed, element (row, d) at
-//     (row / 32) * 32 * head_dim + d * 32 + row % 32
-// so that the 8 consecutive rows an MFMA lane needs for one channel are 16 contiguous
-// bytes and a wavefront's operand load covers 1 KiB of contiguous memory.
+// side 0 = keys, 1 = values. With v_block == 0 both are row-major (row*head_dim + d).
+// With v_block == 32 (f16 pools whose head_dim is a multiple of 16) both are stored in
+// blocks of 32 rows laid out as the MFMA kernels consume them, so that every operand load
+// of a wavefront is 64 lanes x 16 bytes of contiguous memory:
+//   values: block transposed, element (row, d) at
+//       (row/32)*32*head_dim + d*32 + row%32
+//     (a lane's 8 consecutive rows of one channel are 16 contiguous bytes);
+//   keys: 16-byte pieces of 8 channels, grouped by MFMA tile t and channel chunk c, element
+//     (row, d) with kk = row%32, t = (kk/4)%2, i = (kk/8)*4 + kk%4, c = d/8 at
+//       (row/32)*32*head_dim + ((t*(head_dim/8) + c)*16 + i)*8 + d%8
+//     (tile t holds the 16 rows whose scores one lane group receives as 8 consecutive
+//     keys; the lanes (chunk c, row i) of one load instruction are adjacent in memory).
 struct PoolGeom {
     uint32_t kv_heads;
     uint32_t head_dim;
@@ -37,6 +43,35 @@ constexpr uint32_t kVBlock = 32;
 __host__ __device__ inline uint64_t v_offset(const PoolGeom &g, uint32_t row, uint32_t d) {
     if (g.v_block == 0) return uint64_t(row) * g.head_dim + d;
     return uint64_t(row / kVBlock) * (kVBlock * g.head_dim) + uint64_t(d) * kVBlock + row % kVBlock;
+}
+
+// Element offset of (row, d) inside a key plane.
+__host__ __device__ inline uint64_t k_offset(const PoolGeom &g, uint32_t row, uint32_t d) {
+    if (g.v_block == 0) return uint64_t(row) * g.head_dim + d;
+    const uint32_t kk = row % kVBlock;
+    const uint32_t t = (kk >> 2) & 1, i = (kk >> 3) * 4 + (kk & 3);
+    return uint64_t(row / kVBlock) * (kVBlock * g.head_dim) +
+           ((t * (g.head_dim / 8) + d / 8) * 16 + i) * 8 + d % 8;
+}
+
+// Element offset inside a plane of either side.
+__host__ __device__ inline uint64_t kv_offset(const PoolGeom &g, uint32_t side, uint32_t row,
+                                              uint32_t d) {
+    return side ? v_offset(g, row, d) : k_offset(g, row, d);
+}
+
+// f32 -> f16 bits, round-to-nearest-even, overflow to infinity, subnormals rounded, and
+// every NaN stored as sign|0x7e00: the rule of f32_to_f16_bits in
+// crates/wgpu-compute/src/kernels/k1_q4k_gemv.rs:285-329. v_cvt_f16_f32 implements all of
+// it except the NaN payload, which is replaced explicitly.
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float x) {
+    _Float16 h = static_cast<_Float16>(x);
+    uint16_t bits = __builtin_bit_cast(uint16_t, h);
+    uint32_t in = __builtin_bit_cast(uint32_t, x);
+    if ((in & 0x7fffffffu) > 0x7f800000u) {
+        bits = static_cast<uint16_t>(((in >> 16) & 0x8000u) | 0x7e00u);
+    }
+    return bits;
 }
 
 constexpr int kMaxBatchItems = 64;
@@ -125,6 +160,63 @@ struct AttnBatch {
     uint32_t pad;
     AttnItem item[kMaxBatchItems];
 };
+// The kernel argument form of AttnBatch, sized to the batch: kernel arguments are
+// expensive to read on this GPU (a 2.6 KB argument block costs about a microsecond per
+// launch, a scan through 40-byte items several), so small batches get a small block and
+// the workgroup-to-item search runs over a compact array of first-workgroup indices.
+template <int N>
+struct AttnBatchT {
+    uint32_t n;
+    uint32_t total_blocks;
+    uint32_t rows_per_block;
+    uint32_t base_row;  // q_row0 of item 0
+    uint32_t block0[N];
+    uint32_t row0[N];   // q_row0 - base_row
+    AttnItem item[N];
+
+    explicit AttnBatchT(const AttnBatch &b)
+        : n(b.n), total_blocks(b.total_blocks), rows_per_block(b.rows_per_block),
+          base_row(b.n ? b.item[0].q_row0 : 0) {
+        for (int i = 0; i < N; ++i) {
+            const bool live = uint32_t(i) < b.n;
+            item[i] = live ? b.item[i] : AttnItem{};
+            block0[i] = live ? b.item[i].block0 : 0xffffffffu;
+            row0[i] = live ? b.item[i].q_row0 - base_row : 0xffffffffu;
+        }
+    }
+    __device__ __forceinline__ uint32_t find_by_block(uint32_t block) const {
+        uint32_t it = 0;
+        if (N > 1) {
+#pragma unroll 1
+            while (it + 1 < n && block >= block0[it + 1]) ++it;
+        }
+        return it;
+    }
+    __device__ __forceinline__ uint32_t find_by_row(uint32_t row) const {
+        uint32_t it = 0;
+        if (N > 1) {
+#pragma unroll 1
+            while (it + 1 < n && row >= row0[it + 1]) ++it;
+        }
+        return it;
+    }
+};
+
+// Runs CALL with `constexpr int N` set to the smallest of {1, 8, 64} that holds n items.
+#define ITAK_DISPATCH_BATCH(n, CALL) \
+    do {                              \
+        if ((n) <= 1) {               \
+            constexpr int N = 1;      \
+            CALL;                     \
+        } else if ((n) <= 8) {        \
+            constexpr int N = 8;      \
+            CALL;                     \
+        } else {                      \
+            constexpr int N = 64;     \
+            CALL;                     \
+        }                             \
+    } while (0)
+
 struct AttnParams {
     const void *layer_base;
     PoolGeom g;
@@ -132,10 +224,16 @@ struct AttnParams {
     float *out;
     const uint32_t *q_pos;  // optional explicit positions, [sum rows]
     float *ws;              // partials: (head_dim + 2) floats each
+    // Fused append (split-K f16 kernel only): when set, the last `rows` positions of every
+    // item are not in the cache yet; their K/V rows are read from here (row q_row0 + r,
+    // [kv_heads*head_dim] f32 each), written to the cache by the kernel, and attended to.
+    const float *k_new;
+    const float *v_new;
     uint32_t q_heads;
     uint32_t group;         // q_heads / kv_heads
     float scale;
     float softcap;
+    uint32_t dbg;  // experiment switch, 0 in production
 };
 
 // Generic VALU path: f32 or f16 storage, any head_dim <= 256, group <= 64. Partials are in

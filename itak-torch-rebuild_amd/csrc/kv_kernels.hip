@@ -7,20 +7,6 @@
 
 namespace itak {
 
-// f32 -> f16 bits, round-to-nearest-even, overflow to infinity, subnormals rounded, and
-// every NaN stored as sign|0x7e00: the rule of f32_to_f16_bits in
-// crates/wgpu-compute/src/kernels/k1_q4k_gemv.rs:285-329. v_cvt_f16_f32 implements all of
-// it except the NaN payload, which is replaced explicitly.
-__device__ __forceinline__ uint16_t f32_to_f16_bits(float x) {
-    _Float16 h = static_cast<_Float16>(x);
-    uint16_t bits = __builtin_bit_cast(uint16_t, h);
-    uint32_t in = __builtin_bit_cast(uint32_t, x);
-    if ((in & 0x7fffffffu) > 0x7f800000u) {
-        bits = static_cast<uint16_t>(((in >> 16) & 0x8000u) | 0x7e00u);
-    }
-    return bits;
-}
-
 __device__ __forceinline__ void store4(float *dst, const float4 &v) {
     *reinterpret_cast<float4 *>(dst) = v;
 }
@@ -35,9 +21,10 @@ __device__ __forceinline__ void store1(uint16_t *dst, float v) { *dst = f32_to_f
 __device__ __forceinline__ void store1(uint16_t *dst, uint16_t v) { *dst = v; }
 
 // ---------------------------------------------------------------------------- append
-// Thread = one (row, side, kv head, VEC-element chunk) of the new rows. Key planes and
-// row-major value planes take one vector store; blocked value planes take VEC 2-byte
-// stores 64 bytes apart (an append moves a few KiB, so their width does not matter).
+// Thread = one (row, side, kv head, VEC-element chunk) of the new rows. Key planes
+// (row-major or blocked) and row-major value planes take one vector store; blocked value
+// planes take VEC 2-byte stores 64 bytes apart (an append moves a few KiB, so their width
+// does not matter).
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void kv_append_kernel(T *__restrict__ layer_base, PoolGeom g,
                                                         AppendBatch b,
@@ -62,7 +49,8 @@ __global__ __launch_bounds__(256) void kv_append_kernel(T *__restrict__ layer_ba
     if constexpr (VEC == 4) {
         const float4 v = *reinterpret_cast<const float4 *>(src);
         if (side == 0 || g.v_block == 0) {
-            store4(plane + uint64_t(dst_row) * g.head_dim + d, v);
+            // Four channels never straddle an 8-channel piece of the blocked key layout.
+            store4(plane + k_offset(g, dst_row, d), v);
         } else {
             T *dst = plane + v_offset(g, dst_row, d);
             store1(dst, v.x);
@@ -71,8 +59,7 @@ __global__ __launch_bounds__(256) void kv_append_kernel(T *__restrict__ layer_ba
             store1(dst + 3 * kVBlock, v.w);
         }
     } else {
-        const uint64_t off = (side == 0) ? uint64_t(dst_row) * g.head_dim + d : v_offset(g, dst_row, d);
-        store1(plane + off, *src);
+        store1(plane + kv_offset(g, side, dst_row, d), *src);
     }
 }
 
@@ -114,14 +101,13 @@ __global__ __launch_bounds__(256) void kv_zero_rows(T *__restrict__ pool_base, P
     T *plane = pool_base + layer * g.layer_stride + item.slot * g.slot_stride +
                plane_id * g.head_stride;
     const uint64_t total = uint64_t(item.row_to - item.row_from) * g.head_dim;
-    const bool blocked = side == 1 && g.v_block != 0;
+    const bool blocked = g.v_block != 0;
     for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < total; i += gridDim.x * 256ull) {
         if (blocked) {
-            // Consecutive threads walk the rows of one channel: contiguous inside a block.
             const uint32_t rows = item.row_to - item.row_from;
             const uint32_t d = uint32_t(i / rows);
             const uint32_t row = item.row_from + uint32_t(i % rows);
-            plane[v_offset(g, row, d)] = T(0);
+            plane[kv_offset(g, side, row, d)] = T(0);
         } else {
             plane[uint64_t(item.row_from) * g.head_dim + i] = T(0);
         }
@@ -171,7 +157,11 @@ __global__ __launch_bounds__(256) void kv_restore_rows(D *__restrict__ pool_base
         const uint32_t rem = uint32_t(i % (g.kv_heads * chunks));
         const uint32_t head = rem / chunks;
         const uint32_t d = (rem % chunks) * VEC;
-        D *dst = dst_side + head * g.head_stride + uint64_t(L.first_row + row) * g.head_dim + d;
+        // side 1 only gets here with row-major planes; VEC (4 or 8) channels stay inside one
+        // 8-channel piece of the blocked key layout.
+        D *dst = dst_side + head * g.head_stride +
+                 (side ? uint64_t(L.first_row + row) * g.head_dim + d
+                       : k_offset(g, L.first_row + row, d));
         if constexpr (sizeof(S) == 4) {
             store4(dst, *reinterpret_cast<const float4 *>(src + i * VEC));
         } else {
@@ -249,9 +239,7 @@ __global__ __launch_bounds__(256) void kv_restore_scalar(D *__restrict__ pool_ba
         const uint32_t rem = uint32_t(i % (g.kv_heads * g.head_dim));
         const uint32_t head = rem / g.head_dim;
         const uint32_t d = rem % g.head_dim;
-        const uint64_t off = side == 0 ? uint64_t(L.first_row + row) * g.head_dim + d
-                                       : v_offset(g, L.first_row + row, d);
-        store1(dst_side + head * g.head_stride + off, src[i]);
+        store1(dst_side + head * g.head_stride + kv_offset(g, side, L.first_row + row, d), src[i]);
     }
 }
 
@@ -329,9 +317,7 @@ __global__ __launch_bounds__(256) void kv_read_rows(const T *__restrict__ layer_
         const uint32_t rem = uint32_t(i % (g.kv_heads * g.head_dim));
         const uint32_t head = rem / g.head_dim;
         const uint32_t d = rem % g.head_dim;
-        const uint64_t off = side == 0 ? uint64_t(first_row + row) * g.head_dim + d
-                                       : v_offset(g, first_row + row, d);
-        out[i] = src_side[head * g.head_stride + off];
+        out[i] = src_side[head * g.head_stride + kv_offset(g, side, first_row + row, d)];
     }
 }
 

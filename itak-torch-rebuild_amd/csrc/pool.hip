@@ -9,6 +9,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -225,14 +226,26 @@ struct PlanInput {
 // f16 pools at head_dim 128 with up to 64 query vectors per KV head (decode and
 // speculative blocks) take the MFMA split-K kernel; everything else the generic kernel.
 // Either way a second small launch merges the split partials.
-itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, uint32_t n,
-                          const float *q_dev, float *out_dev, const uint32_t *q_pos_dev,
-                          uint64_t q_heads, float scale, float softcap) {
+// True when a batch takes the MFMA split-K kernel (which can also fuse the append).
+bool takes_splitk_f16(const itak_pool *pool, const PlanInput *in, uint32_t n, uint64_t q_heads,
+                      const uint32_t *q_pos_dev) {
     const uint32_t group = uint32_t(q_heads / pool->g.kv_heads);
     uint32_t max_rows = 0;
     for (uint32_t i = 0; i < n; ++i) max_rows = std::max(max_rows, in[i].rows);
-    const bool mfma = pool->elem_f16 && q_pos_dev == nullptr &&
-                      attn_splitk_f16_supports(pool->g, group, max_rows);
+    return pool->elem_f16 && q_pos_dev == nullptr &&
+           attn_splitk_f16_supports(pool->g, group, max_rows);
+}
+
+// k_new / v_new non-null = the rows are not in the cache yet and the kernel appends them
+// (only valid when takes_splitk_f16 holds).
+itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, uint32_t n,
+                          const float *q_dev, float *out_dev, const uint32_t *q_pos_dev,
+                          uint64_t q_heads, float scale, float softcap,
+                          const float *k_new = nullptr, const float *v_new = nullptr) {
+    const uint32_t group = uint32_t(q_heads / pool->g.kv_heads);
+    uint32_t max_rows = 0;
+    for (uint32_t i = 0; i < n; ++i) max_rows = std::max(max_rows, in[i].rows);
+    const bool mfma = takes_splitk_f16(pool, in, n, q_heads, q_pos_dev);
     const uint32_t rpb = mfma ? 0 : attn_generic_rows_per_block(group, pool->g.head_dim);
     if (!mfma && rpb == 0)
         return unsupported(pool->err, "head_dim above 256 or GQA group too wide");
@@ -295,10 +308,15 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         p.out = out_dev;
         p.q_pos = q_pos_dev;
         p.ws = pool->ws;
+        p.k_new = mfma ? k_new : nullptr;
+        p.v_new = mfma ? v_new : nullptr;
         p.q_heads = uint32_t(q_heads);
         p.group = group;
         p.scale = scale;
         p.softcap = softcap;
+        static const int dbg = getenv("ITAK_DBG") ? atoi(getenv("ITAK_DBG")) : 0;
+        static const bool no_combine = getenv("ITAK_DBG_NOCOMBINE") != nullptr;
+        p.dbg = uint32_t(dbg);
         if (mfma) {
             HIP_TRY(pool, launch_attn_splitk_f16(p, b, partials, max_rows, pool->stream),
                     "launch split-K attention");
@@ -306,8 +324,9 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
             HIP_TRY(pool, launch_attn_generic(pool->elem_f16, p, b, partials, pool->stream),
                     "launch attention");
         }
-        HIP_TRY(pool, launch_attn_combine(p, b, partials, total_rows, mfma ? 1 : 0, pool->stream),
-                "launch split merge");
+        if (!no_combine)
+            HIP_TRY(pool, launch_attn_combine(p, b, partials, total_rows, mfma ? 1 : 0, pool->stream),
+                    "launch split merge");
     }
     return ITAK_OK;
 }
@@ -1006,6 +1025,32 @@ itak_status itak_gqa_attention(itak_pool *pool, uint32_t slot, uint64_t layer, c
     return ITAK_OK;
 }
 
+// Append + attend for a validated plan. Decode and speculative blocks on f16 pools run as
+// one launch that appends and attends (plus the split merge); other shapes append first.
+static itak_status step_on_device(itak_pool *pool, uint64_t layer, const itak_batch_item *items,
+                                  uint32_t item_count, const std::vector<PlanInput> &plan,
+                                  const float *q_dev, const float *k_dev, const float *v_dev,
+                                  float *out_dev, uint64_t num_q_heads, float scale,
+                                  float softcap) {
+    // Rows of zero-row items contribute nothing; q/k/v rows are numbered by walking the
+    // items in order, so such items may simply be dropped.
+    std::vector<PlanInput> active;
+    for (const PlanInput &p : plan)
+        if (p.rows) active.push_back(p);
+    const bool fuse = takes_splitk_f16(pool, active.data(), uint32_t(active.size()), num_q_heads,
+                                       nullptr);
+    if (fuse) {
+        for (uint32_t i = 0; i < item_count; ++i)
+            pool->slots[items[i].slot].appended[layer] += items[i].rows;
+        return run_attention(pool, layer, active.data(), uint32_t(active.size()), q_dev, out_dev,
+                             nullptr, num_q_heads, scale, softcap, k_dev, v_dev);
+    }
+    itak_status st = run_append(pool, layer, items, item_count, k_dev, v_dev);
+    if (st != ITAK_OK) return st;
+    return run_attention(pool, layer, active.data(), uint32_t(active.size()), q_dev, out_dev,
+                         nullptr, num_q_heads, scale, softcap);
+}
+
 // Validates one batched step and returns the per-item plan (positions before the append).
 static itak_status plan_step(itak_pool *pool, uint64_t layer, const itak_batch_item *items,
                              uint32_t item_count, uint64_t num_q_heads,
@@ -1043,16 +1088,8 @@ itak_status itak_attention_step_device(itak_pool *pool, uint64_t layer,
     itak_status st = plan_step(pool, layer, items, item_count, num_q_heads, plan);
     if (st != ITAK_OK) return st;
     if (std::isnan(scale)) scale = default_scale(pool->g.head_dim);
-    st = run_append(pool, layer, items, item_count, k_dev, v_dev);
-    if (st != ITAK_OK) return st;
-    // Rows of zero-row items contribute nothing.
-    std::vector<PlanInput> active;
-    for (const PlanInput &p : plan)
-        if (p.rows) active.push_back(p);
-    // run_attention numbers q rows by walking the items in order, so zero-row items may
-    // simply be dropped.
-    return run_attention(pool, layer, active.data(), uint32_t(active.size()), q_dev, out_dev,
-                         nullptr, num_q_heads, scale, softcap);
+    return step_on_device(pool, layer, items, item_count, plan, q_dev, k_dev, v_dev, out_dev,
+                          num_q_heads, scale, softcap);
 }
 
 itak_status itak_attention_device(itak_pool *pool, uint64_t layer, const itak_batch_item *items,
