@@ -23,6 +23,7 @@ FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
+    "-Rpass-analysis=kernel-resource-usage", "-fno-caret-diagnostics",
 ]
 
 
@@ -35,9 +36,21 @@ def _compile(src: str) -> str:
     cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
-    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    lines = [l for l in res.stderr.splitlines() if noise not in l]
+    remarks = [l for l in lines if "-Rpass-analysis=kernel-resource-usage" in l]
+    err = "\n".join(l for l in lines if l not in remarks and "remark" not in l)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+    # No kernel may spill registers to scratch memory: spilled variants of the attention
+    # kernels have produced wrong results on the target, and they are slow anyway.
+    name = "?"
+    for l in remarks:
+        if "Function Name:" in l:
+            name = l.split("Function Name:")[1].split("[")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in l:
+            size = int(l.split("ScratchSize [bytes/lane]:")[1].split("[")[0])
+            if size:
+                raise RuntimeError(f"{src}: kernel {name} spills {size} bytes/lane to scratch")
     if err.strip():
         sys.stderr.write(err + "\n")
     return obj

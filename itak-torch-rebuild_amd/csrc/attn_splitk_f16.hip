@@ -23,32 +23,13 @@
 // (key kp visible to a query at position p iff kp <= p), with the optional softcap
 // cap*tanh(s/cap) of crates/torch-math/src/logits.rs:26-37 applied to the scaled scores.
 #include "internal.h"
+#include "mfma_common.h"
 
 #include <math.h>
 
 namespace itak {
 
 namespace {
-
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-
-constexpr int kD = 128;          // head_dim this kernel is written for
-constexpr int kBlockKeys = 32;   // keys per block (= value plane block)
-constexpr int kQStride = kD + 8; // LDS row stride of the staged queries (halves)
-constexpr float kLog2e = 1.4426950408889634f;
-
-__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-// cap * tanh(x / cap) * log2(e), via exp2; x is a scaled score in natural units.
-__device__ __forceinline__ float softcap_log2(float x, float cap, float inv_cap) {
-    const float y = x * inv_cap;
-    // tanh(y) = 1 - 2 / (exp(2y) + 1); exp2 saturates to inf/0 at the tails, giving +-1.
-    const float e = fast_exp2(y * (2.0f * kLog2e));
-    const float t = 1.0f - 2.0f / (e + 1.0f);
-    return cap * kLog2e * t;
-}
 
 template <int NQ>
 struct WaveState {
@@ -82,63 +63,33 @@ __device__ __forceinline__ void load_block(BlockOperands &b, const uint16_t *kpl
         b.v[dt] = *reinterpret_cast<const half8 *>(vb + dt * 16 * kBlockKeys);
 }
 
-// Fused append for a block that contains new positions [pos0, kv_len): the operands the
-// wavefront holds for those keys are replaced by the converted source rows (bit-identical
-// to what the cache will hold), and the wavefront stores the rows into the planes. No other
-// wavefront reads these positions, so nothing depends on the stores within the launch.
-__device__ __forceinline__ half8 convert8(const float *src) {
-    const float4 a = *reinterpret_cast<const float4 *>(src);
-    const float4 c = *reinterpret_cast<const float4 *>(src + 4);
-    const uint16_t h[8] = {f32_to_f16_bits(a.x), f32_to_f16_bits(a.y), f32_to_f16_bits(a.z),
-                           f32_to_f16_bits(a.w), f32_to_f16_bits(c.x), f32_to_f16_bits(c.y),
-                           f32_to_f16_bits(c.z), f32_to_f16_bits(c.w)};
-    half8 out;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) out[e] = __builtin_bit_cast(_Float16, h[e]);
-    return out;
-}
+// Fused append. The workgroup that owns the blocks holding the new positions
+// [pos0, kv_len) converts the new K/V rows once (all threads, coalesced), keeps them in LDS
+// and stores them into the planes; the wavefront that multiplies such a block replaces the
+// operand elements of the new keys from LDS. No other workgroup reads these positions, so
+// nothing depends on the stores within the launch.
+constexpr int kNewStride = kD + 8;  // LDS row stride of the staged new rows (halves)
 
-__device__ __forceinline__ void patch_and_store_new_rows(BlockOperands &b, uint16_t *kplane,
-                                                         uint16_t *vplane, const float *k_new,
-                                                         const float *v_new, uint32_t row_width,
-                                                         uint32_t kb, uint32_t g, uint32_t i,
-                                                         uint32_t lane, uint32_t pos0,
-                                                         uint32_t kv_len) {
-    // k_new / v_new already point at this item's first new row and this KV head.
+__device__ __forceinline__ void patch_new_rows(BlockOperands &b, const _Float16 *sm_newk,
+                                               const _Float16 *sm_newv, uint32_t kb, uint32_t g,
+                                               uint32_t i, uint32_t pos0, uint32_t kv_len) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         const uint32_t key = kb * kBlockKeys + (i >> 2) * 8 + t * 4 + (i & 3);
         if (key >= pos0 && key < kv_len) {
-            const float *src = k_new + uint64_t(key - pos0) * row_width + g * 8;
+            const _Float16 *src = sm_newk + (key - pos0) * kNewStride + g * 8;
 #pragma unroll
-            for (int s = 0; s < 4; ++s) b.k[t][s] = convert8(src + s * 32);
+            for (int s = 0; s < 4; ++s) b.k[t][s] = *reinterpret_cast<const half8 *>(src + s * 32);
         }
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         const uint32_t key = kb * kBlockKeys + g * 8 + e;
         if (key >= pos0 && key < kv_len) {
-            const float *src = v_new + uint64_t(key - pos0) * row_width + i;
+            const _Float16 *src = sm_newv + (key - pos0) * kNewStride + i;
 #pragma unroll
-            for (int dt = 0; dt < 8; ++dt)
-                b.v[dt][e] = __builtin_bit_cast(_Float16, f32_to_f16_bits(src[dt * 16]));
+            for (int dt = 0; dt < 8; ++dt) b.v[dt][e] = src[dt * 16];
         }
-    }
-    // Store: lane owns channels 2*lane and 2*lane + 1 of every new row in this block.
-    const uint32_t first = max(pos0, kb * kBlockKeys);
-    const uint32_t last = min(kv_len, (kb + 1) * kBlockKeys);
-    for (uint32_t key = first; key < last; ++key) {
-        const float2 kk = *reinterpret_cast<const float2 *>(k_new + uint64_t(key - pos0) * row_width + lane * 2);
-        const float2 vv = *reinterpret_cast<const float2 *>(v_new + uint64_t(key - pos0) * row_width + lane * 2);
-        const uint32_t packed = uint32_t(f32_to_f16_bits(kk.x)) | (uint32_t(f32_to_f16_bits(kk.y)) << 16);
-        const uint32_t kin = key % kBlockKeys;
-        const uint32_t kt = (kin >> 2) & 1, ki = (kin >> 3) * 4 + (kin & 3);
-        *reinterpret_cast<uint32_t *>(kplane + uint64_t(key / kBlockKeys) * (kBlockKeys * kD) +
-                                      ((kt * 16 + (lane >> 2)) * 16 + ki) * 8 + (lane & 3) * 2) = packed;
-        uint16_t *vd = vplane + uint64_t(key / kBlockKeys) * (kBlockKeys * kD) +
-                       (lane * 2) * kBlockKeys + key % kBlockKeys;
-        vd[0] = f32_to_f16_bits(vv.x);
-        vd[kBlockKeys] = f32_to_f16_bits(vv.y);
     }
 }
 
@@ -226,6 +177,8 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
     float *sm_l = sm_m + WAVES * NQ * 16;       // [WAVES][NQ*16]
     float *sm_o = sm_l + WAVES * NQ * 16;       // [WAVES][NQ][8][64][4]
     _Float16 *sm_q = reinterpret_cast<_Float16 *>(sm_o + WAVES * NQ * 8 * 64 * 4);  // [NQ*16][kQStride]
+    _Float16 *sm_newk = sm_q + NQ * 16 * kQStride;  // [kMaxNewRows][kNewStride]
+    _Float16 *sm_newv = sm_newk + kMaxNewRows * kNewStride;
 
     const uint32_t tid = threadIdx.x;
     const uint32_t wave = tid >> 6, lane = tid & 63;
@@ -275,6 +228,32 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
         }
         *reinterpret_cast<half4 *>(sm_q + j * kQStride + c4) = h;
     }
+    const bool owns_new = fused && kb_end * kBlockKeys > item.pos0;
+    if (owns_new) {
+        // rows x {K, V} x 32 chunks of 4 channels: convert, keep in LDS, store to the planes.
+        for (uint32_t f = tid; f < item.rows * 2 * (kD / 4); f += WAVES * 64) {
+            const uint32_t r = f / (2 * (kD / 4)), side = (f / (kD / 4)) & 1, c4 = (f % (kD / 4)) * 4;
+            const float4 a = *reinterpret_cast<const float4 *>((side ? v_new : k_new) +
+                                                               uint64_t(r) * row_width + c4);
+            const uint16_t h0 = f32_to_f16_bits(a.x), h1 = f32_to_f16_bits(a.y);
+            const uint16_t h2 = f32_to_f16_bits(a.z), h3 = f32_to_f16_bits(a.w);
+            uint2 packed{uint32_t(h0) | (uint32_t(h1) << 16), uint32_t(h2) | (uint32_t(h3) << 16)};
+            *reinterpret_cast<uint2 *>((side ? sm_newv : sm_newk) + r * kNewStride + c4) = packed;
+            const uint32_t key = item.pos0 + r, kin = key % kBlockKeys;
+            const uint64_t blk = uint64_t(key / kBlockKeys) * (kBlockKeys * kD);
+            if (side == 0) {
+                const uint32_t kt = (kin >> 2) & 1, ki = (kin >> 3) * 4 + (kin & 3);
+                *reinterpret_cast<uint2 *>(kplane + blk + ((kt * 16 + (c4 >> 3)) * 16 + ki) * 8 +
+                                           (c4 & 7)) = packed;
+            } else {
+                uint16_t *vd = vplane + blk + c4 * kBlockKeys + kin;
+                vd[0] = h0;
+                vd[kBlockKeys] = h1;
+                vd[2 * kBlockKeys] = h2;
+                vd[3 * kBlockKeys] = h3;
+            }
+        }
+    }
     __syncthreads();
 
     if (p.dbg == 1) {  // loads only
@@ -310,8 +289,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
                 const bool has2 = kb2 < kb_end;
                 if (has2) load_block(buf_b, kplane, vplane, kb2, g, jl);
                 if (fused && (kb + 1) * kBlockKeys > item.pos0)
-                    patch_and_store_new_rows(buf_a, kplane, vplane, k_new, v_new, row_width, kb, g,
-                                             jl, lane, item.pos0, item.kv_len);
+                    patch_new_rows(buf_a, sm_newk, sm_newv, kb, g, jl, item.pos0, item.kv_len);
                 process_block<NQ>(st, buf_a, sm_q, kb, g, jl, item.pos0, group, item.kv_len,
                                   softcap, inv_cap);
                 if (!has2) break;
@@ -319,8 +297,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
                 const bool has3 = kb3 < kb_end;
                 if (has3) load_block(buf_a, kplane, vplane, kb3, g, jl);
                 if (fused && (kb2 + 1) * kBlockKeys > item.pos0)
-                    patch_and_store_new_rows(buf_b, kplane, vplane, k_new, v_new, row_width, kb2, g,
-                                             jl, lane, item.pos0, item.kv_len);
+                    patch_new_rows(buf_b, sm_newk, sm_newv, kb2, g, jl, item.pos0, item.kv_len);
                 process_block<NQ>(st, buf_b, sm_q, kb2, g, jl, item.pos0, group, item.kv_len,
                                   softcap, inv_cap);
                 if (!has3) break;
@@ -330,8 +307,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
     } else {
         while (kb < kb_end) {
             if (fused && (kb + 1) * kBlockKeys > item.pos0)
-                patch_and_store_new_rows(buf_a, kplane, vplane, k_new, v_new, row_width, kb, g, jl,
-                                         lane, item.pos0, item.kv_len);
+                patch_new_rows(buf_a, sm_newk, sm_newv, kb, g, jl, item.pos0, item.kv_len);
             process_block<NQ>(st, buf_a, sm_q, kb, g, jl, item.pos0, group, item.kv_len, softcap,
                               inv_cap);
             kb += WAVES;
@@ -412,7 +388,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
 
 bool attn_splitk_f16_supports(const PoolGeom &g, uint32_t group, uint32_t max_rows) {
     return g.v_block == kVBlock && g.head_dim == kD && group >= 1 && max_rows >= 1 &&
-           max_rows * group <= 64;
+           max_rows <= uint32_t(kMaxNewRows) && max_rows * group <= 64;
 }
 
 // Fills splits / keys_per_split / block0 / ws0 for a batch (the caller has set slot, rows,
@@ -453,7 +429,7 @@ hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint3
 #define ITAK_LAUNCH(NQ)                                                                          \
     do {                                                                                         \
         const size_t lds = (size_t(2) * W * NQ * 16 + size_t(W) * NQ * 8 * 64 * 4) * 4 +          \
-                           size_t(NQ) * 16 * kQStride * 2;                                       \
+                           size_t(NQ) * 16 * kQStride * 2 + size_t(2) * kMaxNewRows * (kD + 8) * 2; \
         static size_t granted = 64 * 1024;                                                       \
         if (lds > granted) {                                                                     \
             hipError_t e = hipFuncSetAttribute(                                                  \

@@ -246,8 +246,12 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
     uint32_t max_rows = 0;
     for (uint32_t i = 0; i < n; ++i) max_rows = std::max(max_rows, in[i].rows);
     const bool mfma = takes_splitk_f16(pool, in, n, q_heads, q_pos_dev);
-    const uint32_t rpb = mfma ? 0 : attn_generic_rows_per_block(group, pool->g.head_dim);
-    if (!mfma && rpb == 0)
+    // Blocks of many rows (prefill chunks) on the same pools take the MFMA prefill kernel.
+    const bool prefill = !mfma && pool->elem_f16 && q_pos_dev == nullptr &&
+                         attn_prefill_f16_supports(pool->g, group);
+    const uint32_t rpb =
+        (mfma || prefill) ? 0 : attn_generic_rows_per_block(group, pool->g.head_dim);
+    if (!mfma && !prefill && rpb == 0)
         return unsupported(pool->err, "head_dim above 256 or GQA group too wide");
     const uint32_t tile = attn_generic_tile(pool->g.head_dim);
     constexpr uint64_t kTargetBlocks = 1024;  // about four workgroups per CU
@@ -272,6 +276,8 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         uint32_t partials = 0;
         if (mfma) {
             partials = attn_splitk_f16_plan(pool->g, b, uint32_t(q_heads));
+        } else if (prefill) {
+            attn_prefill_f16_plan(pool->g, b, group);
         } else {
             b.rows_per_block = rpb;
             uint64_t key_work = 0;
@@ -320,6 +326,8 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         if (mfma) {
             HIP_TRY(pool, launch_attn_splitk_f16(p, b, partials, max_rows, pool->stream),
                     "launch split-K attention");
+        } else if (prefill) {
+            HIP_TRY(pool, launch_attn_prefill_f16(p, b, pool->stream), "launch prefill attention");
         } else {
             HIP_TRY(pool, launch_attn_generic(pool->elem_f16, p, b, partials, pool->stream),
                     "launch attention");
