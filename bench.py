@@ -1,15 +1,20 @@
-"""Benchmark of the decode hot path on one MI355X.
+"""Benchmark of the KV-cache + attention hot path on one MI355X.
 
-Workload (BASELINE.json configs[1]): 30B-class decode step, batch 1, 48 layers, 32 Q / 4 KV
-heads, head_dim 128, f16 KV cache at context 4096, K pre-rotated with RoPE base 1e6. One
-step = one token: every layer appends one K/V row (f32 -> f16 RNE) at position 4096 and
-runs GQA flash-decode over the 4097 stored positions. All inputs are resident in HBM before
-the timed region. After each step the cache is truncated back to 4096 positions (a host-side
-length update; nothing is enqueued), so every step does the same work at the same context.
+Default workload (BASELINE.json configs[1], the one the metric is quoted on): 30B-class decode
+step, batch 1, 48 layers, 32 Q / 4 KV heads, head_dim 128, f16 KV cache at context 4096, K
+pre-rotated with RoPE base 1e6. One step = one token: every layer appends one K/V row
+(f32 -> f16 RNE) at position 4096 and runs GQA flash-decode over the 4097 stored positions.
+All inputs are resident in HBM before the timed region. After each step the cache is
+truncated back to 4096 positions (a host-side length update; nothing is enqueued), so every
+step does the same work at the same context.
 
 Prints one JSON line: decode-attention KV GB/s over the algorithmic KV bytes
-(2 * 4097 * 4 * 128 * 2 B per layer), with the roofline figures of the dominant kernel and
+(2 * 4097 * 4 * 128 * 2 B per layer), with the roofline figures of the attention launches and
 the CPU oracle timed on the host cores beside it.
+
+`--workload ragged|verify|prefill` measures the other configurations (continuous batching
+over 16 ragged slots, the speculative verify block, the chunked causal prefill) with the
+same JSON shape; they are secondary measurements, the default line is the contract.
 """
 from __future__ import annotations
 
@@ -22,10 +27,15 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-LAYERS, Q_HEADS, KV_HEADS, D, CTX = 48, 32, 4, 128, 4096
+Q_HEADS, KV_HEADS, D = 32, 4, 128
 ROW = KV_HEADS * D
-KV_BYTES_PER_LAYER = 2 * (CTX + 1) * KV_HEADS * D * 2  # K and V rows visible after the append
 HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+# HBM bytes per decode-layer launch pair measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# and scaled by the same counters on the probe copy of known size (see
+# profiles/decode_ctx4096_traffic.md for the runs and the scaling factors). None = not measured.
+MEASURED_TRAFFIC = {"decode": None}
 
 
 def rope_on_device(x, base):
@@ -42,38 +52,86 @@ def rope_on_device(x, base):
     return torch.cat([(a * c - b * s).float(), (a * s + b * c).float()], dim=-1)
 
 
-def cpu_baseline(budget_s: float = 12.0):
-    """The CPU oracle (a port of the reference's single-threaded Rust path) on the same
-    step: append one row at position 4096, attend over 4097 positions, f16-rounded KV."""
+def cpu_baseline(ctx: int, kv_bytes_per_layer: int, layers: int, budget_s: float = 12.0):
+    """The CPU oracle (a port of the reference's single-threaded Rust path) on the decode
+    step: append one row at position ctx, attend over ctx + 1 positions, f16-rounded KV."""
     import numpy as np
 
     import oracle
 
     rng = np.random.default_rng(0)
-    k = oracle.rope_rows(rng.standard_normal((CTX + 1, KV_HEADS, D), dtype=np.float32), 0, 1e6)
-    k = k.reshape(CTX + 1, ROW)
-    v = rng.standard_normal((CTX + 1, ROW), dtype=np.float32)
+    k = oracle.rope_rows(rng.standard_normal((ctx + 1, KV_HEADS, D), dtype=np.float32), 0, 1e6)
+    k = k.reshape(ctx + 1, ROW)
+    v = rng.standard_normal((ctx + 1, ROW), dtype=np.float32)
     q = rng.standard_normal((1, Q_HEADS * D), dtype=np.float32)
     cache = oracle.KvCache.new([oracle.LayerKind.Global], KV_HEADS, D, store_f16=True)
-    cache.restore_bulk(0, 0, k[:CTX], v[:CTX])
+    cache.restore_bulk(0, 0, k[:ctx], v[:ctx])
     done, spent = 0, 0.0
     while spent < budget_s or done < 4:
         cp = cache.checkpoint(1)
         t0 = time.perf_counter()
-        oracle.attention_step(cache, 0, q, k[CTX:], v[CTX:], Q_HEADS, CTX, threads=1)
+        oracle.attention_step(cache, 0, q, k[ctx:], v[ctx:], Q_HEADS, ctx, threads=1)
         spent += time.perf_counter() - t0
-        cache.rewind_to(cp, CTX)
+        cache.rewind_to(cp, ctx)
         cache.release(cp)
         done += 1
     per_layer = spent / done
     return {
-        "value": round(KV_BYTES_PER_LAYER / per_layer / 1e9, 4),
+        "value": round(kv_bytes_per_layer / per_layer / 1e9, 4),
         "unit": "GB/s",
         "cores": 1,
         "kind": "port",
-        "us_per_token": round(per_layer * LAYERS * 1e6, 1),
-        "sample": f"{done} layer-steps of the same decode step (append + attend over "
-                  f"{CTX + 1} positions), single thread; per-token figure is x{LAYERS} layers",
+        "us_per_token": round(per_layer * layers * 1e6, 1),
+        "sample": f"{done} layer-steps of the decode step (append + attend over {ctx + 1} "
+                  f"positions, 32 Q / 4 KV heads, d=128, f16-rounded KV), single thread; the "
+                  f"per-token figure is x{layers} layers",
+    }
+
+
+class Timer:
+    def __init__(self, torch, stream):
+        self.torch, self.stream = torch, stream
+
+    def __call__(self, fn, reps):
+        torch = self.torch
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        start.record(self.stream)
+        for _ in range(reps):
+            fn()
+        end.record(self.stream)
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) * 1e-3, time.perf_counter() - t0
+
+
+def capture(torch, pool, stream, fn):
+    """One call of fn captured into a HIP graph on a side stream."""
+    cap = torch.cuda.Stream()
+    cap.wait_stream(stream)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(cap):
+        pool.set_stream(cap.cuda_stream)
+        with torch.cuda.graph(graph, stream=cap):
+            fn()
+    torch.cuda.synchronize()
+    pool.set_stream(stream.cuda_stream)
+    return graph
+
+
+def probes(torch, pool, timed, dev):
+    """Launch floor (empty kernel) and a streaming copy of known size on this device."""
+    n = 256 << 20
+    src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    pool.probe_copy_device(src.data_ptr(), dst.data_ptr(), n)
+    copy_s, _ = timed(lambda: pool.probe_copy_device(src.data_ptr(), dst.data_ptr(), n), 5)
+    for _ in range(50):
+        pool.probe_empty_launch()
+    empty_s, _ = timed(pool.probe_empty_launch, 2000)
+    return {
+        "empty_kernel_us_per_launch": round(empty_s / 2000 * 1e6, 3),
+        "copy_256MiB_GBps_read_plus_write": round(2 * n * 5 / copy_s / 1e9, 1),
     }
 
 
@@ -82,14 +140,17 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", choices=["decode", "ragged", "verify", "prefill"],
+                    default="decode")
+    ap.add_argument("--softcap", type=float, default=0.0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-graph", action="store_true", help="time eager launches only")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)",
               file=sys.stderr)
         sys.exit(2)
 
+    import numpy as np
     import torch
 
     from __graft_entry__ import load_package
@@ -98,97 +159,125 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
-
-    pool = pkg.KvPool(LAYERS, KV_HEADS, D, elem="f16", max_slots=1, capacity_rows=CTX + 8,
-                      scrub_on_truncate=False)
     stream = torch.cuda.current_stream()
+    timed = Timer(torch, stream)
+
+    # ---- workload shapes -------------------------------------------------------------
+    wl = args.workload
+    if wl == "decode":
+        layers, slots, rows, lengths = 48, 1, 1, [4096]
+        name = ("configs[1]: 30B-class decode step, batch 1, 48 layers, 32 Q / 4 KV heads, "
+                "head_dim 128, f16 KV, context 4096, append 1 token per layer then flash-decode")
+    elif wl == "ragged":
+        layers, slots, rows = 8, 16, 1
+        lengths = np.random.default_rng(3).integers(256, 16384, size=slots, endpoint=True).tolist()
+        name = ("configs[2]: continuous-batching decode, 16 slots, ragged context 256..16384 "
+                f"(sum {sum(lengths)}), 30B-class heads, f16 KV, 8 of the 48 layers cycled")
+    elif wl == "verify":
+        layers, slots, rows, lengths = 16, 4, 7, [8192] * 4
+        name = ("configs[3]: speculative verify block, 4 slots at context 8192, 7 query rows "
+                "appended and attended causally, 30B-class heads, f16 KV, 16 layers cycled")
+    else:
+        layers, slots, rows, lengths = 4, 1, 2048, [30720]
+        name = ("configs[4]: chunked causal prefill, 2048-row chunk over a 30720-token prefix, "
+                "30B-class heads, f16 KV, f32 accumulate, 4 layers cycled")
+    max_len = max(lengths)
+    kv_bytes_layer = sum(2 * (n + rows) * KV_HEADS * D * 2 for n in lengths)
+    flops_layer = sum(4 * D * Q_HEADS * (rows * n + rows * (rows + 1) // 2) for n in lengths)
+
+    pool = pkg.KvPool(layers, KV_HEADS, D, elem="f16", max_slots=slots,
+                      capacity_rows=max_len + rows + 8, scrub_on_truncate=False)
     pool.set_stream(stream.cuda_stream)
-    cache = pool.acquire()
+    caches = [pool.acquire() for _ in range(slots)]
 
-    # Synthetic inputs, resident in HBM: per-layer prefix K/V, per-layer new K/V row and Q.
-    q = torch.randn(LAYERS, 1, Q_HEADS * D, device=dev)
-    k_new = torch.randn(LAYERS, 1, ROW, device=dev)
-    v_new = torch.randn(LAYERS, 1, ROW, device=dev)
+    # Synthetic inputs, resident in HBM: prefix K/V per layer and slot, new K/V rows and Q.
+    total_rows = slots * rows
+    q = torch.randn(layers, total_rows, Q_HEADS * D, device=dev)
+    k_new = torch.randn(layers, total_rows, ROW, device=dev)
+    v_new = torch.randn(layers, total_rows, ROW, device=dev)
+    if wl == "prefill":  # f16-valued Q/K/V
+        q, k_new, v_new = q.half().float(), k_new.half().float(), v_new.half().float()
     out = torch.empty_like(q)
-    for layer in range(LAYERS):
-        k = rope_on_device(torch.randn(CTX, KV_HEADS, D, device=dev), 1e6).reshape(CTX, ROW)
-        v = torch.randn(CTX, ROW, device=dev)
-        pool.append_device(layer, [(cache, CTX)], k.contiguous().data_ptr(), v.data_ptr())
-        torch.cuda.synchronize()
+    for layer in range(layers):
+        for s, n in enumerate(lengths):
+            k = rope_on_device(torch.randn(n, KV_HEADS, D, device=dev), 1e6).reshape(n, ROW)
+            v = torch.randn(n, ROW, device=dev)
+            pool.append_device(layer, [(caches[s], n)], k.contiguous().data_ptr(), v.data_ptr())
+            torch.cuda.synchronize()
+    items = [(c, rows) for c in caches]
     ptrs = [(q[l].data_ptr(), k_new[l].data_ptr(), v_new[l].data_ptr(), out[l].data_ptr())
-            for l in range(LAYERS)]
-    item = [(cache, 1)]
+            for l in range(layers)]
 
-    def token_step():
-        for layer in range(LAYERS):
+    def step():
+        for layer in range(layers):
             qp, kp, vp, op = ptrs[layer]
-            pool.attention_step_device(layer, item, qp, kp, vp, op, Q_HEADS)
-        pool.truncate([cache], [CTX])
+            pool.attention_step_device(layer, items, qp, kp, vp, op, Q_HEADS,
+                                       softcap=args.softcap)
+        pool.truncate(caches, lengths)
 
     def attention_only():
-        for layer in range(LAYERS):
+        for layer in range(layers):
             qp, _, _, op = ptrs[layer]
-            pool.attention_device(layer, item, qp, op, Q_HEADS)
-
-    def timed(fn, steps):
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        start.record(stream)
-        for _ in range(steps):
-            fn()
-        end.record(stream)
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        return start.elapsed_time(end) * 1e-3, wall  # seconds on the stream, wall seconds
+            pool.attention_device(layer, items, qp, op, Q_HEADS, softcap=args.softcap)
 
     for _ in range(max(args.warmup, 1)):
-        token_step()
+        step()
     torch.cuda.synchronize()
+    probe = probes(torch, pool, timed, dev)
 
-    eager_gpu_s, eager_wall_s = timed(token_step, args.steps)
+    eager_s, eager_wall_s = timed(step, args.steps)
 
-    use_graph = not args.no_graph
-    graph_s = None
-    attn_launch_s = None
-    if use_graph:
-        # One token step (48 appends + 48 decode launches) captured once, replayed per step:
-        # the launch-bound loop a serving engine would keep in a HIP graph.
-        cap = torch.cuda.Stream()
-        cap.wait_stream(stream)
-        g_step, g_attn = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
-        with torch.cuda.stream(cap):
-            pool.set_stream(cap.cuda_stream)
-            with torch.cuda.graph(g_step, stream=cap):
-                token_step()
-            # Attention launches alone, on a cache that holds 4097 positions.
-            pool.append_device(0, item, ptrs[0][1], ptrs[0][2])
-            for layer in range(1, LAYERS):
-                pool.append_device(layer, item, ptrs[layer][1], ptrs[layer][2])
-            with torch.cuda.graph(g_attn, stream=cap):
-                attention_only()
-        torch.cuda.synchronize()
-        pool.set_stream(stream.cuda_stream)
-        for _ in range(max(args.warmup, 1)):
-            g_step.replay()
-        graph_s, _ = timed(g_step.replay, args.steps)
-        for _ in range(max(args.warmup, 1)):
-            g_attn.replay()
-        attn_s, _ = timed(g_attn.replay, args.steps)
-        attn_launch_s = attn_s / (args.steps * LAYERS)
-        pool.truncate([cache], [CTX])
+    # One step (all layers) captured once and replayed: the launch-bound loop a serving
+    # engine keeps in a HIP graph. The attention launches alone are timed the same way on
+    # a cache that already holds the new rows.
+    g_step = capture(torch, pool, stream, step)
+    for layer in range(layers):
+        pool.append_device(layer, items, ptrs[layer][1], ptrs[layer][2])
+    g_attn = capture(torch, pool, stream, attention_only)
+    for _ in range(max(args.warmup, 1)):
+        g_step.replay()
+    step_s = timed(g_step.replay, args.steps)[0] / args.steps
+    for _ in range(max(args.warmup, 1)):
+        g_attn.replay()
+    attn_s = timed(g_attn.replay, args.steps)[0] / (args.steps * layers)
+    pool.truncate(caches, lengths)
 
-    step_s = (graph_s if graph_s is not None else eager_gpu_s) / args.steps
-    bytes_per_token = KV_BYTES_PER_LAYER * LAYERS
-    value = bytes_per_token / step_s / 1e9
-    if attn_launch_s is None:
-        attn_launch_s = eager_gpu_s / (args.steps * LAYERS)
-    achieved = KV_BYTES_PER_LAYER / attn_launch_s / 1e9
+    if wl == "prefill":
+        metric, unit = "prefill attention TFLOP/s (2048-row chunk over 30720 prefix)", "TFLOP/s"
+        value = flops_layer * layers / step_s / 1e12
+        roofline = {
+            "bound": "mfma",
+            "kernel": "attn_prefill_f16_kernel (one launch per layer)",
+            "achieved": round(flops_layer / attn_s / 1e12, 2),
+            "peak": MFMA_F16_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(flops_layer / attn_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+            "traffic": MEASURED_TRAFFIC.get(wl),
+            "us_per_launch": round(attn_s * 1e6, 2),
+            "flops_per_launch": flops_layer,
+        }
+    else:
+        metric, unit = "decode-attn KV GB/s (all layers, ctx 4096)", "GB/s"
+        if wl != "decode":
+            metric = f"decode-attn KV GB/s ({wl})"
+        value = kv_bytes_layer * layers / step_s / 1e9
+        roofline = {
+            "bound": "hbm",
+            "kernel": "attn_splitk_f16_kernel + attn_combine_kernel (the two launches of one "
+                      "layer's attention)",
+            "achieved": round(kv_bytes_layer / attn_s / 1e9, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(kv_bytes_layer / attn_s / 1e9 / HBM_PEAK_GBS, 4),
+            "traffic": MEASURED_TRAFFIC.get(wl),
+            "us_per_launch": round(attn_s * 1e6, 3),
+            "bytes_per_launch": kv_bytes_layer,
+        }
 
     result = {
-        "metric": "decode-attn KV GB/s (all layers, ctx 4096)",
+        "metric": metric,
         "value": round(value, 2),
-        "unit": "GB/s",
+        "unit": unit,
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
@@ -196,35 +285,26 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32 arithmetic over f16 KV",
+        "dtype": "f32 softmax and accumulation over f16 KV (f16 MFMA operands)",
         "data": "synthetic",
         "config": {
-            "workload": "configs[1]: 30B-class decode step, batch 1, 48 layers, 32 Q / 4 KV "
-                        "heads, head_dim 128, f16 KV, context 4096, append 1 token per layer "
-                        "then flash-decode",
-            "launch": "HIP graph replay of one token step" if graph_s is not None else "eager",
-            "kv_bytes_per_token": bytes_per_token,
+            "workload": name,
+            "launch": "HIP graph replay of one step (all layers)",
+            "layers_per_step": layers,
+            "kv_bytes_per_step": kv_bytes_layer * layers,
+            "softcap": args.softcap,
         },
-        "us_per_token": round(step_s * 1e6, 2),
-        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "us_per_token": round(step_s * 1e6 * (48 / layers), 2),
+        "pct_of_hbm_peak": round(100.0 * kv_bytes_layer * layers / step_s / 1e9 / HBM_PEAK_GBS, 2),
         "eager": {
-            "us_per_token_stream": round(eager_gpu_s / args.steps * 1e6, 2),
-            "us_per_token_wall": round(eager_wall_s / args.steps * 1e6, 2),
+            "us_per_step_stream": round(eager_s / args.steps * 1e6, 2),
+            "us_per_step_wall": round(eager_wall_s / args.steps * 1e6, 2),
         },
-        "roofline": {
-            "bound": "hbm",
-            "kernel": "decode attention (one launch per layer)",
-            "achieved": round(achieved, 2),
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
-            "us_per_launch": round(attn_launch_s * 1e6, 3),
-            "bytes_per_launch": KV_BYTES_PER_LAYER,
-        },
+        "device_probes": probe,
+        "roofline": roofline,
     }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline()
+        result["cpu_baseline"] = cpu_baseline(4096, 2 * 4097 * KV_HEADS * D * 2, 48)
     print(json.dumps(result))
     pool.close()
 

@@ -293,6 +293,16 @@ itak_status itak_kv_append_device(itak_pool *pool, uint64_t layer, const itak_ba
 itak_status itak_convert_f32_to_f16_device(itak_pool *pool, const float *src_dev,
                                            uint16_t *dst_dev, uint64_t count);
 
+/* ---- measurement aids (no counterpart in the reference) ------------------------------ */
+
+/* A plain streaming copy of `bytes` (a multiple of 16) on the pool's stream: the kernel of
+   known size that hardware traffic counters are scaled by. */
+itak_status itak_probe_copy_device(itak_pool *pool, const void *src_dev, void *dst_dev,
+                                   uint64_t bytes);
+/* One empty kernel on the pool's stream: timing a run of these gives the per-launch floor
+   of dependent launches on this device. */
+itak_status itak_probe_empty_launch(itak_pool *pool);
+
 #ifdef __cplusplus
 }
 #endif

@@ -110,6 +110,8 @@ PROTOTYPES = {
                                      _f32]),
     "itak_kv_append_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P]),
     "itak_convert_f32_to_f16_device": (_i32, [_P, _P, _P, _u64]),
+    "itak_probe_copy_device": (_i32, [_P, _P, _P, _u64]),
+    "itak_probe_empty_launch": (_i32, [_P]),
 }
 
 _lib = None

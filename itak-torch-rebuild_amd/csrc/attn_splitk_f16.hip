@@ -256,20 +256,6 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
     }
     __syncthreads();
 
-    if (p.dbg == 1) {  // loads only
-        float acc = 0.0f;
-        if (kb < kb_end) {
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int s = 0; s < 4; ++s) acc += float(buf_a.k[t][s][0]);
-#pragma unroll
-            for (int dt = 0; dt < 8; ++dt) acc += float(buf_a.v[dt][0]);
-        }
-        acc += float(sm_q[jl]);
-        if (acc == 1234.5f) p.out[0] = acc;
-        return;
-    }
     WaveState<NQ> st;
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
@@ -315,11 +301,6 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
         }
     }
 
-    if (p.dbg == 2) {  // no merge, no writes
-        float acc = st.m[0] + st.l[0] + st.o[0][0][0] + st.o[0][7][3];
-        if (acc == 1234.5f) p.out[0] = acc;
-        return;
-    }
     // ---- merge the wavefronts through LDS ------------------------------------------------
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
@@ -393,11 +374,25 @@ bool attn_splitk_f16_supports(const PoolGeom &g, uint32_t group, uint32_t max_ro
 
 // Fills splits / keys_per_split / block0 / ws0 for a batch (the caller has set slot, rows,
 // pos0, q_row0, kv_len) and returns the number of partials the launch will write.
+// Wavefronts per workgroup. The 16-vector (decode) kernel is built with four and with
+// eight: eight-wave workgroups halve the partials and measured about 4 % faster on large
+// ragged batches, four-wave ones are faster at a few hundred blocks (context 4096, batch 1);
+// two-wave workgroups were slower everywhere (the merge launch pays for the doubled partials).
+constexpr uint32_t kSplitWaves = 4;
+static uint32_t splitk_waves(const PoolGeom &g, const AttnBatch &b, uint32_t group) {
+    uint64_t blocks = 0;
+    for (uint32_t i = 0; i < b.n; ++i) {
+        if (b.item[i].rows * group > 16) return kSplitWaves;
+        blocks += uint64_t(g.kv_heads) * ((b.item[i].kv_len + kBlockKeys - 1) / kBlockKeys);
+    }
+    return blocks >= 4096 ? 8 : kSplitWaves;
+}
+
 uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads) {
     uint64_t blocks = 0;
     for (uint32_t i = 0; i < b.n; ++i)
         blocks += uint64_t(g.kv_heads) * ((b.item[i].kv_len + kBlockKeys - 1) / kBlockKeys);
-    const uint32_t waves = 4;
+    const uint32_t waves = splitk_waves(g, b, q_heads / g.kv_heads);
     // About four workgroups per CU keeps every SIMD fed; short contexts get one block per
     // wavefront, the least work a workgroup can usefully have.
     constexpr uint64_t kTargetGroups = 1024;
@@ -425,8 +420,8 @@ hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint3
                                   uint32_t max_rows, hipStream_t stream) {
     if (b.total_blocks == 0) return hipSuccess;
     const uint32_t nvec = max_rows * p.group;
-    constexpr int W = 4;
-#define ITAK_LAUNCH(NQ)                                                                          \
+    const uint32_t waves = splitk_waves(p.g, b, p.group);
+#define ITAK_LAUNCH(NQ, W)                                                                       \
     do {                                                                                         \
         const size_t lds = (size_t(2) * W * NQ * 16 + size_t(W) * NQ * 8 * 64 * 4) * 4 +          \
                            size_t(NQ) * 16 * kQStride * 2 + size_t(2) * kMaxNewRows * (kD + 8) * 2; \
@@ -441,14 +436,18 @@ hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint3
         attn_splitk_f16_kernel<NQ, W, N><<<b.total_blocks, W * 64, lds, stream>>>(               \
             p, AttnBatchT<N>(b), total_partials);                                                \
     } while (0)
-#define ITAK_LAUNCH_NQ()             \
-    do {                             \
-        if (nvec <= 16)              \
-            ITAK_LAUNCH(1);          \
-        else if (nvec <= 32)         \
-            ITAK_LAUNCH(2);          \
-        else                         \
-            ITAK_LAUNCH(4);          \
+#define ITAK_LAUNCH_NQ()                \
+    do {                                \
+        if (nvec <= 16) {               \
+            if (waves == 8)             \
+                ITAK_LAUNCH(1, 8);      \
+            else                        \
+                ITAK_LAUNCH(1, 4);      \
+        } else if (nvec <= 32) {        \
+            ITAK_LAUNCH(2, 4);          \
+        } else {                        \
+            ITAK_LAUNCH(4, 4);          \
+        }                               \
     } while (0)
     ITAK_DISPATCH_BATCH(b.n, ITAK_LAUNCH_NQ());
 #undef ITAK_LAUNCH_NQ

@@ -132,6 +132,8 @@ hipError_t launch_read_rows(const void *layer_base, int elem_f16, const PoolGeom
                             hipStream_t stream);
 
 hipError_t launch_convert_f16(const float *src, uint16_t *dst, uint64_t count, hipStream_t stream);
+hipError_t launch_probe_copy(const void *src, void *dst, uint64_t bytes, hipStream_t stream);
+hipError_t launch_probe_empty(hipStream_t stream);
 
 // ---- attention ----------------------------------------------------------------------
 // One item = one slot's query rows against that slot's rows of one layer. Query row r
@@ -233,7 +235,6 @@ struct AttnParams {
     uint32_t group;         // q_heads / kv_heads
     float scale;
     float softcap;
-    uint32_t dbg;  // experiment switch, 0 in production
 };
 
 // Generic VALU path: f32 or f16 storage, any head_dim <= 256, group <= 64. Partials are in

@@ -357,4 +357,34 @@ hipError_t launch_convert_f16(const float *src, uint16_t *dst, uint64_t count, h
     return hipGetLastError();
 }
 
+// ------------------------------------------------------------- measurement aids
+// A plain streaming copy of known size (the yardstick the FETCH_SIZE / WRITE_SIZE counters
+// are scaled by) and an empty kernel (the per-launch floor of a stream of dependent
+// launches).
+__global__ __launch_bounds__(256) void probe_copy_kernel(const uint4 *__restrict__ src,
+                                                         uint4 *__restrict__ dst, uint64_t n) {
+    for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < n; i += gridDim.x * 256ull)
+        dst[i] = src[i];
+}
+
+__global__ void probe_empty_kernel(uint32_t *sink) {
+    if (sink == nullptr) return;
+    if (threadIdx.x == 0xffffffffu) *sink = 0;
+}
+
+hipError_t launch_probe_copy(const void *src, void *dst, uint64_t bytes, hipStream_t stream) {
+    const uint64_t n = bytes / 16;
+    if (n == 0) return hipSuccess;
+    uint64_t blocks = (n + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    probe_copy_kernel<<<uint32_t(blocks), 256, 0, stream>>>(static_cast<const uint4 *>(src),
+                                                            static_cast<uint4 *>(dst), n);
+    return hipGetLastError();
+}
+
+hipError_t launch_probe_empty(hipStream_t stream) {
+    probe_empty_kernel<<<1, 64, 0, stream>>>(nullptr);
+    return hipGetLastError();
+}
+
 }  // namespace itak

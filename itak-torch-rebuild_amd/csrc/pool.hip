@@ -9,7 +9,6 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
-#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -320,9 +319,6 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         p.group = group;
         p.scale = scale;
         p.softcap = softcap;
-        static const int dbg = getenv("ITAK_DBG") ? atoi(getenv("ITAK_DBG")) : 0;
-        static const bool no_combine = getenv("ITAK_DBG_NOCOMBINE") != nullptr;
-        p.dbg = uint32_t(dbg);
         if (mfma) {
             HIP_TRY(pool, launch_attn_splitk_f16(p, b, partials, max_rows, pool->stream),
                     "launch split-K attention");
@@ -332,9 +328,8 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
             HIP_TRY(pool, launch_attn_generic(pool->elem_f16, p, b, partials, pool->stream),
                     "launch attention");
         }
-        if (!no_combine)
-            HIP_TRY(pool, launch_attn_combine(p, b, partials, total_rows, mfma ? 1 : 0, pool->stream),
-                    "launch split merge");
+        HIP_TRY(pool, launch_attn_combine(p, b, partials, total_rows, mfma ? 1 : 0, pool->stream),
+                "launch split merge");
     }
     return ITAK_OK;
 }
@@ -1259,6 +1254,21 @@ itak_status itak_convert_f32_to_f16_device(itak_pool *pool, const float *src_dev
     if (!pool) return ITAK_INVALID_ARGUMENT;
     if (count && (!src_dev || !dst_dev)) return invalid_argument(pool->err, "src or dst is null");
     HIP_TRY(pool, launch_convert_f16(src_dev, dst_dev, count, pool->stream), "launch conversion");
+    return ITAK_OK;
+}
+
+itak_status itak_probe_copy_device(itak_pool *pool, const void *src_dev, void *dst_dev,
+                                   uint64_t bytes) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (bytes && (!src_dev || !dst_dev)) return invalid_argument(pool->err, "src or dst is null");
+    if (bytes % 16 != 0) return invalid_argument(pool->err, "bytes is not a multiple of 16");
+    HIP_TRY(pool, launch_probe_copy(src_dev, dst_dev, bytes, pool->stream), "launch probe copy");
+    return ITAK_OK;
+}
+
+itak_status itak_probe_empty_launch(itak_pool *pool) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    HIP_TRY(pool, launch_probe_empty(pool->stream), "launch empty probe");
     return ITAK_OK;
 }
 

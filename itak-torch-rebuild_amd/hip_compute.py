@@ -272,6 +272,14 @@ class KvPool:
         n = np.asarray(new_lengths, dtype=np.uint64)
         _check(self._h, self._lib.itak_kv_truncate(self._h, _ptr(s), _ptr(n), len(s)))
 
+    def probe_copy_device(self, src_ptr: int, dst_ptr: int, nbytes: int) -> None:
+        """Measurement aid: a plain streaming copy of known size on the pool's stream."""
+        _check(self._h, self._lib.itak_probe_copy_device(self._h, src_ptr, dst_ptr, nbytes))
+
+    def probe_empty_launch(self) -> None:
+        """Measurement aid: one empty kernel on the pool's stream."""
+        _check(self._h, self._lib.itak_probe_empty_launch(self._h))
+
     def convert_f32_to_f16_device(self, src_ptr: int, dst_ptr: int, count: int) -> None:
         _check(self._h, self._lib.itak_convert_f32_to_f16_device(self._h, src_ptr, dst_ptr, count))
 
