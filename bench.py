@@ -34,8 +34,9 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 
 # HBM bytes per decode-layer launch pair measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # and scaled by the same counters on the probe copy of known size (see
-# profiles/decode_ctx4096_traffic.md for the runs and the scaling factors). None = not measured.
-MEASURED_TRAFFIC = {"decode": None}
+# profiles/attn_splitk_f16_decode_ctx4096_traffic.md for the runs and the scaling factors).
+# None = not measured.
+MEASURED_TRAFFIC = {"decode": 10_027_000}
 
 
 def rope_on_device(x, base):
