@@ -27,6 +27,15 @@
 
 #include <math.h>
 
+// Timeline hooks: a measurement build may pre-define these to record timestamps at the
+// numbered points; the library build compiles them to nothing.
+#ifndef ITAK_MARK
+#define ITAK_MARK_BEGIN
+#define ITAK_MARK(i)
+#define ITAK_MARK_END
+#define ITAK_MARK_END2
+#endif
+
 namespace itak {
 
 namespace {
@@ -93,10 +102,33 @@ __device__ __forceinline__ void patch_new_rows(BlockOperands &b, const _Float16 
     }
 }
 
-template <int NQ>
+// Reductions over the four lanes that share a query-vector column (lanes l, l^16, l^32,
+// l^48) with the gfx950 row and half swaps: they run at VALU speed, not through the LDS
+// crossbar. permlane16_swap exchanges the odd rows of its first operand with the even rows
+// of its second, permlane32_swap the upper half of the first with the lower half of the
+// second; with both operands equal, combining the two results folds l with l^16 (l^32).
+__device__ __forceinline__ float column_max(float v) {
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(c[0]), __uint_as_float(c[1]));
+}
+__device__ __forceinline__ float column_sum(float v) {
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(c[0]) + __uint_as_float(c[1]);
+}
+
+// One 32-key block against all NQ tiles of query vectors. FIRST = the wavefront's first
+// block: the running state is written, not rescaled (most decode wavefronts see one block).
+// Up to 32 vectors the Q^T operand lives in registers (qreg), beyond that it is re-read
+// from LDS per block: lane (g, jl) holds channels k*32 + g*8 .. +8 of vector jl.
+template <int NQ, bool FIRST>
 __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &b,
-                                              const _Float16 *sm_q, uint32_t kb, uint32_t g,
-                                              uint32_t jl, uint32_t pos0, uint32_t group,
+                                              const half8 *qreg, const _Float16 *sm_q,
+                                              uint32_t kb, uint32_t g, uint32_t jl,
+                                              const uint32_t *colpos, uint32_t pos0,
                                               uint32_t kv_len, float softcap, float inv_cap) {
     const uint32_t key_base = kb * kBlockKeys + g * 8;  // first of this lane's 8 keys
     const bool tail = (kb + 1) * kBlockKeys > kv_len;
@@ -111,12 +143,15 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
     const bool need_mask = (kb + 1) * kBlockKeys > pos0 + 1;
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
-        // Q^T operand of this tile: lane (g, jl) holds channels k*32 + g*8 .. +8 of vector jl.
         half8 qb[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
-            qb[k] = *reinterpret_cast<const half8 *>(sm_q + (qt * 16 + jl) * kQStride + k * 32 +
-                                                     g * 8);
+        for (int k = 0; k < 4; ++k) {
+            if constexpr (NQ <= 2)
+                qb[k] = qreg[qt * 4 + k];
+            else
+                qb[k] = *reinterpret_cast<const half8 *>(sm_q + (qt * 16 + jl) * kQStride +
+                                                         k * 32 + g * 8);
+        }
         floatx4 s[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -135,7 +170,7 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
             for (int e = 0; e < 8; ++e) sc[e] = softcap_log2(sc[e], softcap, inv_cap);
         }
         if (need_mask) {
-            const uint32_t pos = pos0 + (qt * 16 + jl) / group;  // this column's query position
+            const uint32_t pos = colpos[qt];  // this column's query position
 #pragma unroll
             for (int e = 0; e < 8; ++e)
                 if (key_base + e > pos) sc[e] = -INFINITY;
@@ -143,11 +178,9 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
         float mx = sc[0];
 #pragma unroll
         for (int e = 1; e < 8; ++e) mx = fmaxf(mx, sc[e]);
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(st.m[qt], mx);
+        mx = column_max(mx);
+        const float m_new = FIRST ? mx : fmaxf(st.m[qt], mx);
         const bool dead = m_new == -INFINITY;  // nothing visible to this column so far
-        const float alpha = dead ? 1.0f : fast_exp2(st.m[qt] - m_new);
         float p[8];
         float sum = 0.0f;
 #pragma unroll
@@ -155,20 +188,35 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
             p[e] = dead ? 0.0f : fast_exp2(sc[e] - m_new);
             sum += p[e];
         }
-        st.m[qt] = m_new;
-        st.l[qt] = st.l[qt] * alpha + sum;
         half8 pb;
 #pragma unroll
         for (int e = 0; e < 8; ++e) pb[e] = static_cast<_Float16>(p[e]);
+        if constexpr (FIRST) {
+            st.l[qt] = sum;
 #pragma unroll
-        for (int dt = 0; dt < 8; ++dt) {
-            st.o[qt][dt] *= alpha;
-            st.o[qt][dt] =
-                __builtin_amdgcn_mfma_f32_16x16x32_f16(b.v[dt], pb, st.o[qt][dt], 0, 0, 0);
+            for (int dt = 0; dt < 8; ++dt)
+                st.o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                    b.v[dt], pb, floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+        } else {
+            const float alpha = dead ? 1.0f : fast_exp2(st.m[qt] - m_new);
+            st.l[qt] = st.l[qt] * alpha + sum;
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) {
+                st.o[qt][dt] *= alpha;
+                st.o[qt][dt] =
+                    __builtin_amdgcn_mfma_f32_16x16x32_f16(b.v[dt], pb, st.o[qt][dt], 0, 0, 0);
+            }
         }
+        st.m[qt] = m_new;
     }
 }
 
+// This kernel runs for a few microseconds at decode shapes, so its shape follows latency,
+// not throughput: every global load is issued before anything waits (new rows, then the
+// query vectors, then the wavefront's first K/V block, all unconditional so that the
+// in-order load counter lets the queries be staged while K/V are still in flight),
+// integer divisions are replaced by multiplications with host-made reciprocals, and the
+// bookkeeping the epilogue needs is computed in the shadow of the loads.
 template <int NQ, int WAVES, int N>
 __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams p, AttnBatchT<N> b,
                                                                      uint32_t total_partials) {
@@ -183,58 +231,118 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
     const uint32_t tid = threadIdx.x;
     const uint32_t wave = tid >> 6, lane = tid & 63;
     const uint32_t g = lane >> 4, jl = lane & 15;
+    ITAK_MARK_BEGIN
+    ITAK_MARK(0)
 
+    // Kernel arguments arrive through scalar loads that the compiler would issue one
+    // dependent batch at a time, each a round trip; naming them all in one place makes it
+    // fetch them together.
+    if (N == 1)
+        asm volatile("" ::"s"(p.layer_base), "s"(p.q), "s"(p.out), "s"(p.ws), "s"(p.k_new),
+                     "s"(p.v_new), "s"(p.g.slot_stride), "s"(p.g.head_stride),
+                     "s"(p.g.side_stride), "s"(p.g.kv_heads), "s"(p.q_heads), "s"(p.group),
+                     "s"(p.group_magic), "s"(p.scale), "s"(p.softcap), "s"(total_partials),
+                     "s"(b.item[0].slot), "s"(b.item[0].rows), "s"(b.item[0].pos0),
+                     "s"(b.item[0].q_row0), "s"(b.item[0].kv_len), "s"(b.item[0].splits),
+                     "s"(b.item[0].keys_per_split), "s"(b.item[0].block0), "s"(b.item[0].ws0),
+                     "s"(b.item[0].splits_magic));
     const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
     const uint32_t local = blockIdx.x - item.block0;
-    const uint32_t split = local % item.splits;
-    const uint32_t kv_head = local / item.splits;
-    const uint32_t group = p.group;
+    const uint32_t kv_head = item.splits > 1 ? __umulhi(local, item.splits_magic) : local;
+    const uint32_t split = local - kv_head * item.splits;
+    const uint32_t group = p.group, magic = p.group_magic;
     const uint32_t nvec = item.rows * group;
 
     uint16_t *kplane = static_cast<uint16_t *>(const_cast<void *>(p.layer_base)) +
                        item.slot * p.g.slot_stride + kv_head * p.g.head_stride;
     uint16_t *vplane = kplane + p.g.side_stride;
     const uint32_t row_width = p.g.kv_heads * kD;
-    const bool fused = p.k_new != nullptr;
-    const float *k_new = fused ? p.k_new + uint64_t(item.q_row0) * row_width + kv_head * kD : nullptr;
-    const float *v_new = fused ? p.v_new + uint64_t(item.q_row0) * row_width + kv_head * kD : nullptr;
 
     const uint32_t nblocks = (item.kv_len + kBlockKeys - 1) / kBlockKeys;
     const uint32_t blocks_per_split = item.keys_per_split / kBlockKeys;
     const uint32_t kb_begin = split * blocks_per_split;
     const uint32_t kb_end = min(nblocks, kb_begin + blocks_per_split);
+    const bool fused = p.k_new != nullptr;
+    const bool owns_new = fused && kb_end * kBlockKeys > item.pos0;
+    float *const ws_acc = p.ws;
+    float *const ws_ml = p.ws + uint64_t(total_partials) * kD;
+    ITAK_MARK(1)
 
-    // Start the first block's loads before anything else: this kernel is latency bound.
+    // ---- 1. new K/V rows into registers: rows x {K, V} x 32 chunks of 4 channels, read by
+    // the one workgroup per KV head whose blocks hold the new positions.
+    constexpr int NL = (kMaxNewRows * 2 * (kD / 4) + WAVES * 64 - 1) / (WAVES * 64);
+    float4 nreg[NL];
+    if (owns_new) {
+        const float *k_new = p.k_new + uint64_t(item.q_row0) * row_width + kv_head * kD;
+        const float *v_new = p.v_new + uint64_t(item.q_row0) * row_width + kv_head * kD;
+#pragma unroll
+        for (int u = 0; u < NL; ++u) {
+            const uint32_t f = tid + u * WAVES * 64;
+            const uint32_t r = f >> 6, side = (f >> 5) & 1, c4 = (f & 31) * 4;
+            nreg[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (r < item.rows)
+                nreg[u] = *reinterpret_cast<const float4 *>((side ? v_new : k_new) +
+                                                            uint64_t(r) * row_width + c4);
+        }
+    }
+
+    // ---- 2. query vectors into registers (vector j = query row j / group, Q head
+    // kv_head*group + j % group); padding vectors re-read the last real one and are zeroed
+    // when staged, so the loads need no branch.
+    constexpr int QL = (NQ * 16 * (kD / 4)) / (WAVES * 64);
+    static_assert(QL >= 1, "too many wavefronts for the query tile");
+    float4 qld[QL];
+#pragma unroll
+    for (int u = 0; u < QL; ++u) {
+        const uint32_t f = tid + u * WAVES * 64;
+        const uint32_t j = min(f >> 5, nvec - 1), c4 = (f & 31) * 4;
+        const uint32_t row = (j * magic) >> 16, head = kv_head * group + (j - row * group);
+        qld[u] = *reinterpret_cast<const float4 *>(
+            p.q + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + c4);
+    }
+
+    // ---- 3. the wavefront's first block (a wavefront without one loads the split's first
+    // block and ignores it).
     BlockOperands buf_a;
     [[maybe_unused]] BlockOperands buf_b;
     uint32_t kb = kb_begin + wave;
-    if (kb < kb_end) load_block(buf_a, kplane, vplane, kb, g, jl);
+    const bool has_block = kb < kb_end;
+    load_block(buf_a, kplane, vplane, has_block ? kb : kb_begin, g, jl);
+    ITAK_MARK(2)
 
-    // ---- Q^T as the B operand: lane (g, jl) holds channels s*32 + g*8 .. +8 of vector jl.
-    // The workgroup reads its query vectors once, coalesced, scales and converts them to
-    // f16 into LDS; each wavefront reads its operand registers from there per block.
+    // ---- 4. in the shadow of the loads: what the mask and the epilogue need per column.
+    uint32_t colpos[NQ], colout[NQ], colps[NQ];
+#pragma unroll
+    for (int qt = 0; qt < NQ; ++qt) {
+        const uint32_t j = qt * 16 + jl;
+        const uint32_t row = (j * magic) >> 16, head = kv_head * group + (j - row * group);
+        colpos[qt] = item.pos0 + row;
+        colout[qt] = (item.q_row0 + row) * p.q_heads + head;
+        colps[qt] = item.ws0 + (row * p.q_heads + head) * item.splits + split;
+    }
     const float softcap = p.softcap;
     const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
     const float qscale = softcap > 0.0f ? p.scale : p.scale * kLog2e;
-    for (uint32_t f = tid; f < NQ * 16 * (kD / 4); f += WAVES * 64) {
-        const uint32_t j = f / (kD / 4), c4 = (f % (kD / 4)) * 4;
-        half4 h{0, 0, 0, 0};
-        if (j < nvec) {
-            const uint32_t row = j / group, head = kv_head * group + j % group;
-            const float4 a = *reinterpret_cast<const float4 *>(
-                p.q + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + c4);
-            h = half4{static_cast<_Float16>(a.x * qscale), static_cast<_Float16>(a.y * qscale),
-                      static_cast<_Float16>(a.z * qscale), static_cast<_Float16>(a.w * qscale)};
-        }
+    ITAK_MARK(3)
+
+    // ---- 5. stage Q^T (scaled, f16) and the new rows (f16, also stored to the planes).
+#pragma unroll
+    for (int u = 0; u < QL; ++u) {
+        const uint32_t f = tid + u * WAVES * 64;
+        const uint32_t j = f >> 5, c4 = (f & 31) * 4;
+        const float4 a = qld[u];
+        half4 h{static_cast<_Float16>(a.x * qscale), static_cast<_Float16>(a.y * qscale),
+                static_cast<_Float16>(a.z * qscale), static_cast<_Float16>(a.w * qscale)};
+        if (j >= nvec) h = half4{0, 0, 0, 0};
         *reinterpret_cast<half4 *>(sm_q + j * kQStride + c4) = h;
     }
-    const bool owns_new = fused && kb_end * kBlockKeys > item.pos0;
     if (owns_new) {
-        // rows x {K, V} x 32 chunks of 4 channels: convert, keep in LDS, store to the planes.
-        for (uint32_t f = tid; f < item.rows * 2 * (kD / 4); f += WAVES * 64) {
-            const uint32_t r = f / (2 * (kD / 4)), side = (f / (kD / 4)) & 1, c4 = (f % (kD / 4)) * 4;
-            const float4 a = *reinterpret_cast<const float4 *>((side ? v_new : k_new) +
-                                                               uint64_t(r) * row_width + c4);
+#pragma unroll
+        for (int u = 0; u < NL; ++u) {
+            const uint32_t f = tid + u * WAVES * 64;
+            const uint32_t r = f >> 6, side = (f >> 5) & 1, c4 = (f & 31) * 4;
+            if (r >= item.rows) continue;
+            const float4 a = nreg[u];
             const uint16_t h0 = f32_to_f16_bits(a.x), h1 = f32_to_f16_bits(a.y);
             const uint16_t h2 = f32_to_f16_bits(a.z), h3 = f32_to_f16_bits(a.w);
             uint2 packed{uint32_t(h0) | (uint32_t(h1) << 16), uint32_t(h2) | (uint32_t(h3) << 16)};
@@ -254,59 +362,70 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
             }
         }
     }
+    ITAK_MARK(4)
     __syncthreads();
-
-    WaveState<NQ> st;
+    half8 qreg[NQ <= 2 ? NQ * 4 : 1];
+    if constexpr (NQ <= 2) {
 #pragma unroll
-    for (int qt = 0; qt < NQ; ++qt) {
-        st.m[qt] = -INFINITY;
-        st.l[qt] = 0.0f;
+        for (int qt = 0; qt < NQ; ++qt)
 #pragma unroll
-        for (int dt = 0; dt < 8; ++dt) st.o[qt][dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int k = 0; k < 4; ++k)
+                qreg[qt * 4 + k] = *reinterpret_cast<const half8 *>(
+                    sm_q + (qt * 16 + jl) * kQStride + k * 32 + g * 8);
     }
+    ITAK_MARK(5)
 
     // ---- this wavefront's blocks. Up to 32 query vectors there are registers for two
     // operand sets, so the next block's loads fly while the current one is multiplied; with
     // 64 vectors the accumulators take that room and the other wavefronts hide the latency.
-    if constexpr (NQ <= 2) {
-        if (kb < kb_end) {
-            for (;;) {
-                const uint32_t kb2 = kb + WAVES;
-                const bool has2 = kb2 < kb_end;
-                if (has2) load_block(buf_b, kplane, vplane, kb2, g, jl);
-                if (fused && (kb + 1) * kBlockKeys > item.pos0)
-                    patch_new_rows(buf_a, sm_newk, sm_newv, kb, g, jl, item.pos0, item.kv_len);
-                process_block<NQ>(st, buf_a, sm_q, kb, g, jl, item.pos0, group, item.kv_len,
-                                  softcap, inv_cap);
-                if (!has2) break;
+    WaveState<NQ> st;
+#define ITAK_BLOCK(FIRST, BUF, KB)                                                               \
+    do {                                                                                         \
+        if (fused && ((KB) + 1) * kBlockKeys > item.pos0)                                        \
+            patch_new_rows(BUF, sm_newk, sm_newv, KB, g, jl, item.pos0, item.kv_len);            \
+        process_block<NQ, FIRST>(st, BUF, qreg, sm_q, KB, g, jl, colpos, item.pos0, item.kv_len, \
+                                 softcap, inv_cap);                                              \
+    } while (0)
+    if (has_block) {
+        if constexpr (NQ <= 2) {
+            uint32_t kb2 = kb + WAVES;
+            bool more = kb2 < kb_end;
+            if (more) load_block(buf_b, kplane, vplane, kb2, g, jl);
+            ITAK_BLOCK(true, buf_a, kb);
+            while (more) {
                 const uint32_t kb3 = kb2 + WAVES;
-                const bool has3 = kb3 < kb_end;
-                if (has3) load_block(buf_a, kplane, vplane, kb3, g, jl);
-                if (fused && (kb2 + 1) * kBlockKeys > item.pos0)
-                    patch_new_rows(buf_b, sm_newk, sm_newv, kb2, g, jl, item.pos0, item.kv_len);
-                process_block<NQ>(st, buf_b, sm_q, kb2, g, jl, item.pos0, group, item.kv_len,
-                                  softcap, inv_cap);
-                if (!has3) break;
-                kb = kb3;
+                const bool more3 = kb3 < kb_end;
+                if (more3) load_block(buf_a, kplane, vplane, kb3, g, jl);
+                ITAK_BLOCK(false, buf_b, kb2);
+                if (!more3) break;
+                kb2 = kb3 + WAVES;
+                more = kb2 < kb_end;
+                if (more) load_block(buf_b, kplane, vplane, kb2, g, jl);
+                ITAK_BLOCK(false, buf_a, kb3);
+            }
+        } else {
+            ITAK_BLOCK(true, buf_a, kb);
+            for (kb += WAVES; kb < kb_end; kb += WAVES) {
+                load_block(buf_a, kplane, vplane, kb, g, jl);
+                ITAK_BLOCK(false, buf_a, kb);
             }
         }
     } else {
-        while (kb < kb_end) {
-            if (fused && (kb + 1) * kBlockKeys > item.pos0)
-                patch_new_rows(buf_a, sm_newk, sm_newv, kb, g, jl, item.pos0, item.kv_len);
-            process_block<NQ>(st, buf_a, sm_q, kb, g, jl, item.pos0, group, item.kv_len, softcap,
-                              inv_cap);
-            kb += WAVES;
-            if (kb < kb_end) load_block(buf_a, kplane, vplane, kb, g, jl);
+#pragma unroll
+        for (int qt = 0; qt < NQ; ++qt) {
+            st.m[qt] = -INFINITY;
+            st.l[qt] = 0.0f;
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) st.o[qt][dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
         }
     }
+#undef ITAK_BLOCK
 
     // ---- merge the wavefronts through LDS ------------------------------------------------
+    ITAK_MARK(6)
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
-        float l = st.l[qt];
-        l += __shfl_xor(l, 16);
-        l += __shfl_xor(l, 32);
+        const float l = column_sum(st.l[qt]);
         if (g == 0) {
             sm_m[wave * NQ * 16 + qt * 16 + jl] = st.m[qt];
             sm_l[wave * NQ * 16 + qt * 16 + jl] = l;
@@ -316,53 +435,55 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
             *reinterpret_cast<floatx4 *>(sm_o + (((wave * NQ + qt) * 8 + dt) * 64 + lane) * 4) =
                 st.o[qt][dt];
     }
+    ITAK_MARK(7)
     __syncthreads();
+    ITAK_MARK(8)
 
-    float *ws_acc = p.ws;
-    float *ws_ml = p.ws + uint64_t(total_partials) * kD;
+    // Every LDS read of the merge is issued before the first one is used.
     constexpr int kDtPerWave = 8 / WAVES;  // channel tiles each wavefront finishes
+    const bool final_out = item.splits == 1;
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
         const uint32_t j = qt * 16 + jl;
-        float mw[WAVES], M = -INFINITY;
+        floatx4 ow[kDtPerWave][WAVES];
+        float mw[WAVES], lw[WAVES];
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
             mw[w] = sm_m[w * NQ * 16 + qt * 16 + jl];
-            M = fmaxf(M, mw[w]);
+            lw[w] = sm_l[w * NQ * 16 + qt * 16 + jl];
         }
+#pragma unroll
+        for (int x = 0; x < kDtPerWave; ++x)
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w)
+                ow[x][w] = *reinterpret_cast<const floatx4 *>(
+                    sm_o + (((w * NQ + qt) * 8 + wave * kDtPerWave + x) * 64 + lane) * 4);
+        float M = mw[0];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) M = fmaxf(M, mw[w]);
         float L = 0.0f, wgt[WAVES];
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
             wgt[w] = (mw[w] == -INFINITY) ? 0.0f : fast_exp2(mw[w] - M);
-            L += sm_l[w * NQ * 16 + qt * 16 + jl] * wgt[w];
+            L = fmaf(lw[w], wgt[w], L);
         }
         if (j >= nvec) continue;
-        const uint32_t row = j / group, head = kv_head * group + j % group;
-        const uint64_t ps = item.ws0 + (uint64_t(row) * p.q_heads + head) * item.splits + split;
+        float *dst = final_out ? p.out + uint64_t(colout[qt]) * kD
+                               : ws_acc + uint64_t(colps[qt]) * kD;
+        const float post = final_out ? __builtin_amdgcn_rcpf(L) : 1.0f;
 #pragma unroll
         for (int x = 0; x < kDtPerWave; ++x) {
-            const int dt = wave * kDtPerWave + x;
-            floatx4 acc{0.0f, 0.0f, 0.0f, 0.0f};
+            floatx4 acc = ow[x][0] * wgt[0];
 #pragma unroll
-            for (int w = 0; w < WAVES; ++w)
-                acc += *reinterpret_cast<const floatx4 *>(
-                           sm_o + (((w * NQ + qt) * 8 + dt) * 64 + lane) * 4) *
-                       wgt[w];
-            const uint32_t d = dt * 16 + g * 4;
-            if (item.splits == 1) {
-                const float inv = 1.0f / L;
-                acc *= inv;
-                *reinterpret_cast<floatx4 *>(
-                    p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + d) = acc;
-            } else {
-                *reinterpret_cast<floatx4 *>(ws_acc + ps * kD + d) = acc;
-            }
+            for (int w = 1; w < WAVES; ++w) acc += ow[x][w] * wgt[w];
+            acc *= post;
+            *reinterpret_cast<floatx4 *>(dst + (wave * kDtPerWave + x) * 16 + g * 4) = acc;
         }
-        if (item.splits > 1 && wave == 0 && g == 0) {
-            ws_ml[ps * 2] = M;
-            ws_ml[ps * 2 + 1] = L;
-        }
+        if (!final_out && wave == 0 && g == 0)
+            *reinterpret_cast<float2 *>(ws_ml + uint64_t(colps[qt]) * 2) = make_float2(M, L);
     }
+    ITAK_MARK(9)
+    ITAK_MARK_END
 }
 
 }  // namespace
@@ -406,6 +527,8 @@ uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads)
         it.keys_per_split = uint32_t(bps) * kBlockKeys;
         it.splits = uint32_t((nblocks + bps - 1) / bps);
         if (it.splits == 0) it.splits = 1;
+        it.splits_magic =
+            it.splits > 1 ? uint32_t(((uint64_t(1) << 32) + it.splits - 1) / it.splits) : 0;
         it.block0 = block0;
         it.ws0 = ws0;
         block0 += g.kv_heads * it.splits;
@@ -574,11 +697,116 @@ __global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(AttnParam
     }
 }
 
+// The same merge for head_dim 128, shaped for latency (it runs for about two microseconds
+// per decode layer): grid = (Q head, query row), thread = (4 channels c, split lane sl of 8).
+// A thread issues every load of its first 8 splits, accumulators and (m, l) pairs alike,
+// before it waits for anything, folds them with its own running maximum, and the eight
+// split lanes meet once in LDS. One memory round trip and one barrier.
+template <int N, bool BASE2>
+__global__ __launch_bounds__(256) void attn_combine128_kernel(AttnParams p, AttnBatchT<N> b,
+                                                              uint32_t total_partials) {
+    __shared__ float4 part[256];
+    __shared__ float part_m[8], part_l[8];
+    const uint32_t tid = threadIdx.x;
+    ITAK_MARK_BEGIN
+    ITAK_MARK(0)
+    const uint32_t head = blockIdx.x, grow = blockIdx.y;
+    if (N == 1)  // fetch every kernel argument in one batch of scalar loads
+        asm volatile("" ::"s"(p.out), "s"(p.ws), "s"(p.q_heads), "s"(total_partials),
+                     "s"(b.base_row), "s"(b.item[0].q_row0), "s"(b.item[0].splits),
+                     "s"(b.item[0].ws0));
+    const AttnItem item = b.item[b.find_by_row(grow)];
+    const uint32_t S = item.splits;
+    if (S == 1) return;
+    const uint32_t row = grow - (item.q_row0 - b.base_row);
+    const uint64_t ps0 = item.ws0 + (uint64_t(row) * p.q_heads + head) * S;
+    const uint32_t c = tid & 31, sl = tid >> 5;
+    const float *ws_acc = p.ws + ps0 * 128 + c * 4;
+    const float2 *ws_ml = reinterpret_cast<const float2 *>(p.ws + uint64_t(total_partials) * 128) + ps0;
+    ITAK_MARK(1)
+
+    float m_run = -INFINITY, l_run = 0.0f;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t s0 = 0; s0 < S; s0 += 64) {
+        float4 x[8];
+        float2 ml[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {  // clamped, so the loads need no branch
+            const uint32_t s = min(s0 + sl + u * 8, S - 1);
+            x[u] = *reinterpret_cast<const float4 *>(ws_acc + uint64_t(s) * 128);
+            ml[u] = ws_ml[s];
+        }
+        if (s0 == 0) { ITAK_MARK(2) }
+        float mx = m_run;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (s0 + sl + u * 8 >= S) ml[u].x = -INFINITY;
+            mx = fmaxf(mx, ml[u].x);
+        }
+        if (mx == -INFINITY) continue;  // nothing visible in these splits (nor before)
+        const float alpha = BASE2 ? fast_exp2(m_run - mx) : __expf(m_run - mx);  // 0 at first
+        acc.x *= alpha, acc.y *= alpha, acc.z *= alpha, acc.w *= alpha;
+        l_run *= alpha;
+        m_run = mx;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float w = BASE2 ? fast_exp2(ml[u].x - mx) : __expf(ml[u].x - mx);  // exp(-inf) = 0
+            l_run = fmaf(ml[u].y, w, l_run);
+            acc.x = fmaf(x[u].x, w, acc.x);
+            acc.y = fmaf(x[u].y, w, acc.y);
+            acc.z = fmaf(x[u].z, w, acc.z);
+            acc.w = fmaf(x[u].w, w, acc.w);
+        }
+    }
+    part[tid] = acc;
+    if (c == 0) {
+        part_m[sl] = m_run;
+        part_l[sl] = l_run;
+    }
+    ITAK_MARK(7)
+    __syncthreads();
+    ITAK_MARK(8)
+    if (tid < 32) {
+        float M = part_m[0];
+#pragma unroll
+        for (int l = 1; l < 8; ++l) M = fmaxf(M, part_m[l]);
+        float L = 0.0f;
+        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int l = 0; l < 8; ++l) {
+            const float ml = part_m[l];
+            const float w = ml == -INFINITY ? 0.0f : (BASE2 ? fast_exp2(ml - M) : __expf(ml - M));
+            const float4 y = part[l * 32 + tid];
+            L = fmaf(part_l[l], w, L);
+            sum.x = fmaf(y.x, w, sum.x);
+            sum.y = fmaf(y.y, w, sum.y);
+            sum.z = fmaf(y.z, w, sum.z);
+            sum.w = fmaf(y.w, w, sum.w);
+        }
+        const float inv = 1.0f / L;
+        float *dst = p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * 128;
+        *reinterpret_cast<float4 *>(dst + tid * 4) =
+            make_float4(sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv);
+    }
+    ITAK_MARK(9)
+    ITAK_MARK_END2
+}
+
 hipError_t launch_attn_combine(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                uint32_t total_rows, int base2, hipStream_t stream) {
     bool any = false;
     for (uint32_t i = 0; i < b.n; ++i) any = any || b.item[i].splits > 1;
     if (!any || total_rows == 0) return hipSuccess;
+    if (p.g.head_dim == 128) {
+        const dim3 grid(p.q_heads, total_rows);
+        if (base2)
+            ITAK_DISPATCH_BATCH(b.n, (attn_combine128_kernel<N, true><<<grid, 256, 0, stream>>>(
+                                         p, AttnBatchT<N>(b), total_partials)));
+        else
+            ITAK_DISPATCH_BATCH(b.n, (attn_combine128_kernel<N, false><<<grid, 256, 0, stream>>>(
+                                         p, AttnBatchT<N>(b), total_partials)));
+        return hipGetLastError();
+    }
     ITAK_DISPATCH_BATCH(b.n, (attn_combine_kernel<N><<<total_rows * p.q_heads, kCombineThreads, 0,
                                                       stream>>>(p, AttnBatchT<N>(b), total_partials,
                                                                 base2)));

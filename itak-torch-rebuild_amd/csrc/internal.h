@@ -153,7 +153,7 @@ struct AttnItem {
     uint32_t keys_per_split;
     uint32_t block0;        // first workgroup index of the item
     uint32_t ws0;           // first partial index of the item
-    uint32_t pad;
+    uint32_t splits_magic;  // ceil(2^32 / splits) for splits > 1: x / splits == mulhi(x, magic), x < 2^16
 };
 struct AttnBatch {
     uint32_t n;
@@ -233,6 +233,7 @@ struct AttnParams {
     const float *v_new;
     uint32_t q_heads;
     uint32_t group;         // q_heads / kv_heads
+    uint32_t group_magic;   // ceil(2^16 / group): j / group == (j * magic) >> 16 for j < 64
     float scale;
     float softcap;
 };

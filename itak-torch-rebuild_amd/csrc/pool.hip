@@ -317,6 +317,7 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         p.v_new = mfma ? v_new : nullptr;
         p.q_heads = uint32_t(q_heads);
         p.group = group;
+        p.group_magic = (65536u + group - 1) / group;
         p.scale = scale;
         p.softcap = softcap;
         if (mfma) {
