@@ -27,6 +27,8 @@
 
 #include <math.h>
 
+#include <algorithm>
+
 // Timeline hooks: a measurement build may pre-define these to record timestamps at the
 // numbered points; the library build compiles them to nothing.
 #ifndef ITAK_MARK
@@ -493,40 +495,105 @@ bool attn_splitk_f16_supports(const PoolGeom &g, uint32_t group, uint32_t max_ro
            max_rows <= uint32_t(kMaxNewRows) && max_rows * group <= 64;
 }
 
-// Fills splits / keys_per_split / block0 / ws0 for a batch (the caller has set slot, rows,
-// pos0, q_row0, kv_len) and returns the number of partials the launch will write.
-// Wavefronts per workgroup. The 16-vector (decode) kernel is built with four and with
-// eight: eight-wave workgroups halve the partials and measured about 4 % faster on large
-// ragged batches, four-wave ones are faster at a few hundred blocks (context 4096, batch 1);
-// two-wave workgroups were slower everywhere (the merge launch pays for the doubled partials).
-constexpr uint32_t kSplitWaves = 4;
-static uint32_t splitk_waves(const PoolGeom &g, const AttnBatch &b, uint32_t group) {
+// ---- variants and planning ---------------------------------------------------------------
+// The kernel is built for 16, 32 and 64 query vectors per KV head (NQ = 1, 2, 4 tiles) and,
+// for 16 vectors, with four or eight wavefronts per workgroup: eight-wave workgroups halve
+// the partials and win on large batches, four-wave ones are faster at a few hundred blocks
+// (context 4096, batch 1); two-wave workgroups lose everywhere, because the partials they
+// double are paid for at the kernel boundary and in the merge launch.
+struct Variant {
+    int nq, waves, index;
+};
+static Variant pick_variant(const PoolGeom &g, const AttnBatch &b, uint32_t group) {
+    uint32_t nvec = 0;
     uint64_t blocks = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
-        if (b.item[i].rows * group > 16) return kSplitWaves;
+        nvec = std::max(nvec, b.item[i].rows * group);
         blocks += uint64_t(g.kv_heads) * ((b.item[i].kv_len + kBlockKeys - 1) / kBlockKeys);
     }
-    return blocks >= 4096 ? 8 : kSplitWaves;
+    if (nvec > 32) return {4, 4, 3};
+    if (nvec > 16) return {2, 4, 2};
+    return blocks >= 4096 ? Variant{1, 8, 1} : Variant{1, 4, 0};
+}
+static size_t variant_lds(int nq, int waves) {
+    return (size_t(2) * waves * nq * 16 + size_t(waves) * nq * 8 * 64 * 4) * 4 +
+           size_t(nq) * 16 * kQStride * 2 + size_t(2) * kMaxNewRows * kNewStride * 2;
+}
+template <int NQ, int W>
+static hipError_t grant_lds(size_t lds) {
+    static size_t granted = 64 * 1024;
+    if (lds <= granted) return hipSuccess;
+    // The attribute is per kernel function: set it on each batch-size instantiation.
+    hipError_t e = hipFuncSetAttribute(
+        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 1>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 8>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 64>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+    if (e == hipSuccess) granted = lds;
+    return e;
+}
+// Workgroups of a variant the device holds at once (registers and LDS decide), asked of the
+// runtime once per variant. A launch of at most this many workgroups runs in one wave of
+// dispatch, so its duration is that of its largest workgroup.
+template <int NQ, int W>
+static uint32_t resident_groups() {
+    static uint32_t cached = 0;
+    if (cached) return cached;
+    const size_t lds = variant_lds(NQ, W);
+    int per_cu = 0, cus = 0, dev = 0;
+    if (grant_lds<NQ, W>(lds) != hipSuccess || hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(
+            &per_cu, reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 1>), W * 64,
+            lds) != hipSuccess ||
+        per_cu < 1 || cus < 1) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    cached = uint32_t(per_cu) * uint32_t(cus);
+    return cached;
+}
+static uint32_t variant_capacity(const Variant &v) {
+    switch (v.index) {
+        case 0: return resident_groups<1, 4>();
+        case 1: return resident_groups<1, 8>();
+        case 2: return resident_groups<2, 4>();
+        default: return resident_groups<4, 4>();
+    }
 }
 
+// Fills splits / keys_per_split / block0 / ws0 for a batch (the caller has set slot, rows,
+// pos0, q_row0, kv_len) and returns the number of partials the launch will write.
+// Every (item, KV head) is cut into equal runs of at most T blocks, T the smallest run for
+// which the whole batch fits the device in one wave of dispatch; a run is never shorter
+// than one block per wavefront.
 uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads) {
+    const Variant v = pick_variant(g, b, q_heads / g.kv_heads);
+    const uint64_t capacity = variant_capacity(v);
     uint64_t blocks = 0;
     for (uint32_t i = 0; i < b.n; ++i)
         blocks += uint64_t(g.kv_heads) * ((b.item[i].kv_len + kBlockKeys - 1) / kBlockKeys);
-    const uint32_t waves = splitk_waves(g, b, q_heads / g.kv_heads);
-    // About four workgroups per CU keeps every SIMD fed; short contexts get one block per
-    // wavefront, the least work a workgroup can usefully have.
-    constexpr uint64_t kTargetGroups = 1024;
-    uint64_t bps = (blocks + kTargetGroups - 1) / kTargetGroups;
-    bps = (bps + waves - 1) / waves * waves;
-    if (bps < waves) bps = waves;
+    uint64_t T = std::max<uint64_t>((blocks + capacity - 1) / capacity, uint64_t(v.waves));
+    for (;; ++T) {
+        uint64_t groups = 0;
+        for (uint32_t i = 0; i < b.n; ++i) {
+            const uint64_t nb = (b.item[i].kv_len + kBlockKeys - 1) / kBlockKeys;
+            groups += uint64_t(g.kv_heads) * std::max<uint64_t>((nb + T - 1) / T, 1);
+        }
+        if (groups <= capacity || T >= blocks) break;
+    }
     uint32_t block0 = 0, ws0 = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         AttnItem &it = b.item[i];
         const uint32_t nblocks = (it.kv_len + kBlockKeys - 1) / kBlockKeys;
-        it.keys_per_split = uint32_t(bps) * kBlockKeys;
-        it.splits = uint32_t((nblocks + bps - 1) / bps);
-        if (it.splits == 0) it.splits = 1;
+        it.splits = std::max<uint32_t>(uint32_t((nblocks + T - 1) / T), 1);
+        const uint32_t bps = std::max<uint32_t>((nblocks + it.splits - 1) / it.splits, 1);
+        it.splits = std::max<uint32_t>((nblocks + bps - 1) / bps, 1);
+        it.keys_per_split = bps * kBlockKeys;
         it.splits_magic =
             it.splits > 1 ? uint32_t(((uint64_t(1) << 32) + it.splits - 1) / it.splits) : 0;
         it.block0 = block0;
@@ -541,36 +608,25 @@ uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads)
 
 hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                   uint32_t max_rows, hipStream_t stream) {
+    (void)max_rows;
     if (b.total_blocks == 0) return hipSuccess;
-    const uint32_t nvec = max_rows * p.group;
-    const uint32_t waves = splitk_waves(p.g, b, p.group);
-#define ITAK_LAUNCH(NQ, W)                                                                       \
-    do {                                                                                         \
-        const size_t lds = (size_t(2) * W * NQ * 16 + size_t(W) * NQ * 8 * 64 * 4) * 4 +          \
-                           size_t(NQ) * 16 * kQStride * 2 + size_t(2) * kMaxNewRows * (kD + 8) * 2; \
-        static size_t granted = 64 * 1024;                                                       \
-        if (lds > granted) {                                                                     \
-            hipError_t e = hipFuncSetAttribute(                                                  \
-                reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, N>),               \
-                hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));                           \
-            if (e != hipSuccess) return e;                                                       \
-            granted = lds;                                                                       \
-        }                                                                                        \
-        attn_splitk_f16_kernel<NQ, W, N><<<b.total_blocks, W * 64, lds, stream>>>(               \
-            p, AttnBatchT<N>(b), total_partials);                                                \
+    const Variant v = pick_variant(p.g, b, p.group);
+#define ITAK_LAUNCH(NQ, W)                                                                \
+    do {                                                                                  \
+        const size_t lds = variant_lds(NQ, W);                                            \
+        hipError_t e = grant_lds<NQ, W>(lds);                                             \
+        if (e != hipSuccess) return e;                                                    \
+        attn_splitk_f16_kernel<NQ, W, N><<<b.total_blocks, W * 64, lds, stream>>>(        \
+            p, AttnBatchT<N>(b), total_partials);                                         \
     } while (0)
-#define ITAK_LAUNCH_NQ()                \
-    do {                                \
-        if (nvec <= 16) {               \
-            if (waves == 8)             \
-                ITAK_LAUNCH(1, 8);      \
-            else                        \
-                ITAK_LAUNCH(1, 4);      \
-        } else if (nvec <= 32) {        \
-            ITAK_LAUNCH(2, 4);          \
-        } else {                        \
-            ITAK_LAUNCH(4, 4);          \
-        }                               \
+#define ITAK_LAUNCH_NQ()               \
+    do {                               \
+        switch (v.index) {             \
+            case 0: ITAK_LAUNCH(1, 4); break; \
+            case 1: ITAK_LAUNCH(1, 8); break; \
+            case 2: ITAK_LAUNCH(2, 4); break; \
+            default: ITAK_LAUNCH(4, 4); break; \
+        }                              \
     } while (0)
     ITAK_DISPATCH_BATCH(b.n, ITAK_LAUNCH_NQ());
 #undef ITAK_LAUNCH_NQ
