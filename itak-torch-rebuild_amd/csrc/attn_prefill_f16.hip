@@ -19,6 +19,8 @@
 #include "internal.h"
 #include "mfma_common.h"
 
+#include <stdlib.h>
+
 namespace itak {
 
 namespace {
@@ -36,7 +38,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_prefill_f16_kernel(AttnParam
     __shared__ __attribute__((aligned(16))) uint16_t lds_v[2][kBlockElems];
 
     const uint32_t tid = threadIdx.x;
-    const uint32_t wave = tid >> 6, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const uint32_t g = lane >> 4, jl = lane & 15;
 
     const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
@@ -242,16 +244,277 @@ __global__ __launch_bounds__(kWaves * 64) void attn_prefill_f16_kernel(AttnParam
     }
 }
 
+
+// ---- two wavefronts per SIMD ------------------------------------------------------------
+// Same tiling of the problem, half the query vectors per workgroup: 128 vectors, 32 per
+// wavefront (2 MFMA column tiles), at most 256 registers, so that two workgroups share a
+// compute unit and one wavefront's softmax runs under the other's MFMAs. The softmax keeps a
+// *reference* maximum per column instead of the exact running maximum:
+//   * the reference enters the score MFMA as its initial accumulator (-ref), so the product
+//     comes out as s - ref and the exponent needs no subtraction;
+//   * the reference moves only when some score of the block exceeds it by more than
+//     kRefSlack (P is bounded by 2^kRefSlack, far inside f16 and f32 range), which after
+//     the first blocks is rare: the cross-lane maximum, the rescale of the accumulators and
+//     the branch around them leave the common path. The result is the same softmax: every
+//     term of numerator and denominator carries the same factor 2^-ref.
+// A column with nothing visible yet has ref = 0 and threshold -inf, so its first finite
+// score sets the reference exactly.
+constexpr int kTiles2 = 2;
+constexpr int kVecPerWave2 = kTiles2 * 16;            // 32
+constexpr int kVecPerGroup2 = kWaves * kVecPerWave2;  // 128
+constexpr float kRefSlack = 8.0f;
+
+__device__ __forceinline__ float column_max4(float v) {
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(c[0]), __uint_as_float(c[1]));
+}
+__device__ __forceinline__ float column_sum4(float v) {
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(c[0]) + __uint_as_float(c[1]);
+}
+
+template <int N, bool SOFTCAP>
+__global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnParams p,
+                                                                           AttnBatchT<N> b) {
+    __shared__ __attribute__((aligned(16))) uint16_t lds_k[2][kBlockElems];
+    __shared__ __attribute__((aligned(16))) uint16_t lds_v[2][kBlockElems];
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const uint32_t g = lane >> 4, jl = lane & 15;
+
+    const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
+    const uint32_t group = p.group;
+    const uint32_t rows_per_group = kVecPerGroup2 / group;
+    const uint32_t rows_per_wave = kVecPerWave2 / group;
+    const uint32_t local = blockIdx.x - item.block0;
+    const uint32_t kv_head = local % p.g.kv_heads;
+    const uint32_t tiles = (item.rows + rows_per_group - 1) / rows_per_group;
+    const uint32_t tile = tiles - 1 - local / p.g.kv_heads;  // longest first
+    const uint32_t row_begin = tile * rows_per_group + wave * rows_per_wave;
+    const uint32_t wg_row_end = min(item.rows, (tile + 1) * rows_per_group);
+
+    const uint16_t *kplane = static_cast<const uint16_t *>(p.layer_base) +
+                             item.slot * p.g.slot_stride + kv_head * p.g.head_stride;
+    const uint16_t *vplane = kplane + p.g.side_stride;
+
+    const uint32_t nblocks = (item.pos0 + wg_row_end + kBlockKeys - 1) / kBlockKeys;
+    const uint32_t wave_row_end = min(item.rows, row_begin + rows_per_wave);
+    const uint32_t wave_blocks =
+        row_begin < item.rows ? (item.pos0 + wave_row_end + kBlockKeys - 1) / kBlockKeys : 0;
+    const uint32_t first_masked = (item.pos0 + row_begin + 1) / kBlockKeys;
+
+    const uint4 *kg = reinterpret_cast<const uint4 *>(kplane) + tid;
+    const uint4 *vg = reinterpret_cast<const uint4 *>(vplane) + tid;
+    constexpr uint32_t kBlockVec = kBlockElems / 8;
+    uint4 pre0 = kg[0], pre1 = kg[256], pre2 = vg[0], pre3 = vg[256];
+
+    const float softcap = p.softcap;
+    const float inv_cap = SOFTCAP ? 1.0f / softcap : 0.0f;
+    const float qscale = SOFTCAP ? p.scale : p.scale * kLog2e;
+    half8 qb[kTiles2][4];
+    uint32_t colpos[kTiles2];
+#pragma unroll
+    for (int qt = 0; qt < kTiles2; ++qt) {
+        const uint32_t j = qt * 16 + jl;
+        const uint32_t row = row_begin + j / group;
+        colpos[qt] = item.pos0 + row;
+        if (row < item.rows) {
+            const uint32_t head = kv_head * group + j % group;
+            const float *qp = p.q + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + g * 8;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const float4 a = *reinterpret_cast<const float4 *>(qp + s * 32);
+                const float4 c = *reinterpret_cast<const float4 *>(qp + s * 32 + 4);
+                qb[qt][s] = half8{static_cast<_Float16>(a.x * qscale), static_cast<_Float16>(a.y * qscale),
+                                  static_cast<_Float16>(a.z * qscale), static_cast<_Float16>(a.w * qscale),
+                                  static_cast<_Float16>(c.x * qscale), static_cast<_Float16>(c.y * qscale),
+                                  static_cast<_Float16>(c.z * qscale), static_cast<_Float16>(c.w * qscale)};
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) qb[qt][s] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+    }
+
+    float ref[kTiles2], thr[kTiles2], l[kTiles2];
+    floatx4 negref[kTiles2];
+    floatx4 o[kTiles2][8];
+#pragma unroll
+    for (int qt = 0; qt < kTiles2; ++qt) {
+        ref[qt] = 0.0f;
+        thr[qt] = -INFINITY;
+        l[qt] = 0.0f;
+        negref[qt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) o[qt][dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    {
+        uint4 *kd = reinterpret_cast<uint4 *>(lds_k[0]) + tid;
+        uint4 *vd = reinterpret_cast<uint4 *>(lds_v[0]) + tid;
+        kd[0] = pre0;
+        kd[256] = pre1;
+        vd[0] = pre2;
+        vd[256] = pre3;
+    }
+    __syncthreads();
+
+    for (uint32_t kb = 0; kb < nblocks; ++kb) {
+        const uint32_t buf = kb & 1;
+        if (kb + 1 < nblocks) {
+            const uint64_t off = uint64_t(kb + 1) * kBlockVec;
+            pre0 = kg[off];
+            pre1 = kg[off + 256];
+            pre2 = vg[off];
+            pre3 = vg[off + 256];
+        }
+
+        if (kb < wave_blocks) {
+            const uint32_t key_base = kb * kBlockKeys + g * 8;
+            floatx4 x[kTiles2][2];
+            {
+                half8 ka[2][4];
+                const uint16_t *kl = lds_k[buf] + (g * 16 + jl) * 8;
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+                        ka[t][s] =
+                            *reinterpret_cast<const half8 *>(kl + ((t * 16 + s * 4) * 16) * 8);
+#pragma unroll
+                for (int qt = 0; qt < kTiles2; ++qt)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        floatx4 s = negref[qt];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+                            s = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[t][k], qb[qt][k], s, 0, 0, 0);
+                        x[qt][t] = s;
+                    }
+            }
+            half8 va[8];
+            const uint16_t *vl = lds_v[buf] + jl * kBlockKeys + g * 8;
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt)
+                va[dt] = *reinterpret_cast<const half8 *>(vl + dt * 16 * kBlockKeys);
+
+            if constexpr (SOFTCAP) {  // negref stays zero: x is the raw scaled score here
+#pragma unroll
+                for (int qt = 0; qt < kTiles2; ++qt)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        x[qt][e >> 2][e & 3] =
+                            softcap_log2(x[qt][e >> 2][e & 3], softcap, inv_cap) - ref[qt];
+            }
+            if (kb >= first_masked) {
+#pragma unroll
+                for (int qt = 0; qt < kTiles2; ++qt)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (key_base + e > colpos[qt]) x[qt][e >> 2][e & 3] = -INFINITY;
+                if ((kb + 1) * kBlockKeys > item.kv_len) {
+                    // Rows past the stored length may hold stale data: keep them out of P.V.
+#pragma unroll
+                    for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (key_base + e >= item.kv_len) va[dt][e] = _Float16(0.0f);
+                }
+            }
+            float lmax[kTiles2];
+            bool over = false;
+#pragma unroll
+            for (int qt = 0; qt < kTiles2; ++qt) {
+                float mx = fmaxf(fmaxf(x[qt][0][0], x[qt][0][1]), x[qt][0][2]);
+                mx = fmaxf(fmaxf(mx, x[qt][0][3]), x[qt][1][0]);
+                mx = fmaxf(fmaxf(mx, x[qt][1][1]), x[qt][1][2]);
+                lmax[qt] = fmaxf(mx, x[qt][1][3]);
+                over = over || lmax[qt] > thr[qt];
+            }
+            if (__builtin_amdgcn_ballot_w64(over) != 0) {
+                // Some column's scores ran past its reference (or it saw its first key).
+#pragma unroll
+                for (int qt = 0; qt < kTiles2; ++qt) {
+                    const float cm = column_max4(lmax[qt]);
+                    const bool live = thr[qt] != -INFINITY;
+                    float delta = live ? fmaxf(cm, 0.0f) : cm;
+                    if (cm == -INFINITY) delta = 0.0f;
+                    const float alpha = live ? fast_exp2(-delta) : 1.0f;
+                    ref[qt] += delta;
+                    if (cm != -INFINITY) thr[qt] = kRefSlack;
+                    l[qt] *= alpha;
+#pragma unroll
+                    for (int dt = 0; dt < 8; ++dt) o[qt][dt] *= alpha;
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) x[qt][t][r] -= delta;
+                    if constexpr (!SOFTCAP) {
+                        const float nr = -ref[qt];
+                        negref[qt] = floatx4{nr, nr, nr, nr};
+                    }
+                }
+            }
+#pragma unroll
+            for (int qt = 0; qt < kTiles2; ++qt) {
+                float pe[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pe[e] = fast_exp2(x[qt][e >> 2][e & 3]);
+                half8 pb;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pb[e] = static_cast<_Float16>(pe[e]);
+                l[qt] += ((pe[0] + pe[1]) + (pe[2] + pe[3])) + ((pe[4] + pe[5]) + (pe[6] + pe[7]));
+#pragma unroll
+                for (int dt = 0; dt < 8; ++dt)
+                    o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[dt], pb, o[qt][dt], 0, 0, 0);
+            }
+        }
+
+        if (kb + 1 < nblocks) {
+            uint4 *kd = reinterpret_cast<uint4 *>(lds_k[buf ^ 1]) + tid;
+            uint4 *vd = reinterpret_cast<uint4 *>(lds_v[buf ^ 1]) + tid;
+            kd[0] = pre0;
+            kd[256] = pre1;
+            vd[0] = pre2;
+            vd[256] = pre3;
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int qt = 0; qt < kTiles2; ++qt) {
+        const float lt = column_sum4(l[qt]);
+        const uint32_t j = qt * 16 + jl;
+        const uint32_t row = row_begin + j / group, head = kv_head * group + j % group;
+        if (row >= item.rows) continue;
+        const float inv = 1.0f / lt;
+        float *dst = p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + g * 4;
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt)
+            *reinterpret_cast<floatx4 *>(dst + dt * 16) = o[qt][dt] * inv;
+    }
+}
+
 }  // namespace
 
+static bool use_old_prefill() {
+    static const bool old = getenv("ITAK_PREFILL_OLD") != nullptr;
+    return old;
+}
+
 bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group) {
-    return g.v_block == kVBlock && g.head_dim == kD && group >= 1 && group <= uint32_t(kVecPerWave) &&
-           kVecPerWave % group == 0;
+    return g.v_block == kVBlock && g.head_dim == kD && group >= 1 &&
+           group <= uint32_t(kVecPerWave2) && kVecPerWave2 % group == 0;
 }
 
 // Fills block0 for a batch (slot, rows, pos0, q_row0, kv_len already set).
 void attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group) {
-    const uint32_t rows_per_group = kVecPerGroup / group;
+    const uint32_t rows_per_group = (use_old_prefill() ? kVecPerGroup : kVecPerGroup2) / group;
     uint32_t block0 = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         AttnItem &it = b.item[i];
@@ -267,8 +530,16 @@ void attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group) {
 
 hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, hipStream_t stream) {
     if (b.total_blocks == 0) return hipSuccess;
-    ITAK_DISPATCH_BATCH(b.n, (attn_prefill_f16_kernel<N><<<b.total_blocks, kWaves * 64, 0, stream>>>(
-                                 p, AttnBatchT<N>(b))));
+    if (use_old_prefill()) {
+        ITAK_DISPATCH_BATCH(b.n, (attn_prefill_f16_kernel<N><<<b.total_blocks, kWaves * 64, 0, stream>>>(
+                                     p, AttnBatchT<N>(b))));
+    } else if (p.softcap > 0.0f) {
+        ITAK_DISPATCH_BATCH(b.n, (attn_prefill2_f16_kernel<N, true><<<b.total_blocks, kWaves * 64, 0,
+                                                                      stream>>>(p, AttnBatchT<N>(b))));
+    } else {
+        ITAK_DISPATCH_BATCH(b.n, (attn_prefill2_f16_kernel<N, false><<<b.total_blocks, kWaves * 64, 0,
+                                                                       stream>>>(p, AttnBatchT<N>(b))));
+    }
     return hipGetLastError();
 }
 

@@ -292,3 +292,30 @@ def test_reduced_prefill_matches_the_oracle_on_every_row():
                                      oracle.AttentionParams(softcap=softcap), threads=THREADS)
         assert max_abs(out.cpu().numpy().reshape(-1), want) <= 2e-3
         pool.close()
+
+
+def test_prefill_with_scores_that_climb_and_fall_along_the_context():
+    # Key magnitudes ramp up and down along the context, so the softmax reference maximum
+    # moves many times, by little and by a lot, and long runs of keys sit far below it; group sizes 8 and 2; with and without softcap.
+    rng = np.random.default_rng(8)
+    for q_heads, prefix, chunk, softcap in ((32, 700, 90, 0.0), (8, 259, 77, 0.0), (32, 420, 40, 50.0)):
+        n = prefix + chunk
+        ramp = 0.25 + 1.5 * np.abs(np.sin(np.arange(n, dtype=np.float32) * (7.0 / n)))[:, None]
+        k, v = normal(rng, n, ROW) * ramp, normal(rng, n, ROW)
+        q = normal(rng, chunk, q_heads * D)
+        pool = P().KvPool(1, KV_HEADS, D, elem="f16", capacity_rows=n)
+        pool.set_stream(torch.cuda.current_stream().cuda_stream)
+        cache = pool.acquire()
+        kd, vd, qd = dev(k), dev(v), dev(q)
+        out = torch.empty_like(qd)
+        pool.append_device(0, [(cache, prefix)], kd.data_ptr(), vd.data_ptr())
+        pool.attention_step_device(0, [(cache, chunk)], qd.data_ptr(), kd[prefix:].data_ptr(),
+                                   vd[prefix:].data_ptr(), out.data_ptr(), q_heads,
+                                   softcap=softcap)
+        torch.cuda.synchronize()
+        ref = oracle_cache(1, KV_HEADS, D, True)
+        ref.restore_bulk(0, 0, k[:prefix], v[:prefix])
+        want = oracle.attention_step(ref, 0, q, k[prefix:], v[prefix:], q_heads, prefix,
+                                     oracle.AttentionParams(softcap=softcap), threads=THREADS)
+        assert max_abs(out.cpu().numpy().reshape(-1), want) <= 2e-3
+        pool.close()
