@@ -277,11 +277,32 @@ __device__ __forceinline__ float column_sum4(float v) {
     return __uint_as_float(c[0]) + __uint_as_float(c[1]);
 }
 
+// K/V blocks travel HBM -> LDS without passing through registers (global_load_lds_dwordx4:
+// lane i of the instruction writes 16 bytes at M0 + 16*i) into a ring of kStages stages, so
+// loads for three blocks ahead are in flight while one is multiplied; the latency of a
+// miss is about a microsecond, more than two block times. The instruction is issued from
+// inline assembly: the compiler then neither tracks it (it would make every LDS read wait
+// for all of them) nor needs to, because the only consumer is ordered by the explicit
+// s_waitcnt vmcnt + s_barrier at the top of each iteration.
+constexpr int kStages = 4;
+constexpr int kStageBytes = 2 * kBlockElems * 2;  // one key block + one value block
+
+__device__ __forceinline__ void lds_dma16(const void *src, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(src), "s"(lds_addr)
+                 : "memory");
+}
+// s_waitcnt vmcnt(n), other counters untouched.
+template <int n>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
+}
+
 template <int N, bool SOFTCAP>
 __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnParams p,
                                                                            AttnBatchT<N> b) {
-    __shared__ __attribute__((aligned(16))) uint16_t lds_k[2][kBlockElems];
-    __shared__ __attribute__((aligned(16))) uint16_t lds_v[2][kBlockElems];
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds_ring[];  // [kStages][K block | V block]
 
     const uint32_t tid = threadIdx.x;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -308,10 +329,31 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
         row_begin < item.rows ? (item.pos0 + wave_row_end + kBlockKeys - 1) / kBlockKeys : 0;
     const uint32_t first_masked = (item.pos0 + row_begin + 1) / kBlockKeys;
 
+    // Each wavefront moves two 1 KiB pieces of the key block and two of the value block.
     const uint4 *kg = reinterpret_cast<const uint4 *>(kplane) + tid;
-    const uint4 *vg = reinterpret_cast<const uint4 *>(vplane) + tid;
+    // Value pieces are permuted on the way in: LDS position dt*64 + g*16 + jl holds the
+    // 16 bytes (channel dt*16 + jl, keys g*8 .. g*8+7), so that the operand read of a
+    // wavefront is linear in the lane number like the key read (the plane's own order,
+    // channel-major, would make 16 consecutive lanes read at a 64-byte stride: bank
+    // conflicts). The pieces of one load still come from one contiguous KiB.
+    const uint4 *vg = reinterpret_cast<const uint4 *>(vplane) + (wave * 16 + jl) * 4 + g;
     constexpr uint32_t kBlockVec = kBlockElems / 8;
-    uint4 pre0 = kg[0], pre1 = kg[256], pre2 = vg[0], pre3 = vg[256];
+    const uint32_t ring_base =
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)(lds_ring);  // LDS byte address
+    const uint32_t dma_base = ring_base + wave * 1024;
+    auto issue_block = [&](uint32_t kb) {
+        // Past the end the last block is fetched again into a stage nobody reads: the
+        // number of loads in flight stays the same in every iteration.
+        const uint64_t off = uint64_t(min(kb, nblocks - 1)) * kBlockVec;
+        const uint32_t dst = dma_base + (kb % kStages) * kStageBytes;
+        lds_dma16(kg + off, dst);
+        lds_dma16(kg + off + 256, dst + 4096);
+        lds_dma16(vg + off, dst + 8192);
+        lds_dma16(vg + off + 256, dst + 12288);
+    };
+    issue_block(0);
+    issue_block(1);
+    issue_block(2);
 
     const float softcap = p.softcap;
     const float inv_cap = SOFTCAP ? 1.0f / softcap : 0.0f;
@@ -354,32 +396,22 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
         for (int dt = 0; dt < 8; ++dt) o[qt][dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
-    {
-        uint4 *kd = reinterpret_cast<uint4 *>(lds_k[0]) + tid;
-        uint4 *vd = reinterpret_cast<uint4 *>(lds_v[0]) + tid;
-        kd[0] = pre0;
-        kd[256] = pre1;
-        vd[0] = pre2;
-        vd[256] = pre3;
-    }
-    __syncthreads();
-
     for (uint32_t kb = 0; kb < nblocks; ++kb) {
-        const uint32_t buf = kb & 1;
-        if (kb + 1 < nblocks) {
-            const uint64_t off = uint64_t(kb + 1) * kBlockVec;
-            pre0 = kg[off];
-            pre1 = kg[off + 256];
-            pre2 = vg[off];
-            pre3 = vg[off + 256];
-        }
+        // This thread's pieces of block kb have landed (the 8 loads of the next two blocks
+        // may still fly); after the barrier everybody's have, and everybody is done with
+        // block kb - 1, whose stage the loads for block kb + 3 may now overwrite.
+        wait_vmcnt<8>();
+        __builtin_amdgcn_s_barrier();
+        issue_block(kb + 3);
+        const uint16_t *lds_k = lds_ring + (kb % kStages) * (kStageBytes / 2);
+        const uint16_t *lds_v = lds_k + kBlockElems;
 
         if (kb < wave_blocks) {
             const uint32_t key_base = kb * kBlockKeys + g * 8;
             floatx4 x[kTiles2][2];
             {
                 half8 ka[2][4];
-                const uint16_t *kl = lds_k[buf] + (g * 16 + jl) * 8;
+                const uint16_t *kl = lds_k + (g * 16 + jl) * 8;
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -398,10 +430,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
                     }
             }
             half8 va[8];
-            const uint16_t *vl = lds_v[buf] + jl * kBlockKeys + g * 8;
+            const uint16_t *vl = lds_v + lane * 8;
 #pragma unroll
             for (int dt = 0; dt < 8; ++dt)
-                va[dt] = *reinterpret_cast<const half8 *>(vl + dt * 16 * kBlockKeys);
+                va[dt] = *reinterpret_cast<const half8 *>(vl + dt * 64 * 8);
 
             if constexpr (SOFTCAP) {  // negref stays zero: x is the raw scaled score here
 #pragma unroll
@@ -475,16 +507,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
             }
         }
 
-        if (kb + 1 < nblocks) {
-            uint4 *kd = reinterpret_cast<uint4 *>(lds_k[buf ^ 1]) + tid;
-            uint4 *vd = reinterpret_cast<uint4 *>(lds_v[buf ^ 1]) + tid;
-            kd[0] = pre0;
-            kd[256] = pre1;
-            vd[0] = pre2;
-            vd[256] = pre3;
-        }
-        __syncthreads();
     }
+    wait_vmcnt<0>();  // the surplus loads of the last iterations
 
 #pragma unroll
     for (int qt = 0; qt < kTiles2; ++qt) {
@@ -528,19 +552,30 @@ void attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group) {
     b.rows_per_block = rows_per_group;
 }
 
+template <int N, bool SOFTCAP>
+static hipError_t launch_prefill2(const AttnParams &p, const AttnBatch &b, hipStream_t stream) {
+    constexpr size_t lds = size_t(kStages) * kStageBytes;
+    static const hipError_t granted = hipFuncSetAttribute(
+        reinterpret_cast<const void *>(&attn_prefill2_f16_kernel<N, SOFTCAP>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+    if (granted != hipSuccess) return granted;
+    attn_prefill2_f16_kernel<N, SOFTCAP><<<b.total_blocks, kWaves * 64, lds, stream>>>(p, AttnBatchT<N>(b));
+    return hipGetLastError();
+}
+
 hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, hipStream_t stream) {
     if (b.total_blocks == 0) return hipSuccess;
     if (use_old_prefill()) {
         ITAK_DISPATCH_BATCH(b.n, (attn_prefill_f16_kernel<N><<<b.total_blocks, kWaves * 64, 0, stream>>>(
                                      p, AttnBatchT<N>(b))));
-    } else if (p.softcap > 0.0f) {
-        ITAK_DISPATCH_BATCH(b.n, (attn_prefill2_f16_kernel<N, true><<<b.total_blocks, kWaves * 64, 0,
-                                                                      stream>>>(p, AttnBatchT<N>(b))));
-    } else {
-        ITAK_DISPATCH_BATCH(b.n, (attn_prefill2_f16_kernel<N, false><<<b.total_blocks, kWaves * 64, 0,
-                                                                       stream>>>(p, AttnBatchT<N>(b))));
+        return hipGetLastError();
     }
-    return hipGetLastError();
+    hipError_t e = hipSuccess;
+    if (p.softcap > 0.0f)
+        ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill2<N, true>(p, b, stream)));
+    else
+        ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill2<N, false>(p, b, stream)));
+    return e;
 }
 
 }  // namespace itak
