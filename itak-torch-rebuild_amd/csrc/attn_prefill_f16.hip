@@ -1,255 +1,26 @@
 // Chunked causal prefill attention for gfx950, f16 KV, head_dim 128: QK^T and PV on
 // v_mfma_f32_16x16x32_f16, everything else (scale, softcap, mask, online softmax) in f32.
 //
-// One workgroup of four wavefronts owns (item, kv head, tile of 256 query vectors), where a
+// One workgroup of four wavefronts owns (item, kv head, tile of 128 query vectors), where a
 // query vector is one query row of one Q head of the KV group: with a group of 8 that is
-// 32 consecutive rows x 8 heads, all reading the same K and V. Each wavefront keeps 64 of
-// the vectors (4 MFMA column tiles): Q^T as f16 B-operands in registers for the whole
-// kernel, O^T as f32 accumulators. The workgroup walks the context in 32-key blocks; every
-// block of the key plane and of the value plane is copied once from HBM into LDS (the
-// planes are stored as the MFMA consumes them, so the copy is a straight 2 x 8 KiB move and
-// operand reads from LDS are conflict free), double buffered so the next block's loads are
-// in flight while the current one is multiplied. Per block and column tile:
-//   S^T = K . Q^T (8 MFMA), scale/softcap/causal mask, online softmax in the lane's own
-//   column (max over 8 keys in registers + two cross-lane steps), O^T += V^T . P^T (8 MFMA),
-// with the accumulator rescale skipped while the running maximum does not move.
+// 16 consecutive rows x 8 heads, all reading the same K and V. Each wavefront keeps 32 of
+// the vectors (2 MFMA column tiles): Q^T as f16 B-operands in registers for the whole
+// kernel, O^T as f32 accumulators; at most 256 registers, so two workgroups share a compute
+// unit and one wavefront's softmax runs under another's MFMAs. The workgroup walks the
+// context in 32-key blocks. Per block and column tile:
+//   S^T = K . Q^T (8 MFMA), softcap / causal mask, softmax in the lane's own column,
+//   O^T += V^T . P^T (8 MFMA).
 //
-// The chunk's own K/V rows are appended before this kernel runs; row r of the chunk sits at
-// position pos0 + r and sees keys <= its position (attention.rs:77-85 with no window).
-#include "internal.h"
-#include "mfma_common.h"
-
-#include <stdlib.h>
-
-namespace itak {
-
-namespace {
-
-constexpr int kWaves = 4;
-constexpr int kTiles = 4;                       // MFMA column tiles (16 vectors) per wavefront
-constexpr int kVecPerWave = kTiles * 16;        // 64
-constexpr int kVecPerGroup = kWaves * kVecPerWave;  // 256 query vectors per workgroup
-constexpr int kBlockElems = kBlockKeys * kD;    // 4096 halves = 8 KiB per plane block
-
-template <int N>
-__global__ __launch_bounds__(kWaves * 64) void attn_prefill_f16_kernel(AttnParams p,
-                                                                       AttnBatchT<N> b) {
-    __shared__ __attribute__((aligned(16))) uint16_t lds_k[2][kBlockElems];
-    __shared__ __attribute__((aligned(16))) uint16_t lds_v[2][kBlockElems];
-
-    const uint32_t tid = threadIdx.x;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-    const uint32_t g = lane >> 4, jl = lane & 15;
-
-    const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
-    const uint32_t group = p.group;
-    const uint32_t rows_per_group = kVecPerGroup / group;  // query rows per workgroup
-    const uint32_t rows_per_wave = kVecPerWave / group;
-    const uint32_t local = blockIdx.x - item.block0;
-    const uint32_t kv_head = local % p.g.kv_heads;
-    // Later row tiles see more keys and run longer: hand them out first.
-    const uint32_t tiles = (item.rows + rows_per_group - 1) / rows_per_group;
-    const uint32_t tile = tiles - 1 - local / p.g.kv_heads;
-    const uint32_t row_begin = tile * rows_per_group + wave * rows_per_wave;  // this wave's rows
-    const uint32_t wg_row_end = min(item.rows, (tile + 1) * rows_per_group);
-
-    const uint16_t *kplane = static_cast<const uint16_t *>(p.layer_base) +
-                             item.slot * p.g.slot_stride + kv_head * p.g.head_stride;
-    const uint16_t *vplane = kplane + p.g.side_stride;
-
-    // Blocks the workgroup needs: up to the position of its last row.
-    const uint32_t nblocks = (item.pos0 + wg_row_end + kBlockKeys - 1) / kBlockKeys;
-    // This wavefront stops multiplying once its own last row has seen everything.
-    const uint32_t wave_row_end = min(item.rows, row_begin + rows_per_wave);
-    const uint32_t wave_blocks =
-        row_begin < item.rows ? (item.pos0 + wave_row_end + kBlockKeys - 1) / kBlockKeys : 0;
-    const uint32_t first_masked = (item.pos0 + row_begin + 1) / kBlockKeys;  // block holding keys > pos of the first row
-
-    // ---- stage block 0 ------------------------------------------------------------------
-    // Each thread moves 2 x 16 bytes of the key block and of the value block.
-    const uint4 *kg = reinterpret_cast<const uint4 *>(kplane) + tid;
-    const uint4 *vg = reinterpret_cast<const uint4 *>(vplane) + tid;
-    constexpr uint32_t kBlockVec = kBlockElems / 8;  // uint4 per block
-    uint4 pre0 = kg[0], pre1 = kg[256], pre2 = vg[0], pre3 = vg[256];
-
-    // ---- Q^T operands: lane (g, jl) of tile qt holds channels s*32 + g*8 .. +8 of vector
-    // qt*16 + jl, scaled and converted to f16 once.
-    const float softcap = p.softcap;
-    const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
-    const float qscale = softcap > 0.0f ? p.scale : p.scale * kLog2e;
-    half8 qb[kTiles][4];
-#pragma unroll
-    for (int qt = 0; qt < kTiles; ++qt) {
-        const uint32_t j = qt * 16 + jl;
-        const uint32_t row = row_begin + j / group;
-        if (row < item.rows) {
-            const uint32_t head = kv_head * group + j % group;
-            const float *qp = p.q + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + g * 8;
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const float4 a = *reinterpret_cast<const float4 *>(qp + s * 32);
-                const float4 c = *reinterpret_cast<const float4 *>(qp + s * 32 + 4);
-                qb[qt][s] = half8{static_cast<_Float16>(a.x * qscale), static_cast<_Float16>(a.y * qscale),
-                                  static_cast<_Float16>(a.z * qscale), static_cast<_Float16>(a.w * qscale),
-                                  static_cast<_Float16>(c.x * qscale), static_cast<_Float16>(c.y * qscale),
-                                  static_cast<_Float16>(c.z * qscale), static_cast<_Float16>(c.w * qscale)};
-            }
-        } else {
-#pragma unroll
-            for (int s = 0; s < 4; ++s) qb[qt][s] = half8{0, 0, 0, 0, 0, 0, 0, 0};
-        }
-    }
-
-    float m[kTiles], l[kTiles];
-    floatx4 o[kTiles][8];
-#pragma unroll
-    for (int qt = 0; qt < kTiles; ++qt) {
-        m[qt] = -INFINITY;
-        l[qt] = 0.0f;
-#pragma unroll
-        for (int dt = 0; dt < 8; ++dt) o[qt][dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-    }
-
-    {
-        uint4 *kd = reinterpret_cast<uint4 *>(lds_k[0]) + tid;
-        uint4 *vd = reinterpret_cast<uint4 *>(lds_v[0]) + tid;
-        kd[0] = pre0;
-        kd[256] = pre1;
-        vd[0] = pre2;
-        vd[256] = pre3;
-    }
-    __syncthreads();
-
-    for (uint32_t kb = 0; kb < nblocks; ++kb) {
-        const uint32_t buf = kb & 1;
-        if (kb + 1 < nblocks) {
-            const uint64_t off = uint64_t(kb + 1) * kBlockVec;
-            pre0 = kg[off];
-            pre1 = kg[off + 256];
-            pre2 = vg[off];
-            pre3 = vg[off + 256];
-        }
-
-        if (kb < wave_blocks) {
-            // Operands of this block come from LDS (same byte layout as the planes). First
-            // all four score tiles (key operands live), then softmax and P.V per tile (value
-            // operands live): the two operand sets never hold registers at the same time.
-            const uint32_t key_base = kb * kBlockKeys + g * 8;
-            const bool need_mask = kb >= first_masked;
-            float sc[kTiles][8];
-            {
-                half8 ka[2][4];
-                const uint16_t *kl = lds_k[buf] + (g * 16 + jl) * 8;
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int s = 0; s < 4; ++s)
-                        ka[t][s] =
-                            *reinterpret_cast<const half8 *>(kl + ((t * 16 + s * 4) * 16) * 8);
-#pragma unroll
-                for (int qt = 0; qt < kTiles; ++qt) {
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        floatx4 s{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                        for (int k = 0; k < 4; ++k)
-                            s = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[t][k], qb[qt][k], s, 0, 0, 0);
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) sc[qt][t * 4 + r] = s[r];
-                    }
-                }
-            }
-            half8 va[8];
-            const uint16_t *vl = lds_v[buf] + jl * kBlockKeys + g * 8;
-#pragma unroll
-            for (int dt = 0; dt < 8; ++dt)
-                va[dt] = *reinterpret_cast<const half8 *>(vl + dt * 16 * kBlockKeys);
-            if ((kb + 1) * kBlockKeys > item.kv_len) {
-                // Rows past the stored length may hold stale data: keep them out of P.V.
-#pragma unroll
-                for (int dt = 0; dt < 8; ++dt)
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (key_base + e >= item.kv_len) va[dt][e] = _Float16(0.0f);
-            }
-#pragma unroll
-            for (int qt = 0; qt < kTiles; ++qt) {
-                if (softcap > 0.0f) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        sc[qt][e] = softcap_log2(sc[qt][e], softcap, inv_cap);
-                }
-                if (need_mask) {
-                    const uint32_t pos = item.pos0 + row_begin + (qt * 16 + jl) / group;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (key_base + e > pos) sc[qt][e] = -INFINITY;
-                }
-                float mx = sc[qt][0];
-#pragma unroll
-                for (int e = 1; e < 8; ++e) mx = fmaxf(mx, sc[qt][e]);
-                mx = fmaxf(mx, __shfl_xor(mx, 16));
-                mx = fmaxf(mx, __shfl_xor(mx, 32));
-                const float m_new = fmaxf(m[qt], mx);
-                const bool dead = m_new == -INFINITY;
-                // Rescale only when some column's maximum moved (wave-uniform decision).
-                const bool moved = m_new != m[qt];
-                if (__builtin_amdgcn_ballot_w64(moved) != 0) {
-                    const float alpha = dead ? 1.0f : fast_exp2(m[qt] - m_new);
-                    l[qt] *= alpha;
-#pragma unroll
-                    for (int dt = 0; dt < 8; ++dt) o[qt][dt] *= alpha;
-                    m[qt] = m_new;
-                }
-                float sum = 0.0f;
-                half8 pb;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float pe = dead ? 0.0f : fast_exp2(sc[qt][e] - m_new);
-                    sum += pe;
-                    pb[e] = static_cast<_Float16>(pe);
-                }
-                l[qt] += sum;
-#pragma unroll
-                for (int dt = 0; dt < 8; ++dt)
-                    o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[dt], pb, o[qt][dt], 0, 0, 0);
-            }
-        }
-
-        if (kb + 1 < nblocks) {
-            uint4 *kd = reinterpret_cast<uint4 *>(lds_k[buf ^ 1]) + tid;
-            uint4 *vd = reinterpret_cast<uint4 *>(lds_v[buf ^ 1]) + tid;
-            kd[0] = pre0;
-            kd[256] = pre1;
-            vd[0] = pre2;
-            vd[256] = pre3;
-        }
-        __syncthreads();
-    }
-
-    // ---- normalise and write --------------------------------------------------------------
-#pragma unroll
-    for (int qt = 0; qt < kTiles; ++qt) {
-        float lt = l[qt];
-        lt += __shfl_xor(lt, 16);
-        lt += __shfl_xor(lt, 32);
-        const uint32_t j = qt * 16 + jl;
-        const uint32_t row = row_begin + j / group, head = kv_head * group + j % group;
-        if (row >= item.rows) continue;
-        const float inv = 1.0f / lt;
-        float *dst = p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + g * 4;
-#pragma unroll
-        for (int dt = 0; dt < 8; ++dt)
-            *reinterpret_cast<floatx4 *>(dst + dt * 16) = o[qt][dt] * inv;
-    }
-}
-
-
-// ---- two wavefronts per SIMD ------------------------------------------------------------
-// Same tiling of the problem, half the query vectors per workgroup: 128 vectors, 32 per
-// wavefront (2 MFMA column tiles), at most 256 registers, so that two workgroups share a
-// compute unit and one wavefront's softmax runs under the other's MFMAs. The softmax keeps a
-// *reference* maximum per column instead of the exact running maximum:
+// K/V blocks travel HBM -> LDS without passing through registers (global_load_lds_dwordx4:
+// lane i of the instruction writes 16 bytes at M0 + 16*i) into a ring of four stages, so
+// the loads of three blocks are in flight while one is multiplied; the latency of a miss is
+// about a microsecond, more than two block times. The planes are stored as the MFMA
+// consumes them, so the key block is a straight 8 KiB copy; the 16-byte pieces of the value
+// block are permuted on the way in (the source address of such a load is free per lane, the
+// destination is lane-linear) so that every operand read of a wavefront is one KiB of
+// consecutive LDS: no bank conflicts.
+//
+// The softmax keeps a *reference* maximum per column instead of the exact running maximum:
 //   * the reference enters the score MFMA as its initial accumulator (-ref), so the product
 //     comes out as s - ref and the exponent needs no subtraction;
 //   * the reference moves only when some score of the block exceeds it by more than
@@ -259,9 +30,21 @@ __global__ __launch_bounds__(kWaves * 64) void attn_prefill_f16_kernel(AttnParam
 //     term of numerator and denominator carries the same factor 2^-ref.
 // A column with nothing visible yet has ref = 0 and threshold -inf, so its first finite
 // score sets the reference exactly.
-constexpr int kTiles2 = 2;
-constexpr int kVecPerWave2 = kTiles2 * 16;            // 32
-constexpr int kVecPerGroup2 = kWaves * kVecPerWave2;  // 128
+//
+// The chunk's own K/V rows are appended before this kernel runs; row r of the chunk sits at
+// position pos0 + r and sees keys <= its position (attention.rs:77-85 with no window).
+#include "internal.h"
+#include "mfma_common.h"
+
+namespace itak {
+
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kTiles = 2;                           // MFMA column tiles (16 vectors) per wavefront
+constexpr int kVecPerWave = kTiles * 16;            // 32
+constexpr int kVecPerGroup = kWaves * kVecPerWave;  // 128 query vectors per workgroup
+constexpr int kBlockElems = kBlockKeys * kD;        // 4096 halves = 8 KiB per plane block
 constexpr float kRefSlack = 8.0f;
 
 __device__ __forceinline__ float column_max4(float v) {
@@ -277,13 +60,9 @@ __device__ __forceinline__ float column_sum4(float v) {
     return __uint_as_float(c[0]) + __uint_as_float(c[1]);
 }
 
-// K/V blocks travel HBM -> LDS without passing through registers (global_load_lds_dwordx4:
-// lane i of the instruction writes 16 bytes at M0 + 16*i) into a ring of kStages stages, so
-// loads for three blocks ahead are in flight while one is multiplied; the latency of a
-// miss is about a microsecond, more than two block times. The instruction is issued from
-// inline assembly: the compiler then neither tracks it (it would make every LDS read wait
-// for all of them) nor needs to, because the only consumer is ordered by the explicit
-// s_waitcnt vmcnt + s_barrier at the top of each iteration.
+// The direct-to-LDS load is issued from inline assembly: the compiler then neither tracks it
+// (it would make every LDS read wait for all of them) nor needs to, because the only consumer
+// is ordered by the explicit s_waitcnt vmcnt + s_barrier at the top of each iteration.
 constexpr int kStages = 4;
 constexpr int kStageBytes = 2 * kBlockElems * 2;  // one key block + one value block
 
@@ -300,7 +79,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 template <int N, bool SOFTCAP>
-__global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnParams p,
+__global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnParams p,
                                                                            AttnBatchT<N> b) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lds_ring[];  // [kStages][K block | V block]
 
@@ -310,8 +89,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
 
     const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
     const uint32_t group = p.group;
-    const uint32_t rows_per_group = kVecPerGroup2 / group;
-    const uint32_t rows_per_wave = kVecPerWave2 / group;
+    const uint32_t rows_per_group = kVecPerGroup / group;
+    const uint32_t rows_per_wave = kVecPerWave / group;
     const uint32_t local = blockIdx.x - item.block0;
     const uint32_t kv_head = local % p.g.kv_heads;
     const uint32_t tiles = (item.rows + rows_per_group - 1) / rows_per_group;
@@ -358,10 +137,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
     const float softcap = p.softcap;
     const float inv_cap = SOFTCAP ? 1.0f / softcap : 0.0f;
     const float qscale = SOFTCAP ? p.scale : p.scale * kLog2e;
-    half8 qb[kTiles2][4];
-    uint32_t colpos[kTiles2];
+    half8 qb[kTiles][4];
+    uint32_t colpos[kTiles];
 #pragma unroll
-    for (int qt = 0; qt < kTiles2; ++qt) {
+    for (int qt = 0; qt < kTiles; ++qt) {
         const uint32_t j = qt * 16 + jl;
         const uint32_t row = row_begin + j / group;
         colpos[qt] = item.pos0 + row;
@@ -383,11 +162,11 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
         }
     }
 
-    float ref[kTiles2], thr[kTiles2], l[kTiles2];
-    floatx4 negref[kTiles2];
-    floatx4 o[kTiles2][8];
+    float ref[kTiles], thr[kTiles], l[kTiles];
+    floatx4 negref[kTiles];
+    floatx4 o[kTiles][8];
 #pragma unroll
-    for (int qt = 0; qt < kTiles2; ++qt) {
+    for (int qt = 0; qt < kTiles; ++qt) {
         ref[qt] = 0.0f;
         thr[qt] = -INFINITY;
         l[qt] = 0.0f;
@@ -408,7 +187,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
 
         if (kb < wave_blocks) {
             const uint32_t key_base = kb * kBlockKeys + g * 8;
-            floatx4 x[kTiles2][2];
+            floatx4 x[kTiles][2];
             {
                 half8 ka[2][4];
                 const uint16_t *kl = lds_k + (g * 16 + jl) * 8;
@@ -419,7 +198,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
                         ka[t][s] =
                             *reinterpret_cast<const half8 *>(kl + ((t * 16 + s * 4) * 16) * 8);
 #pragma unroll
-                for (int qt = 0; qt < kTiles2; ++qt)
+                for (int qt = 0; qt < kTiles; ++qt)
 #pragma unroll
                     for (int t = 0; t < 2; ++t) {
                         floatx4 s = negref[qt];
@@ -437,7 +216,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
 
             if constexpr (SOFTCAP) {  // negref stays zero: x is the raw scaled score here
 #pragma unroll
-                for (int qt = 0; qt < kTiles2; ++qt)
+                for (int qt = 0; qt < kTiles; ++qt)
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
                         x[qt][e >> 2][e & 3] =
@@ -445,7 +224,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
             }
             if (kb >= first_masked) {
 #pragma unroll
-                for (int qt = 0; qt < kTiles2; ++qt)
+                for (int qt = 0; qt < kTiles; ++qt)
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
                         if (key_base + e > colpos[qt]) x[qt][e >> 2][e & 3] = -INFINITY;
@@ -458,10 +237,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
                             if (key_base + e >= item.kv_len) va[dt][e] = _Float16(0.0f);
                 }
             }
-            float lmax[kTiles2];
+            float lmax[kTiles];
             bool over = false;
 #pragma unroll
-            for (int qt = 0; qt < kTiles2; ++qt) {
+            for (int qt = 0; qt < kTiles; ++qt) {
                 float mx = fmaxf(fmaxf(x[qt][0][0], x[qt][0][1]), x[qt][0][2]);
                 mx = fmaxf(fmaxf(mx, x[qt][0][3]), x[qt][1][0]);
                 mx = fmaxf(fmaxf(mx, x[qt][1][1]), x[qt][1][2]);
@@ -471,7 +250,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
             if (__builtin_amdgcn_ballot_w64(over) != 0) {
                 // Some column's scores ran past its reference (or it saw its first key).
 #pragma unroll
-                for (int qt = 0; qt < kTiles2; ++qt) {
+                for (int qt = 0; qt < kTiles; ++qt) {
                     const float cm = column_max4(lmax[qt]);
                     const bool live = thr[qt] != -INFINITY;
                     float delta = live ? fmaxf(cm, 0.0f) : cm;
@@ -493,7 +272,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
                 }
             }
 #pragma unroll
-            for (int qt = 0; qt < kTiles2; ++qt) {
+            for (int qt = 0; qt < kTiles; ++qt) {
                 float pe[8];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) pe[e] = fast_exp2(x[qt][e >> 2][e & 3]);
@@ -511,7 +290,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
     wait_vmcnt<0>();  // the surplus loads of the last iterations
 
 #pragma unroll
-    for (int qt = 0; qt < kTiles2; ++qt) {
+    for (int qt = 0; qt < kTiles; ++qt) {
         const float lt = column_sum4(l[qt]);
         const uint32_t j = qt * 16 + jl;
         const uint32_t row = row_begin + j / group, head = kv_head * group + j % group;
@@ -524,21 +303,17 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill2_f16_kernel(AttnP
     }
 }
 
-}  // namespace
 
-static bool use_old_prefill() {
-    static const bool old = getenv("ITAK_PREFILL_OLD") != nullptr;
-    return old;
-}
+}  // namespace
 
 bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group) {
     return g.v_block == kVBlock && g.head_dim == kD && group >= 1 &&
-           group <= uint32_t(kVecPerWave2) && kVecPerWave2 % group == 0;
+           group <= uint32_t(kVecPerWave) && kVecPerWave % group == 0;
 }
 
 // Fills block0 for a batch (slot, rows, pos0, q_row0, kv_len already set).
 void attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group) {
-    const uint32_t rows_per_group = (use_old_prefill() ? kVecPerGroup : kVecPerGroup2) / group;
+    const uint32_t rows_per_group = kVecPerGroup / group;
     uint32_t block0 = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         AttnItem &it = b.item[i];
@@ -553,28 +328,23 @@ void attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group) {
 }
 
 template <int N, bool SOFTCAP>
-static hipError_t launch_prefill2(const AttnParams &p, const AttnBatch &b, hipStream_t stream) {
+static hipError_t launch_prefill(const AttnParams &p, const AttnBatch &b, hipStream_t stream) {
     constexpr size_t lds = size_t(kStages) * kStageBytes;
     static const hipError_t granted = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(&attn_prefill2_f16_kernel<N, SOFTCAP>),
+        reinterpret_cast<const void *>(&attn_prefill_f16_kernel<N, SOFTCAP>),
         hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
     if (granted != hipSuccess) return granted;
-    attn_prefill2_f16_kernel<N, SOFTCAP><<<b.total_blocks, kWaves * 64, lds, stream>>>(p, AttnBatchT<N>(b));
+    attn_prefill_f16_kernel<N, SOFTCAP><<<b.total_blocks, kWaves * 64, lds, stream>>>(p, AttnBatchT<N>(b));
     return hipGetLastError();
 }
 
 hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, hipStream_t stream) {
     if (b.total_blocks == 0) return hipSuccess;
-    if (use_old_prefill()) {
-        ITAK_DISPATCH_BATCH(b.n, (attn_prefill_f16_kernel<N><<<b.total_blocks, kWaves * 64, 0, stream>>>(
-                                     p, AttnBatchT<N>(b))));
-        return hipGetLastError();
-    }
     hipError_t e = hipSuccess;
     if (p.softcap > 0.0f)
-        ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill2<N, true>(p, b, stream)));
+        ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, true>(p, b, stream)));
     else
-        ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill2<N, false>(p, b, stream)));
+        ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, false>(p, b, stream)));
     return e;
 }
 
