@@ -14,7 +14,9 @@ the CPU oracle timed on the host cores beside it.
 
 `--workload ragged|verify|prefill` measures the other configurations (continuous batching
 over 16 ragged slots, the speculative verify block, the chunked causal prefill) with the
-same JSON shape; they are secondary measurements, the default line is the contract.
+same JSON shape; `--workload restore|append` measures the cache-maintenance kernels (the
+48-layer prefix-snapshot gather of configs[4]; the append of a 2048-row chunk). They are
+secondary measurements, the default line is the contract.
 """
 from __future__ import annotations
 
@@ -89,6 +91,100 @@ def cpu_baseline(ctx: int, kv_bytes_per_layer: int, layers: int, budget_s: float
     }
 
 
+def cache_maintenance(args, pkg, torch, dev, stream, timed):
+    """restore: the 8192-token x 48-layer prefix snapshot of configs[4] gathered into the
+    device cache (f16 rows copied raw, f32 rows converted like append), from a source in HBM
+    (the kernel's own speed) and from pinned host memory (what a session start pays: the
+    host link). append: a 2048-row chunk per layer, f32 -> f16, into a cache of 30720 rows."""
+    layers, tokens = 48, 8192
+    if args.workload == "append":
+        layers, prefix, chunk = 8, 30720, 2048
+        pool = pkg.KvPool(layers, KV_HEADS, D, elem="f16", max_slots=1,
+                          capacity_rows=prefix + chunk, scrub_on_truncate=False)
+        pool.set_stream(stream.cuda_stream)
+        cache = pool.acquire()
+        k = torch.randn(layers, chunk, ROW, device=dev)
+        v = torch.randn(layers, chunk, ROW, device=dev)
+        zero = torch.zeros(prefix, ROW, device=dev)
+        for layer in range(layers):
+            pool.append_device(layer, [(cache, prefix)], zero.data_ptr(), zero.data_ptr())
+
+        def step():
+            for layer in range(layers):
+                pool.append_device(layer, [(cache, chunk)], k[layer].data_ptr(), v[layer].data_ptr())
+            pool.truncate([cache], [prefix])
+
+        for _ in range(max(args.warmup, 1)):
+            step()
+        graph = capture(torch, pool, stream, step)
+        pool.truncate([cache], [prefix])
+        graph.replay()
+        step_s = timed(graph.replay, args.steps)[0] / args.steps
+        bytes_layer = chunk * 2 * ROW * (4 + 2)
+        gbs = bytes_layer * layers / step_s / 1e9
+        result = {
+            "metric": "KV append GB/s (2048-row chunk, f32 -> f16, bytes read + written)",
+            "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 5),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+            "data": "synthetic",
+            "config": {"workload": "append of a 2048-row chunk per layer into a 30720-row f16 cache, "
+                                   "8 layers cycled, HIP graph replay", "layers_per_step": layers},
+            "roofline": {"bound": "hbm", "kernel": "kv_append_kernel", "achieved": round(gbs, 2),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                         "traffic": None, "us_per_launch": round(step_s / layers * 1e6, 3),
+                         "bytes_per_launch": bytes_layer},
+        }
+        pool.close()
+        return result
+
+    pool = pkg.KvPool(layers, KV_HEADS, D, elem="f16", max_slots=1, capacity_rows=tokens,
+                      scrub_on_truncate=False)
+    pool.set_stream(stream.cuda_stream)
+    cache = pool.acquire()
+    elems = layers * tokens * ROW
+    dev_k = torch.randn(layers, tokens, ROW, device=dev).half()
+    dev_v = torch.randn(layers, tokens, ROW, device=dev).half()
+    pin_k16, pin_v16 = dev_k.cpu().pin_memory(), dev_v.cpu().pin_memory()
+    pin_k32, pin_v32 = dev_k.float().cpu().pin_memory(), dev_v.float().cpu().pin_memory()
+
+    def restore_from(k, v, f16):
+        def run():
+            cache.restore_snapshot_ptrs(tokens, [(0, tokens, k[l].data_ptr(), v[l].data_ptr())
+                                                 for l in range(layers)], src_f16=f16)
+            pool.truncate([cache], [0])
+        run()
+        reps = max(3, min(args.steps, 20))
+        return timed(run, reps)[0] / reps
+
+    dst_bytes = 2 * elems * 2
+    t_dev = restore_from(dev_k, dev_v, True)
+    t_pin16 = restore_from(pin_k16, pin_v16, True)
+    t_pin32 = restore_from(pin_k32, pin_v32, False)
+    gbs = 2 * dst_bytes / t_dev / 1e9  # reads the f16 source and writes the planes
+    result = {
+        "metric": "prefix-snapshot restore GB/s (48 layers x 8192 rows, source in HBM, bytes read + written)",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(t_dev * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "configs[4] restore: 8192-token x 48-layer snapshot gathered into the "
+                               "f16 device cache", "snapshot_bytes_f16": dst_bytes},
+        "from_pinned_host": {
+            "f16_rows_ms": round(t_pin16 * 1e3, 3),
+            "f16_rows_GBps_over_link": round(dst_bytes / t_pin16 / 1e9, 2),
+            "f32_rows_ms": round(t_pin32 * 1e3, 3),
+            "f32_rows_GBps_over_link": round(2 * dst_bytes / t_pin32 / 1e9, 2),
+        },
+        "roofline": {"bound": "hbm", "kernel": "kv_restore_rows + kv_restore_v_blocked (all layers, "
+                                               "two launches)",
+                     "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "us_per_launch": round(t_dev / 2 * 1e6, 2), "bytes_per_launch": dst_bytes},
+    }
+    pool.close()
+    return result
+
+
 class Timer:
     def __init__(self, torch, stream):
         self.torch, self.stream = torch, stream
@@ -141,7 +237,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["decode", "ragged", "verify", "prefill"],
+    ap.add_argument("--workload", choices=["decode", "ragged", "verify", "prefill", "restore", "append"],
                     default="decode")
     ap.add_argument("--softcap", type=float, default=0.0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -165,6 +261,9 @@ def main():
 
     # ---- workload shapes -------------------------------------------------------------
     wl = args.workload
+    if wl in ("restore", "append"):
+        print(json.dumps(cache_maintenance(args, pkg, torch, dev, stream, timed)))
+        return
     if wl == "decode":
         layers, slots, rows, lengths = 48, 1, 1, [4096]
         name = ("configs[1]: 30B-class decode step, batch 1, 48 layers, 32 Q / 4 KV heads, "
@@ -286,7 +385,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32 softmax and accumulation over f16 KV (f16 MFMA operands)",
+        "dtype": "f16",
         "data": "synthetic",
         "config": {
             "workload": name,
@@ -294,6 +393,7 @@ def main():
             "layers_per_step": layers,
             "kv_bytes_per_step": kv_bytes_layer * layers,
             "softcap": args.softcap,
+            "arithmetic": "f16 KV and MFMA operands, f32 scores, softmax and accumulation",
         },
         "us_per_token": round(step_s * 1e6 * (48 / layers), 2),
         "pct_of_hbm_peak": round(100.0 * kv_bytes_layer * layers / step_s / 1e9 / HBM_PEAK_GBS, 2),

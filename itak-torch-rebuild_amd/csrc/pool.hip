@@ -342,6 +342,37 @@ float default_scale(uint64_t head_dim) {  // attention.rs:35-37
 // Appends `rows` rows per item from device sources; the caller has validated everything.
 itak_status run_append(itak_pool *pool, uint64_t layer, const itak_batch_item *items, uint32_t n,
                        const float *k_dev, const float *v_dev) {
+    // A long run of rows into blocked planes (a prefill chunk) goes in two parts: the rows up
+    // to the next 32-row boundary through the row kernel, the block-aligned rest through the
+    // gather kernels of the snapshot restore, which transpose whole value blocks in LDS and
+    // store 16 bytes per thread instead of 2. The rows after the run inside its last block
+    // are beyond the slot's length; the gather writes zeros there, which is what they hold.
+    constexpr uint32_t kChunkRows = 4 * kVBlock;
+    if (n == 1 && pool->elem_f16 && pool->g.v_block != 0 && items[0].rows >= kChunkRows) {
+        const uint32_t slot = items[0].slot, rows = items[0].rows;
+        const uint32_t pos0 = uint32_t(pool->slots[slot].appended[layer]);
+        const uint32_t head_rows = (kVBlock - pos0 % kVBlock) % kVBlock;
+        if (head_rows) {
+            AppendBatch b{};
+            b.n = 1;
+            b.total_rows = head_rows;
+            b.item[0] = AppendItem{slot, head_rows, pos0, 0};
+            HIP_TRY(pool, launch_append(layer_base(pool, layer), 1, pool->g, b, k_dev, v_dev,
+                                        pool->stream),
+                    "launch append");
+        }
+        RestoreBatch rb{};
+        rb.n = 1;
+        rb.max_rows = rows - head_rows;
+        rb.slot = slot;
+        rb.layer[0] = RestoreLayer{k_dev + uint64_t(head_rows) * pool->row,
+                                   v_dev + uint64_t(head_rows) * pool->row, uint32_t(layer),
+                                   rows - head_rows, pos0 + head_rows, 0};
+        HIP_TRY(pool, launch_restore(pool->base, 1, 0, pool->g, rb, pool->stream),
+                "launch chunk append");
+        pool->slots[slot].appended[layer] += rows;
+        return ITAK_OK;
+    }
     uint32_t src_row = 0;
     for (uint32_t first = 0; first < n; first += kMaxBatchItems) {
         const uint32_t count = std::min<uint32_t>(kMaxBatchItems, n - first);

@@ -117,6 +117,35 @@ def test_append_is_bit_exact_against_the_oracle(elem, kv_heads, head_dim):
             assert gk.tobytes() == ck.tobytes() and gv.tobytes() == cv.tobytes()
 
 
+@pytest.mark.parametrize("start,rows", [(0, 128), (45, 300), (64, 129), (31, 2048)])
+def test_chunk_append_is_bit_exact_and_leaves_its_neighbours_alone(start, rows):
+    # A long run of rows appended in one call (a prefill chunk) at aligned and unaligned
+    # positions: device bytes equal the host conversion, the rows before the run keep their
+    # bytes, the rows after it are still zero.
+    import torch
+
+    kv_heads, head_dim = 4, 128
+    width = kv_heads * head_dim
+    rng = np.random.default_rng(start * 7 + rows)
+    n = start + rows
+    k, v = normal(rng, n, width), normal(rng, n, width)
+    k[start + 1, 5], v[start + 2, 7], k[n - 1, 0] = np.nan, np.inf, 65520.0
+    pool = P().KvPool(1, kv_heads, head_dim, elem="f16", capacity_rows=n + 70)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    cache = pool.acquire()
+    kd, vd = torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda()
+    for p in range(start):  # one row at a time
+        pool.append_device(0, [(cache, 1)], kd[p:].data_ptr(), vd[p:].data_ptr())
+    pool.append_device(0, [(cache, rows)], kd[start:].data_ptr(), vd[start:].data_ptr())
+    assert cache.next_position(0) == n
+    gk, gv = cache.read_raw(0)
+    want_k, want_v = oracle.f32_to_f16_array(k), oracle.f32_to_f16_array(v)
+    assert np.array_equal(gk[:n].reshape(n, width), want_k)
+    assert np.array_equal(gv[:n].reshape(n, width), want_v)
+    assert not gk[n:].any() and not gv[n:].any()
+    pool.close()
+
+
 def test_f32_to_f16_conversion_matches_the_oracle_on_every_rounding_class():
     import torch
 
