@@ -36,14 +36,14 @@
 #include "internal.h"
 #include "mfma_common.h"
 
+#include <algorithm>
+
 namespace itak {
 
 namespace {
 
 constexpr int kWaves = 4;
-constexpr int kTiles = 2;                           // MFMA column tiles (16 vectors) per wavefront
-constexpr int kVecPerWave = kTiles * 16;            // 32
-constexpr int kVecPerGroup = kWaves * kVecPerWave;  // 128 query vectors per workgroup
+constexpr int kMaxTiles = 2;  // MFMA column tiles (16 query vectors) per wavefront: 1 or 2
 constexpr int kBlockElems = kBlockKeys * kD;        // 4096 halves = 8 KiB per plane block
 constexpr float kRefSlack = 8.0f;
 
@@ -78,9 +78,12 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
 }
 
-template <int N, bool SOFTCAP>
+template <int N, bool SOFTCAP, int kTiles>
 __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnParams p,
-                                                                           AttnBatchT<N> b) {
+                                                                           AttnBatchT<N> b,
+                                                                           uint32_t total_partials) {
+    constexpr int kVecPerWave = kTiles * 16;
+    constexpr int kVecPerGroup = kWaves * kVecPerWave;  // query vectors per workgroup
     extern __shared__ __attribute__((aligned(16))) uint16_t lds_ring[];  // [kStages][K block | V block]
 
     const uint32_t tid = threadIdx.x;
@@ -91,10 +94,12 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     const uint32_t group = p.group;
     const uint32_t rows_per_group = kVecPerGroup / group;
     const uint32_t rows_per_wave = kVecPerWave / group;
+    // Workgroup -> (row tile, kv head, split of the context).
     const uint32_t local = blockIdx.x - item.block0;
-    const uint32_t kv_head = local % p.g.kv_heads;
+    const uint32_t unit = local / item.splits, split = local - unit * item.splits;
+    const uint32_t kv_head = unit % p.g.kv_heads;
     const uint32_t tiles = (item.rows + rows_per_group - 1) / rows_per_group;
-    const uint32_t tile = tiles - 1 - local / p.g.kv_heads;  // longest first
+    const uint32_t tile = tiles - 1 - unit / p.g.kv_heads;  // longest first
     const uint32_t row_begin = tile * rows_per_group + wave * rows_per_wave;
     const uint32_t wg_row_end = min(item.rows, (tile + 1) * rows_per_group);
 
@@ -102,7 +107,11 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                              item.slot * p.g.slot_stride + kv_head * p.g.head_stride;
     const uint16_t *vplane = kplane + p.g.side_stride;
 
-    const uint32_t nblocks = (item.pos0 + wg_row_end + kBlockKeys - 1) / kBlockKeys;
+    // Blocks of this workgroup: its split's run, cut at the last block its rows can see.
+    const uint32_t blocks_per_split = item.keys_per_split / kBlockKeys;
+    const uint32_t kb_begin = split * blocks_per_split;
+    const uint32_t nblocks = min((item.pos0 + wg_row_end + kBlockKeys - 1) / kBlockKeys,
+                                 kb_begin + blocks_per_split);
     const uint32_t wave_row_end = min(item.rows, row_begin + rows_per_wave);
     const uint32_t wave_blocks =
         row_begin < item.rows ? (item.pos0 + wave_row_end + kBlockKeys - 1) / kBlockKeys : 0;
@@ -130,9 +139,12 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
         lds_dma16(vg + off, dst + 8192);
         lds_dma16(vg + off + 256, dst + 12288);
     };
-    issue_block(0);
-    issue_block(1);
-    issue_block(2);
+    const bool any_block = kb_begin < nblocks;  // a split past the rows' horizon has none
+    if (any_block) {
+        issue_block(kb_begin);
+        issue_block(kb_begin + 1);
+        issue_block(kb_begin + 2);
+    }
 
     const float softcap = p.softcap;
     const float inv_cap = SOFTCAP ? 1.0f / softcap : 0.0f;
@@ -175,7 +187,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
         for (int dt = 0; dt < 8; ++dt) o[qt][dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
-    for (uint32_t kb = 0; kb < nblocks; ++kb) {
+    for (uint32_t kb = kb_begin; kb < nblocks; ++kb) {
         // This thread's pieces of block kb have landed (the 8 loads of the next two blocks
         // may still fly); after the barrier everybody's have, and everybody is done with
         // block kb - 1, whose stage the loads for block kb + 3 may now overwrite.
@@ -287,64 +299,123 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
         }
 
     }
-    wait_vmcnt<0>();  // the surplus loads of the last iterations
+    if (any_block) wait_vmcnt<0>();  // the surplus loads of the last iterations
 
+    // One split: the normalised output. Several: the partial (m, l, acc[128]) of this split
+    // in the log2 domain, merged by the combine launch; a column that saw nothing writes
+    // m = -inf and zeros.
+    const bool final_out = item.splits == 1;
+    float *const ws_acc = p.ws;
+    float *const ws_ml = p.ws + uint64_t(total_partials) * kD;
 #pragma unroll
     for (int qt = 0; qt < kTiles; ++qt) {
         const float lt = column_sum4(l[qt]);
         const uint32_t j = qt * 16 + jl;
         const uint32_t row = row_begin + j / group, head = kv_head * group + j % group;
         if (row >= item.rows) continue;
-        const float inv = 1.0f / lt;
-        float *dst = p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + g * 4;
+        if (final_out) {
+            const float inv = 1.0f / lt;
+            float *dst = p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + g * 4;
 #pragma unroll
-        for (int dt = 0; dt < 8; ++dt)
-            *reinterpret_cast<floatx4 *>(dst + dt * 16) = o[qt][dt] * inv;
+            for (int dt = 0; dt < 8; ++dt)
+                *reinterpret_cast<floatx4 *>(dst + dt * 16) = o[qt][dt] * inv;
+        } else {
+            const uint64_t ps = item.ws0 + (uint64_t(row) * p.q_heads + head) * item.splits + split;
+            float *dst = ws_acc + ps * kD + g * 4;
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) *reinterpret_cast<floatx4 *>(dst + dt * 16) = o[qt][dt];
+            if (g == 0)
+                *reinterpret_cast<float2 *>(ws_ml + ps * 2) =
+                    make_float2(thr[qt] == -INFINITY ? -INFINITY : ref[qt], lt);
+        }
     }
 }
-
 
 }  // namespace
 
 bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group) {
-    return g.v_block == kVBlock && g.head_dim == kD && group >= 1 &&
-           group <= uint32_t(kVecPerWave) && kVecPerWave % group == 0;
+    return g.v_block == kVBlock && g.head_dim == kD && group >= 1 && group <= 16 &&
+           16 % group == 0;
 }
 
-// Fills block0 for a batch (slot, rows, pos0, q_row0, kv_len already set).
-void attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group) {
-    const uint32_t rows_per_group = kVecPerGroup / group;
-    uint32_t block0 = 0;
+// Up to 64 query vectors per KV head (speculative blocks) take one 16-vector tile per
+// wavefront, so that all four wavefronts of the workgroup have columns; more take two.
+static int tiles_for(const AttnBatch &b, uint32_t group) {
+    uint32_t nvec = 0;
+    for (uint32_t i = 0; i < b.n; ++i) nvec = std::max(nvec, b.item[i].rows * group);
+    return nvec <= uint32_t(kWaves * 16) ? 1 : kMaxTiles;
+}
+
+// Fills splits / keys_per_split / block0 / ws0 for a batch (slot, rows, pos0, q_row0, kv_len
+// already set) and returns the number of partials the launch will write. A unit is one
+// (row tile, KV head) of an item; the context of every unit is cut into equal runs of at
+// most T blocks, T the smallest run length for which the launch has at least two
+// workgroups per compute unit's worth of work units, and never shorter than 8 blocks
+// (a workgroup needs that many to amortise filling its load pipeline).
+uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, uint32_t q_heads) {
+    const uint32_t rows_per_group = uint32_t(tiles_for(b, group) * kWaves * 16) / group;
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        (void)hipGetLastError();
+    const uint64_t target = uint64_t(2) * uint64_t(cus > 0 ? cus : 256);
+    uint64_t unit_blocks = 0;
+    for (uint32_t i = 0; i < b.n; ++i) {
+        const uint64_t units = uint64_t(g.kv_heads) * ((b.item[i].rows + rows_per_group - 1) / rows_per_group);
+        unit_blocks += units * ((b.item[i].kv_len + kBlockKeys - 1) / kBlockKeys);
+    }
+    const uint64_t T = std::max<uint64_t>((unit_blocks + target - 1) / target, 8);
+    uint32_t block0 = 0, ws0 = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         AttnItem &it = b.item[i];
-        it.splits = 1;
-        it.keys_per_split = it.kv_len;
+        const uint32_t nblocks = (it.kv_len + kBlockKeys - 1) / kBlockKeys;
+        const uint32_t units = g.kv_heads * ((it.rows + rows_per_group - 1) / rows_per_group);
+        uint32_t splits = std::max<uint32_t>(uint32_t((nblocks + T - 1) / T), 1);
+        const uint32_t bps = std::max<uint32_t>((nblocks + splits - 1) / splits, 1);
+        splits = std::max<uint32_t>((nblocks + bps - 1) / bps, 1);
+        it.splits = splits;
+        it.keys_per_split = bps * kBlockKeys;
+        it.splits_magic = 0;
         it.block0 = block0;
-        it.ws0 = 0;
-        block0 += g.kv_heads * ((it.rows + rows_per_group - 1) / rows_per_group);
+        it.ws0 = ws0;
+        block0 += units * splits;
+        if (splits > 1) ws0 += it.rows * q_heads * splits;
     }
     b.total_blocks = block0;
     b.rows_per_block = rows_per_group;
+    return ws0;
 }
 
-template <int N, bool SOFTCAP>
-static hipError_t launch_prefill(const AttnParams &p, const AttnBatch &b, hipStream_t stream) {
+template <int N, bool SOFTCAP, int TILES>
+static hipError_t launch_prefill(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                                 hipStream_t stream) {
     constexpr size_t lds = size_t(kStages) * kStageBytes;
     static const hipError_t granted = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(&attn_prefill_f16_kernel<N, SOFTCAP>),
+        reinterpret_cast<const void *>(&attn_prefill_f16_kernel<N, SOFTCAP, TILES>),
         hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
     if (granted != hipSuccess) return granted;
-    attn_prefill_f16_kernel<N, SOFTCAP><<<b.total_blocks, kWaves * 64, lds, stream>>>(p, AttnBatchT<N>(b));
+    attn_prefill_f16_kernel<N, SOFTCAP, TILES><<<b.total_blocks, kWaves * 64, lds, stream>>>(
+        p, AttnBatchT<N>(b), total_partials);
     return hipGetLastError();
 }
 
-hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, hipStream_t stream) {
+hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                                   hipStream_t stream) {
     if (b.total_blocks == 0) return hipSuccess;
     hipError_t e = hipSuccess;
+    const bool one = tiles_for(b, p.group) == 1;
+#define ITAK_LAUNCH_TILES(SC)                                                                  \
+    do {                                                                                       \
+        if (one)                                                                               \
+            ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, SC, 1>(p, b, total_partials, stream))); \
+        else                                                                                   \
+            ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, SC, 2>(p, b, total_partials, stream))); \
+    } while (0)
     if (p.softcap > 0.0f)
-        ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, true>(p, b, stream)));
+        ITAK_LAUNCH_TILES(true);
     else
-        ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, false>(p, b, stream)));
+        ITAK_LAUNCH_TILES(false);
+#undef ITAK_LAUNCH_TILES
     return e;
 }
 

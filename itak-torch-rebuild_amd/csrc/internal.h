@@ -253,10 +253,13 @@ bool attn_splitk_f16_supports(const PoolGeom &g, uint32_t group, uint32_t max_ro
 uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads);
 hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                   uint32_t max_rows, hipStream_t stream);
-// MFMA prefill path: same pools, any number of rows, group dividing 64; no splits.
+// MFMA block path (speculative blocks and prefill chunks): same pools, any number of rows,
+// group dividing 16; K/V staged through LDS, split over the context when the launch would
+// otherwise not fill the device. Partials are in log2 domain (combine with base2 = 1).
 bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group);
-void attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group);
-hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, hipStream_t stream);
+uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, uint32_t q_heads);
+hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                                   hipStream_t stream);
 // Merge of split partials; total_rows = query rows of the batch.
 hipError_t launch_attn_combine(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                uint32_t total_rows, int base2, hipStream_t stream);

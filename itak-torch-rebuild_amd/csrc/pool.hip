@@ -231,7 +231,12 @@ bool takes_splitk_f16(const itak_pool *pool, const PlanInput *in, uint32_t n, ui
     const uint32_t group = uint32_t(q_heads / pool->g.kv_heads);
     uint32_t max_rows = 0;
     for (uint32_t i = 0; i < n; ++i) max_rows = std::max(max_rows, in[i].rows);
-    return pool->elem_f16 && q_pos_dev == nullptr &&
+    // Decode and speculative blocks (up to 64 query vectors per KV head, up to 8 new rows):
+    // the split-K kernel, which also appends the new rows. Its 64-vector variant and the
+    // block kernel (wavefronts split the query vectors, K/V shared through LDS) attend at the
+    // same speed on a 7-row block; the fused append decides (one launch less per layer).
+    constexpr uint32_t max_vec = 64;
+    return pool->elem_f16 && q_pos_dev == nullptr && max_rows * group <= max_vec &&
            attn_splitk_f16_supports(pool->g, group, max_rows);
 }
 
@@ -276,7 +281,7 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         if (mfma) {
             partials = attn_splitk_f16_plan(pool->g, b, uint32_t(q_heads));
         } else if (prefill) {
-            attn_prefill_f16_plan(pool->g, b, group);
+            partials = attn_prefill_f16_plan(pool->g, b, group, uint32_t(q_heads));
         } else {
             b.rows_per_block = rpb;
             uint64_t key_work = 0;
@@ -324,12 +329,14 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
             HIP_TRY(pool, launch_attn_splitk_f16(p, b, partials, max_rows, pool->stream),
                     "launch split-K attention");
         } else if (prefill) {
-            HIP_TRY(pool, launch_attn_prefill_f16(p, b, pool->stream), "launch prefill attention");
+            HIP_TRY(pool, launch_attn_prefill_f16(p, b, partials, pool->stream),
+                    "launch block attention");
         } else {
             HIP_TRY(pool, launch_attn_generic(pool->elem_f16, p, b, partials, pool->stream),
                     "launch attention");
         }
-        HIP_TRY(pool, launch_attn_combine(p, b, partials, total_rows, mfma ? 1 : 0, pool->stream),
+        HIP_TRY(pool, launch_attn_combine(p, b, partials, total_rows, (mfma || prefill) ? 1 : 0,
+                                          pool->stream),
                 "launch split merge");
     }
     return ITAK_OK;

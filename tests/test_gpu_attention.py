@@ -269,3 +269,32 @@ def test_speculative_round_trip_rewind_restores_the_exact_continuation():
     with pytest.raises(P().StepFailed) as e:
         spec.cache_release(handle)
     assert "not this cache's live checkpoint" in e.value.detail
+
+
+@pytest.mark.parametrize("rows,ctx,softcap", [(9, 3000, 0.0), (40, 5000, 0.0), (130, 2100, 25.0)])
+def test_mid_size_blocks_split_over_the_context(rows, ctx, softcap):
+    # Blocks too long for the decode kernel and too short to fill the device by rows alone:
+    # the block kernel cuts the context into splits and the merge launch joins them.
+    # Row r at position ctx + r sees keys 0..ctx+r (causal inside the block).
+    import torch
+
+    q_heads, kv_heads, d = 32, 4, 128
+    rng = np.random.default_rng(rows)
+    n = ctx + rows
+    k, v = normal(rng, n, kv_heads * d), normal(rng, n, kv_heads * d)
+    q = normal(rng, rows, q_heads * d)
+    pool = P().KvPool(1, kv_heads, d, elem="f16", capacity_rows=n)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    cache = pool.acquire()
+    kd, vd, qd = [torch.from_numpy(a).cuda() for a in (k, v, q)]
+    out = torch.empty_like(qd)
+    pool.append_device(0, [(cache, ctx)], kd.data_ptr(), vd.data_ptr())
+    pool.attention_step_device(0, [(cache, rows)], qd.data_ptr(), kd[ctx:].data_ptr(),
+                               vd[ctx:].data_ptr(), out.data_ptr(), q_heads, softcap=softcap)
+    torch.cuda.synchronize()
+    ref = oracle.KvCache.new([oracle.LayerKind.Global], kv_heads, d, store_f16=True)
+    ref.restore_bulk(0, 0, k[:ctx], v[:ctx])
+    want = oracle.attention_step(ref, 0, q, k[ctx:], v[ctx:], q_heads, ctx,
+                                 oracle.AttentionParams(softcap=softcap), threads=8)
+    assert max_abs(out.cpu().numpy().reshape(-1), want) <= 2e-3
+    pool.close()
