@@ -34,11 +34,10 @@ ROW = KV_HEADS * D
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
-# HBM bytes per decode-layer launch pair measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# and scaled by the same counters on the probe copy of known size (see
-# profiles/attn_splitk_f16_decode_ctx4096_traffic.md for the runs and the scaling factors).
-# None = not measured.
-MEASURED_TRAFFIC = {"decode": 10_027_000}
+# HBM bytes per layer (all launches of the layer's attention) measured with rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE and scaled by the same counters on the probe copy of known size
+# (profiles/*_traffic.md hold the runs and the scaling factors). Missing = not measured.
+MEASURED_TRAFFIC = {"decode": 9_949_357, "ragged": 216_849_858, "prefill": 290_163_333}
 
 
 def rope_on_device(x, base):
@@ -130,7 +129,8 @@ def cache_maintenance(args, pkg, torch, dev, stream, timed):
             "data": "synthetic",
             "config": {"workload": "append of a 2048-row chunk per layer into a 30720-row f16 cache, "
                                    "8 layers cycled, HIP graph replay", "layers_per_step": layers},
-            "roofline": {"bound": "hbm", "kernel": "kv_append_kernel", "achieved": round(gbs, 2),
+            "roofline": {"bound": "hbm", "kernel": "kv_restore_rows + kv_restore_v_blocked (chunk append: "
+                                                   "two launches per layer)", "achieved": round(gbs, 2),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                          "traffic": None, "us_per_launch": round(step_s / layers * 1e6, 3),
                          "bytes_per_launch": bytes_layer},
@@ -363,8 +363,8 @@ def main():
         value = kv_bytes_layer * layers / step_s / 1e9
         roofline = {
             "bound": "hbm",
-            "kernel": "attn_splitk_f16_kernel + attn_combine_kernel (the two launches of one "
-                      "layer's attention)",
+            "kernel": "attn_splitk_f16_kernel + attn_combine128_kernel (the two launches of "
+                      "one layer's attention)",
             "achieved": round(kv_bytes_layer / attn_s / 1e9, 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
