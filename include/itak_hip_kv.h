@@ -62,7 +62,17 @@ enum {
     ITAK_INVALID_ARGUMENT = 17, /* null pointer, unknown slot, unknown enum value */
     ITAK_NO_FREE_SLOT = 18,     /* every slot of the pool is in use */
     ITAK_CAPACITY_EXCEEDED = 19,/* a slot would outgrow the pool's per-slot row capacity */
-    ITAK_UNSUPPORTED = 20       /* a shape or layer kind this build has no kernel for */
+    ITAK_UNSUPPORTED = 20,      /* a shape or layer kind this build has no kernel for */
+    /* itak_kv::KvError (crates/itak-kv/src/error.rs:13-124), the variants the snapshot path
+       raises; messages are its Display text (error.rs:141-188). */
+    ITAK_KV_BAD_MAGIC = 21,
+    ITAK_KV_UNSUPPORTED_VERSION = 22,   /* a = version */
+    ITAK_KV_TRUNCATED = 23,             /* a = expected bytes, b = actual */
+    ITAK_KV_CHECKSUM_MISMATCH = 24,     /* a = stored, b = computed */
+    ITAK_KV_INCONSISTENT_SNAPSHOT = 25,
+    ITAK_KV_GEOMETRY_MISMATCH = 26,
+    ITAK_KV_FINGERPRINT_MISMATCH = 27,
+    ITAK_KV_INCOHERENT_CACHE = 28
 };
 
 /* Storage / source element types. */
@@ -133,6 +143,30 @@ typedef struct itak_snapshot_layer {
     const void *keys;   /* [rows][kv_heads][head_dim], oldest first */
     const void *values; /* same shape */
 } itak_snapshot_layer;
+
+/* The fixed part of an ITKV v1 snapshot (crates/itak-kv/src/snapshot.rs:13-29): the
+   geometry of itak_kv::KvGeometry (snapshot.rs:57-65) plus token count and fingerprint. */
+typedef struct itak_itkv_header {
+    uint64_t token_count;
+    uint64_t num_kv_heads;
+    uint64_t head_dim;
+    uint64_t layer_count;
+    uint64_t fingerprint_len;
+    uint64_t fingerprint_offset; /* decode: byte offset of the UTF-8 fingerprint in the buffer */
+    uint64_t encoded_len;        /* decode: bytes consumed, trailing checksum included */
+} itak_itkv_header;
+
+/* One layer of an ITKV snapshot: its 28-byte header (snapshot.rs:24-26) and where its
+   rows sit in the encoded buffer (f32 little-endian, keys then values). */
+typedef struct itak_itkv_layer {
+    uint32_t kind; /* ITAK_LAYER_* */
+    uint32_t reserved;
+    uint64_t window; /* 0 for a global layer */
+    uint64_t first_position;
+    uint64_t rows;
+    uint64_t keys_offset;
+    uint64_t values_offset;
+} itak_itkv_layer;
 
 /* ---- library ------------------------------------------------------------------ */
 
@@ -227,6 +261,51 @@ itak_status itak_kv_release(itak_pool *pool, uint32_t slot, const itak_checkpoin
    layer (RewindOutOfRange) or a slot with a live checkpoint (CheckpointBusy). */
 itak_status itak_kv_truncate(itak_pool *pool, const uint32_t *slots, const uint64_t *new_lengths,
                              uint32_t count);
+
+/* ---- prefix snapshots: itak_kv (crates/itak-kv/src) ------------------------------------ */
+
+/* hash::prefix_hash, prefix_discriminator, checksum (hash.rs:44-61): FNV-1a 64. */
+uint64_t itak_kv_prefix_hash(const uint32_t *tokens, uint64_t count);
+uint64_t itak_kv_prefix_discriminator(const uint32_t *tokens, uint64_t count);
+uint64_t itak_kv_checksum(const void *bytes, uint64_t count);
+
+/* The three calls below take no pool: after a failure itak_last_error(NULL) and
+   itak_last_error_info(NULL, ..) return the refusal, per thread. */
+
+/* KvSnapshot::validate (snapshot.rs:187-236) of a snapshot held by the caller: `blocks`
+   layer blocks whose key / value arrays hold key_floats[i] / value_floats[i] floats. */
+itak_status itak_itkv_validate(const itak_itkv_header *header, const itak_itkv_layer *layers,
+                               uint64_t blocks, const uint64_t *key_floats,
+                               const uint64_t *value_floats);
+/* KvSnapshot::to_bytes (snapshot.rs:381-403): validates, then writes the versioned byte
+   format. With out == NULL only *written (the size) is set. */
+itak_status itak_itkv_encode(const itak_itkv_header *header, const char *fingerprint,
+                             const itak_itkv_layer *layers, uint64_t blocks,
+                             const float *const *keys, const uint64_t *key_floats,
+                             const float *const *values, const uint64_t *value_floats, void *out,
+                             uint64_t capacity, uint64_t *written);
+/* KvSnapshot::from_bytes (snapshot.rs:405-509): strict decode. Rows are not copied: each
+   layer's keys_offset / values_offset locate its f32 rows inside `bytes`. Fills at most
+   layers_capacity entries; a smaller capacity than header->layer_count is refused after the
+   header has been filled, so a caller may size its array from a first call with 0. */
+itak_status itak_itkv_decode(const void *bytes, uint64_t len, itak_itkv_header *header,
+                             itak_itkv_layer *layers, uint64_t layers_capacity);
+
+/* KvSnapshot::capture (snapshot.rs:247-302) of a slot, written straight as ITKV v1 bytes
+   into host memory: refuses a slot whose layers disagree on position (IncoherentCache),
+   reads every layer's visible rows back as f32 (the rows of an f16 pool widen exactly) and
+   appends the checksum. With out == NULL only *written (the size) is set. */
+itak_status itak_kv_capture_itkv(itak_pool *pool, uint32_t slot, const char *fingerprint,
+                                 uint64_t fingerprint_len, void *out, uint64_t capacity,
+                                 uint64_t *written);
+/* KvSnapshot::from_bytes followed by restore_checked (snapshot.rs:351-371) into a fresh
+   slot: the snapshot's geometry must be the pool's, and, when expected_fingerprint is not
+   NULL, its fingerprint the expected one. The rows are gathered from `bytes` in place when
+   the device can read them there (pinned host or device memory, 4-byte aligned payload),
+   otherwise staged. An f32 snapshot into an f16 pool converts exactly as append does. */
+itak_status itak_kv_restore_itkv(itak_pool *pool, uint32_t slot, const void *bytes, uint64_t len,
+                                 const char *expected_fingerprint,
+                                 uint64_t expected_fingerprint_len);
 
 /* ---- attention over one slot, host pointers ---------------------------------------- */
 

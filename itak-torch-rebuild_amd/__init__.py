@@ -21,10 +21,24 @@ from .hip_compute import (  # noqa: F401
     gqa_attention,
     kv_head_for_query_head,
 )
+from .itak_kv import (  # noqa: F401
+    KvError,
+    KvGeometry,
+    KvSnapshot,
+    LayerSnapshot,
+    SNAPSHOT_FORMAT_VERSION,
+    capture_bytes,
+    checksum,
+    prefix_discriminator,
+    prefix_hash,
+    restore_bytes,
+)
 from . import _native  # noqa: F401
 
 __all__ = [
     "AttentionError", "AttentionParams", "AttentionRequest", "CacheView", "Checkpoint",
     "GlimmerConfig", "HipCompute", "KvCache", "KvPool", "LayerKind", "LayerStats",
     "PositionCache", "StepFailed", "gqa_attention", "kv_head_for_query_head",
+    "KvError", "KvGeometry", "KvSnapshot", "LayerSnapshot", "SNAPSHOT_FORMAT_VERSION",
+    "capture_bytes", "checksum", "prefix_discriminator", "prefix_hash", "restore_bytes",
 ]

@@ -19,7 +19,11 @@ STATUS_NAMES = {
     12: "CheckpointRangeExceeded", 13: "BulkRestoreNotFresh", 14: "RewindOutOfRange",
     15: "StepFailed", 16: "HipError", 17: "InvalidArgument", 18: "NoFreeSlot",
     19: "CapacityExceeded", 20: "Unsupported",
+    21: "BadMagic", 22: "UnsupportedVersion", 23: "Truncated", 24: "ChecksumMismatch",
+    25: "InconsistentSnapshot", 26: "GeometryMismatch", 27: "FingerprintMismatch",
+    28: "IncoherentCache",
 }
+KV_ERROR_FIRST, KV_ERROR_LAST = 21, 28
 ELEM_F32, ELEM_F16 = 0, 1
 LAYER_GLOBAL, LAYER_WINDOWED = 0, 1
 POOL_SCRUB_ON_TRUNCATE = 1
@@ -64,6 +68,19 @@ class SnapshotLayer(C.Structure):
                 ("values", C.c_void_p)]
 
 
+class ItkvHeader(C.Structure):
+    _fields_ = [("token_count", C.c_uint64), ("num_kv_heads", C.c_uint64),
+                ("head_dim", C.c_uint64), ("layer_count", C.c_uint64),
+                ("fingerprint_len", C.c_uint64), ("fingerprint_offset", C.c_uint64),
+                ("encoded_len", C.c_uint64)]
+
+
+class ItkvLayer(C.Structure):
+    _fields_ = [("kind", C.c_uint32), ("reserved", C.c_uint32), ("window", C.c_uint64),
+                ("first_position", C.c_uint64), ("rows", C.c_uint64),
+                ("keys_offset", C.c_uint64), ("values_offset", C.c_uint64)]
+
+
 _P = C.c_void_p
 _u32, _u64, _f32, _i32 = C.c_uint32, C.c_uint64, C.c_float, C.c_int32
 
@@ -89,6 +106,15 @@ PROTOTYPES = {
     "itak_kv_append": (_i32, [_P, _u32, _u64, _P, _u64, _P, _u64, _u64]),
     "itak_kv_restore_bulk": (_i32, [_P, _u32, _u64, _u64, _P, _u64, _P, _u64, _u32]),
     "itak_kv_restore_snapshot": (_i32, [_P, _u32, _u64, C.POINTER(SnapshotLayer), _u64, _u32]),
+    "itak_kv_prefix_hash": (_u64, [_P, _u64]),
+    "itak_kv_prefix_discriminator": (_u64, [_P, _u64]),
+    "itak_kv_checksum": (_u64, [_P, _u64]),
+    "itak_itkv_validate": (_i32, [C.POINTER(ItkvHeader), C.POINTER(ItkvLayer), _u64, _P, _P]),
+    "itak_itkv_encode": (_i32, [C.POINTER(ItkvHeader), C.c_char_p, C.POINTER(ItkvLayer), _u64, _P,
+                                _P, _P, _P, _P, _u64, C.POINTER(_u64)]),
+    "itak_itkv_decode": (_i32, [_P, _u64, C.POINTER(ItkvHeader), C.POINTER(ItkvLayer), _u64]),
+    "itak_kv_capture_itkv": (_i32, [_P, _u32, C.c_char_p, _u64, _P, _u64, C.POINTER(_u64)]),
+    "itak_kv_restore_itkv": (_i32, [_P, _u32, _P, _u64, C.c_char_p, _u64]),
     "itak_kv_stats": (_i32, [_P, _u32, C.POINTER(LayerStatsRaw)]),
     "itak_kv_read_rows": (_i32, [_P, _u32, _u64, _u64, _u64, _P, _P, _P]),
     "itak_kv_read_raw": (_i32, [_P, _u32, _u64, _P, _P]),

@@ -132,6 +132,8 @@ hipError_t launch_read_rows(const void *layer_base, int elem_f16, const PoolGeom
                             hipStream_t stream);
 
 hipError_t launch_convert_f16(const float *src, uint16_t *dst, uint64_t count, hipStream_t stream);
+// f16 bits -> f32, exact (the widening a snapshot capture of an f16 pool needs).
+hipError_t launch_widen_f16(const uint16_t *src, float *dst, uint64_t count, hipStream_t stream);
 hipError_t launch_probe_copy(const void *src, void *dst, uint64_t bytes, hipStream_t stream);
 hipError_t launch_probe_empty(hipStream_t stream);
 

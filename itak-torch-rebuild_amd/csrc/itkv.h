@@ -1,0 +1,68 @@
+// The ITKV v1 snapshot wire format (crates/itak-kv/src/snapshot.rs:13-29) and the FNV-1a
+// hashes of crates/itak-kv/src/hash.rs, host side. Nothing here touches the device: the
+// format fixes a byte-serial checksum over the whole file, so encoding and decoding are
+// host work; the rows themselves move between the encoded buffer and the device planes
+// through the gather / readback kernels.
+#pragma once
+
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+namespace itak {
+
+constexpr uint64_t kFnvOffset = 0xcbf29ce484222325ull;     // hash.rs:14
+constexpr uint64_t kFnvPrime = 0x00000100000001b3ull;      // hash.rs:16
+constexpr uint64_t kFnvAltOffset = 0x84222325cbf29ce4ull;  // hash.rs:21
+constexpr uint32_t kItkvVersion = 1;                       // snapshot.rs:53
+constexpr uint64_t kItkvLayerHeaderLen = 28;               // snapshot.rs:51
+
+uint64_t fnv1a64(const uint8_t *bytes, uint64_t count, uint64_t basis);           // hash.rs:24-31
+uint64_t fnv1a64_tokens(const uint32_t *tokens, uint64_t count, uint64_t basis);  // hash.rs:35-41
+
+// A refusal of itak_kv::KvError (crates/itak-kv/src/error.rs:13-124); `message` is its
+// Display text (error.rs:141-188).
+struct ItkvError {
+    int32_t code = 0;
+    std::string message;
+    uint64_t a = 0, b = 0;  // the variant's integers, in declaration order
+};
+
+struct ItkvLayer {
+    uint32_t kind = 0;  // 0 global, 1 windowed
+    uint64_t window = 0;
+    uint64_t first_position = 0;
+    uint64_t rows = 0;
+    uint64_t keys_offset = 0;    // byte offsets into the encoded buffer
+    uint64_t values_offset = 0;
+};
+
+struct ItkvHeader {
+    uint64_t token_count = 0;
+    uint64_t num_kv_heads = 0;
+    uint64_t head_dim = 0;
+    uint64_t layer_count = 0;
+    uint64_t fingerprint_len = 0;
+    uint64_t fingerprint_offset = 0;
+    uint64_t encoded_len = 0;
+};
+
+// KvSnapshot::validate (snapshot.rs:187-236). `blocks` is the number of layer blocks the
+// snapshot carries (layers.len()); key_floats / value_floats their lengths.
+bool itkv_validate(const ItkvHeader &h, const ItkvLayer *layers, uint64_t blocks,
+                   const uint64_t *key_floats, const uint64_t *value_floats, ItkvError &err);
+
+// KvSnapshot::from_bytes (snapshot.rs:405-509): strict; fills offsets instead of copying rows.
+bool itkv_decode(const uint8_t *bytes, uint64_t len, ItkvHeader &h, std::vector<ItkvLayer> &layers,
+                 ItkvError &err);
+
+// Bytes of everything before the row payload, and of the whole encoding (payload and the
+// trailing checksum included), for a header whose layers carry `rows` rows each.
+uint64_t itkv_header_len(const ItkvHeader &h);
+bool itkv_encoded_len(const ItkvHeader &h, const ItkvLayer *layers, uint64_t *out);
+// Writes magic .. layer headers (snapshot.rs:383-403) and fills the payload offsets.
+void itkv_write_header(uint8_t *out, const ItkvHeader &h, const char *fingerprint,
+                       ItkvLayer *layers);
+
+}  // namespace itak

@@ -357,6 +357,21 @@ hipError_t launch_convert_f16(const float *src, uint16_t *dst, uint64_t count, h
     return hipGetLastError();
 }
 
+// f16 -> f32 is exact for every half (crates/gguf/src/dequant.rs:12-34 is the host rule).
+__global__ __launch_bounds__(256) void widen_f16_to_f32(const uint16_t *__restrict__ src,
+                                                        float *__restrict__ dst, uint64_t count) {
+    for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < count; i += gridDim.x * 256ull)
+        dst[i] = static_cast<float>(__builtin_bit_cast(_Float16, src[i]));
+}
+
+hipError_t launch_widen_f16(const uint16_t *src, float *dst, uint64_t count, hipStream_t stream) {
+    if (count == 0) return hipSuccess;
+    uint64_t blocks = (count + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    widen_f16_to_f32<<<uint32_t(blocks), 256, 0, stream>>>(src, dst, count);
+    return hipGetLastError();
+}
+
 // ------------------------------------------------------------- measurement aids
 // A plain streaming copy of known size (the yardstick the FETCH_SIZE / WRITE_SIZE counters
 // are scaled by) and an empty kernel (the per-launch floor of a stream of dependent

@@ -4,6 +4,7 @@
 // All validation happens here, in the reference's order, before anything is enqueued.
 #include "../../include/itak_hip_kv.h"
 #include "internal.h"
+#include "itkv.h"
 
 #include <algorithm>
 #include <cmath>
@@ -456,6 +457,39 @@ PtrKind classify(const void *p, const void **usable) {
     return PtrKind::PlainHost;
 }
 
+// Rows the gather kernel cannot read where they lie: ordinary host memory, or a source that
+// is not aligned to its element size (the payload of an encoded snapshot starts wherever
+// its fingerprint ends).
+bool must_stage(const void *p, uint64_t elem_bytes) {
+    const void *usable;
+    return classify(p, &usable) == PtrKind::PlainHost ||
+           reinterpret_cast<uintptr_t>(p) % elem_bytes != 0;
+}
+
+itak_status set_itkv_error(ErrorState &e, const ItkvError &err) {
+    return set_error(e, err.code, "snapshot", err.a, err.b, 0, 0, "%s", err.message.c_str());
+}
+
+ItkvHeader to_internal(const itak_itkv_header &h) {
+    ItkvHeader r;
+    r.token_count = h.token_count;
+    r.num_kv_heads = h.num_kv_heads;
+    r.head_dim = h.head_dim;
+    r.layer_count = h.layer_count;
+    r.fingerprint_len = h.fingerprint_len;
+    return r;
+}
+std::vector<ItkvLayer> to_internal(const itak_itkv_layer *layers, uint64_t n) {
+    std::vector<ItkvLayer> r(n);
+    for (uint64_t i = 0; i < n; ++i) {
+        r[i].kind = layers[i].kind;
+        r[i].window = layers[i].window;
+        r[i].first_position = layers[i].first_position;
+        r[i].rows = layers[i].rows;
+    }
+    return r;
+}
+
 }  // namespace
 
 // ======================================================================== public ABI
@@ -722,9 +756,8 @@ static itak_status restore_layers(itak_pool *pool, uint32_t slot, Slot &s,
     for (uint64_t i = 0; i < count; ++i) {
         if (layers[i].rows == 0) continue;
         const uint64_t bytes = layers[i].rows * pool->row * src_bytes_per_elem;
-        const void *unused;
-        if (classify(layers[i].keys, &unused) == PtrKind::PlainHost) stage_need += align_up(bytes, 256);
-        if (classify(layers[i].values, &unused) == PtrKind::PlainHost) stage_need += align_up(bytes, 256);
+        if (must_stage(layers[i].keys, src_bytes_per_elem)) stage_need += align_up(bytes, 256);
+        if (must_stage(layers[i].values, src_bytes_per_elem)) stage_need += align_up(bytes, 256);
     }
     unsigned char *temp = nullptr;
     if (stage_need) HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&temp), stage_need), "allocate restore staging");
@@ -741,7 +774,8 @@ static itak_status restore_layers(itak_pool *pool, uint32_t slot, Slot &s,
             const void *src[2] = {L.keys, L.values};
             for (int side = 0; side < 2; ++side) {
                 const void *usable;
-                if (classify(src[side], &usable) != PtrKind::PlainHost) {
+                if (!must_stage(src[side], src_bytes_per_elem)) {
+                    classify(src[side], &usable);
                     src[side] = usable;
                     continue;
                 }
@@ -835,6 +869,209 @@ itak_status itak_kv_restore_snapshot(itak_pool *pool, uint32_t slot, uint64_t to
     if (token_count > pool->rows_limit)
         return capacity_exceeded(pool->err, 0, token_count, pool->rows_limit);
     return restore_layers(pool, slot, *s, layers, nullptr, layer_count, src_elem);
+}
+
+// ---- itak_kv: hashes, the ITKV codec, capture and restore of encoded snapshots ----------
+
+uint64_t itak_kv_prefix_hash(const uint32_t *tokens, uint64_t count) {  // hash.rs:44-46
+    return fnv1a64_tokens(tokens, tokens ? count : 0, kFnvOffset);
+}
+uint64_t itak_kv_prefix_discriminator(const uint32_t *tokens, uint64_t count) {  // hash.rs:52-54
+    return fnv1a64_tokens(tokens, tokens ? count : 0, kFnvAltOffset);
+}
+uint64_t itak_kv_checksum(const void *bytes, uint64_t count) {  // hash.rs:59-61
+    return fnv1a64(static_cast<const uint8_t *>(bytes), bytes ? count : 0, kFnvOffset);
+}
+
+itak_status itak_itkv_validate(const itak_itkv_header *header, const itak_itkv_layer *layers,
+                               uint64_t blocks, const uint64_t *key_floats,
+                               const uint64_t *value_floats) {
+    ErrorState &e = g_create_error;
+    if (!header || (blocks && (!layers || !key_floats || !value_floats)))
+        return invalid_argument(e, "header, layers or the float counts are null");
+    ItkvError err;
+    const std::vector<ItkvLayer> ls = to_internal(layers, blocks);
+    if (!itkv_validate(to_internal(*header), ls.data(), blocks, key_floats, value_floats, err))
+        return set_itkv_error(e, err);
+    return ITAK_OK;
+}
+
+itak_status itak_itkv_encode(const itak_itkv_header *header, const char *fingerprint,
+                             const itak_itkv_layer *layers, uint64_t blocks,
+                             const float *const *keys, const uint64_t *key_floats,
+                             const float *const *values, const uint64_t *value_floats, void *out,
+                             uint64_t capacity, uint64_t *written) {
+    ErrorState &e = g_create_error;
+    itak_status st = itak_itkv_validate(header, layers, blocks, key_floats, value_floats);
+    if (st != ITAK_OK) return st;
+    if (!written) return invalid_argument(e, "written is null");
+    if (header->fingerprint_len && !fingerprint) return invalid_argument(e, "fingerprint is null");
+    if (header->num_kv_heads > UINT32_MAX || header->head_dim > UINT32_MAX ||
+        header->layer_count > UINT32_MAX || header->fingerprint_len > UINT32_MAX)
+        return invalid_argument(e, "a header field does not fit the 32-bit wire field");
+    ItkvHeader h = to_internal(*header);
+    std::vector<ItkvLayer> ls = to_internal(layers, blocks);
+    uint64_t total = 0;
+    if (!itkv_encoded_len(h, ls.data(), &total)) return size_overflow(e, "encoded snapshot");
+    *written = total;
+    if (!out) return ITAK_OK;
+    if (capacity < total) return invalid_argument(e, "output buffer is smaller than the encoding");
+    uint8_t *bytes = static_cast<uint8_t *>(out);
+    itkv_write_header(bytes, h, fingerprint, ls.data());
+    for (uint64_t i = 0; i < blocks; ++i) {
+        if (key_floats[i] && (!keys || !keys[i] || !values || !values[i]))
+            return invalid_argument(e, "a layer's keys or values is null");
+        if (key_floats[i]) {  // f32 little-endian is this host's own representation
+            memcpy(bytes + ls[i].keys_offset, keys[i], key_floats[i] * 4);
+            memcpy(bytes + ls[i].values_offset, values[i], value_floats[i] * 4);
+        }
+    }
+    const uint64_t sum = fnv1a64(bytes, total - 8, kFnvOffset);
+    for (int b = 0; b < 8; ++b) bytes[total - 8 + b] = uint8_t(sum >> (8 * b));
+    return ITAK_OK;
+}
+
+itak_status itak_itkv_decode(const void *bytes, uint64_t len, itak_itkv_header *header,
+                             itak_itkv_layer *layers, uint64_t layers_capacity) {
+    ErrorState &e = g_create_error;
+    if (!bytes || !header) return invalid_argument(e, "bytes or header is null");
+    ItkvHeader h;
+    std::vector<ItkvLayer> ls;
+    ItkvError err;
+    if (!itkv_decode(static_cast<const uint8_t *>(bytes), len, h, ls, err))
+        return set_itkv_error(e, err);
+    *header = itak_itkv_header{h.token_count,     h.num_kv_heads,       h.head_dim, h.layer_count,
+                               h.fingerprint_len, h.fingerprint_offset, h.encoded_len};
+    if (layers_capacity < ls.size())
+        return invalid_argument(e, "layers_capacity is smaller than the snapshot's layer count");
+    for (size_t i = 0; i < ls.size(); ++i)
+        layers[i] = itak_itkv_layer{ls[i].kind, 0, ls[i].window, ls[i].first_position, ls[i].rows,
+                                    ls[i].keys_offset, ls[i].values_offset};
+    return ITAK_OK;
+}
+
+itak_status itak_kv_capture_itkv(itak_pool *pool, uint32_t slot, const char *fingerprint,
+                                 uint64_t fingerprint_len, void *out, uint64_t capacity,
+                                 uint64_t *written) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    if (!written) return invalid_argument(pool->err, "written is null");
+    if (fingerprint_len && !fingerprint) return invalid_argument(pool->err, "fingerprint is null");
+    if (fingerprint_len > UINT32_MAX) return invalid_argument(pool->err, "fingerprint too long");
+    // snapshot.rs:249-262: one sequence, every layer at the same position.
+    const uint64_t token_count = s->appended[0];
+    for (uint64_t i = 0; i < pool->cfg.layer_count; ++i)
+        if (s->appended[i] != token_count)
+            return set_error(pool->err, ITAK_KV_INCOHERENT_CACHE, "snapshot", token_count,
+                             s->appended[i], i, 0,
+                             "incoherent cache: layer 0 has appended %llu positions but layer %llu "
+                             "has appended %llu; a snapshot is one sequence",
+                             ULL(token_count), ULL(i), ULL(s->appended[i]));
+    ItkvHeader h;
+    h.token_count = token_count;
+    h.num_kv_heads = pool->g.kv_heads;
+    h.head_dim = pool->g.head_dim;
+    h.layer_count = pool->cfg.layer_count;
+    h.fingerprint_len = fingerprint_len;
+    std::vector<ItkvLayer> ls(h.layer_count);
+    for (ItkvLayer &l : ls) l.rows = token_count;  // global layers: every row, from position 0
+    uint64_t total = 0;
+    if (!itkv_encoded_len(h, ls.data(), &total)) return size_overflow(pool->err, "encoded snapshot");
+    *written = total;
+    if (!out) return ITAK_OK;
+    if (capacity < total)
+        return invalid_argument(pool->err, "output buffer is smaller than the encoding");
+    uint8_t *bytes = static_cast<uint8_t *>(out);
+    itkv_write_header(bytes, h, fingerprint, ls.data());
+    // Rows come back through the readback kernel in chunks that bound the staging buffer:
+    // planes -> [row][kv_head][d] in the pool's element type, widened to f32 for an f16 pool.
+    const uint64_t chunk_rows = std::max<uint64_t>(1, (uint64_t(16) << 20) / (pool->row * 4));
+    const uint64_t raw = align_up(chunk_rows * pool->row * pool->elem_bytes, 256);
+    const uint64_t wide = align_up(chunk_rows * pool->row * 4, 256);
+    itak_status st = ensure_stage(pool, 2 * raw + (pool->elem_f16 ? 2 * wide : 0));
+    if (st != ITAK_OK) return st;
+    for (uint64_t layer = 0; layer < h.layer_count; ++layer) {
+        for (uint64_t first = 0; first < token_count; first += chunk_rows) {
+            const uint64_t rows = std::min(chunk_rows, token_count - first);
+            const uint64_t elems = rows * pool->row;
+            unsigned char *kd = pool->stage, *vd = pool->stage + raw;
+            HIP_TRY(pool,
+                    launch_read_rows(layer_base(pool, layer), pool->elem_f16, pool->g, slot,
+                                     uint32_t(first), uint32_t(rows), kd, vd, pool->stream),
+                    "launch row readback");
+            const void *ksrc = kd, *vsrc = vd;
+            if (pool->elem_f16) {
+                float *kw = reinterpret_cast<float *>(pool->stage + 2 * raw);
+                float *vw = reinterpret_cast<float *>(pool->stage + 2 * raw + wide);
+                HIP_TRY(pool,
+                        launch_widen_f16(reinterpret_cast<const uint16_t *>(kd), kw, elems, pool->stream),
+                        "launch widening");
+                HIP_TRY(pool,
+                        launch_widen_f16(reinterpret_cast<const uint16_t *>(vd), vw, elems, pool->stream),
+                        "launch widening");
+                ksrc = kw;
+                vsrc = vw;
+            }
+            HIP_TRY(pool,
+                    hipMemcpyAsync(bytes + ls[layer].keys_offset + first * pool->row * 4, ksrc,
+                                   elems * 4, hipMemcpyDeviceToHost, pool->stream),
+                    "download keys");
+            HIP_TRY(pool,
+                    hipMemcpyAsync(bytes + ls[layer].values_offset + first * pool->row * 4, vsrc,
+                                   elems * 4, hipMemcpyDeviceToHost, pool->stream),
+                    "download values");
+            // The staging buffer is reused by the next chunk.
+            HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after readback");
+        }
+    }
+    const uint64_t sum = fnv1a64(bytes, total - 8, kFnvOffset);
+    for (int b = 0; b < 8; ++b) bytes[total - 8 + b] = uint8_t(sum >> (8 * b));
+    return ITAK_OK;
+}
+
+itak_status itak_kv_restore_itkv(itak_pool *pool, uint32_t slot, const void *bytes, uint64_t len,
+                                 const char *expected_fingerprint,
+                                 uint64_t expected_fingerprint_len) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    if (!bytes) return invalid_argument(pool->err, "bytes is null");
+    // The decoder walks the bytes on the host (header fields, then the checksum over all of
+    // them); a device-resident buffer would have to be copied first.
+    const void *unused;
+    if (classify(bytes, &unused) == PtrKind::Device)
+        return invalid_argument(pool->err, "an encoded snapshot is decoded on the host: pass host memory");
+    ItkvHeader h;
+    std::vector<ItkvLayer> ls;
+    ItkvError err;
+    const uint8_t *b8 = static_cast<const uint8_t *>(bytes);
+    if (!itkv_decode(b8, len, h, ls, err)) return set_itkv_error(pool->err, err);
+    // restore_checked (snapshot.rs:351-371): geometry first, then the fingerprint.
+    bool same = h.layer_count == pool->cfg.layer_count && h.num_kv_heads == pool->g.kv_heads &&
+                h.head_dim == pool->g.head_dim;
+    for (size_t i = 0; same && i < ls.size(); ++i) same = ls[i].kind == ITAK_LAYER_GLOBAL;
+    if (!same)
+        return set_error(pool->err, ITAK_KV_GEOMETRY_MISMATCH, "snapshot", 0, 0, 0, 0,
+                         "geometry mismatch: snapshot geometry (%llu layers, %llu KV heads, head "
+                         "dim %llu) differs from the required geometry (%llu layers, %llu KV "
+                         "heads, head dim %llu)",
+                         ULL(h.layer_count), ULL(h.num_kv_heads), ULL(h.head_dim),
+                         ULL(pool->cfg.layer_count), ULL(pool->g.kv_heads), ULL(pool->g.head_dim));
+    if (expected_fingerprint &&
+        (expected_fingerprint_len != h.fingerprint_len ||
+         memcmp(expected_fingerprint, b8 + h.fingerprint_offset, h.fingerprint_len) != 0))
+        return set_error(pool->err, ITAK_KV_FINGERPRINT_MISMATCH, "snapshot", 0, 0, 0, 0,
+                         "model fingerprint mismatch: need %.*s, snapshot carries %.*s",
+                         int(std::min<uint64_t>(expected_fingerprint_len, 400)), expected_fingerprint,
+                         int(std::min<uint64_t>(h.fingerprint_len, 400)),
+                         reinterpret_cast<const char *>(b8 + h.fingerprint_offset));
+    std::vector<itak_snapshot_layer> layers(ls.size());
+    for (size_t i = 0; i < ls.size(); ++i)
+        layers[i] = itak_snapshot_layer{ls[i].first_position, ls[i].rows, b8 + ls[i].keys_offset,
+                                        b8 + ls[i].values_offset};
+    return itak_kv_restore_snapshot(pool, slot, h.token_count, layers.data(), layers.size(),
+                                    ITAK_ELEM_F32);
 }
 
 itak_status itak_kv_stats(itak_pool *pool, uint32_t slot, itak_layer_stats *out) {
