@@ -356,6 +356,33 @@ itak_status itak_attention_step_device(itak_pool *pool, uint64_t layer,
                                        const float *q_dev, const float *k_dev, const float *v_dev,
                                        float *out_dev, uint64_t num_q_heads, float scale,
                                        float softcap);
+/* What Q and K go through between their projections and attention in the reference's
+   model (crates/muse-glimmer/src/model.rs:445-451, crates/cpu-compute/src/cpu.rs:598-622):
+   a per-head RMSNorm under one [head_dim] weight each (torch_math::rms_norm,
+   crates/torch-math/src/norm.rs:21-52) and RoPE at the row's position
+   (rope_interleaved.rs:65-116 or rope.rs:63-116). */
+typedef struct itak_prep_params {
+    const float *q_norm_weight; /* device, [head_dim]; NULL = Q is not normed */
+    const float *k_norm_weight; /* device, [head_dim]; NULL = K is not normed */
+    float eps;                  /* > 0 when a weight is given */
+    float rope_base;            /* > 1: rotate Q and K; 0: no rotation (a global, NoPE layer) */
+    uint32_t rope_interleaved;  /* 1: adjacent pairs (llama.cpp NORM), 0: half split (NEOX) */
+    uint32_t rotary_dim;        /* even, <= head_dim; 0 = head_dim */
+} itak_prep_params;
+
+/* itak_attention_step_device preceded by the fused preparation of the resident chain
+   (crates/wgpu-compute/src/kernels/k9_attn_prep.rs:1-60: the Q and K norms, the rotations
+   and the append as one dispatch) and followed by the attention gate
+   (CpuCompute::attn_gate, cpu.rs:657-673): q_dev and k_dev are the raw projections; norms
+   and rotation run as one launch, the append is part of the attention launch, and with
+   gate_dev != NULL ([sum rows][q_heads*head_dim]) out = attention * sigmoid(gate). Numerics
+   are those of the reference's CPU path (f64 norm, f64 angles), not of its f32 shader. */
+itak_status itak_attention_prep_step_device(itak_pool *pool, uint64_t layer,
+                                            const itak_batch_item *items, uint32_t item_count,
+                                            const float *q_dev, const float *k_dev,
+                                            const float *v_dev, const float *gate_dev,
+                                            float *out_dev, uint64_t num_q_heads, float scale,
+                                            float softcap, const itak_prep_params *prep);
 /* The attention half alone: query row r of item i attends at position
    len_i - rows_i + r, i.e. over rows the slot already holds (gqa_attention over the
    slot's view, attention.rs:104-215, with the last rows_i positions as queries). */

@@ -68,6 +68,12 @@ class SnapshotLayer(C.Structure):
                 ("values", C.c_void_p)]
 
 
+class PrepParams(C.Structure):
+    _fields_ = [("q_norm_weight", C.c_void_p), ("k_norm_weight", C.c_void_p), ("eps", C.c_float),
+                ("rope_base", C.c_float), ("rope_interleaved", C.c_uint32),
+                ("rotary_dim", C.c_uint32)]
+
+
 class ItkvHeader(C.Structure):
     _fields_ = [("token_count", C.c_uint64), ("num_kv_heads", C.c_uint64),
                 ("head_dim", C.c_uint64), ("layer_count", C.c_uint64),
@@ -132,6 +138,8 @@ PROTOTYPES = {
     "itak_compute_cache_release": (_i32, [_P, _u32, C.POINTER(CheckpointRaw)]),
     "itak_attention_step_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P, _P, _P,
                                           _u64, _f32, _f32]),
+    "itak_attention_prep_step_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P, _P, _P,
+                                               _P, _u64, _f32, _f32, C.POINTER(PrepParams)]),
     "itak_attention_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P, _u64, _f32,
                                      _f32]),
     "itak_kv_append_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P]),

@@ -137,6 +137,30 @@ hipError_t launch_widen_f16(const uint16_t *src, float *dst, uint64_t count, hip
 hipError_t launch_probe_copy(const void *src, void *dst, uint64_t bytes, hipStream_t stream);
 hipError_t launch_probe_empty(hipStream_t stream);
 
+// ---- attention preparation (per-head RMSNorm + RoPE of Q and K) and the output gate ------
+struct PrepArgs {
+    const float *q_in;      // [total_rows][q_heads*head_dim]
+    const float *k_in;      // [total_rows][kv_heads*head_dim]
+    float *q_out;
+    float *k_out;
+    const float *q_weight;  // [head_dim] or null: no norm
+    const float *k_weight;
+    float eps;
+    float rope_base;        // > 1 rotates, otherwise no rotation
+    uint32_t interleaved;   // 1: pairs (2i, 2i+1); 0: pairs (i, i + rotary_dim/2)
+    uint32_t rotary_dim;
+    uint32_t head_dim;
+    uint32_t q_heads;
+    uint32_t kv_heads;
+    uint32_t total_rows;
+    uint32_t n;                      // items
+    uint32_t row0[kMaxBatchItems];   // first row of item i (rows are laid out item after item)
+    uint32_t pos0[kMaxBatchItems];   // position of that row
+};
+hipError_t launch_attn_prep(const PrepArgs &a, hipStream_t stream);
+// out[i] *= sigmoid(gate[i]) (CpuCompute::attn_gate, cpu.rs:657-673).
+hipError_t launch_attn_gate(float *out, const float *gate, uint64_t count, hipStream_t stream);
+
 // ---- attention ----------------------------------------------------------------------
 // One item = one slot's query rows against that slot's rows of one layer. Query row r
 // sits at position pos0 + r unless q_pos is given. A workgroup owns (item, row block,

@@ -61,6 +61,8 @@ struct itak_pool {
     uint64_t stage_bytes = 0;
     float *ws = nullptr;
     uint64_t ws_floats = 0;
+    float *prep = nullptr;  // prepared Q and K rows of a prep step
+    uint64_t prep_floats = 0;
     mutable ErrorState err;
 };
 
@@ -208,6 +210,20 @@ itak_status ensure_workspace(itak_pool *pool, uint64_t floats) {
         HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&pool->ws), want * sizeof(float)),
                 "allocate split workspace");
         pool->ws_floats = want;
+    }
+    return ITAK_OK;
+}
+
+itak_status ensure_prep(itak_pool *pool, uint64_t floats) {
+    if (floats > pool->prep_floats) {
+        HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize before growing prep scratch");
+        if (pool->prep) HIP_TRY(pool, hipFree(pool->prep), "free prep scratch");
+        pool->prep = nullptr;
+        pool->prep_floats = 0;
+        uint64_t want = std::max<uint64_t>(floats + floats / 2, 1u << 16);
+        HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&pool->prep), want * sizeof(float)),
+                "allocate prep scratch");
+        pool->prep_floats = want;
     }
     return ITAK_OK;
 }
@@ -605,6 +621,7 @@ void itak_pool_destroy(itak_pool *pool) {
     if (pool->base) (void)hipFree(pool->base);
     if (pool->stage) (void)hipFree(pool->stage);
     if (pool->ws) (void)hipFree(pool->ws);
+    if (pool->prep) (void)hipFree(pool->prep);
     delete pool;
 }
 
@@ -1369,6 +1386,84 @@ itak_status itak_attention_step_device(itak_pool *pool, uint64_t layer,
     if (std::isnan(scale)) scale = default_scale(pool->g.head_dim);
     return step_on_device(pool, layer, items, item_count, plan, q_dev, k_dev, v_dev, out_dev,
                           num_q_heads, scale, softcap);
+}
+
+itak_status itak_attention_prep_step_device(itak_pool *pool, uint64_t layer,
+                                            const itak_batch_item *items, uint32_t item_count,
+                                            const float *q_dev, const float *k_dev,
+                                            const float *v_dev, const float *gate_dev,
+                                            float *out_dev, uint64_t num_q_heads, float scale,
+                                            float softcap, const itak_prep_params *prep) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (item_count == 0) return ITAK_OK;
+    if (!items || !q_dev || !k_dev || !v_dev || !out_dev || !prep)
+        return invalid_argument(pool->err, "items, a device tensor or prep is null");
+    const uint32_t D = pool->g.head_dim;
+    // torch-math's refusals (norm.rs:32-38, rope_interleaved.rs:72-99), by name.
+    if ((prep->q_norm_weight || prep->k_norm_weight) && !(std::isfinite(prep->eps) && prep->eps > 0.0f))
+        return set_error(pool->err, ITAK_STEP_FAILED, "rms_norm", 0, 0, 0, 0,
+                         "rms_norm: eps must be finite and > 0");
+    const bool rotate = prep->rope_base != 0.0f;
+    const uint32_t rotary = prep->rotary_dim ? prep->rotary_dim : D;
+    if (rotate) {
+        if (D < 2 || D % 2 != 0)
+            return set_error(pool->err, ITAK_STEP_FAILED, "attention", 0, 0, 0, 0,
+                             "rope: head_dim must be even and >= 2");
+        if (rotary < 2 || rotary % 2 != 0 || rotary > D)
+            return set_error(pool->err, ITAK_STEP_FAILED, "attention", 0, 0, 0, 0,
+                             "rope: rotary_dim must be even, >= 2, and <= head_dim");
+        if (!std::isfinite(prep->rope_base) || prep->rope_base <= 1.0f)
+            return set_error(pool->err, ITAK_STEP_FAILED, "attention", 0, 0, 0, 0,
+                             "rope: base must be finite and > 1");
+    } else if (D % 2 != 0) {
+        return unsupported(pool->err, "attention preparation needs an even head_dim");
+    }
+    std::vector<PlanInput> plan;
+    itak_status st = plan_step(pool, layer, items, item_count, num_q_heads, plan);
+    if (st != ITAK_OK) return st;
+    uint64_t total_rows = 0;
+    for (const PlanInput &p : plan) total_rows += p.rows;
+    if (total_rows == 0) return ITAK_OK;
+    const uint64_t q_width = num_q_heads * D, k_width = pool->row;
+    st = ensure_prep(pool, total_rows * (q_width + k_width));
+    if (st != ITAK_OK) return st;
+    float *q_prep = pool->prep, *k_prep = pool->prep + total_rows * q_width;
+    uint32_t row = 0;
+    for (uint32_t first = 0; first < item_count; first += kMaxBatchItems) {
+        const uint32_t count = std::min<uint32_t>(kMaxBatchItems, item_count - first);
+        PrepArgs a{};
+        a.q_in = q_dev + uint64_t(row) * q_width;
+        a.k_in = k_dev + uint64_t(row) * k_width;
+        a.q_out = q_prep + uint64_t(row) * q_width;
+        a.k_out = k_prep + uint64_t(row) * k_width;
+        a.q_weight = prep->q_norm_weight;
+        a.k_weight = prep->k_norm_weight;
+        a.eps = prep->eps;
+        a.rope_base = rotate ? prep->rope_base : 0.0f;
+        a.interleaved = prep->rope_interleaved ? 1 : 0;
+        a.rotary_dim = rotary;
+        a.head_dim = D;
+        a.q_heads = uint32_t(num_q_heads);
+        a.kv_heads = pool->g.kv_heads;
+        a.n = count;
+        uint32_t chunk_rows = 0;
+        for (uint32_t i = 0; i < count; ++i) {
+            a.row0[i] = chunk_rows;
+            a.pos0[i] = plan[first + i].pos0;
+            chunk_rows += plan[first + i].rows;
+        }
+        a.total_rows = chunk_rows;
+        HIP_TRY(pool, launch_attn_prep(a, pool->stream), "launch attention preparation");
+        row += chunk_rows;
+    }
+    if (std::isnan(scale)) scale = default_scale(D);
+    st = step_on_device(pool, layer, items, item_count, plan, q_prep, k_prep, v_dev, out_dev,
+                        num_q_heads, scale, softcap);
+    if (st != ITAK_OK) return st;
+    if (gate_dev)
+        HIP_TRY(pool, launch_attn_gate(out_dev, gate_dev, total_rows * q_width, pool->stream),
+                "launch attention gate");
+    return ITAK_OK;
 }
 
 itak_status itak_attention_device(itak_pool *pool, uint64_t layer, const itak_batch_item *items,

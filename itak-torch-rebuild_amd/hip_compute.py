@@ -254,6 +254,20 @@ class KvPool:
             self._h, layer, raw, n, q_ptr, k_ptr, v_ptr, out_ptr, num_q_heads,
             math.nan if scale is None else scale, softcap))
 
+    def attention_prep_step_device(self, layer: int, items, q_ptr: int, k_ptr: int, v_ptr: int,
+                                   out_ptr: int, num_q_heads: int, *, q_norm_ptr: int = 0,
+                                   k_norm_ptr: int = 0, eps: float = 1e-6, rope_base: float = 0.0,
+                                   interleaved: bool = True, rotary_dim: int = 0, gate_ptr: int = 0,
+                                   scale: float = float("nan"), softcap: float = 0.0) -> None:
+        """Per-head RMSNorm + RoPE of the raw Q/K projections, append, attention, gate: the
+        steps of muse-glimmer/src/model.rs:445-464 around Compute::attention, device tensors."""
+        arr, n = self._items(items)
+        prep = N.PrepParams(q_norm_ptr or None, k_norm_ptr or None, eps, rope_base,
+                            1 if interleaved else 0, rotary_dim)
+        _check(self._h, self._lib.itak_attention_prep_step_device(
+            self._h, layer, arr, n, q_ptr, k_ptr, v_ptr, gate_ptr or None, out_ptr, num_q_heads,
+            scale, softcap, C.byref(prep)), "attention")
+
     def attention_device(self, layer: int, items, q_ptr: int, out_ptr: int, num_q_heads: int,
                          scale: Optional[float] = None, softcap: float = 0.0) -> None:
         """Attend with each item's last `rows` stored positions as the queries' positions."""

@@ -85,6 +85,13 @@ def lib():
         L.orc_prefix_hash.restype = C.c_uint64
         L.orc_prefix_hash.argtypes = [C.c_void_p, C.c_size_t]
         L.orc_rope_half_split.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_float]
+        L.orc_rope_half_split_partial.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t,
+                                                  C.c_uint64, C.c_float]
+        L.orc_rope_interleaved.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t,
+                                           C.c_uint64, C.c_float]
+        L.orc_rms_norm.argtypes = [C.c_void_p, C.c_void_p, C.c_float, C.c_size_t, C.c_void_p]
+        L.orc_sigmoid.restype = C.c_float
+        L.orc_sigmoid.argtypes = [C.c_float]
         L.orc_logit_softcap.restype = C.c_float
         L.orc_logit_softcap.argtypes = [C.c_float, C.c_float]
         L.orc_cache_new.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64,
@@ -257,6 +264,69 @@ def rope_rows(x: np.ndarray, first_position: int, base: float) -> np.ndarray:
     out[..., :half] = (a * c - b * s).astype(np.float32)
     out[..., half:] = (a * s + b * c).astype(np.float32)
     return out
+
+
+def rope_interleaved(x: np.ndarray, position: int, base: float, rotary_dim: Optional[int] = None) -> np.ndarray:
+    """torch_math::rope_interleaved(_partial) (rope_interleaved.rs:65-116) on one head row."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    lib().orc_rope_interleaved(x.ctypes.data, out.ctypes.data, x.size, rotary_dim or x.size,
+                               position, base)
+    return out
+
+
+def rope_half_split_partial(x: np.ndarray, position: int, base: float, rotary_dim: Optional[int] = None) -> np.ndarray:
+    """torch_math::rope(_partial) (rope.rs:63-116) on one head row."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    lib().orc_rope_half_split_partial(x.ctypes.data, out.ctypes.data, x.size, rotary_dim or x.size,
+                                      position, base)
+    return out
+
+
+def rms_norm(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:
+    """torch_math::rms_norm (norm.rs:21-52) on one row."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(weight, dtype=np.float32)
+    assert x.size == w.size and x.size > 0
+    out = np.empty_like(x)
+    lib().orc_rms_norm(x.ctypes.data, w.ctypes.data, eps, x.size, out.ctypes.data)
+    return out
+
+
+def sigmoid(x: float) -> float:
+    """cpu-compute/src/cpu.rs:162-169."""
+    return float(lib().orc_sigmoid(C.c_float(x)))
+
+
+def attn_gate(attn_out: np.ndarray, gate: np.ndarray) -> np.ndarray:
+    """CpuCompute::attn_gate (cpu.rs:657-673): a * sigmoid(g), f32."""
+    a = np.ascontiguousarray(attn_out, dtype=np.float32).reshape(-1)
+    g = np.ascontiguousarray(gate, dtype=np.float32).reshape(-1)
+    assert a.size == g.size
+    s = np.array([sigmoid(float(v)) for v in g], dtype=np.float32)
+    return (a * s).astype(np.float32)
+
+
+def attention_prep(rows: np.ndarray, heads: int, head_dim: int, first_position: int,
+                   norm_weight: Optional[np.ndarray], eps: float, rope_base: float,
+                   interleaved: bool = True, rotary_dim: Optional[int] = None) -> np.ndarray:
+    """What one of Q or K goes through between its projection and attention: per-head RMSNorm
+    (muse-glimmer/src/model.rs:445-451 -> CpuCompute::rms_norm, cpu.rs:445-475) and then RoPE per
+    head at the row's position (cpu.rs:598-622, rope_row cpu.rs:398-418). norm_weight None skips
+    the norm, rope_base 0 the rotation (a global, NoPE layer). rows: [n][heads*head_dim]."""
+    x = np.ascontiguousarray(rows, dtype=np.float32).reshape(-1, heads, head_dim)
+    out = np.empty_like(x)
+    for r in range(x.shape[0]):
+        for h in range(heads):
+            row = x[r, h]
+            if norm_weight is not None:
+                row = rms_norm(row, norm_weight, eps)
+            if rope_base > 0:
+                fn = rope_interleaved if interleaved else rope_half_split_partial
+                row = fn(row, first_position + r, rope_base, rotary_dim)
+            out[r, h] = row
+    return out.reshape(x.shape[0], heads * head_dim)
 
 
 def logit_softcap(x: float, cap: float) -> float:

@@ -249,6 +249,67 @@ void orc_rope_half_split(const float *in, float *out, size_t head_dim, uint64_t 
     }
 }
 
+/* torch-math/src/rope.rs:63-116 (half-split pairing: channel i with i + rotary_dim/2) with a
+   rotary_dim that may be smaller than head_dim; the tail passes through. */
+void orc_rope_half_split_partial(const float *in, float *out, size_t head_dim, size_t rotary_dim,
+                                 uint64_t position, float base) {
+    size_t half = rotary_dim / 2;
+    double pos = (double)position;
+    double base64 = (double)base;
+    for (size_t i = 0; i < head_dim; i++) {
+        out[i] = in[i];
+    }
+    for (size_t i = 0; i < half; i++) {
+        double exponent = -((double)(2 * i)) / (double)rotary_dim;
+        double angle = pos * pow(base64, exponent);
+        double s = sin(angle), c = cos(angle);
+        double x = (double)in[i], y = (double)in[i + half];
+        out[i] = (float)(x * c - y * s);
+        out[i + half] = (float)(x * s + y * c);
+    }
+}
+
+/* torch-math/src/rope_interleaved.rs:65-116 (adjacent pairing: channels 2i and 2i+1). */
+void orc_rope_interleaved(const float *in, float *out, size_t head_dim, size_t rotary_dim,
+                          uint64_t position, float base) {
+    double pos = (double)position;
+    double base64 = (double)base;
+    for (size_t i = 0; i < head_dim; i++) {
+        out[i] = in[i];
+    }
+    for (size_t i = 0; i < rotary_dim / 2; i++) {
+        double exponent = -((double)(2 * i)) / (double)rotary_dim;
+        double angle = pos * pow(base64, exponent);
+        double s = sin(angle), c = cos(angle);
+        double x = (double)in[2 * i], y = (double)in[2 * i + 1];
+        out[2 * i] = (float)(x * c - y * s);
+        out[2 * i + 1] = (float)(x * s + y * c);
+    }
+}
+
+/* torch-math/src/norm.rs:21-52: mean of squares and the scaled product in f64, one rounding
+   to f32 per element. */
+void orc_rms_norm(const float *in, const float *weight, float eps, size_t n, float *out) {
+    double sum = 0.0;
+    for (size_t i = 0; i < n; i++) {
+        sum += (double)in[i] * (double)in[i];
+    }
+    double mean_sq = sum / (double)n;
+    double inv_rms = 1.0 / sqrt(mean_sq + (double)eps);
+    for (size_t i = 0; i < n; i++) {
+        out[i] = (float)((double)in[i] * inv_rms * (double)weight[i]);
+    }
+}
+
+/* cpu-compute/src/cpu.rs:162-169. */
+float orc_sigmoid(float x) {
+    if (x >= 0.0f) {
+        return 1.0f / (1.0f + expf(-x));
+    }
+    float e = expf(x);
+    return e / (1.0f + e);
+}
+
 /* torch-math/src/logits.rs:36. */
 float orc_logit_softcap(float x, float cap) { return cap * tanhf(x / cap); }
 

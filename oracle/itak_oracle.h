@@ -89,6 +89,12 @@ uint64_t orc_prefix_hash(const uint32_t *tokens, size_t n);
 /* Half-split RoPE with float64 angles (torch-math/src/rope.rs:99-116); input generation only. */
 void orc_rope_half_split(const float *in, float *out, size_t head_dim, uint64_t position, float base);
 /* cap * tanh(x / cap) in f32 (torch-math/src/logits.rs:26-37). */
+void orc_rope_half_split_partial(const float *in, float *out, size_t head_dim, size_t rotary_dim,
+                                 uint64_t position, float base);
+void orc_rope_interleaved(const float *in, float *out, size_t head_dim, size_t rotary_dim,
+                          uint64_t position, float base);
+void orc_rms_norm(const float *in, const float *weight, float eps, size_t n, float *out);
+float orc_sigmoid(float x);
 float orc_logit_softcap(float x, float cap);
 
 /*

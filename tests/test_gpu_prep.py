@@ -1,0 +1,150 @@
+"""The fused attention preparation (per-head RMSNorm + RoPE of Q and K), append, attention
+and gate as one device step, against the oracle's composition of the reference's CPU steps
+(crates/muse-glimmer/src/model.rs:445-464, crates/cpu-compute/src/cpu.rs:445-475, 586-673).
+
+Bars: prepared K rows in an f32 cache within 1e-6 of the oracle's (the reference pins its own
+fused kernel against the unfused chain at 1e-5, crates/wgpu-compute/tests/fused_kernels.rs:
+408-431), V rows exact; outputs within 1e-5 relative on f32 KV and 2e-3 max-abs on f16 KV."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import max_abs, normal, pkg, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def P():
+    return pkg()
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def run_case(elem, q_heads, kv_heads, d, ctx, rows, norm, rope_base, interleaved, rotary, gate,
+             seed=0, slots=1):
+    rng = np.random.default_rng(seed)
+    width = kv_heads * d
+    pool = P().KvPool(1, kv_heads, d, elem=elem, max_slots=slots, capacity_rows=ctx + 13 * (slots - 1) + rows + 8)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    qw = (1.0 + 0.1 * normal(rng, d)) if norm else None
+    kw = (1.0 + 0.1 * normal(rng, d)) if norm else None
+    eps = 1e-6
+    caches, refs, qs, ks, vs, gs = [], [], [], [], [], []
+    for s in range(slots):
+        cache = pool.acquire()
+        ref = oracle.KvCache.new([oracle.LayerKind.Global], kv_heads, d, store_f16=(elem == "f16"))
+        n0 = ctx + 13 * s
+        k0 = oracle.attention_prep(normal(rng, n0, width), kv_heads, d, 0, kw, eps, rope_base,
+                                   interleaved, rotary or None)
+        v0 = normal(rng, n0, width)
+        if n0:
+            k0d, v0d = dev(k0), dev(v0)
+            pool.append_device(0, [(cache, n0)], k0d.data_ptr(), v0d.data_ptr())
+            torch.cuda.synchronize()
+            ref.restore_bulk(0, 0, k0, v0)
+        caches.append(cache); refs.append(ref)
+        qs.append(3.0 * normal(rng, rows, q_heads * d)); ks.append(2.0 * normal(rng, rows, width))
+        vs.append(normal(rng, rows, width)); gs.append(2.0 * normal(rng, rows, q_heads * d))
+    q, k, v, g = (np.concatenate(x) for x in (qs, ks, vs, gs))
+    qd, kd, vd, gd = dev(q), dev(k), dev(v), dev(g)
+    qwd, kwd = (dev(qw), dev(kw)) if norm else (None, None)  # kept alive across the call
+    out = torch.empty_like(qd)
+    pool.attention_prep_step_device(
+        0, [(c, rows) for c in caches], qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(),
+        q_heads, q_norm_ptr=qwd.data_ptr() if norm else 0,
+        k_norm_ptr=kwd.data_ptr() if norm else 0, eps=eps, rope_base=rope_base,
+        interleaved=interleaved, rotary_dim=rotary, gate_ptr=gd.data_ptr() if gate else 0)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    for s in range(slots):
+        n0 = ctx + 13 * s
+        qp = oracle.attention_prep(qs[s], q_heads, d, n0, qw, eps, rope_base, interleaved, rotary or None)
+        kp = oracle.attention_prep(ks[s], kv_heads, d, n0, kw, eps, rope_base, interleaved, rotary or None)
+        want = oracle.attention_step(refs[s], 0, qp, kp, vs[s], q_heads, n0, threads=8)
+        if gate:
+            want = oracle.attn_gate(want, gs[s])
+        mine = got[s * rows:(s + 1) * rows].reshape(-1)
+        if elem == "f32":
+            assert rel_err(mine, want) <= 1e-5
+        else:
+            assert max_abs(mine, want) <= 2e-3
+        # The appended rows: prepared keys, untouched values.
+        _, gk, gv = caches[s].read_rows(0, n0, rows)
+        if elem == "f32":
+            assert max_abs(gk.reshape(rows, width), kp) <= 1e-6
+            assert gv.reshape(rows, width).tobytes() == vs[s].tobytes()
+        else:
+            # A prepared key that differs from the oracle's in its last f32 bit can round to
+            # the neighbouring half: one f16 ulp at most.
+            ulp = np.abs(gk.reshape(rows, width).view(np.int16).astype(np.int32)
+                         - oracle.f32_to_f16_array(kp).view(np.int16).astype(np.int32))
+            assert ulp.max() <= 1
+            assert np.array_equal(gv.reshape(rows, width), oracle.f32_to_f16_array(vs[s]))
+        assert caches[s].next_position(0) == n0 + rows
+    pool.close()
+
+
+@pytest.mark.parametrize("elem", ["f32", "f16"])
+def test_decode_step_with_norms_interleaved_rope_and_gate(elem):
+    run_case(elem, 32, 4, 128, ctx=300, rows=1, norm=True, rope_base=1e6, interleaved=True,
+             rotary=0, gate=True)
+
+
+def test_long_positions_need_the_f64_angle_law():
+    # At position ~100,000 an f32 angle is off by several 1e-3 rad; the f32 cache rows must
+    # still be within 1e-6 of the oracle's.
+    run_case("f32", 8, 2, 64, ctx=0, rows=3, norm=True, rope_base=1e4, interleaved=True, rotary=0,
+             gate=False, seed=1)
+    rng = np.random.default_rng(2)
+    d, kv_heads, q_heads, pos = 128, 4, 32, 100_000
+    pool = P().KvPool(1, kv_heads, d, elem="f32", capacity_rows=pos + 4)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    cache = pool.acquire()
+    zeros = torch.zeros(pos, kv_heads * d, device="cuda")
+    pool.append_device(0, [(cache, pos)], zeros.data_ptr(), zeros.data_ptr())
+    q, k, v = normal(rng, 1, q_heads * d), normal(rng, 1, kv_heads * d), normal(rng, 1, kv_heads * d)
+    out = torch.empty(1, q_heads * d, device="cuda")
+    qd, kd, vd = dev(q), dev(k), dev(v)
+    pool.attention_prep_step_device(0, [(cache, 1)], qd.data_ptr(), kd.data_ptr(), vd.data_ptr(),
+                                    out.data_ptr(), q_heads, rope_base=1e4, interleaved=True)
+    torch.cuda.synchronize()
+    _, gk, _ = cache.read_rows(0, pos, 1)
+    want = oracle.attention_prep(k, kv_heads, d, pos, None, 1e-6, 1e4, True)
+    assert max_abs(gk.reshape(1, -1), want) <= 1e-6
+    pool.close()
+
+
+@pytest.mark.parametrize("rows,interleaved,rotary,norm,rope_base", [
+    (7, True, 0, True, 1e6), (7, False, 0, True, 1e4), (5, False, 64, False, 1e4),
+    (5, True, 32, True, 5e5), (1, True, 0, True, 0.0), (200, True, 0, True, 1e6)])
+def test_blocks_pairings_partial_rotary_and_nope(rows, interleaved, rotary, norm, rope_base):
+    run_case("f16", 32, 4, 128, ctx=150, rows=rows, norm=norm, rope_base=rope_base,
+             interleaved=interleaved, rotary=rotary, gate=(rows < 100), seed=rows)
+
+
+def test_several_slots_each_at_its_own_position():
+    run_case("f16", 32, 4, 128, ctx=90, rows=1, norm=True, rope_base=1e6, interleaved=True, rotary=0,
+             gate=True, seed=5, slots=5)
+    run_case("f32", 8, 2, 64, ctx=40, rows=3, norm=True, rope_base=1e4, interleaved=False, rotary=0,
+             gate=True, seed=6, slots=3)
+
+
+def test_bad_preparation_parameters_are_refused_by_name():
+    pool = P().KvPool(1, 4, 128, elem="f16", capacity_rows=16)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    cache = pool.acquire()
+    t = torch.zeros(1, 32 * 128, device="cuda")
+    w = torch.ones(128, device="cuda")
+    args = (0, [(cache, 1)], t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), 32)
+    for kw, text in ((dict(q_norm_ptr=w.data_ptr(), eps=0.0), "eps must be finite and > 0"),
+                     (dict(rope_base=1.0), "base must be finite and > 1"),
+                     (dict(rope_base=1e4, rotary_dim=130), "rotary_dim must be even"),
+                     (dict(rope_base=1e4, rotary_dim=3), "rotary_dim must be even")):
+        with pytest.raises(P().StepFailed) as e:
+            pool.attention_prep_step_device(*args, **kw)
+        assert text in str(e.value)
+    assert cache.next_position(0) == 0  # nothing was appended by a refused step
+    pool.close()
