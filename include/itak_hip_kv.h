@@ -101,6 +101,15 @@ typedef struct itak_pool_config {
     uint64_t capacity_rows; /* positions one slot can hold per global layer */
     int32_t device;         /* HIP device ordinal */
     uint32_t flags;         /* ITAK_POOL_* */
+    /* Windowed layers only: rows a layer's device ring holds beyond its window (0 = 64). A
+       step appends its whole block before its queries run, so the ring must still hold the
+       window of the block's first row after the last row has landed; the same spare rows let
+       a rewind drop positions without saved copies. It bounds the rows one device step may
+       carry on a windowed layer, max_round_tokens of a checkpoint, and how far a truncate may
+       go back (the chunk_cap of the reference's resident session,
+       crates/wgpu-compute/src/session.rs:235-249, 5376-5428). A ring is window +
+       ring_headroom rows, rounded up to a multiple of 32. */
+    uint64_t ring_headroom;
 } itak_pool_config;
 
 /* The fields of the last refusal, in the order the Rust variant declares them
@@ -209,6 +218,9 @@ uint64_t itak_kv_num_kv_heads(const itak_pool *pool); /* cache.rs:379-381 */
 uint64_t itak_kv_head_dim(const itak_pool *pool);     /* cache.rs:384-386 */
 /* KvCache::layer_kind (cache.rs:403-405). */
 itak_status itak_kv_layer_kind(itak_pool *pool, uint64_t layer, uint32_t *kind, uint64_t *window);
+/* Storage rows of one layer of one slot: capacity_rows on a global layer, the ring length on
+   a windowed one (what itak_kv_read_raw returns). */
+itak_status itak_kv_storage_rows(itak_pool *pool, uint64_t layer, uint64_t *out);
 /* KvCache::stored_len (cache.rs:408-410). */
 itak_status itak_kv_stored_len(itak_pool *pool, uint32_t slot, uint64_t layer, uint64_t *out);
 /* KvCache::next_position (cache.rs:413-415). */

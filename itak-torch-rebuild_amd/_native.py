@@ -41,6 +41,7 @@ class PoolConfig(C.Structure):
         ("capacity_rows", C.c_uint64),
         ("device", C.c_int32),
         ("flags", C.c_uint32),
+        ("ring_headroom", C.c_uint64),
     ]
 
 
@@ -107,6 +108,7 @@ PROTOTYPES = {
     "itak_kv_num_kv_heads": (_u64, [_P]),
     "itak_kv_head_dim": (_u64, [_P]),
     "itak_kv_layer_kind": (_i32, [_P, _u64, C.POINTER(_u32), C.POINTER(_u64)]),
+    "itak_kv_storage_rows": (_i32, [_P, _u64, C.POINTER(_u64)]),
     "itak_kv_stored_len": (_i32, [_P, _u32, _u64, C.POINTER(_u64)]),
     "itak_kv_next_position": (_i32, [_P, _u32, _u64, C.POINTER(_u64)]),
     "itak_kv_append": (_i32, [_P, _u32, _u64, _P, _u64, _P, _u64, _u64]),

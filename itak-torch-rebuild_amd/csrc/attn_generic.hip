@@ -5,7 +5,8 @@
 // kernels elsewhere in this directory cover the shapes the engine actually serves.
 //
 // Semantics follow gqa_attention in crates/attention/src/attention.rs:104-215: a key at
-// position kp is visible to a query at position p iff kp <= p (global layers), query head
+// position kp is visible to a query at position p iff kp <= p and, on a windowed layer,
+// kp > p - window (attention.rs:77-85), query head
 // h reads KV head h / group, scores are dot(q, k) * scale, softmax over the visible keys,
 // output = sum of weights * values. The reference's two-pass softmax becomes an online
 // softmax over key tiles; sums are f32.
@@ -78,8 +79,9 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p, At
     // last row can see.
     uint32_t kend = item.kv_len;
     if (p.q_pos == nullptr) kend = min(kend, item.pos0 + row_end);
-    const uint32_t k_begin = min(kend, split * item.keys_per_split);
+    const uint32_t k_begin = min(kend, item.kv_lo + split * item.keys_per_split);
     const uint32_t k_end = min(kend, k_begin + item.keys_per_split);
+    const uint32_t ring = p.ring_blocks * 32;
 
     const T *kplane = static_cast<const T *>(p.layer_base) + item.slot * p.g.slot_stride +
                       kv_head * p.g.head_stride;
@@ -122,11 +124,12 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p, At
             const uint32_t kj = i / sh.ncol, c = (i % sh.ncol) * VEC;
             float kv[VEC], vv[VEC];
             if (kj < tn) {
-                const uint64_t koff = k_offset(p.g, t0 + kj, c);  // VEC channels share a piece
+                const uint32_t srow = ring ? (t0 + kj) % ring : t0 + kj;
+                const uint64_t koff = k_offset(p.g, srow, c);  // VEC channels share a piece
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     kv[e] = to_f32(kplane[koff + e]);
-                    vv[e] = to_f32(vplane[v_offset(p.g, t0 + kj, c + e)]);
+                    vv[e] = to_f32(vplane[v_offset(p.g, srow, c + e)]);
                 }
             } else {
 #pragma unroll
@@ -168,7 +171,8 @@ __global__ __launch_bounds__(kThreads) void attn_generic_kernel(AttnParams p, At
                     float v = s[i] * p.scale;
                     if (p.softcap > 0.0f) v = p.softcap * tanhf(v / p.softcap);
                     const uint32_t kp = t0 + j;
-                    if (j >= tn || kp > pos) v = -INFINITY;
+                    if (j >= tn || kp > pos || kp < lowest_visible(pos, p.window, item.kv_lo))
+                        v = -INFINITY;
                     Ss[r * TILE + j] = v;
                 }
             }

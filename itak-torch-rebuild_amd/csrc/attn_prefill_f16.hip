@@ -78,7 +78,9 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
 }
 
-template <int N, bool SOFTCAP, int kTiles>
+// RING = the layer is windowed (blocks start at the window, live in a ring, the mask has a
+// lower edge); global layers run the instantiation without any of it.
+template <int N, bool SOFTCAP, int kTiles, bool RING>
 __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnParams p,
                                                                            AttnBatchT<N> b,
                                                                            uint32_t total_partials) {
@@ -107,15 +109,30 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                              item.slot * p.g.slot_stride + kv_head * p.g.head_stride;
     const uint16_t *vplane = kplane + p.g.side_stride;
 
-    // Blocks of this workgroup: its split's run, cut at the last block its rows can see.
+    // Blocks of this workgroup: its split's run of the blocks its rows can see (on a windowed
+    // layer those start at the window of the workgroup's first row, not at the item's).
     const uint32_t blocks_per_split = item.keys_per_split / kBlockKeys;
-    const uint32_t kb_begin = split * blocks_per_split;
-    const uint32_t nblocks = min((item.pos0 + wg_row_end + kBlockKeys - 1) / kBlockKeys,
-                                 kb_begin + blocks_per_split);
+    const uint32_t window = RING ? p.window : 0, kv_lo = RING ? item.kv_lo : 0;
+    const uint32_t wg_lo =
+        lowest_visible(item.pos0 + min(tile * rows_per_group, item.rows - 1), window, kv_lo);
+    const uint32_t kb_begin = wg_lo / kBlockKeys + split * blocks_per_split;
+    // (Rows that stand ahead of the stored length see all of it and nothing more.)
+    const uint32_t nblocks =
+        min((min(item.pos0 + wg_row_end, item.kv_len) + kBlockKeys - 1) / kBlockKeys,
+            kb_begin + blocks_per_split);
     const uint32_t wave_row_end = min(item.rows, row_begin + rows_per_wave);
     const uint32_t wave_blocks =
-        row_begin < item.rows ? (item.pos0 + wave_row_end + kBlockKeys - 1) / kBlockKeys : 0;
-    const uint32_t first_masked = (item.pos0 + row_begin + 1) / kBlockKeys;
+        row_begin < item.rows
+            ? (min(item.pos0 + wave_row_end, item.kv_len) + kBlockKeys - 1) / kBlockKeys
+            : 0;
+    const uint32_t first_masked = (min(item.pos0 + row_begin, item.kv_len - 1) + 1) / kBlockKeys;
+    // Lower edge: blocks before wave_first hold nothing this wavefront's rows see; blocks
+    // before low_masked_end hold positions too old for some of them.
+    const uint32_t item_lo = lowest_visible(item.pos0, window, kv_lo);
+    const uint32_t wave_first =
+        lowest_visible(item.pos0 + min(row_begin, item.rows - 1), window, kv_lo) / kBlockKeys;
+    const uint32_t low_masked_end =
+        (lowest_visible(item.pos0 + wave_row_end - 1, window, kv_lo) + kBlockKeys - 1) / kBlockKeys;
 
     // Each wavefront moves two 1 KiB pieces of the key block and two of the value block.
     const uint4 *kg = reinterpret_cast<const uint4 *>(kplane) + tid;
@@ -129,10 +146,15 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     const uint32_t ring_base =
         (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)(lds_ring);  // LDS byte address
     const uint32_t dma_base = ring_base + wave * 1024;
+    // Storage block of the next block to fetch: position blocks are consecutive, so it climbs
+    // by one and wraps at the end of a windowed layer's ring.
+    const uint32_t ring_blocks = RING ? p.ring_blocks : 1;
+    uint32_t next_sb = RING ? kb_begin % ring_blocks : 0;
     auto issue_block = [&](uint32_t kb) {
         // Past the end the last block is fetched again into a stage nobody reads: the
         // number of loads in flight stays the same in every iteration.
-        const uint64_t off = uint64_t(min(kb, nblocks - 1)) * kBlockVec;
+        const uint64_t off = uint64_t(RING ? next_sb : min(kb, nblocks - 1)) * kBlockVec;
+        if (RING && kb + 1 < nblocks) next_sb = next_sb + 1 == ring_blocks ? 0 : next_sb + 1;
         const uint32_t dst = dma_base + (kb % kStages) * kStageBytes;
         lds_dma16(kg + off, dst);
         lds_dma16(kg + off + 256, dst + 4096);
@@ -150,12 +172,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     const float inv_cap = SOFTCAP ? 1.0f / softcap : 0.0f;
     const float qscale = SOFTCAP ? p.scale : p.scale * kLog2e;
     half8 qb[kTiles][4];
-    uint32_t colpos[kTiles];
+    uint32_t colpos[kTiles], collo[kTiles];
 #pragma unroll
     for (int qt = 0; qt < kTiles; ++qt) {
         const uint32_t j = qt * 16 + jl;
         const uint32_t row = row_begin + j / group;
-        colpos[qt] = item.pos0 + row;
+        colpos[qt] = min(item.pos0 + row, item.kv_len - 1);
+        collo[qt] = lowest_visible(item.pos0 + row, window, kv_lo);
         if (row < item.rows) {
             const uint32_t head = kv_head * group + j % group;
             const float *qp = p.q + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + g * 8;
@@ -197,7 +220,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
         const uint16_t *lds_k = lds_ring + (kb % kStages) * (kStageBytes / 2);
         const uint16_t *lds_v = lds_k + kBlockElems;
 
-        if (kb < wave_blocks) {
+        if (kb < wave_blocks && (!RING || kb >= wave_first)) {
             const uint32_t key_base = kb * kBlockKeys + g * 8;
             floatx4 x[kTiles][2];
             {
@@ -236,6 +259,21 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                     for (int e = 0; e < 8; ++e)
                         x[qt][e >> 2][e & 3] =
                             softcap_log2(x[qt][e >> 2][e & 3], softcap, inv_cap) - ref[qt];
+            }
+            if (RING && kb < low_masked_end) {
+#pragma unroll
+                for (int qt = 0; qt < kTiles; ++qt)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (key_base + e < collo[qt]) x[qt][e >> 2][e & 3] = -INFINITY;
+                if (kb * kBlockKeys < item_lo) {
+                    // Ring rows older than anything the item's queries see may be stale.
+#pragma unroll
+                    for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (key_base + e < item_lo) va[dt][e] = _Float16(0.0f);
+                }
             }
             if (kb >= first_masked) {
 #pragma unroll
@@ -355,7 +393,18 @@ static int tiles_for(const AttnBatch &b, uint32_t group) {
 // most T blocks, T the smallest run length for which the launch has at least two
 // workgroups per compute unit's worth of work units, and never shorter than 8 blocks
 // (a workgroup needs that many to amortise filling its load pipeline).
-uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, uint32_t q_heads) {
+// Key blocks one (row tile, KV head) unit of an item walks at most: everything up to the
+// item's end on a global layer, the window of its first row plus its own rows on a windowed
+// one (the kernel starts each workgroup at its own first visible block).
+static uint32_t unit_block_count(const AttnItem &it, uint32_t rows_per_group, uint32_t window) {
+    const uint32_t all = item_block_count(it);
+    if (window == 0) return all;
+    const uint32_t span = window + std::min(rows_per_group, it.rows) + 2 * kBlockKeys - 2;
+    return std::min(all, span / kBlockKeys);
+}
+
+uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, uint32_t q_heads,
+                               uint32_t window) {
     const uint32_t rows_per_group = uint32_t(tiles_for(b, group) * kWaves * 16) / group;
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess ||
@@ -365,13 +414,13 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
     uint64_t unit_blocks = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         const uint64_t units = uint64_t(g.kv_heads) * ((b.item[i].rows + rows_per_group - 1) / rows_per_group);
-        unit_blocks += units * ((b.item[i].kv_len + kBlockKeys - 1) / kBlockKeys);
+        unit_blocks += units * unit_block_count(b.item[i], rows_per_group, window);
     }
     const uint64_t T = std::max<uint64_t>((unit_blocks + target - 1) / target, 8);
     uint32_t block0 = 0, ws0 = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         AttnItem &it = b.item[i];
-        const uint32_t nblocks = (it.kv_len + kBlockKeys - 1) / kBlockKeys;
+        const uint32_t nblocks = unit_block_count(it, rows_per_group, window);
         const uint32_t units = g.kv_heads * ((it.rows + rows_per_group - 1) / rows_per_group);
         uint32_t splits = std::max<uint32_t>(uint32_t((nblocks + T - 1) / T), 1);
         const uint32_t bps = std::max<uint32_t>((nblocks + splits - 1) / splits, 1);
@@ -389,15 +438,15 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
     return ws0;
 }
 
-template <int N, bool SOFTCAP, int TILES>
+template <int N, bool SOFTCAP, int TILES, bool RING>
 static hipError_t launch_prefill(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                  hipStream_t stream) {
     constexpr size_t lds = size_t(kStages) * kStageBytes;
     static const hipError_t granted = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(&attn_prefill_f16_kernel<N, SOFTCAP, TILES>),
+        reinterpret_cast<const void *>(&attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING>),
         hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
     if (granted != hipSuccess) return granted;
-    attn_prefill_f16_kernel<N, SOFTCAP, TILES><<<b.total_blocks, kWaves * 64, lds, stream>>>(
+    attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING><<<b.total_blocks, kWaves * 64, lds, stream>>>(
         p, AttnBatchT<N>(b), total_partials);
     return hipGetLastError();
 }
@@ -407,17 +456,25 @@ hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, uint
     if (b.total_blocks == 0) return hipSuccess;
     hipError_t e = hipSuccess;
     const bool one = tiles_for(b, p.group) == 1;
-#define ITAK_LAUNCH_TILES(SC)                                                                  \
+#define ITAK_LAUNCH_TILES(SC, RING)                                                            \
     do {                                                                                       \
         if (one)                                                                               \
-            ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, SC, 1>(p, b, total_partials, stream))); \
+            ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, SC, 1, RING>(p, b, total_partials, stream))); \
         else                                                                                   \
-            ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, SC, 2>(p, b, total_partials, stream))); \
+            ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, SC, 2, RING>(p, b, total_partials, stream))); \
+    } while (0)
+#define ITAK_LAUNCH_RING(SC)              \
+    do {                                  \
+        if (p.ring_blocks)                \
+            ITAK_LAUNCH_TILES(SC, true);  \
+        else                              \
+            ITAK_LAUNCH_TILES(SC, false); \
     } while (0)
     if (p.softcap > 0.0f)
-        ITAK_LAUNCH_TILES(true);
+        ITAK_LAUNCH_RING(true);
     else
-        ITAK_LAUNCH_TILES(false);
+        ITAK_LAUNCH_RING(false);
+#undef ITAK_LAUNCH_RING
 #undef ITAK_LAUNCH_TILES
     return e;
 }

@@ -59,6 +59,11 @@ struct BlockOperands {
     half8 v[8];     // [channel tile dt]
 };
 
+// Position block kb lives in storage block kb % ring_blocks on a windowed layer.
+__device__ __forceinline__ uint32_t storage_block(uint32_t kb, uint32_t ring_blocks) {
+    return ring_blocks ? kb % ring_blocks : kb;
+}
+
 __device__ __forceinline__ void load_block(BlockOperands &b, const uint16_t *kplane,
                                            const uint16_t *vplane, uint32_t kb, uint32_t g,
                                            uint32_t i) {
@@ -131,23 +136,27 @@ __device__ __forceinline__ float column_sum(float v) {
 // block: the running state is written, not rescaled (most decode wavefronts see one block).
 // Up to 32 vectors the Q^T operand lives in registers (qreg), beyond that it is re-read
 // from LDS per block: lane (g, jl) holds channels k*32 + g*8 .. +8 of vector jl.
-template <int NQ, bool FIRST>
+template <int NQ, bool FIRST, bool RING>
 __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &b,
                                               const half8 *qreg, const _Float16 *sm_q,
                                               uint32_t kb, uint32_t g, uint32_t jl,
-                                              const uint32_t *colpos, uint32_t pos0,
-                                              uint32_t kv_len, float softcap, float inv_cap) {
+                                              const uint32_t *colpos, const uint32_t *collo,
+                                              uint32_t pos0, uint32_t kv_len, uint32_t lo_min,
+                                              uint32_t lo_max, float softcap, float inv_cap) {
     const uint32_t key_base = kb * kBlockKeys + g * 8;  // first of this lane's 8 keys
-    const bool tail = (kb + 1) * kBlockKeys > kv_len;
+    const bool tail = (kb + 1) * kBlockKeys > kv_len || (RING && kb * kBlockKeys < lo_min);
     if (tail) {
-        // Rows past the stored length may hold stale data: keep them out of P.V even as 0*x.
+        // Rows past the stored length, and ring rows older than anything the block's queries
+        // see, may hold stale data: keep them out of P.V even as 0*x.
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
             for (int e = 0; e < 8; ++e)
-                if (key_base + e >= kv_len) b.v[dt][e] = _Float16(0.0f);
+                if (key_base + e >= kv_len || (RING && key_base + e < lo_min))
+                    b.v[dt][e] = _Float16(0.0f);
     }
-    const bool need_mask = (kb + 1) * kBlockKeys > pos0 + 1;
+    const bool need_mask =
+        (kb + 1) * kBlockKeys > pos0 + 1 || (RING && kb * kBlockKeys < lo_max);
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
         half8 qb[4];
@@ -178,9 +187,10 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
         }
         if (need_mask) {
             const uint32_t pos = colpos[qt];  // this column's query position
+            const uint32_t lo = RING ? collo[qt] : 0;  // and the oldest position it sees
 #pragma unroll
             for (int e = 0; e < 8; ++e)
-                if (key_base + e > pos) sc[e] = -INFINITY;
+                if (key_base + e > pos || (RING && key_base + e < lo)) sc[e] = -INFINITY;
         }
         float mx = sc[0];
 #pragma unroll
@@ -224,7 +234,9 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
 // in-order load counter lets the queries be staged while K/V are still in flight),
 // integer divisions are replaced by multiplications with host-made reciprocals, and the
 // bookkeeping the epilogue needs is computed in the shadow of the loads.
-template <int NQ, int WAVES, int N>
+// RING = the layer is windowed: blocks start at the window, live in a ring, and the mask has a
+// lower edge. Global layers run the instantiation without any of it.
+template <int NQ, int WAVES, int N, bool RING>
 __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams p, AttnBatchT<N> b,
                                                                      uint32_t total_partials) {
     extern __shared__ float lds[];
@@ -252,7 +264,8 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
                      "s"(b.item[0].slot), "s"(b.item[0].rows), "s"(b.item[0].pos0),
                      "s"(b.item[0].q_row0), "s"(b.item[0].kv_len), "s"(b.item[0].splits),
                      "s"(b.item[0].keys_per_split), "s"(b.item[0].block0), "s"(b.item[0].ws0),
-                     "s"(b.item[0].splits_magic));
+                     "s"(b.item[0].splits_magic), "s"(b.item[0].kv_lo), "s"(p.window),
+                     "s"(p.ring_blocks));
     const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
     const uint32_t local = blockIdx.x - item.block0;
     const uint32_t kv_head = item.splits > 1 ? __umulhi(local, item.splits_magic) : local;
@@ -267,8 +280,10 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
 
     const uint32_t nblocks = (item.kv_len + kBlockKeys - 1) / kBlockKeys;
     const uint32_t blocks_per_split = item.keys_per_split / kBlockKeys;
-    const uint32_t kb_begin = split * blocks_per_split;
+    const uint32_t kb_begin = (RING ? item_first_block(item) : 0) + split * blocks_per_split;
     const uint32_t kb_end = min(nblocks, kb_begin + blocks_per_split);
+    const uint32_t ring_blocks = RING ? p.ring_blocks : 0;
+    const uint32_t window = RING ? p.window : 0, kv_lo = RING ? item.kv_lo : 0;
     const bool fused = p.k_new != nullptr;
     const bool owns_new = fused && kb_end * kBlockKeys > item.pos0;
     float *const ws_acc = p.ws;
@@ -314,16 +329,21 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
     [[maybe_unused]] BlockOperands buf_b;
     uint32_t kb = kb_begin + wave;
     const bool has_block = kb < kb_end;
-    load_block(buf_a, kplane, vplane, has_block ? kb : kb_begin, g, jl);
+    load_block(buf_a, kplane, vplane, storage_block(has_block ? kb : kb_begin, ring_blocks), g, jl);
     ITAK_MARK(2)
 
     // ---- 4. in the shadow of the loads: what the mask and the epilogue need per column.
-    uint32_t colpos[NQ], colout[NQ], colps[NQ];
+    uint32_t colpos[NQ], collo[NQ], colout[NQ], colps[NQ];
+    const uint32_t lo_min = lowest_visible(item.pos0, window, kv_lo);
+    const uint32_t lo_max = lowest_visible(item.pos0 + item.rows - 1, window, kv_lo);
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
         const uint32_t j = qt * 16 + jl;
         const uint32_t row = (j * magic) >> 16, head = kv_head * group + (j - row * group);
-        colpos[qt] = item.pos0 + row;
+        // A query ahead of the stored rows sees them all: for the mask its position is the
+        // last stored one (its window still follows from where it really stands).
+        colpos[qt] = min(item.pos0 + row, item.kv_len - 1);
+        collo[qt] = lowest_visible(item.pos0 + row, window, kv_lo);
         colout[qt] = (item.q_row0 + row) * p.q_heads + head;
         colps[qt] = item.ws0 + (row * p.q_heads + head) * item.splits + split;
     }
@@ -355,7 +375,8 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
             uint2 packed{uint32_t(h0) | (uint32_t(h1) << 16), uint32_t(h2) | (uint32_t(h3) << 16)};
             *reinterpret_cast<uint2 *>((side ? sm_newv : sm_newk) + r * kNewStride + c4) = packed;
             const uint32_t key = item.pos0 + r, kin = key % kBlockKeys;
-            const uint64_t blk = uint64_t(key / kBlockKeys) * (kBlockKeys * kD);
+            const uint64_t blk =
+                uint64_t(storage_block(key / kBlockKeys, ring_blocks)) * (kBlockKeys * kD);
             if (side == 0) {
                 const uint32_t kt = (kin >> 2) & 1, ki = (kin >> 3) * 4 + (kin & 3);
                 *reinterpret_cast<uint2 *>(kplane + blk + ((kt * 16 + (c4 >> 3)) * 16 + ki) * 8 +
@@ -390,30 +411,31 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
     do {                                                                                         \
         if (fused && ((KB) + 1) * kBlockKeys > item.pos0)                                        \
             patch_new_rows(BUF, sm_newk, sm_newv, KB, g, jl, item.pos0, item.kv_len);            \
-        process_block<NQ, FIRST>(st, BUF, qreg, sm_q, KB, g, jl, colpos, item.pos0, item.kv_len, \
+        process_block<NQ, FIRST, RING>(st, BUF, qreg, sm_q, KB, g, jl, colpos, collo,                  \
+                                 min(item.pos0, item.kv_len - 1), item.kv_len, lo_min, lo_max,   \
                                  softcap, inv_cap);                                              \
     } while (0)
     if (has_block) {
         if constexpr (NQ <= 2) {
             uint32_t kb2 = kb + WAVES;
             bool more = kb2 < kb_end;
-            if (more) load_block(buf_b, kplane, vplane, kb2, g, jl);
+            if (more) load_block(buf_b, kplane, vplane, storage_block(kb2, ring_blocks), g, jl);
             ITAK_BLOCK(true, buf_a, kb);
             while (more) {
                 const uint32_t kb3 = kb2 + WAVES;
                 const bool more3 = kb3 < kb_end;
-                if (more3) load_block(buf_a, kplane, vplane, kb3, g, jl);
+                if (more3) load_block(buf_a, kplane, vplane, storage_block(kb3, ring_blocks), g, jl);
                 ITAK_BLOCK(false, buf_b, kb2);
                 if (!more3) break;
                 kb2 = kb3 + WAVES;
                 more = kb2 < kb_end;
-                if (more) load_block(buf_b, kplane, vplane, kb2, g, jl);
+                if (more) load_block(buf_b, kplane, vplane, storage_block(kb2, ring_blocks), g, jl);
                 ITAK_BLOCK(false, buf_a, kb3);
             }
         } else {
             ITAK_BLOCK(true, buf_a, kb);
             for (kb += WAVES; kb < kb_end; kb += WAVES) {
-                load_block(buf_a, kplane, vplane, kb, g, jl);
+                load_block(buf_a, kplane, vplane, storage_block(kb, ring_blocks), g, jl);
                 ITAK_BLOCK(false, buf_a, kb);
             }
         }
@@ -514,7 +536,7 @@ static Variant pick_variant(const PoolGeom &g, const AttnBatch &b, uint32_t grou
     uint64_t blocks = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         nvec = std::max(nvec, b.item[i].rows * group);
-        blocks += uint64_t(g.kv_heads) * ((b.item[i].kv_len + kBlockKeys - 1) / kBlockKeys);
+        blocks += uint64_t(g.kv_heads) * item_block_count(b.item[i]);
     }
     if (nvec > 32) return {4, 4, 3};
     if (nvec > 16) return {2, 4, 2};
@@ -529,15 +551,17 @@ static hipError_t grant_lds(size_t lds) {
     static size_t granted = 64 * 1024;
     if (lds <= granted) return hipSuccess;
     // The attribute is per kernel function: set it on each batch-size instantiation.
-    hipError_t e = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 1>),
-        hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
-    if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 8>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
-    if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 64>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+    const void *kernels[] = {
+        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 1, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 8, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 64, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 1, true>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 8, true>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 64, true>)};
+    hipError_t e = hipSuccess;
+    for (const void *k : kernels)
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
     if (e == hipSuccess) granted = lds;
     return e;
 }
@@ -553,7 +577,7 @@ static uint32_t resident_groups() {
     if (grant_lds<NQ, W>(lds) != hipSuccess || hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
         hipOccupancyMaxActiveBlocksPerMultiprocessor(
-            &per_cu, reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 1>), W * 64,
+            &per_cu, reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 1, false>), W * 64,
             lds) != hipSuccess ||
         per_cu < 1 || cus < 1) {
         (void)hipGetLastError();
@@ -580,13 +604,12 @@ uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads)
     const Variant v = pick_variant(g, b, q_heads / g.kv_heads);
     const uint64_t capacity = variant_capacity(v);
     uint64_t blocks = 0;
-    for (uint32_t i = 0; i < b.n; ++i)
-        blocks += uint64_t(g.kv_heads) * ((b.item[i].kv_len + kBlockKeys - 1) / kBlockKeys);
+    for (uint32_t i = 0; i < b.n; ++i) blocks += uint64_t(g.kv_heads) * item_block_count(b.item[i]);
     uint64_t T = std::max<uint64_t>((blocks + capacity - 1) / capacity, uint64_t(v.waves));
     for (;; ++T) {
         uint64_t groups = 0;
         for (uint32_t i = 0; i < b.n; ++i) {
-            const uint64_t nb = (b.item[i].kv_len + kBlockKeys - 1) / kBlockKeys;
+            const uint64_t nb = item_block_count(b.item[i]);
             groups += uint64_t(g.kv_heads) * std::max<uint64_t>((nb + T - 1) / T, 1);
         }
         if (groups <= capacity || T >= blocks) break;
@@ -594,7 +617,7 @@ uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads)
     uint32_t block0 = 0, ws0 = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         AttnItem &it = b.item[i];
-        const uint32_t nblocks = (it.kv_len + kBlockKeys - 1) / kBlockKeys;
+        const uint32_t nblocks = item_block_count(it);
         it.splits = std::max<uint32_t>(uint32_t((nblocks + T - 1) / T), 1);
         const uint32_t bps = std::max<uint32_t>((nblocks + it.splits - 1) / it.splits, 1);
         it.splits = std::max<uint32_t>((nblocks + bps - 1) / bps, 1);
@@ -621,8 +644,12 @@ hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint3
         const size_t lds = variant_lds(NQ, W);                                            \
         hipError_t e = grant_lds<NQ, W>(lds);                                             \
         if (e != hipSuccess) return e;                                                    \
-        attn_splitk_f16_kernel<NQ, W, N><<<b.total_blocks, W * 64, lds, stream>>>(        \
-            p, AttnBatchT<N>(b), total_partials);                                         \
+        if (p.ring_blocks)                                                                \
+            attn_splitk_f16_kernel<NQ, W, N, true><<<b.total_blocks, W * 64, lds, stream>>>(  \
+                p, AttnBatchT<N>(b), total_partials);                                     \
+        else                                                                              \
+            attn_splitk_f16_kernel<NQ, W, N, false><<<b.total_blocks, W * 64, lds, stream>>>( \
+                p, AttnBatchT<N>(b), total_partials);                                     \
     } while (0)
 #define ITAK_LAUNCH_NQ()               \
     do {                               \

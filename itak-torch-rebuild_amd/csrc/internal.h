@@ -80,12 +80,14 @@ constexpr int kMaxBatchItems = 64;
 struct AppendItem {
     uint32_t slot;
     uint32_t rows;
-    uint32_t pos0;      // storage row of the item's first new row
+    uint32_t pos0;      // position of the item's first new row
     uint32_t src_row0;  // row offset of the item inside k_src / v_src
 };
 struct AppendBatch {
     uint32_t n;
     uint32_t total_rows;
+    uint32_t ring;      // storage rows of a windowed layer's ring (position p lives in row p % ring); 0 = row p
+    uint32_t pad;
     AppendItem item[kMaxBatchItems];
 };
 hipError_t launch_append(void *layer_base, int elem_f16, const PoolGeom &g, const AppendBatch &b,
@@ -127,9 +129,11 @@ hipError_t launch_restore(void *pool_base, int dst_f16, int src_f16, const PoolG
                           const RestoreBatch &b, hipStream_t stream);
 
 // ---- row readback: planes -> [row][kv_head][d] ---------------------------------------
+// Row r of the output is position first_row + r, read from storage row (first_row + r) % ring
+// when ring != 0.
 hipError_t launch_read_rows(const void *layer_base, int elem_f16, const PoolGeom &g, uint32_t slot,
-                            uint32_t first_row, uint32_t rows, void *keys_out, void *values_out,
-                            hipStream_t stream);
+                            uint32_t first_row, uint32_t rows, uint32_t ring, void *keys_out,
+                            void *values_out, hipStream_t stream);
 
 hipError_t launch_convert_f16(const float *src, uint16_t *dst, uint64_t count, hipStream_t stream);
 // f16 bits -> f32, exact (the widening a snapshot capture of an f16 pool needs).
@@ -163,7 +167,10 @@ hipError_t launch_attn_gate(float *out, const float *gate, uint64_t count, hipSt
 
 // ---- attention ----------------------------------------------------------------------
 // One item = one slot's query rows against that slot's rows of one layer. Query row r
-// sits at position pos0 + r unless q_pos is given. A workgroup owns (item, row block,
+// sits at position pos0 + r unless q_pos is given. A query at position p sees the keys at
+// positions max(kv_lo, p + 1 - window) .. min(p, kv_len - 1) (window 0 = no lower bound but
+// kv_lo); on a windowed layer position kp lives in storage row kp % (32 * ring_blocks), so
+// that 32-position blocks stay whole and in order inside the ring. A workgroup owns (item, row block,
 // kv head, split of the key range) and writes either the final output (splits == 1) or
 // a partial (m, l, acc[head_dim]) per query vector; a second, small launch merges the
 // partials of each (row, Q head). Partials live in `ws`: first total_partials*head_dim
@@ -180,7 +187,13 @@ struct AttnItem {
     uint32_t block0;        // first workgroup index of the item
     uint32_t ws0;           // first partial index of the item
     uint32_t splits_magic;  // ceil(2^32 / splits) for splits > 1: x / splits == mulhi(x, magic), x < 2^16
+    uint32_t kv_lo;         // oldest position any query of the item may see (0 on global layers)
 };
+// Key blocks (32 positions) an item's queries can touch: [first, end).
+__host__ __device__ inline uint32_t item_first_block(const AttnItem &it) { return it.kv_lo / 32; }
+__host__ __device__ inline uint32_t item_block_count(const AttnItem &it) {
+    return (it.kv_len + 31) / 32 - it.kv_lo / 32;
+}
 struct AttnBatch {
     uint32_t n;
     uint32_t total_blocks;
@@ -262,7 +275,14 @@ struct AttnParams {
     uint32_t group_magic;   // ceil(2^16 / group): j / group == (j * magic) >> 16 for j < 64
     float scale;
     float softcap;
+    uint32_t window;        // attention window of the layer (cache.rs:36-48); 0 = global
+    uint32_t ring_blocks;   // 32-row blocks of the layer's storage ring; 0 = rows are positions
 };
+// The oldest position a query at `pos` sees (attention.rs:77-85 and the view's oldest row).
+__host__ __device__ inline uint32_t lowest_visible(uint32_t pos, uint32_t window, uint32_t kv_lo) {
+    const uint32_t lo = (window != 0 && pos + 1 > window) ? pos + 1 - window : 0;
+    return lo > kv_lo ? lo : kv_lo;
+}
 
 // Generic VALU path: f32 or f16 storage, any head_dim <= 256, group <= 64. Partials are in
 // natural-log domain (combine with base2 = 0).
@@ -283,7 +303,8 @@ hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint3
 // group dividing 16; K/V staged through LDS, split over the context when the launch would
 // otherwise not fill the device. Partials are in log2 domain (combine with base2 = 1).
 bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group);
-uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, uint32_t q_heads);
+uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, uint32_t q_heads,
+                               uint32_t window);
 hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                    hipStream_t stream);
 // Merge of split partials; total_rows = query rows of the batch.

@@ -43,7 +43,8 @@ __global__ __launch_bounds__(256) void kv_append_kernel(T *__restrict__ layer_ba
     uint32_t it = 0;
     while (it + 1 < b.n && row >= b.item[it + 1].src_row0) ++it;
     const AppendItem item = b.item[it];
-    const uint32_t dst_row = item.pos0 + (row - item.src_row0);
+    uint32_t dst_row = item.pos0 + (row - item.src_row0);
+    if (b.ring) dst_row %= b.ring;  // cache.rs:168-173 with the device ring in place of the window
     const float *src = (side ? v_src : k_src) + (uint64_t(row) * g.kv_heads + head) * g.head_dim + d;
     T *plane = layer_base + item.slot * g.slot_stride + side * g.side_stride + head * g.head_stride;
     if constexpr (VEC == 4) {
@@ -305,7 +306,8 @@ hipError_t launch_restore(void *pool_base, int dst_f16, int src_f16, const PoolG
 template <typename T>
 __global__ __launch_bounds__(256) void kv_read_rows(const T *__restrict__ layer_base, PoolGeom g,
                                                     uint32_t slot, uint32_t first_row,
-                                                    uint32_t rows, T *__restrict__ keys_out,
+                                                    uint32_t rows, uint32_t ring,
+                                                    T *__restrict__ keys_out,
                                                     T *__restrict__ values_out) {
     const uint32_t side = blockIdx.y;
     T *out = side ? values_out : keys_out;
@@ -317,13 +319,14 @@ __global__ __launch_bounds__(256) void kv_read_rows(const T *__restrict__ layer_
         const uint32_t rem = uint32_t(i % (g.kv_heads * g.head_dim));
         const uint32_t head = rem / g.head_dim;
         const uint32_t d = rem % g.head_dim;
-        out[i] = src_side[head * g.head_stride + kv_offset(g, side, first_row + row, d)];
+        const uint32_t srow = ring ? (first_row + row) % ring : first_row + row;
+        out[i] = src_side[head * g.head_stride + kv_offset(g, side, srow, d)];
     }
 }
 
 hipError_t launch_read_rows(const void *layer_base, int elem_f16, const PoolGeom &g, uint32_t slot,
-                            uint32_t first_row, uint32_t rows, void *keys_out, void *values_out,
-                            hipStream_t stream) {
+                            uint32_t first_row, uint32_t rows, uint32_t ring, void *keys_out,
+                            void *values_out, hipStream_t stream) {
     if (rows == 0) return hipSuccess;
     const uint64_t total = uint64_t(rows) * g.kv_heads * g.head_dim;
     uint32_t bx = uint32_t((total + 255) / 256);
@@ -331,11 +334,11 @@ hipError_t launch_read_rows(const void *layer_base, int elem_f16, const PoolGeom
     dim3 grid(bx, 2, 1);
     if (elem_f16) {
         kv_read_rows<uint16_t><<<grid, 256, 0, stream>>>(
-            static_cast<const uint16_t *>(layer_base), g, slot, first_row, rows,
+            static_cast<const uint16_t *>(layer_base), g, slot, first_row, rows, ring,
             static_cast<uint16_t *>(keys_out), static_cast<uint16_t *>(values_out));
     } else {
         kv_read_rows<float><<<grid, 256, 0, stream>>>(
-            static_cast<const float *>(layer_base), g, slot, first_row, rows,
+            static_cast<const float *>(layer_base), g, slot, first_row, rows, ring,
             static_cast<float *>(keys_out), static_cast<float *>(values_out));
     }
     return hipGetLastError();

@@ -31,7 +31,19 @@ struct Slot {
     uint64_t cache_id = 0;
     uint64_t next_serial = 0;
     std::vector<uint64_t> appended;  // per layer: positions appended == next position
+    // Per layer: one past the highest position ever written into the storage since it was
+    // last fresh. Positions in [appended, high) were dropped by a rewind; on a windowed layer
+    // their rows still sit in the ring and alias the positions one ring length below them.
+    std::vector<uint64_t> high;
     LiveCheckpoint cp;
+};
+
+// One layer of the pattern (attention::LayerKind, cache.rs:36-48) and where it lives.
+struct LayerInfo {
+    bool windowed = false;
+    uint32_t index = 0;   // among the layers of its kind, which are stored together
+    uint64_t window = 0;  // attention window; 0 on a global layer
+    uint32_t ring = 0;    // storage rows of the ring (a multiple of 32); 0 on a global layer
 };
 
 struct ErrorState {
@@ -46,12 +58,24 @@ uint64_t g_next_cache_id = 1;  // cache.rs:32
 
 struct itak_pool {
     itak_pool_config cfg{};
+    // Global layers and windowed layers are two groups of planes with their own row capacity:
+    // `g` (capacity_rows per plane) and `gw` (the longest ring per plane). Within a group the
+    // layers are consecutive, so the kernels that walk several layers take (group base,
+    // group geometry, index within the group).
     PoolGeom g{};
+    PoolGeom gw{};
+    std::vector<LayerInfo> layers;
+    uint32_t global_layers = 0, windowed_layers = 0;
+    // Rows a windowed layer's ring holds beyond its window: the longest block one step may
+    // append there and the deepest rewind (crates/wgpu-compute/src/session.rs:235-249,
+    // 5376-5428 give the algebra).
+    uint64_t headroom = 0;
     int elem_f16 = 0;
     uint32_t elem_bytes = 4;
     uint64_t row = 0;         // kv_heads * head_dim
-    uint64_t rows_limit = 0;  // positions a slot may hold (the configured capacity)
-    unsigned char *base = nullptr;
+    uint64_t rows_limit = 0;  // positions a slot may hold on a global layer (the configured capacity)
+    unsigned char *base = nullptr;    // global layers
+    unsigned char *base_w = nullptr;  // windowed layers (inside the same allocation)
     uint64_t bytes = 0;
     hipStream_t stream = nullptr;
     std::vector<Slot> slots;
@@ -184,8 +208,28 @@ Slot *find_slot(itak_pool *pool, uint32_t slot) {
     return &pool->slots[slot];
 }
 
+const PoolGeom &geom_of(const itak_pool *pool, uint64_t layer) {
+    return pool->layers[layer].windowed ? pool->gw : pool->g;
+}
+
 void *layer_base(itak_pool *pool, uint64_t layer) {
-    return pool->base + layer * pool->g.layer_stride * pool->elem_bytes;
+    const LayerInfo &L = pool->layers[layer];
+    return (L.windowed ? pool->base_w : pool->base) +
+           L.index * geom_of(pool, layer).layer_stride * pool->elem_bytes;
+}
+
+// Positions stored and visible (cache.rs:154-159) and the oldest of them (cache.rs:162-164).
+uint64_t stored_of(const itak_pool *pool, const Slot &s, uint64_t layer) {
+    const LayerInfo &L = pool->layers[layer];
+    return L.windowed ? std::min(s.appended[layer], L.window) : s.appended[layer];
+}
+uint64_t first_visible(const itak_pool *pool, const Slot &s, uint64_t layer) {
+    return s.appended[layer] - stored_of(pool, s, layer);
+}
+
+void advance(Slot &s, uint64_t layer, uint64_t rows) {
+    s.appended[layer] += rows;
+    s.high[layer] = std::max(s.high[layer], s.appended[layer]);
 }
 
 itak_status ensure_stage(itak_pool *pool, uint64_t bytes) {
@@ -236,6 +280,7 @@ struct PlanInput {
     uint32_t rows;
     uint32_t pos0;
     uint32_t kv_len;
+    uint32_t kv_lo;  // oldest position the item's queries may see
 };
 
 // Builds the work list and launches the attention kernels. q/out are device pointers.
@@ -254,7 +299,7 @@ bool takes_splitk_f16(const itak_pool *pool, const PlanInput *in, uint32_t n, ui
     // same speed on a 7-row block; the fused append decides (one launch less per layer).
     constexpr uint32_t max_vec = 64;
     return pool->elem_f16 && q_pos_dev == nullptr && max_rows * group <= max_vec &&
-           attn_splitk_f16_supports(pool->g, group, max_rows);
+           attn_splitk_f16_supports(pool->g, group, max_rows);  // g and gw differ in capacity only
 }
 
 // k_new / v_new non-null = the rows are not in the cache yet and the kernel appends them
@@ -276,6 +321,9 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         return unsupported(pool->err, "head_dim above 256 or GQA group too wide");
     const uint32_t tile = attn_generic_tile(pool->g.head_dim);
     constexpr uint64_t kTargetBlocks = 1024;  // about four workgroups per CU
+    const LayerInfo &L = pool->layers[layer];
+    const PoolGeom &geom = geom_of(pool, layer);
+    const uint32_t window = uint32_t(std::min<uint64_t>(L.window, 0xffffffffu));
 
     uint32_t q_row0 = 0;
     for (uint32_t first = 0; first < n; first += kMaxBatchItems) {
@@ -291,32 +339,34 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
             it.pos0 = pi.pos0;
             it.q_row0 = q_row0;
             it.kv_len = pi.kv_len;
+            it.kv_lo = pi.kv_lo;
             q_row0 += pi.rows;
             total_rows += pi.rows;
         }
         uint32_t partials = 0;
         if (mfma) {
-            partials = attn_splitk_f16_plan(pool->g, b, uint32_t(q_heads));
+            partials = attn_splitk_f16_plan(geom, b, uint32_t(q_heads));
         } else if (prefill) {
-            partials = attn_prefill_f16_plan(pool->g, b, group, uint32_t(q_heads));
+            partials = attn_prefill_f16_plan(geom, b, group, uint32_t(q_heads), window);
         } else {
             b.rows_per_block = rpb;
             uint64_t key_work = 0;
             for (uint32_t i = 0; i < count; ++i) {
                 const uint64_t qblocks = (b.item[i].rows + rpb - 1) / rpb;
-                key_work += qblocks * pool->g.kv_heads * b.item[i].kv_len;
+                key_work += qblocks * pool->g.kv_heads * (b.item[i].kv_len - b.item[i].kv_lo);
             }
             const uint64_t kps = align_up(
                 std::max<uint64_t>((key_work + kTargetBlocks - 1) / kTargetBlocks, tile), tile);
             uint32_t block0 = 0;
             for (uint32_t i = 0; i < count; ++i) {
                 AttnItem &it = b.item[i];
+                const uint32_t keys = it.kv_len - it.kv_lo;
                 it.keys_per_split = uint32_t(kps);
-                it.splits = uint32_t((it.kv_len + kps - 1) / kps);
+                it.splits = uint32_t((keys + kps - 1) / kps);
                 if (it.splits == 0) it.splits = 1;
                 if (it.splits > 1024) {  // the merge kernel holds at most 1024 weights
-                    it.keys_per_split = uint32_t(align_up((it.kv_len + 1023) / 1024, tile));
-                    it.splits = (it.kv_len + it.keys_per_split - 1) / it.keys_per_split;
+                    it.keys_per_split = uint32_t(align_up((keys + 1023) / 1024, tile));
+                    it.splits = (keys + it.keys_per_split - 1) / it.keys_per_split;
                 }
                 const uint32_t qblocks = (it.rows + rpb - 1) / rpb;
                 it.block0 = block0;
@@ -330,7 +380,9 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         if (st != ITAK_OK) return st;
         AttnParams p{};
         p.layer_base = layer_base(pool, layer);
-        p.g = pool->g;
+        p.g = geom;
+        p.window = window;
+        p.ring_blocks = L.ring / kVBlock;
         p.q = q_dev;
         p.out = out_dev;
         p.q_pos = q_pos_dev;
@@ -372,7 +424,10 @@ itak_status run_append(itak_pool *pool, uint64_t layer, const itak_batch_item *i
     // store 16 bytes per thread instead of 2. The rows after the run inside its last block
     // are beyond the slot's length; the gather writes zeros there, which is what they hold.
     constexpr uint32_t kChunkRows = 4 * kVBlock;
-    if (n == 1 && pool->elem_f16 && pool->g.v_block != 0 && items[0].rows >= kChunkRows) {
+    const LayerInfo &L = pool->layers[layer];
+    const PoolGeom &geom = geom_of(pool, layer);
+    if (n == 1 && !L.windowed && pool->elem_f16 && pool->g.v_block != 0 &&
+        items[0].rows >= kChunkRows) {
         const uint32_t slot = items[0].slot, rows = items[0].rows;
         const uint32_t pos0 = uint32_t(pool->slots[slot].appended[layer]);
         const uint32_t head_rows = (kVBlock - pos0 % kVBlock) % kVBlock;
@@ -390,11 +445,11 @@ itak_status run_append(itak_pool *pool, uint64_t layer, const itak_batch_item *i
         rb.max_rows = rows - head_rows;
         rb.slot = slot;
         rb.layer[0] = RestoreLayer{k_dev + uint64_t(head_rows) * pool->row,
-                                   v_dev + uint64_t(head_rows) * pool->row, uint32_t(layer),
+                                   v_dev + uint64_t(head_rows) * pool->row, L.index,
                                    rows - head_rows, pos0 + head_rows, 0};
         HIP_TRY(pool, launch_restore(pool->base, 1, 0, pool->g, rb, pool->stream),
                 "launch chunk append");
-        pool->slots[slot].appended[layer] += rows;
+        advance(pool->slots[slot], layer, rows);
         return ITAK_OK;
     }
     uint32_t src_row = 0;
@@ -402,6 +457,7 @@ itak_status run_append(itak_pool *pool, uint64_t layer, const itak_batch_item *i
         const uint32_t count = std::min<uint32_t>(kMaxBatchItems, n - first);
         AppendBatch b{};
         b.n = count;
+        b.ring = L.ring;
         const uint32_t chunk_row0 = src_row;
         for (uint32_t i = 0; i < count; ++i) {
             const itak_batch_item &bi = items[first + i];
@@ -413,18 +469,24 @@ itak_status run_append(itak_pool *pool, uint64_t layer, const itak_batch_item *i
         }
         b.total_rows = src_row - chunk_row0;
         HIP_TRY(pool,
-                launch_append(layer_base(pool, layer), pool->elem_f16, pool->g, b,
+                launch_append(layer_base(pool, layer), pool->elem_f16, geom, b,
                               k_dev + uint64_t(chunk_row0) * pool->row,
                               v_dev + uint64_t(chunk_row0) * pool->row, pool->stream),
                 "launch append");
     }
-    for (uint32_t i = 0; i < n; ++i) pool->slots[items[i].slot].appended[layer] += items[i].rows;
+    for (uint32_t i = 0; i < n; ++i) advance(pool->slots[items[i].slot], layer, items[i].rows);
     return ITAK_OK;
 }
 
 // The append preconditions of KvCache::append (cache.rs:445-471) for `rows` consecutive
 // positions starting at the layer's next one; returns how many rows may be appended
 // before a refusal (rows if none) and leaves that refusal in the error state.
+// Positions a slot may hold on a layer: the configured capacity on a global layer; a ring
+// never fills, its positions only have to stay well inside 32 bits.
+uint64_t position_limit(const itak_pool *pool, uint64_t layer) {
+    return pool->layers[layer].windowed ? 0xfff00000ull : pool->rows_limit;
+}
+
 itak_status check_append_rows(itak_pool *pool, Slot &s, uint64_t layer, uint64_t rows,
                               uint64_t *ok_rows) {
     uint64_t ok = rows;
@@ -437,17 +499,30 @@ itak_status check_append_rows(itak_pool *pool, Slot &s, uint64_t layer, uint64_t
             st = range_exceeded(pool->err, layer, start + ok, limit);
         }
     }
-    if (start + ok > pool->rows_limit) {
-        ok = pool->rows_limit > start ? pool->rows_limit - start : 0;
-        st = capacity_exceeded(pool->err, layer, start + ok + 1, pool->rows_limit);
+    const uint64_t rows_limit = position_limit(pool, layer);
+    if (start + ok > rows_limit) {
+        ok = rows_limit > start ? rows_limit - start : 0;
+        st = capacity_exceeded(pool->err, layer, start + ok + 1, rows_limit);
     }
     *ok_rows = ok;
     return st;
 }
 
+// A block of a device step lands in a windowed layer's ring before its queries run, so it
+// may be at most as long as the ring's headroom over the window.
+itak_status check_block_rows(itak_pool *pool, uint64_t layer, uint64_t rows) {
+    const LayerInfo &L = pool->layers[layer];
+    if (!L.windowed || rows <= L.ring - L.window) return ITAK_OK;
+    return set_error(pool->err, ITAK_CAPACITY_EXCEEDED, nullptr, layer, rows, L.ring - L.window, 0,
+                     "a block of %llu rows does not fit the %llu rows of ring headroom of windowed "
+                     "layer %llu; split the block or build the pool with a larger ring_headroom",
+                     ULL(rows), ULL(L.ring - L.window), ULL(layer));
+}
+
+// Zero fill of rows [row_from, row_to) of every global layer of the listed slots.
 itak_status scrub_rows(itak_pool *pool, const ZeroBatch &zb) {
     HIP_TRY(pool,
-            launch_zero_rows(pool->base, pool->elem_f16, pool->g, 0, pool->cfg.layer_count, zb,
+            launch_zero_rows(pool->base, pool->elem_f16, pool->g, 0, pool->global_layers, zb,
                              pool->stream),
             "launch row scrub");
     return ITAK_OK;
@@ -546,14 +621,11 @@ itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out) {
     uint64_t row = 0;
     if (__builtin_mul_overflow(config->num_kv_heads, config->head_dim, &row))
         return size_overflow(e, "kv row length");
-    if (any_windowed) {
-        for (uint32_t i = 0; i < config->layer_count; ++i) {
-            if (config->layer_kinds[i] != ITAK_LAYER_WINDOWED) continue;
-            uint64_t slots = 0;
-            if (__builtin_mul_overflow(config->windows[i], row, &slots))
-                return size_overflow(e, "windowed layer storage");
-        }
-        return unsupported(e, "windowed (ring) layers have no device storage in this build");
+    for (uint32_t i = 0; any_windowed && i < config->layer_count; ++i) {
+        if (config->layer_kinds[i] != ITAK_LAYER_WINDOWED) continue;
+        uint64_t slots = 0;
+        if (__builtin_mul_overflow(config->windows[i], row, &slots))  // cache.rs:131-137
+            return size_overflow(e, "windowed layer storage");
     }
     if (config->elem != ITAK_ELEM_F32 && config->elem != ITAK_ELEM_F16)
         return invalid_argument(e, "elem is neither ITAK_ELEM_F32 nor ITAK_ELEM_F16");
@@ -562,46 +634,88 @@ itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out) {
     if (config->capacity_rows > (1ull << 30) || config->head_dim > (1u << 16) ||
         config->num_kv_heads > (1u << 16))
         return size_overflow(e, "global layer storage");
+    const uint64_t headroom = config->ring_headroom ? config->ring_headroom : 64;
+    if (headroom > (1ull << 20)) return size_overflow(e, "windowed layer storage");
     const uint64_t elem_bytes = config->elem == ITAK_ELEM_F16 ? 2 : 4;
     // f16 pools whose head_dim suits the MFMA kernels keep value planes in transposed
     // 32-row blocks; their planes are padded to whole blocks.
     const bool v_blocked = config->elem == ITAK_ELEM_F16 && config->head_dim % 16 == 0;
+
+    // The pattern: global layers share one group of planes, windowed layers another whose
+    // planes hold the longest ring. A ring is window + headroom rows rounded up to whole
+    // 32-row blocks, so that a 32-position block is also a 32-row block of the ring.
+    std::vector<LayerInfo> layers(config->layer_count);
+    uint32_t n_global = 0, n_windowed = 0;
+    uint64_t max_ring = 0;
+    for (uint32_t i = 0; i < config->layer_count; ++i) {
+        LayerInfo &L = layers[i];
+        L.windowed = config->layer_kinds && config->layer_kinds[i] == ITAK_LAYER_WINDOWED;
+        if (!L.windowed) {
+            L.index = n_global++;
+            continue;
+        }
+        L.index = n_windowed++;
+        L.window = config->windows[i];
+        if (L.window > (1ull << 30)) return size_overflow(e, "windowed layer storage");
+        L.ring = uint32_t(align_up(L.window + headroom, kVBlock));
+        max_ring = std::max<uint64_t>(max_ring, L.ring);
+    }
+    auto make_geom = [&](uint64_t plane_rows, uint64_t layer_count, PoolGeom &g,
+                         uint64_t &bytes) -> bool {
+        uint64_t head_stride, side_stride, slot_stride, layer_stride, total;
+        if (__builtin_mul_overflow(plane_rows, config->head_dim, &head_stride) ||
+            __builtin_mul_overflow(head_stride, config->num_kv_heads, &side_stride) ||
+            __builtin_mul_overflow(side_stride, uint64_t(2), &slot_stride) ||
+            __builtin_mul_overflow(slot_stride, uint64_t(config->max_slots), &layer_stride) ||
+            __builtin_mul_overflow(layer_stride, layer_count, &total) ||
+            __builtin_mul_overflow(total, elem_bytes, &bytes))
+            return false;
+        g.kv_heads = uint32_t(config->num_kv_heads);
+        g.head_dim = uint32_t(config->head_dim);
+        g.capacity = uint32_t(plane_rows);
+        g.max_slots = config->max_slots;
+        g.v_block = v_blocked ? kVBlock : 0;
+        g.head_stride = head_stride;
+        g.side_stride = side_stride;
+        g.slot_stride = slot_stride;
+        g.layer_stride = layer_stride;
+        return true;
+    };
     const uint64_t plane_rows =
         v_blocked ? align_up(config->capacity_rows, kVBlock) : config->capacity_rows;
-    uint64_t head_stride, side_stride, slot_stride, layer_stride, total, bytes;
-    if (__builtin_mul_overflow(plane_rows, config->head_dim, &head_stride) ||
-        __builtin_mul_overflow(head_stride, config->num_kv_heads, &side_stride) ||
-        __builtin_mul_overflow(side_stride, uint64_t(2), &slot_stride) ||
-        __builtin_mul_overflow(slot_stride, uint64_t(config->max_slots), &layer_stride) ||
-        __builtin_mul_overflow(layer_stride, uint64_t(config->layer_count), &total) ||
-        __builtin_mul_overflow(total, elem_bytes, &bytes))
+    PoolGeom g{}, gw{};
+    uint64_t bytes_g = 0, bytes_w = 0, bytes = 0;
+    if (!make_geom(plane_rows, n_global, g, bytes_g))
+        return size_overflow(e, "global layer storage");
+    if (!make_geom(max_ring, n_windowed, gw, bytes_w))
+        return size_overflow(e, "windowed layer storage");
+    bytes_g = align_up(bytes_g, 256);
+    if (__builtin_add_overflow(bytes_g, bytes_w, &bytes) || bytes == 0)
         return size_overflow(e, "global layer storage");
 
     hipError_t he = hipSetDevice(config->device);
     if (he != hipSuccess) return hip_error(e, he, "select device");
     itak_pool *pool = new itak_pool();
     pool->cfg = *config;
-    pool->cfg.layer_kinds = nullptr;  // all global; the caller's arrays are not retained
+    pool->cfg.layer_kinds = nullptr;  // the caller's arrays are not retained: see `layers`
     pool->cfg.windows = nullptr;
+    pool->layers = std::move(layers);
+    pool->global_layers = n_global;
+    pool->windowed_layers = n_windowed;
+    pool->headroom = headroom;
     pool->elem_f16 = config->elem == ITAK_ELEM_F16;
     pool->elem_bytes = uint32_t(elem_bytes);
     pool->row = row;
-    pool->g.kv_heads = uint32_t(config->num_kv_heads);
-    pool->g.head_dim = uint32_t(config->head_dim);
-    pool->g.capacity = uint32_t(plane_rows);
-    pool->g.max_slots = config->max_slots;
-    pool->g.v_block = v_blocked ? kVBlock : 0;
+    pool->g = g;
+    pool->gw = gw;
     pool->rows_limit = config->capacity_rows;
-    pool->g.head_stride = head_stride;
-    pool->g.side_stride = side_stride;
-    pool->g.slot_stride = slot_stride;
-    pool->g.layer_stride = layer_stride;
     pool->bytes = bytes;
     he = hipMalloc(reinterpret_cast<void **>(&pool->base), bytes);
     if (he != hipSuccess) {
         delete pool;
         return hip_error(e, he, "allocate KV pool");
     }
+    pool->base_w = pool->base + bytes_g;
     // Fresh storage is all zero bytes, as the reference's ring storage is
     // (cache.rs:139) and as the scrub guarantee needs.
     he = hipMemset(pool->base, 0, bytes);
@@ -649,6 +763,7 @@ itak_status itak_slot_acquire(itak_pool *pool, uint32_t *slot) {
         s.in_use = true;
         s.cache_id = g_next_cache_id++;
         s.appended.assign(pool->cfg.layer_count, 0);
+        s.high.assign(pool->cfg.layer_count, 0);
         *slot = i;
         return ITAK_OK;
     }
@@ -661,7 +776,13 @@ itak_status itak_slot_reset(itak_pool *pool, uint32_t slot) {
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
     uint64_t max_rows = 0;
-    for (uint64_t a : s->appended) max_rows = std::max(max_rows, a);
+    bool ring_used = false;
+    for (uint64_t l = 0; l < s->high.size(); ++l) {
+        if (pool->layers[l].windowed)
+            ring_used = ring_used || s->high[l] > 0;
+        else
+            max_rows = std::max(max_rows, s->high[l]);
+    }
     if (max_rows > 0) {
         ZeroBatch zb{};
         zb.n = 1;
@@ -670,7 +791,18 @@ itak_status itak_slot_reset(itak_pool *pool, uint32_t slot) {
         itak_status st = scrub_rows(pool, zb);
         if (st != ITAK_OK) return st;
     }
+    if (ring_used) {  // the whole ring of every windowed layer
+        ZeroBatch zb{};
+        zb.n = 1;
+        zb.max_rows = pool->gw.capacity;
+        zb.item[0] = ZeroItem{slot, 0, pool->gw.capacity, 0};
+        HIP_TRY(pool,
+                launch_zero_rows(pool->base_w, pool->elem_f16, pool->gw, 0, pool->windowed_layers,
+                                 zb, pool->stream),
+                "launch ring scrub");
+    }
     std::fill(s->appended.begin(), s->appended.end(), 0);
+    std::fill(s->high.begin(), s->high.end(), 0);
     s->built = false;
     s->cp = LiveCheckpoint{};
     s->next_serial = 0;
@@ -692,8 +824,16 @@ uint64_t itak_kv_head_dim(const itak_pool *pool) { return pool ? pool->g.head_di
 itak_status itak_kv_layer_kind(itak_pool *pool, uint64_t layer, uint32_t *kind, uint64_t *window) {
     if (!pool) return ITAK_INVALID_ARGUMENT;
     if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
-    if (kind) *kind = ITAK_LAYER_GLOBAL;
-    if (window) *window = 0;
+    if (kind) *kind = pool->layers[layer].windowed ? ITAK_LAYER_WINDOWED : ITAK_LAYER_GLOBAL;
+    if (window) *window = pool->layers[layer].window;
+    return ITAK_OK;
+}
+
+itak_status itak_kv_storage_rows(itak_pool *pool, uint64_t layer, uint64_t *out) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
+    if (!out) return invalid_argument(pool->err, "out is null");
+    *out = pool->layers[layer].windowed ? pool->layers[layer].ring : pool->rows_limit;
     return ITAK_OK;
 }
 
@@ -702,12 +842,17 @@ itak_status itak_kv_stored_len(itak_pool *pool, uint32_t slot, uint64_t layer, u
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
     if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
-    *out = s->appended[layer];  // global layer: stored == appended (cache.rs:154-159)
+    *out = stored_of(pool, *s, layer);  // cache.rs:154-159
     return ITAK_OK;
 }
 
 itak_status itak_kv_next_position(itak_pool *pool, uint32_t slot, uint64_t layer, uint64_t *out) {
-    return itak_kv_stored_len(pool, slot, layer, out);
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    Slot *s = find_slot(pool, slot);
+    if (!s) return invalid_argument(pool->err, "slot is not in use");
+    if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
+    *out = s->appended[layer];
+    return ITAK_OK;
 }
 
 itak_status itak_kv_append(itak_pool *pool, uint32_t slot, uint64_t layer, const float *k,
@@ -725,8 +870,8 @@ itak_status itak_kv_append(itak_pool *pool, uint32_t slot, uint64_t layer, const
     if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
     if (position != s->appended[layer])
         return out_of_order(pool->err, layer, s->appended[layer], position);
-    if (position >= pool->rows_limit)
-        return capacity_exceeded(pool->err, layer, position + 1, pool->rows_limit);
+    if (position >= position_limit(pool, layer))
+        return capacity_exceeded(pool->err, layer, position + 1, position_limit(pool, layer));
     if (!k || !v) return invalid_argument(pool->err, "k or v is null");
     const uint64_t bytes = pool->row * sizeof(float);
     itak_status st = ensure_stage(pool, 2 * bytes);
@@ -756,6 +901,8 @@ itak_status itak_kv_append_device(itak_pool *pool, uint64_t layer, const itak_ba
         uint64_t ok = 0;
         itak_status st = check_append_rows(pool, *s, layer, items[i].rows, &ok);
         if (st != ITAK_OK) return st;
+        st = check_block_rows(pool, layer, items[i].rows);
+        if (st != ITAK_OK) return st;
     }
     return run_append(pool, layer, items, item_count, k_dev, v_dev);
 }
@@ -780,45 +927,82 @@ static itak_status restore_layers(itak_pool *pool, uint32_t slot, Slot &s,
     if (stage_need) HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&temp), stage_need), "allocate restore staging");
     uint64_t temp_off = 0;
     itak_status st = ITAK_OK;
-    for (uint64_t first = 0; first < count && st == ITAK_OK; first += kMaxRestoreLayers) {
-        const uint64_t n = std::min<uint64_t>(kMaxRestoreLayers, count - first);
-        RestoreBatch b{};
-        b.slot = slot;
-        for (uint64_t i = 0; i < n; ++i) {
-            const itak_snapshot_layer &L = layers[first + i];
-            if (L.rows == 0) continue;
-            const uint64_t bytes = L.rows * pool->row * src_bytes_per_elem;
-            const void *src[2] = {L.keys, L.values};
-            for (int side = 0; side < 2; ++side) {
-                const void *usable;
-                if (!must_stage(src[side], src_bytes_per_elem)) {
-                    classify(src[side], &usable);
-                    src[side] = usable;
-                    continue;
-                }
-                hipError_t he = hipMemcpyAsync(temp + temp_off, src[side], bytes,
-                                               hipMemcpyHostToDevice, pool->stream);
-                if (he != hipSuccess) {
-                    st = hip_error(pool->err, he, "stage snapshot rows");
-                    break;
-                }
-                src[side] = temp + temp_off;
-                temp_off += align_up(bytes, 256);
+    // One gather batch per group of planes (global, windowed), launched when it fills up. A
+    // windowed layer's rows go to storage rows position % ring: one run, or two when the
+    // positions wrap past the end of the ring (session.rs:320-346 states the same split).
+    RestoreBatch batch[2] = {};
+    batch[0].slot = batch[1].slot = slot;
+    // A ring that was filled and then rewound to empty still holds the old rows; a restore
+    // that writes fewer rows than the window must find zeros around them, as in a fresh cache.
+    for (uint64_t i = 0; i < count; ++i) {
+        const uint64_t layer = layer_ids ? layer_ids[i] : i;
+        const LayerInfo &info = pool->layers[layer];
+        if (!info.windowed || s.high[layer] == 0) continue;
+        ZeroBatch zb{};
+        zb.n = 1;
+        zb.max_rows = info.ring;
+        zb.item[0] = ZeroItem{slot, 0, info.ring, 0};
+        hipError_t e = launch_zero_rows(pool->base_w, pool->elem_f16, pool->gw, info.index,
+                                        info.index + 1, zb, pool->stream);
+        if (e != hipSuccess) {
+            if (temp) (void)hipFree(temp);
+            return hip_error(pool->err, e, "launch ring scrub");
+        }
+    }
+    auto flush = [&](int w) -> itak_status {
+        if (batch[w].n == 0) return ITAK_OK;
+        hipError_t e = launch_restore(w ? pool->base_w : pool->base, pool->elem_f16,
+                                      src_elem == ITAK_ELEM_F16, w ? pool->gw : pool->g, batch[w],
+                                      pool->stream);
+        batch[w].n = 0;
+        batch[w].max_rows = 0;
+        return e == hipSuccess ? ITAK_OK : hip_error(pool->err, e, "launch restore gather");
+    };
+    for (uint64_t i = 0; i < count && st == ITAK_OK; ++i) {
+        const itak_snapshot_layer &L = layers[i];
+        if (L.rows == 0) continue;
+        const uint64_t layer = layer_ids ? layer_ids[i] : i;
+        const LayerInfo &info = pool->layers[layer];
+        const uint64_t bytes = L.rows * pool->row * src_bytes_per_elem;
+        const void *src[2] = {L.keys, L.values};
+        for (int side = 0; side < 2; ++side) {
+            const void *usable;
+            if (!must_stage(src[side], src_bytes_per_elem)) {
+                classify(src[side], &usable);
+                src[side] = usable;
+                continue;
             }
-            if (st != ITAK_OK) break;
-            RestoreLayer &R = b.layer[b.n++];
-            R.keys = src[0];
-            R.values = src[1];
-            R.layer = uint32_t(layer_ids ? layer_ids[first + i] : first + i);
-            R.rows = uint32_t(L.rows);
-            R.first_row = uint32_t(L.first_position);  // global layer: slot_of(p) == p
-            b.max_rows = std::max(b.max_rows, R.rows);
+            hipError_t he = hipMemcpyAsync(temp + temp_off, src[side], bytes, hipMemcpyHostToDevice,
+                                           pool->stream);
+            if (he != hipSuccess) {
+                st = hip_error(pool->err, he, "stage snapshot rows");
+                break;
+            }
+            src[side] = temp + temp_off;
+            temp_off += align_up(bytes, 256);
         }
         if (st != ITAK_OK) break;
-        hipError_t he = launch_restore(pool->base, pool->elem_f16, src_elem == ITAK_ELEM_F16,
-                                       pool->g, b, pool->stream);
-        if (he != hipSuccess) st = hip_error(pool->err, he, "launch restore gather");
+        const int w = info.windowed ? 1 : 0;
+        uint64_t done = 0;
+        while (done < L.rows && st == ITAK_OK) {
+            const uint64_t position = L.first_position + done;
+            const uint64_t row = info.windowed ? position % info.ring : position;
+            const uint64_t run =
+                info.windowed ? std::min<uint64_t>(L.rows - done, info.ring - row) : L.rows - done;
+            if (batch[w].n == kMaxRestoreLayers) st = flush(w);
+            if (st != ITAK_OK) break;
+            RestoreLayer &R = batch[w].layer[batch[w].n++];
+            const uint64_t skip = done * pool->row * src_bytes_per_elem;
+            R.keys = static_cast<const unsigned char *>(src[0]) + skip;
+            R.values = static_cast<const unsigned char *>(src[1]) + skip;
+            R.layer = info.index;
+            R.rows = uint32_t(run);
+            R.first_row = uint32_t(row);
+            batch[w].max_rows = std::max(batch[w].max_rows, R.rows);
+            done += run;
+        }
     }
+    for (int w = 0; w < 2 && st == ITAK_OK; ++w) st = flush(w);
     hipError_t he = hipStreamSynchronize(pool->stream);
     if (st == ITAK_OK && he != hipSuccess) st = hip_error(pool->err, he, "synchronize after restore");
     if (temp) (void)hipFree(temp);
@@ -826,6 +1010,7 @@ static itak_status restore_layers(itak_pool *pool, uint32_t slot, Slot &s,
     for (uint64_t i = 0; i < count; ++i) {
         const uint64_t layer = layer_ids ? layer_ids[i] : i;
         s.appended[layer] = layers[i].first_position + layers[i].rows;  // cache.rs:568
+        s.high[layer] = s.appended[layer];
     }
     return ITAK_OK;
 }
@@ -842,10 +1027,18 @@ itak_status itak_kv_restore_bulk(itak_pool *pool, uint32_t slot, uint64_t layer,
     const uint64_t rows = keys_len / pool->row;
     if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
     if (s->appended[layer] != 0) return not_fresh(pool->err, layer, s->appended[layer]);
-    if (first_position != 0)
+    if (pool->layers[layer].windowed) {
+        if (rows > pool->layers[layer].window)
+            return shape_mismatch(pool->err, "bulk restore rows (windowed layer)",
+                                  pool->layers[layer].window, rows);
+    } else if (first_position != 0) {
         return shape_mismatch(pool->err, "bulk restore first position (global layer)", 0,
                               first_position);
-    if (rows > pool->rows_limit) return capacity_exceeded(pool->err, layer, rows, pool->rows_limit);
+    }
+    if (first_position > position_limit(pool, layer) ||
+        rows > position_limit(pool, layer) - first_position)
+        return capacity_exceeded(pool->err, layer, first_position + rows,
+                                 position_limit(pool, layer));
     if (rows && (!keys || !values)) return invalid_argument(pool->err, "keys or values is null");
     itak_snapshot_layer L{first_position, rows, keys, values};
     return restore_layers(pool, slot, *s, &L, &layer, 1, src_elem);
@@ -858,33 +1051,43 @@ itak_status itak_kv_restore_snapshot(itak_pool *pool, uint32_t slot, uint64_t to
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
     if (!layers) return invalid_argument(pool->err, "layers is null");
-    // KvSnapshot::validate (snapshot.rs:187-236) for an all-global geometry.
+    // KvSnapshot::validate (snapshot.rs:187-236) against the pool's own pattern.
     if (layer_count != pool->cfg.layer_count)
         return set_error(pool->err, ITAK_STEP_FAILED, "restore_snapshot", layer_count,
                          pool->cfg.layer_count, 0, 0,
                          "snapshot carries %llu layer blocks but its geometry has %llu layers",
                          ULL(layer_count), ULL(pool->cfg.layer_count));
     for (uint64_t i = 0; i < layer_count; ++i) {
-        if (layers[i].first_position != 0)
+        const LayerInfo &info = pool->layers[i];
+        const uint64_t expected_rows =
+            info.windowed ? std::min(token_count, info.window) : token_count;
+        const uint64_t expected_first = token_count - expected_rows;
+        if (layers[i].first_position != expected_first) {
+            char kind[64] = "Global";
+            if (info.windowed)
+                snprintf(kind, sizeof(kind), "Windowed { window: %llu }", ULL(info.window));
             return set_error(pool->err, ITAK_STEP_FAILED, "restore_snapshot", i,
-                             layers[i].first_position, 0, 0,
-                             "layer %llu: first stored position is %llu but 0 follows from token "
-                             "count %llu and kind Global",
-                             ULL(i), ULL(layers[i].first_position), ULL(token_count));
-        if (layers[i].rows != token_count)
+                             layers[i].first_position, expected_first, 0,
+                             "layer %llu: first stored position is %llu but %llu follows from token "
+                             "count %llu and kind %s",
+                             ULL(i), ULL(layers[i].first_position), ULL(expected_first),
+                             ULL(token_count), kind);
+        }
+        if (layers[i].rows != expected_rows)
             return set_error(pool->err, ITAK_STEP_FAILED, "restore_snapshot", i, layers[i].rows,
-                             token_count, 0,
+                             expected_rows, 0,
                              "layer %llu: holds %llu rows but %llu rows were expected", ULL(i),
-                             ULL(layers[i].rows), ULL(token_count));
-        if (token_count && (!layers[i].keys || !layers[i].values))
+                             ULL(layers[i].rows), ULL(expected_rows));
+        if (expected_rows && (!layers[i].keys || !layers[i].values))
             return invalid_argument(pool->err, "a layer's keys or values is null");
     }
     // KvSnapshot::restore builds a fresh cache (snapshot.rs:321-334): every layer must be
     // fresh here, checked for all layers before any is touched.
     for (uint64_t i = 0; i < layer_count; ++i)
         if (s->appended[i] != 0) return not_fresh(pool->err, i, s->appended[i]);
-    if (token_count > pool->rows_limit)
-        return capacity_exceeded(pool->err, 0, token_count, pool->rows_limit);
+    for (uint64_t i = 0; i < layer_count; ++i)
+        if (token_count > position_limit(pool, i))
+            return capacity_exceeded(pool->err, i, token_count, position_limit(pool, i));
     return restore_layers(pool, slot, *s, layers, nullptr, layer_count, src_elem);
 }
 
@@ -991,8 +1194,16 @@ itak_status itak_kv_capture_itkv(itak_pool *pool, uint32_t slot, const char *fin
     h.head_dim = pool->g.head_dim;
     h.layer_count = pool->cfg.layer_count;
     h.fingerprint_len = fingerprint_len;
+    // snapshot.rs:264-295: every row of a global layer, the last `window` rows of a windowed
+    // one, oldest first.
     std::vector<ItkvLayer> ls(h.layer_count);
-    for (ItkvLayer &l : ls) l.rows = token_count;  // global layers: every row, from position 0
+    for (uint64_t i = 0; i < h.layer_count; ++i) {
+        const LayerInfo &info = pool->layers[i];
+        ls[i].kind = info.windowed ? ITAK_LAYER_WINDOWED : ITAK_LAYER_GLOBAL;
+        ls[i].window = info.window;
+        ls[i].rows = stored_of(pool, *s, i);
+        ls[i].first_position = token_count - ls[i].rows;
+    }
     uint64_t total = 0;
     if (!itkv_encoded_len(h, ls.data(), &total)) return size_overflow(pool->err, "encoded snapshot");
     *written = total;
@@ -1009,13 +1220,15 @@ itak_status itak_kv_capture_itkv(itak_pool *pool, uint32_t slot, const char *fin
     itak_status st = ensure_stage(pool, 2 * raw + (pool->elem_f16 ? 2 * wide : 0));
     if (st != ITAK_OK) return st;
     for (uint64_t layer = 0; layer < h.layer_count; ++layer) {
-        for (uint64_t first = 0; first < token_count; first += chunk_rows) {
-            const uint64_t rows = std::min(chunk_rows, token_count - first);
+        for (uint64_t first = 0; first < ls[layer].rows; first += chunk_rows) {
+            const uint64_t rows = std::min(chunk_rows, ls[layer].rows - first);
             const uint64_t elems = rows * pool->row;
             unsigned char *kd = pool->stage, *vd = pool->stage + raw;
             HIP_TRY(pool,
-                    launch_read_rows(layer_base(pool, layer), pool->elem_f16, pool->g, slot,
-                                     uint32_t(first), uint32_t(rows), kd, vd, pool->stream),
+                    launch_read_rows(layer_base(pool, layer), pool->elem_f16, geom_of(pool, layer),
+                                     slot, uint32_t(ls[layer].first_position + first),
+                                     uint32_t(rows), pool->layers[layer].ring, kd, vd,
+                                     pool->stream),
                     "launch row readback");
             const void *ksrc = kd, *vsrc = vd;
             if (pool->elem_f16) {
@@ -1067,7 +1280,10 @@ itak_status itak_kv_restore_itkv(itak_pool *pool, uint32_t slot, const void *byt
     // restore_checked (snapshot.rs:351-371): geometry first, then the fingerprint.
     bool same = h.layer_count == pool->cfg.layer_count && h.num_kv_heads == pool->g.kv_heads &&
                 h.head_dim == pool->g.head_dim;
-    for (size_t i = 0; same && i < ls.size(); ++i) same = ls[i].kind == ITAK_LAYER_GLOBAL;
+    for (size_t i = 0; same && i < ls.size(); ++i)
+        same = pool->layers[i].windowed
+                   ? (ls[i].kind == ITAK_LAYER_WINDOWED && ls[i].window == pool->layers[i].window)
+                   : ls[i].kind == ITAK_LAYER_GLOBAL;
     if (!same)
         return set_error(pool->err, ITAK_KV_GEOMETRY_MISMATCH, "snapshot", 0, 0, 0, 0,
                          "geometry mismatch: snapshot geometry (%llu layers, %llu KV heads, head "
@@ -1097,13 +1313,18 @@ itak_status itak_kv_stats(itak_pool *pool, uint32_t slot, itak_layer_stats *out)
     if (!s) return invalid_argument(pool->err, "slot is not in use");
     if (!out) return invalid_argument(pool->err, "out is null");
     for (uint32_t i = 0; i < pool->cfg.layer_count; ++i) {
-        out[i] = itak_layer_stats{i, ITAK_LAYER_GLOBAL, 0, 0, s->appended[i], s->appended[i]};
+        const LayerInfo &info = pool->layers[i];
+        out[i] = itak_layer_stats{i, uint32_t(info.windowed ? ITAK_LAYER_WINDOWED : ITAK_LAYER_GLOBAL),
+                                  0, info.window, s->appended[i], stored_of(pool, *s, i)};
     }
     return ITAK_OK;
 }
 
+// `first` is a position (a storage row on a global layer, which is the same thing); `ring`
+// maps positions to storage rows on a windowed layer, 0 reads storage rows as they lie.
 static itak_status read_rows_common(itak_pool *pool, uint32_t slot, uint64_t layer, uint64_t first,
-                                    uint64_t rows, void *keys_out, void *values_out) {
+                                    uint64_t rows, uint32_t ring, void *keys_out,
+                                    void *values_out) {
     if (rows == 0 || (!keys_out && !values_out)) return ITAK_OK;
     const uint64_t bytes = rows * pool->row * pool->elem_bytes;
     itak_status st = ensure_stage(pool, 2 * align_up(bytes, 256));
@@ -1111,8 +1332,8 @@ static itak_status read_rows_common(itak_pool *pool, uint32_t slot, uint64_t lay
     void *kd = keys_out ? pool->stage : nullptr;
     void *vd = values_out ? pool->stage + align_up(bytes, 256) : nullptr;
     HIP_TRY(pool,
-            launch_read_rows(layer_base(pool, layer), pool->elem_f16, pool->g, slot,
-                             uint32_t(first), uint32_t(rows), kd, vd, pool->stream),
+            launch_read_rows(layer_base(pool, layer), pool->elem_f16, geom_of(pool, layer), slot,
+                             uint32_t(first), uint32_t(rows), ring, kd, vd, pool->stream),
             "launch row readback");
     if (keys_out)
         HIP_TRY(pool, hipMemcpyAsync(keys_out, kd, bytes, hipMemcpyDeviceToHost, pool->stream),
@@ -1131,12 +1352,14 @@ itak_status itak_kv_read_rows(itak_pool *pool, uint32_t slot, uint64_t layer, ui
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
     if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
-    const uint64_t stored = s->appended[layer];
+    const uint64_t stored = stored_of(pool, *s, layer);
     if (first > stored || rows > stored - first)
         return shape_mismatch(pool->err, "visible rows", stored, first + rows);
+    const uint64_t oldest = first_visible(pool, *s, layer);
     if (positions_out)
-        for (uint64_t i = 0; i < rows; ++i) positions_out[i] = first + i;  // cache.rs:878-883
-    return read_rows_common(pool, slot, layer, first, rows, keys_out, values_out);
+        for (uint64_t i = 0; i < rows; ++i) positions_out[i] = oldest + first + i;  // cache.rs:878-883
+    return read_rows_common(pool, slot, layer, oldest + first, rows, pool->layers[layer].ring,
+                            keys_out, values_out);
 }
 
 itak_status itak_kv_read_raw(itak_pool *pool, uint32_t slot, uint64_t layer, void *keys_out,
@@ -1145,7 +1368,8 @@ itak_status itak_kv_read_raw(itak_pool *pool, uint32_t slot, uint64_t layer, voi
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
     if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
-    return read_rows_common(pool, slot, layer, 0, pool->rows_limit, keys_out, values_out);
+    const uint64_t rows = pool->layers[layer].windowed ? pool->layers[layer].ring : pool->rows_limit;
+    return read_rows_common(pool, slot, layer, 0, rows, 0, keys_out, values_out);
 }
 
 itak_status itak_kv_checkpoint_active(itak_pool *pool, uint32_t slot, int32_t *out) {
@@ -1162,9 +1386,30 @@ itak_status itak_kv_checkpoint(itak_pool *pool, uint32_t slot, uint64_t max_roun
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
     if (!out) return invalid_argument(pool->err, "out is null");
-    // cache.rs:635-651; with no windowed layer there is no CheckpointTooDeep bound.
+    // cache.rs:635-651, in order.
     if (s->cp.live) return checkpoint_busy(pool->err);
     if (max_round_tokens == 0) return zero_dimension(pool->err, "max_round_tokens");
+    uint64_t smallest_window = 0, windowed = 0;
+    for (const LayerInfo &L : pool->layers)
+        if (L.windowed) {
+            smallest_window = windowed ? std::min(smallest_window, L.window) : L.window;
+            ++windowed;
+        }
+    if (windowed && max_round_tokens > smallest_window)
+        return set_error(pool->err, ITAK_CHECKPOINT_TOO_DEEP, nullptr, max_round_tokens,
+                         smallest_window, 0, 0,
+                         "checkpoint round bound %llu exceeds the smallest sliding window %llu: a "
+                         "round that long would overwrite a ring slot twice and no rewind could be "
+                         "exact",
+                         ULL(max_round_tokens), ULL(smallest_window));
+    // The device keeps no copies of evicted rows: the ring's headroom is what lets a round be
+    // undone, so a round may not be longer than it.
+    if (windowed && max_round_tokens > pool->headroom)
+        return set_error(pool->err, ITAK_CAPACITY_EXCEEDED, nullptr, 0, max_round_tokens,
+                         pool->headroom, 0,
+                         "a round of up to %llu tokens does not fit the %llu rows of ring headroom "
+                         "of the windowed layers; build the pool with a larger ring_headroom",
+                         ULL(max_round_tokens), ULL(pool->headroom));
     s->next_serial += 1;
     s->cp.live = true;
     s->cp.serial = s->next_serial;
@@ -1173,7 +1418,9 @@ itak_status itak_kv_checkpoint(itak_pool *pool, uint32_t slot, uint64_t max_roun
     out->cache_id = s->cache_id;
     out->serial = s->cp.serial;
     out->max_round_tokens = max_round_tokens;
-    out->saved_bytes = 0;  // global layers save no rows: rewind is truncation (cache.rs:675-677)
+    // What the reference's snapshot of the evictable ring slots would hold (cache.rs:678-697):
+    // reported for accounting; the device saves nothing, the rows stay in the ring's headroom.
+    out->saved_bytes = windowed * max_round_tokens * 2 * pool->row * 4;
     return ITAK_OK;
 }
 
@@ -1194,17 +1441,40 @@ itak_status itak_kv_checkpoint_bases(itak_pool *pool, uint32_t slot, const itak_
     return ITAK_OK;
 }
 
+// A windowed layer can drop positions only while the rows written above the target have not
+// wrapped onto rows the target's view still needs: with H the highest position ever written
+// plus one, position x is overwritten once x + ring < H, and the view after the rewind starts
+// at target - window, so H - target may be at most ring - window.
+static itak_status check_ring_rewind(itak_pool *pool, const Slot &s, uint64_t target) {
+    for (uint64_t li = 0; li < s.appended.size(); ++li) {
+        const LayerInfo &L = pool->layers[li];
+        if (!L.windowed || target >= s.appended[li]) continue;
+        if (s.high[li] - target > L.ring - L.window)
+            return set_error(pool->err, ITAK_CAPACITY_EXCEEDED, nullptr, li, s.high[li] - target,
+                             L.ring - L.window, 0,
+                             "dropping windowed layer %llu back to position %llu discards rows up to "
+                             "%llu positions ahead of it, past the %llu rows of ring headroom; reset "
+                             "the slot instead",
+                             ULL(li), ULL(target), ULL(s.high[li] - target), ULL(L.ring - L.window));
+    }
+    return ITAK_OK;
+}
+
 // Drops positions >= target on every layer of the slot (the caller validated the range).
+// Global layers truncate (cache.rs:788-791); windowed layers only move their length back: the
+// dropped rows stay in the ring's headroom, out of every later query's window, until the
+// positions are appended again.
 static itak_status truncate_slots(itak_pool *pool, const uint32_t *slots, const uint64_t *targets,
                                   uint32_t count) {
-    if (pool->cfg.flags & ITAK_POOL_SCRUB_ON_TRUNCATE) {
+    if ((pool->cfg.flags & ITAK_POOL_SCRUB_ON_TRUNCATE) && pool->global_layers) {
         for (uint32_t first = 0; first < count; first += kMaxBatchItems) {
             const uint32_t n = std::min<uint32_t>(kMaxBatchItems, count - first);
             ZeroBatch zb{};
             for (uint32_t i = 0; i < n; ++i) {
                 const Slot &s = pool->slots[slots[first + i]];
                 uint64_t max_len = 0;
-                for (uint64_t a : s.appended) max_len = std::max(max_len, a);
+                for (uint64_t li = 0; li < s.appended.size(); ++li)
+                    if (!pool->layers[li].windowed) max_len = std::max(max_len, s.appended[li]);
                 if (max_len <= targets[first + i]) continue;
                 zb.item[zb.n++] = ZeroItem{slots[first + i], uint32_t(targets[first + i]),
                                            uint32_t(max_len), 0};
@@ -1216,7 +1486,11 @@ static itak_status truncate_slots(itak_pool *pool, const uint32_t *slots, const 
     }
     for (uint32_t i = 0; i < count; ++i) {
         Slot &s = pool->slots[slots[i]];
-        for (uint64_t &a : s.appended) a = std::min(a, targets[i]);  // cache.rs:788-791,814
+        for (uint64_t li = 0; li < s.appended.size(); ++li) {
+            s.appended[li] = std::min(s.appended[li], targets[i]);  // cache.rs:788-791,814
+            // Scrubbed or not, a global layer's dropped rows are never read again.
+            if (!pool->layers[li].windowed) s.high[li] = s.appended[li];
+        }
     }
     return ITAK_OK;
 }
@@ -1234,6 +1508,8 @@ itak_status itak_kv_rewind_to(itak_pool *pool, uint32_t slot, const itak_checkpo
         if (target < base || target > s->appended[li])
             return rewind_range(pool->err, li, base, s->appended[li], target);
     }
+    st = check_ring_rewind(pool, *s, target);
+    if (st != ITAK_OK) return st;
     return truncate_slots(pool, &slot, &target, 1);
 }
 
@@ -1259,6 +1535,8 @@ itak_status itak_kv_truncate(itak_pool *pool, const uint32_t *slots, const uint6
         for (uint64_t li = 0; li < s->appended.size(); ++li)
             if (new_lengths[i] > s->appended[li])
                 return rewind_range(pool->err, li, 0, s->appended[li], new_lengths[i]);
+        itak_status st = check_ring_rewind(pool, *s, new_lengths[i]);
+        if (st != ITAK_OK) return st;
     }
     return truncate_slots(pool, slots, new_lengths, count);
 }
@@ -1282,10 +1560,18 @@ itak_status itak_gqa_attention(itak_pool *pool, uint32_t slot, uint64_t layer, c
         return non_divisible(pool->err, num_q_heads, pool->g.kv_heads);
     if (!q || !out || !query_positions)
         return invalid_argument(pool->err, "q, out or query_positions is null");
-    const uint64_t stored = s->appended[layer];
-    // A global layer's view holds positions 0..stored: a query sees at least position 0
-    // unless the view is empty (attention.rs:160-173).
-    if (stored == 0) return no_visible_keys(pool->err, query_positions[0]);
+    // The view holds positions oldest..appended; a query sees those at or below its own
+    // position and inside its window (attention.rs:77-85,160-173).
+    const uint64_t appended = s->appended[layer];
+    const uint64_t oldest = first_visible(pool, *s, layer);
+    const uint64_t window = pool->layers[layer].window;
+    for (uint64_t i = 0; i < num_queries; ++i) {
+        const uint64_t p = query_positions[i];
+        const uint64_t newest_seen = std::min(p + 1, appended);  // exclusive
+        const uint64_t oldest_seen =
+            std::max(oldest, (window && p + 1 > window) ? p + 1 - window : 0);
+        if (newest_seen <= oldest_seen) return no_visible_keys(pool->err, p);
+    }
     if (std::isnan(scale)) scale = default_scale(pool->g.head_dim);
 
     bool consecutive = true;
@@ -1311,7 +1597,7 @@ itak_status itak_gqa_attention(itak_pool *pool, uint32_t slot, uint64_t layer, c
     }
     PlanInput pi{slot, uint32_t(num_queries),
                  uint32_t(std::min<uint64_t>(query_positions[0], 0xffffffffu - num_queries)),
-                 uint32_t(stored)};
+                 uint32_t(appended), uint32_t(oldest)};
     st = run_attention(pool, layer, &pi, 1, qd, od, consecutive ? nullptr : pd, num_q_heads, scale,
                        softcap);
     if (st != ITAK_OK) return st;
@@ -1337,7 +1623,7 @@ static itak_status step_on_device(itak_pool *pool, uint64_t layer, const itak_ba
                                        nullptr);
     if (fuse) {
         for (uint32_t i = 0; i < item_count; ++i)
-            pool->slots[items[i].slot].appended[layer] += items[i].rows;
+            advance(pool->slots[items[i].slot], layer, items[i].rows);
         return run_attention(pool, layer, active.data(), uint32_t(active.size()), q_dev, out_dev,
                              nullptr, num_q_heads, scale, softcap, k_dev, v_dev);
     }
@@ -1364,9 +1650,15 @@ static itak_status plan_step(itak_pool *pool, uint64_t layer, const itak_batch_i
         uint64_t ok = 0;
         itak_status st = check_append_rows(pool, *s, layer, items[i].rows, &ok);
         if (st != ITAK_OK) return st;
+        st = check_block_rows(pool, layer, items[i].rows);
+        if (st != ITAK_OK) return st;
         const uint64_t base = s->appended[layer];
+        // The block's first row still sees its whole window: the rows below the view of the
+        // block's end are kept by the ring's headroom.
+        const uint64_t window = pool->layers[layer].window;
+        const uint64_t lo = (window && base + 1 > window) ? base + 1 - window : 0;
         plan.push_back(PlanInput{items[i].slot, items[i].rows, uint32_t(base),
-                                 uint32_t(base + items[i].rows)});
+                                 uint32_t(base + items[i].rows), uint32_t(lo)});
     }
     return ITAK_OK;
 }
@@ -1486,8 +1778,10 @@ itak_status itak_attention_device(itak_pool *pool, uint64_t layer, const itak_ba
         if (len == 0) return no_visible_keys(pool->err, 0);
         if (items[i].rows > len)
             return shape_mismatch(pool->err, "query rows", len, items[i].rows);
+        // The newest `rows` positions query the view as it stands: nothing older than the
+        // view's first row is promised to be in the ring.
         plan.push_back(PlanInput{items[i].slot, items[i].rows, uint32_t(len - items[i].rows),
-                                 uint32_t(len)});
+                                 uint32_t(len), uint32_t(first_visible(pool, *s, layer))});
     }
     if (std::isnan(scale)) scale = default_scale(pool->g.head_dim);
     return run_attention(pool, layer, plan.data(), uint32_t(plan.size()), q_dev, out_dev, nullptr,
@@ -1555,20 +1849,37 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
     float *vd = reinterpret_cast<float *>(pool->stage + 2 * q_bytes + kv_bytes);
     HIP_TRY(pool, hipMemcpyAsync(kd, k, k_len * 4, hipMemcpyHostToDevice, pool->stream), "upload k");
     HIP_TRY(pool, hipMemcpyAsync(vd, v, v_len * 4, hipMemcpyHostToDevice, pool->stream), "upload v");
-    itak_batch_item item{slot, uint32_t(ok_rows)};
-    st = run_append(pool, layer, &item, 1, kd, vd);
-    if (st != ITAK_OK) return st;
+    // The reference appends and attends row by row (cpu.rs:586-646). Here a block is appended
+    // whole and attended under the causal mask, which is the same thing on a global layer; on
+    // a windowed layer a block may be as long as the ring's headroom, so longer inputs go in
+    // several blocks.
+    const LayerInfo &L = pool->layers[layer];
+    const uint64_t block_cap = L.windowed ? L.ring - L.window : std::max<uint64_t>(rows, 1);
     if (refusal != ITAK_OK) {
+        for (uint64_t done = 0; done < ok_rows; done += block_cap) {
+            itak_batch_item item{slot, uint32_t(std::min(block_cap, ok_rows - done))};
+            st = run_append(pool, layer, &item, 1, kd + done * pool->row, vd + done * pool->row);
+            if (st != ITAK_OK) return st;
+        }
         HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after append");
         pool->err = saved;
         pool->err.info.code = ITAK_STEP_FAILED;
         return ITAK_STEP_FAILED;
     }
     HIP_TRY(pool, hipMemcpyAsync(qd, q, q_len * 4, hipMemcpyHostToDevice, pool->stream), "upload q");
-    PlanInput pi{slot, uint32_t(rows), uint32_t(appended), uint32_t(appended + rows)};
-    st = run_attention(pool, layer, &pi, 1, qd, od, nullptr, num_q_heads,
-                       default_scale(pool->g.head_dim), softcap);  // AttentionParams::new(), cpu.rs:584
-    if (st != ITAK_OK) return st;
+    for (uint64_t done = 0; done < rows; done += block_cap) {
+        const uint64_t n = std::min(block_cap, rows - done);
+        itak_batch_item item{slot, uint32_t(n)};
+        st = run_append(pool, layer, &item, 1, kd + done * pool->row, vd + done * pool->row);
+        if (st != ITAK_OK) return st;
+        const uint64_t base = appended + done;
+        const uint64_t lo = (L.window && base + 1 > L.window) ? base + 1 - L.window : 0;
+        PlanInput pi{slot, uint32_t(n), uint32_t(base), uint32_t(base + n), uint32_t(lo)};
+        st = run_attention(pool, layer, &pi, 1, qd + done * q_width, od + done * q_width, nullptr,
+                           num_q_heads, default_scale(pool->g.head_dim),
+                           softcap);  // AttentionParams::new(), cpu.rs:584
+        if (st != ITAK_OK) return st;
+    }
     HIP_TRY(pool, hipMemcpyAsync(out, od, q_len * 4, hipMemcpyDeviceToHost, pool->stream),
             "download attention output");
     HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after attention");

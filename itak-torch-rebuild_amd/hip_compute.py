@@ -180,7 +180,7 @@ class KvPool:
 
     def __init__(self, pattern: Union[int, Sequence[LayerKind]], num_kv_heads: int, head_dim: int,
                  *, elem: str = "f16", max_slots: int = 1, capacity_rows: int = 4096,
-                 device: int = 0, scrub_on_truncate: bool = True):
+                 device: int = 0, scrub_on_truncate: bool = True, ring_headroom: int = 0):
         if isinstance(pattern, int):
             pattern = [LayerKind.Global] * pattern
         self.pattern = list(pattern)
@@ -201,6 +201,7 @@ class KvPool:
         cfg.capacity_rows = capacity_rows
         cfg.device = device
         cfg.flags = N.POOL_SCRUB_ON_TRUNCATE if scrub_on_truncate else 0
+        cfg.ring_headroom = ring_headroom
         handle = C.c_void_p()
         self._h = None
         self._lib = N.load()
@@ -330,10 +331,10 @@ class KvCache:
 
     @staticmethod
     def new(pattern: Sequence[LayerKind], num_kv_heads: int, head_dim: int, *, elem: str = "f32",
-            capacity_rows: int = 4096, device: int = 0) -> "KvCache":
+            capacity_rows: int = 4096, device: int = 0, ring_headroom: int = 0) -> "KvCache":
         """KvCache::new: a private one-slot pool. f32 storage is the reference's."""
         pool = KvPool(pattern, num_kv_heads, head_dim, elem=elem, max_slots=1,
-                      capacity_rows=capacity_rows, device=device)
+                      capacity_rows=capacity_rows, device=device, ring_headroom=ring_headroom)
         cache = pool.acquire()
         cache._owns_pool = True
         return cache
@@ -424,7 +425,9 @@ class KvCache:
 
     def read_raw(self, layer: int):
         """Every storage row of the layer, visible or not: (keys, values)."""
-        shape = (self.pool.capacity_rows, self.pool.num_kv_heads, self.pool.head_dim)
+        rows = C.c_uint64()
+        _check(self._h, self._lib.itak_kv_storage_rows(self._h, layer, C.byref(rows)))
+        shape = (rows.value, self.pool.num_kv_heads, self.pool.head_dim)
         keys = np.empty(shape, dtype=self.pool.np_elem)
         vals = np.empty(shape, dtype=self.pool.np_elem)
         _check(self._h, self._lib.itak_kv_read_raw(self._h, self.slot, layer, _ptr(keys),

@@ -147,6 +147,11 @@ def test_matches_the_oracle_on_seeded_shapes(elem, n, qh, kvh, d, nq, softcap):
     got = P().gqa_attention(q, nq, qh, positions, g.view(0), P().AttentionParams(**params))
     want = oracle.gqa_attention(q, nq, qh, positions, c.view(0), oracle.AttentionParams(**params))
     assert (rel_err(got, want) <= F32_REL) if elem == "f32" else (max_abs(got, want) <= F16_ABS)
+    # Consecutive positions ahead of the stored rows: every query sees the whole cache.
+    positions = list(range(n + 2, n + 2 + nq))
+    got = P().gqa_attention(q, nq, qh, positions, g.view(0), P().AttentionParams(**params))
+    want = oracle.gqa_attention(q, nq, qh, positions, c.view(0), oracle.AttentionParams(**params))
+    assert (rel_err(got, want) <= F32_REL) if elem == "f32" else (max_abs(got, want) <= F16_ABS)
 
 
 def glimmer_cfg(layers=2, q_heads=8, kv_heads=2, d=16):
