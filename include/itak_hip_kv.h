@@ -72,7 +72,15 @@ enum {
     ITAK_KV_INCONSISTENT_SNAPSHOT = 25,
     ITAK_KV_GEOMETRY_MISMATCH = 26,
     ITAK_KV_FINGERPRINT_MISMATCH = 27,
-    ITAK_KV_INCOHERENT_CACHE = 28
+    ITAK_KV_INCOHERENT_CACHE = 28,
+    /* The variants the prefix store adds (crates/itak-kv/src/store.rs). */
+    ITAK_KV_EMPTY_PREFIX = 29,
+    ITAK_KV_TOKEN_COUNT_MISMATCH = 30,    /* a = snapshot, b = tokens */
+    ITAK_KV_PREFIX_HASH_MISMATCH = 31,    /* a = stored, b = computed */
+    ITAK_KV_SNAPSHOT_TOKEN_MISMATCH = 32, /* a = entry, b = snapshot */
+    ITAK_KV_ENTRY_TOO_LARGE = 33,         /* a = bytes, b = cap */
+    ITAK_KV_INVALID_CONFIG = 34,
+    ITAK_KV_IO = 35                       /* what = context, a = errno; message as std::io::Error prints it */
 };
 
 /* Storage / source element types. */
@@ -318,6 +326,94 @@ itak_status itak_kv_capture_itkv(itak_pool *pool, uint32_t slot, const char *fin
 itak_status itak_kv_restore_itkv(itak_pool *pool, uint32_t slot, const void *bytes, uint64_t len,
                                  const char *expected_fingerprint,
                                  uint64_t expected_fingerprint_len);
+
+/* ---- persistent prefix store (crates/itak-kv/src/store.rs) ------------------------- */
+
+/* itak_kv::PrefixStore (store.rs:128-543): one file per entry under a root directory, keyed by
+   token prefix, bounded by a byte cap with LRU eviction. Entry files are the reference's
+   byte for byte (store.rs:5-22), so both implementations serve each other's directories.
+   Host code: a store works without a device. Not thread-safe, like the reference's. */
+typedef struct itak_store itak_store;
+
+/* store.rs:77-91. */
+typedef struct itak_store_entry {
+    char file_name[96];
+    uint64_t prefix_hash;
+    uint64_t token_count;
+    uint64_t bytes;
+    uint64_t created_unix;
+    uint64_t last_used_unix;
+} itak_store_entry;
+
+/* store.rs:108-116. */
+typedef struct itak_store_stats {
+    uint64_t entries;
+    uint64_t total_bytes;
+    uint64_t max_bytes;
+} itak_store_stats;
+
+/* store.rs:94-105. token_count == 0 means no stored prefix matched. The matched ids are the
+   first token_count ids of the query (verified equal). `snapshot` points at the verified
+   ITKV v1 bytes inside the store's staging buffer (pinned host memory when a device is
+   present, so itak_kv_restore_itkv gathers from it in place); valid until the next call on
+   this store. */
+typedef struct itak_prefix_hit {
+    uint64_t token_count;
+    const void *snapshot;
+    uint64_t snapshot_len;
+    char file_name[96];
+} itak_prefix_hit;
+
+/* itak_kv::now_unix (store.rs:120-126). */
+uint64_t itak_kv_now_unix(void);
+/* PrefixStore::open (store.rs:147-168): creates the root if needed and indexes every
+   well-formed entry; malformed files are named in the refusal log and left alone. */
+itak_status itak_store_open(const char *root, uint64_t max_bytes, itak_store **out);
+void itak_store_close(itak_store *store);
+/* Message / fields of the last failure on this store (NULL: of the last failed open on this
+   thread). Messages are KvError's Display text (crates/itak-kv/src/error.rs:141-188). */
+const char *itak_store_last_error(const itak_store *store);
+itak_status itak_store_last_error_info(const itak_store *store, itak_error_info *out);
+/* What the reference writes to its diag channel when it refuses an entry or skips a restore:
+   one line per refusal, accumulated until cleared. */
+const char *itak_store_refusals(const itak_store *store);
+void itak_store_clear_refusals(itak_store *store);
+/* PrefixStore::rescan (store.rs:204-224). */
+itak_status itak_store_rescan(itak_store *store);
+/* PrefixStore::stats (store.rs:185-192). */
+itak_status itak_store_get_stats(itak_store *store, itak_store_stats *out);
+/* PrefixStore::entries (store.rs:177-182): longest prefix first. With out == NULL only
+   *count is set. */
+itak_status itak_store_entries(itak_store *store, itak_store_entry *out, uint64_t capacity,
+                               uint64_t *count);
+/* PrefixStore::put (store.rs:236-300) of an encoded snapshot: strict decode (the refusals of
+   KvSnapshot::from_bytes), token count against the ids, the cap, atomic write, LRU eviction. */
+itak_status itak_store_put(itak_store *store, const uint32_t *tokens, uint64_t token_count,
+                           const void *snapshot, uint64_t snapshot_len, uint64_t now);
+/* PrefixStore::lookup (store.rs:314-357): the longest stored prefix of `query` that passes
+   every trust check (store.rs:364-452). expected_geometry (num_kv_heads, head_dim, layer_count
+   are read) with expected_layers (kind, window) and fingerprint are optional requirements
+   (NULL = none). A verified hit is restamped to `now`. */
+itak_status itak_store_lookup(itak_store *store, const uint32_t *query, uint64_t query_len,
+                              const itak_itkv_header *expected_geometry,
+                              const itak_itkv_layer *expected_layers, const char *fingerprint,
+                              uint64_t fingerprint_len, uint64_t now, itak_prefix_hit *hit);
+/* ResidentSession::restore_prefix_from_store
+   (crates/wgpu-compute/src/session.rs:5000-5053): looks `tokens` up under the pool's own
+   pattern and the fingerprint and restores the hit into the (fresh) slot. *matched = tokens
+   now in the slot, 0 when nothing was restored (no hit, slot not fresh, hit refused by the
+   install checks: named in the refusal log, slot untouched). Only a device failure is an
+   error. */
+itak_status itak_store_restore_prefix(itak_store *store, itak_pool *pool, uint32_t slot,
+                                      const uint32_t *tokens, uint64_t token_count,
+                                      const char *fingerprint, uint64_t fingerprint_len,
+                                      uint64_t now, uint64_t *matched);
+/* ResidentSession::capture_and_store_prefix (session.rs:5056-5094): the slot must stand at
+   exactly token_count positions; its rows are captured as ITKV v1 and put under `tokens`. */
+itak_status itak_store_capture_and_put(itak_store *store, itak_pool *pool, uint32_t slot,
+                                       const uint32_t *tokens, uint64_t token_count,
+                                       const char *fingerprint, uint64_t fingerprint_len,
+                                       uint64_t now);
 
 /* ---- attention over one slot, host pointers ---------------------------------------- */
 

@@ -33,6 +33,17 @@ from .itak_kv import (  # noqa: F401
     prefix_hash,
     restore_bytes,
 )
+from .prefix_store import (  # noqa: F401
+    EntryMeta,
+    PrefixHit,
+    PrefixStore,
+    StoreConfig,
+    StoreStats,
+    max_bytes_from,
+    now_unix,
+    prefix_store_enabled,
+    prefix_store_enabled_from,
+)
 from . import _native  # noqa: F401
 
 __all__ = [
@@ -41,4 +52,6 @@ __all__ = [
     "PositionCache", "StepFailed", "gqa_attention", "kv_head_for_query_head",
     "KvError", "KvGeometry", "KvSnapshot", "LayerSnapshot", "SNAPSHOT_FORMAT_VERSION",
     "capture_bytes", "checksum", "prefix_discriminator", "prefix_hash", "restore_bytes",
+    "EntryMeta", "PrefixHit", "PrefixStore", "StoreConfig", "StoreStats", "max_bytes_from",
+    "now_unix", "prefix_store_enabled", "prefix_store_enabled_from",
 ]

@@ -22,8 +22,10 @@ STATUS_NAMES = {
     21: "BadMagic", 22: "UnsupportedVersion", 23: "Truncated", 24: "ChecksumMismatch",
     25: "InconsistentSnapshot", 26: "GeometryMismatch", 27: "FingerprintMismatch",
     28: "IncoherentCache",
+    29: "EmptyPrefix", 30: "TokenCountMismatch", 31: "PrefixHashMismatch",
+    32: "SnapshotTokenMismatch", 33: "EntryTooLarge", 34: "InvalidConfig", 35: "Io",
 }
-KV_ERROR_FIRST, KV_ERROR_LAST = 21, 28
+KV_ERROR_FIRST, KV_ERROR_LAST = 21, 35
 ELEM_F32, ELEM_F16 = 0, 1
 LAYER_GLOBAL, LAYER_WINDOWED = 0, 1
 POOL_SCRUB_ON_TRUNCATE = 1
@@ -88,6 +90,21 @@ class ItkvLayer(C.Structure):
                 ("keys_offset", C.c_uint64), ("values_offset", C.c_uint64)]
 
 
+class StoreEntry(C.Structure):
+    _fields_ = [("file_name", C.c_char * 96), ("prefix_hash", C.c_uint64),
+                ("token_count", C.c_uint64), ("bytes", C.c_uint64), ("created_unix", C.c_uint64),
+                ("last_used_unix", C.c_uint64)]
+
+
+class StoreStats(C.Structure):
+    _fields_ = [("entries", C.c_uint64), ("total_bytes", C.c_uint64), ("max_bytes", C.c_uint64)]
+
+
+class PrefixHit(C.Structure):
+    _fields_ = [("token_count", C.c_uint64), ("snapshot", C.c_void_p),
+                ("snapshot_len", C.c_uint64), ("file_name", C.c_char * 96)]
+
+
 _P = C.c_void_p
 _u32, _u64, _f32, _i32 = C.c_uint32, C.c_uint64, C.c_float, C.c_int32
 
@@ -145,6 +162,22 @@ PROTOTYPES = {
     "itak_attention_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P, _u64, _f32,
                                      _f32]),
     "itak_kv_append_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P]),
+    "itak_kv_now_unix": (_u64, []),
+    "itak_store_open": (_i32, [C.c_char_p, _u64, C.POINTER(_P)]),
+    "itak_store_close": (None, [_P]),
+    "itak_store_last_error": (C.c_char_p, [_P]),
+    "itak_store_last_error_info": (_i32, [_P, C.POINTER(ErrorInfo)]),
+    "itak_store_refusals": (C.c_char_p, [_P]),
+    "itak_store_clear_refusals": (None, [_P]),
+    "itak_store_rescan": (_i32, [_P]),
+    "itak_store_get_stats": (_i32, [_P, C.POINTER(StoreStats)]),
+    "itak_store_entries": (_i32, [_P, C.POINTER(StoreEntry), _u64, C.POINTER(_u64)]),
+    "itak_store_put": (_i32, [_P, _P, _u64, _P, _u64, _u64]),
+    "itak_store_lookup": (_i32, [_P, _P, _u64, C.POINTER(ItkvHeader), C.POINTER(ItkvLayer),
+                                 C.c_char_p, _u64, _u64, C.POINTER(PrefixHit)]),
+    "itak_store_restore_prefix": (_i32, [_P, _P, _u32, _P, _u64, C.c_char_p, _u64, _u64,
+                                         C.POINTER(_u64)]),
+    "itak_store_capture_and_put": (_i32, [_P, _P, _u32, _P, _u64, C.c_char_p, _u64, _u64]),
     "itak_convert_f32_to_f16_device": (_i32, [_P, _P, _P, _u64]),
     "itak_probe_copy_device": (_i32, [_P, _P, _P, _u64]),
     "itak_probe_empty_launch": (_i32, [_P]),
