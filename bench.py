@@ -14,7 +14,9 @@ the CPU oracle timed on the host cores beside it.
 
 `--workload ragged|verify|prefill` measures the other configurations (continuous batching
 over 16 ragged slots, the speculative verify block, the chunked causal prefill) with the
-same JSON shape; `--workload restore|append` measures the cache-maintenance kernels (the
+same JSON shape; `--workload hybrid` a decode step over the reference model's own layer
+pattern (three sliding-window layers of 2048 to one global layer, crates/attention/src/
+cache.rs:66-84) at context 32768; `--workload restore|append` measures the cache-maintenance kernels (the
 48-layer prefix-snapshot gather of configs[4]; the append of a 2048-row chunk). They are
 secondary measurements, the default line is the contract.
 """
@@ -237,8 +239,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["decode", "ragged", "verify", "prefill", "restore", "append"],
-                    default="decode")
+    ap.add_argument("--workload", choices=["decode", "ragged", "verify", "prefill", "hybrid",
+                                           "restore", "append"], default="decode")
     ap.add_argument("--softcap", type=float, default=0.0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -277,15 +279,28 @@ def main():
         layers, slots, rows, lengths = 16, 4, 7, [8192] * 4
         name = ("configs[3]: speculative verify block, 4 slots at context 8192, 7 query rows "
                 "appended and attended causally, 30B-class heads, f16 KV, 16 layers cycled")
+    elif wl == "hybrid":
+        layers, slots, rows, lengths = 8, 1, 1, [32768]
+        name = ("hybrid decode step: sliding-window layers (window 2048) and global layers 3:1, "
+                "the pattern of the reference's 52-layer model, batch 1, context 32768, 30B-class "
+                "heads, f16 KV, 8 layers cycled (6 windowed, 2 global)")
     else:
         layers, slots, rows, lengths = 4, 1, 2048, [30720]
         name = ("configs[4]: chunked causal prefill, 2048-row chunk over a 30720-token prefix, "
                 "30B-class heads, f16 KV, f32 accumulate, 4 layers cycled")
     max_len = max(lengths)
-    kv_bytes_layer = sum(2 * (n + rows) * KV_HEADS * D * 2 for n in lengths)
+    window = 2048
+    pattern = [pkg.LayerKind.Global] * layers
+    if wl == "hybrid":  # glimmer_layer_pattern: every fourth layer global
+        pattern = [pkg.LayerKind.Global if (i + 1) % 4 == 0 else pkg.LayerKind.windowed(window)
+                   for i in range(layers)]
+    # Rows a layer's attention reads per slot: everything stored, or the window.
+    visible = [[min(n + rows, window + rows - 1) if kind.is_windowed else n + rows for n in lengths]
+               for kind in pattern]
+    kv_bytes_layer = sum(sum(2 * r * KV_HEADS * D * 2 for r in per) for per in visible) // layers
     flops_layer = sum(4 * D * Q_HEADS * (rows * n + rows * (rows + 1) // 2) for n in lengths)
 
-    pool = pkg.KvPool(layers, KV_HEADS, D, elem="f16", max_slots=slots,
+    pool = pkg.KvPool(pattern, KV_HEADS, D, elem="f16", max_slots=slots,
                       capacity_rows=max_len + rows + 8, scrub_on_truncate=False)
     pool.set_stream(stream.cuda_stream)
     caches = [pool.acquire() for _ in range(slots)]
@@ -301,8 +316,14 @@ def main():
     for layer in range(layers):
         for s, n in enumerate(lengths):
             k = rope_on_device(torch.randn(n, KV_HEADS, D, device=dev), 1e6).reshape(n, ROW)
+            k = k.contiguous()
             v = torch.randn(n, ROW, device=dev)
-            pool.append_device(layer, [(caches[s], n)], k.contiguous().data_ptr(), v.data_ptr())
+            if pattern[layer].is_windowed:  # the last `window` rows, where a prefill leaves them
+                first = max(0, n - window)
+                caches[s].restore_bulk_ptr(layer, first, k[first:].data_ptr(), v[first:].data_ptr(),
+                                           (n - first) * ROW, src_f16=False)
+            else:
+                pool.append_device(layer, [(caches[s], n)], k.data_ptr(), v.data_ptr())
             torch.cuda.synchronize()
     items = [(c, rows) for c in caches]
     ptrs = [(q[l].data_ptr(), k_new[l].data_ptr(), v_new[l].data_ptr(), out[l].data_ptr())
@@ -395,7 +416,7 @@ def main():
             "softcap": args.softcap,
             "arithmetic": "f16 KV and MFMA operands, f32 scores, softmax and accumulation",
         },
-        "us_per_token": round(step_s * 1e6 * (48 / layers), 2),
+        "us_per_token": round(step_s * 1e6 * ((52 if wl == "hybrid" else 48) / layers), 2),
         "pct_of_hbm_peak": round(100.0 * kv_bytes_layer * layers / step_s / 1e9 / HBM_PEAK_GBS, 2),
         "eager": {
             "us_per_step_stream": round(eager_s / args.steps * 1e6, 2),
