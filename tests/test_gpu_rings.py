@@ -540,3 +540,53 @@ def test_snapshots_of_a_hybrid_cache_round_trip_and_match_the_oracles_bytes(elem
     assert e.value.variant == "GeometryMismatch"
     other_pool.close()
     pool.close()
+
+
+# ---------------------------------------------------------------- Compute::attention mirror
+
+
+@pytest.mark.parametrize("elem", ["f32", "f16"])
+def test_compute_attention_on_a_hybrid_model_takes_any_number_of_rows(elem):
+    # cpu.rs:586-646 on the reference model's kind of pattern: the host-pointer call appends
+    # and attends row by row in the reference, so a prompt longer than the device ring's
+    # headroom (and longer than the window) must come out the same, and decoding on from it
+    # too.
+    rng = np.random.default_rng(41)
+    SW, G = P().LayerKind.SlidingWindow, P().LayerKind.Global
+    cfg = P().GlimmerConfig(layers=[SW, SW, G], q_heads=8, kv_heads=2, key_length=16,
+                            value_length=16, sliding_window=20)
+    ref = oracle.KvCache.new([oracle.LayerKind.windowed(20), oracle.LayerKind.windowed(20),
+                              oracle.LayerKind.Global], cfg.kv_heads, cfg.key_length,
+                             store_f16=(elem == "f16"))
+    hc = P().HipCompute.new(elem=elem, capacity_rows=512)
+    cache = P().PositionCache()
+    for rows in (150, 1, 1, 70, 1):
+        for layer, kind in enumerate(cfg.layers):
+            q = normal(rng, rows, cfg.q_width())
+            k = normal(rng, rows, cfg.k_width())
+            v = normal(rng, rows, cfg.v_width())
+            got = hc.attention(P().AttentionRequest(q, k, v, layer, kind, cfg), cache)
+            want = oracle.attention_step(ref, layer, q, k, v, cfg.q_heads, cache.position(),
+                                         threads=8)
+            if elem == "f32":
+                assert rel_err(got, want) <= 1e-5, (rows, layer)
+            else:
+                assert max_abs(got, want) <= 2e-3, (rows, layer)
+        cache.advance(rows)
+    dev = hc.kv_cache()
+    for layer in range(3):
+        assert dev.next_position(layer) == 223
+        assert view_snapshot(dev, layer) == view_snapshot(ref, layer)
+    # A speculative round through the Compute-level calls, on the hybrid cache.
+    cp = hc.cache_checkpoint(4)
+    rcp = ref.checkpoint(4)
+    for layer, kind in enumerate(cfg.layers):
+        q, k, v = normal(rng, 4, cfg.q_width()), normal(rng, 4, cfg.k_width()), normal(rng, 4, cfg.v_width())
+        hc.attention(P().AttentionRequest(q, k, v, layer, kind, cfg), cache)
+        oracle.attention_step(ref, layer, q, k, v, cfg.q_heads, 223, threads=8)
+    hc.cache_rewind(cp, 225)
+    ref.rewind_to(rcp, 225)
+    hc.cache_release(cp)
+    ref.release(rcp)
+    for layer in range(3):
+        assert view_snapshot(dev, layer) == view_snapshot(ref, layer)
