@@ -35,6 +35,10 @@ struct Slot {
     // last fresh. Positions in [appended, high) were dropped by a rewind; on a windowed layer
     // their rows still sit in the ring and alias the positions one ring length below them.
     std::vector<uint64_t> high;
+    // Per layer: the oldest position the storage was ever given. 0 for a sequence appended
+    // from its start; the first restored position of a windowed layer filled from a snapshot,
+    // which carries only the last `window` rows: nothing below it can come back into view.
+    std::vector<uint64_t> floor;
     LiveCheckpoint cp;
 };
 
@@ -764,6 +768,7 @@ itak_status itak_slot_acquire(itak_pool *pool, uint32_t *slot) {
         s.cache_id = g_next_cache_id++;
         s.appended.assign(pool->cfg.layer_count, 0);
         s.high.assign(pool->cfg.layer_count, 0);
+        s.floor.assign(pool->cfg.layer_count, 0);
         *slot = i;
         return ITAK_OK;
     }
@@ -803,6 +808,7 @@ itak_status itak_slot_reset(itak_pool *pool, uint32_t slot) {
     }
     std::fill(s->appended.begin(), s->appended.end(), 0);
     std::fill(s->high.begin(), s->high.end(), 0);
+    std::fill(s->floor.begin(), s->floor.end(), 0);
     s->built = false;
     s->cp = LiveCheckpoint{};
     s->next_serial = 0;
@@ -1011,6 +1017,7 @@ static itak_status restore_layers(itak_pool *pool, uint32_t slot, Slot &s,
         const uint64_t layer = layer_ids ? layer_ids[i] : i;
         s.appended[layer] = layers[i].first_position + layers[i].rows;  // cache.rs:568
         s.high[layer] = s.appended[layer];
+        s.floor[layer] = layers[i].first_position;
     }
     return ITAK_OK;
 }
@@ -1449,6 +1456,10 @@ static itak_status check_ring_rewind(itak_pool *pool, const Slot &s, uint64_t ta
     for (uint64_t li = 0; li < s.appended.size(); ++li) {
         const LayerInfo &L = pool->layers[li];
         if (!L.windowed || target >= s.appended[li]) continue;
+        // A layer restored from a snapshot holds nothing older than the snapshot's first row:
+        // the view of a target below first + window would reach under it.
+        if (s.floor[li] > 0 && target < s.floor[li] + L.window)
+            return rewind_range(pool->err, li, s.floor[li] + L.window, s.appended[li], target);
         if (s.high[li] - target > L.ring - L.window)
             return set_error(pool->err, ITAK_CAPACITY_EXCEEDED, nullptr, li, s.high[li] - target,
                              L.ring - L.window, 0,

@@ -334,6 +334,42 @@ def test_bulk_restore_refusals_on_rings_are_named():
     assert e.value == E("BulkRestoreNotFresh", layer=0, appended=13)
 
 
+def test_a_ring_rewound_to_empty_restores_like_a_fresh_one():
+    # restore_bulk needs a fresh layer (cache.rs:524-529); a layer rewound to position 0 is
+    # fresh by that rule, and rows the restore does not write must read as a fresh cache's
+    # zeros, not as what the ring held before.
+    cache = P().KvCache.new([W(4)], 1, 2)
+    ref = oracle.KvCache.new([oracle.LayerKind.windowed(4)], 1, 2)
+    for p in range(12):
+        append(cache, 0, 1, 2, p)
+    cache.pool.truncate([cache.slot], [0])
+    rows = np.arange(1, 7, dtype=np.float32).reshape(3, 2)
+    cache.restore_bulk(0, 10, rows, rows)   # positions 10..12; position 9 is in view, unwritten
+    ref.restore_bulk(0, 10, rows, rows)
+    assert cache.next_position(0) == 13 and cache.stored_len(0) == 4
+    assert view_snapshot(cache, 0) == view_snapshot(ref, 0)
+    assert cache.view(0).key(0, 0).tolist() == [0.0, 0.0]
+
+
+def test_a_restored_ring_cannot_be_cut_back_under_its_snapshot():
+    # A snapshot of a windowed layer carries its last `window` rows only: a length below
+    # first + window would put rows in view that the slot never held.
+    pool = P().KvPool([W(8)], 1, 2, elem="f32", ring_headroom=16)
+    cache = pool.acquire()
+    rows = np.arange(16, dtype=np.float32).reshape(8, 2)
+    cache.restore_bulk(0, 40, rows, rows)          # positions 40..47
+    for p in range(48, 52):
+        cache.append(0, [float(p)] * 2, [float(p)] * 2, p)
+    pool.truncate([cache.slot], [49])
+    assert cache.view(0).rows()[0].tolist() == list(range(41, 49))
+    with pytest.raises(P().AttentionError) as e:
+        pool.truncate([cache.slot], [47])
+    assert e.value == E("RewindOutOfRange", layer=0, base=48, appended=49, target=47)
+    pool.truncate([cache.slot], [48])
+    assert cache.view(0).rows()[0].tolist() == list(range(40, 48))
+    pool.close()
+
+
 # ------------------------------------------------------------------------------ attention
 
 
