@@ -19,8 +19,9 @@
 // same MFMA, so K and V are read from HBM once per group. Scores, softmax state and
 // accumulators are f32; P and Q enter the MFMA as f16.
 //
-// Semantics: gqa_attention in crates/attention/src/attention.rs:104-215 on a global layer
-// (key kp visible to a query at position p iff kp <= p), with the optional softcap
+// Semantics: gqa_attention in crates/attention/src/attention.rs:104-215 (key kp visible to a
+// query at position p iff kp <= p and, on a windowed layer, kp > p - window), with the
+// optional softcap
 // cap*tanh(s/cap) of crates/torch-math/src/logits.rs:26-37 applied to the scaled scores.
 #include "internal.h"
 #include "mfma_common.h"
