@@ -428,9 +428,12 @@ itak_status itak_gqa_attention(itak_pool *pool, uint32_t slot, uint64_t layer, c
 
 /* ---- CpuCompute, per slot (crates/cpu-compute/src/cpu.rs) --------------------------- */
 
-/* Compute::attention on a global (NoPE) layer (cpu.rs:506-655): checks whole rows,
-   cross-checks cache_position against the slot's position for `layer`, then for
-   each row appends its K/V and attends at its own position. q is
+/* Compute::attention (cpu.rs:506-655): checks whole rows, cross-checks cache_position
+   against the slot's position for `layer`, then for each row appends its K/V and
+   attends at its own position. On a windowed (sliding-window) layer Q and K are first
+   rotated with the interleaved RoPE at rope_freq_base_swa, each row at its own position;
+   global layers are NoPE and pass through unrotated (cpu.rs:594-622; the base is
+   GlimmerConfig::rope_freq_base_swa and is not looked at on a global layer). q is
    [rows][q_heads*head_dim], k and v [rows][kv_heads*head_dim]; out has q_len
    elements. The slot is never advanced past what was appended: a failed call
    leaves it ahead of the caller's position and the next call refuses until
@@ -438,7 +441,7 @@ itak_status itak_gqa_attention(itak_pool *pool, uint32_t slot, uint64_t layer, c
 itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t layer, const float *q,
                                    uint64_t q_len, const float *k, uint64_t k_len, const float *v,
                                    uint64_t v_len, uint64_t num_q_heads, uint64_t cache_position,
-                                   float softcap, float *out);
+                                   float softcap, float rope_freq_base_swa, float *out);
 /* CpuCompute::cache_checkpoint / cache_rewind / cache_release (cpu.rs:270-339): the
    KvCache calls plus the "no KV state exists yet" refusals before a first forward. */
 itak_status itak_compute_cache_checkpoint(itak_pool *pool, uint32_t slot,

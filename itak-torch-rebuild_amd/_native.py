@@ -151,7 +151,7 @@ PROTOTYPES = {
     "itak_kv_truncate": (_i32, [_P, _P, _P, _u32]),
     "itak_gqa_attention": (_i32, [_P, _u32, _u64, _P, _u64, _u64, _u64, _P, _u64, _f32, _f32, _P]),
     "itak_compute_attention": (_i32, [_P, _u32, _u64, _P, _u64, _P, _u64, _P, _u64, _u64, _u64,
-                                      _f32, _P]),
+                                      _f32, _f32, _P]),
     "itak_compute_cache_checkpoint": (_i32, [_P, _u32, _u64, C.POINTER(CheckpointRaw)]),
     "itak_compute_cache_rewind": (_i32, [_P, _u32, C.POINTER(CheckpointRaw), _u64]),
     "itak_compute_cache_release": (_i32, [_P, _u32, C.POINTER(CheckpointRaw)]),

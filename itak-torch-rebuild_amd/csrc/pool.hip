@@ -1802,7 +1802,7 @@ itak_status itak_attention_device(itak_pool *pool, uint64_t layer, const itak_ba
 itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t layer, const float *q,
                                    uint64_t q_len, const float *k, uint64_t k_len, const float *v,
                                    uint64_t v_len, uint64_t num_q_heads, uint64_t cache_position,
-                                   float softcap, float *out) {
+                                   float softcap, float rope_freq_base_swa, float *out) {
     if (!pool) return ITAK_INVALID_ARGUMENT;
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
@@ -1843,6 +1843,17 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
         return ITAK_STEP_FAILED;
     }
     if (!q || !k || !v || !out) return invalid_argument(pool->err, "q, k, v or out is null");
+    // Sliding-window layers rotate Q and K (cpu.rs:594-622); torch_math::rope_interleaved's
+    // refusals (rope_interleaved.rs:72-99) surface under the attention step.
+    const bool rotate = pool->layers[layer].windowed;
+    if (rotate) {
+        if (pool->g.head_dim < 2 || pool->g.head_dim % 2 != 0)
+            return set_error(pool->err, ITAK_STEP_FAILED, step, 0, 0, 0, 0,
+                             "rope: head_dim must be even and >= 2");
+        if (!std::isfinite(rope_freq_base_swa) || rope_freq_base_swa <= 1.0f)
+            return set_error(pool->err, ITAK_STEP_FAILED, step, 0, 0, 0, 0,
+                             "rope: base must be finite and > 1");
+    }
 
     // Row-at-a-time appends stop at the first refusal (cpu.rs:623-631): rows before it are
     // in the cache when the call fails, exactly as in the reference.
@@ -1860,6 +1871,23 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
     float *vd = reinterpret_cast<float *>(pool->stage + 2 * q_bytes + kv_bytes);
     HIP_TRY(pool, hipMemcpyAsync(kd, k, k_len * 4, hipMemcpyHostToDevice, pool->stream), "upload k");
     HIP_TRY(pool, hipMemcpyAsync(vd, v, v_len * 4, hipMemcpyHostToDevice, pool->stream), "upload v");
+    HIP_TRY(pool, hipMemcpyAsync(qd, q, q_len * 4, hipMemcpyHostToDevice, pool->stream), "upload q");
+    if (rotate) {  // in place on the staged rows, row i at position appended + i
+        PrepArgs a{};
+        a.q_in = a.q_out = qd;
+        a.k_in = a.k_out = kd;
+        a.rope_base = rope_freq_base_swa;
+        a.interleaved = 1;
+        a.rotary_dim = pool->g.head_dim;
+        a.head_dim = pool->g.head_dim;
+        a.q_heads = uint32_t(num_q_heads);
+        a.kv_heads = pool->g.kv_heads;
+        a.total_rows = uint32_t(rows);
+        a.n = 1;
+        a.row0[0] = 0;
+        a.pos0[0] = uint32_t(appended);
+        HIP_TRY(pool, launch_attn_prep(a, pool->stream), "launch rope");
+    }
     // The reference appends and attends row by row (cpu.rs:586-646). Here a block is appended
     // whole and attended under the causal mask, which is the same thing on a global layer; on
     // a windowed layer a block may be as long as the ring's headroom, so longer inputs go in
@@ -1877,7 +1905,6 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
         pool->err.info.code = ITAK_STEP_FAILED;
         return ITAK_STEP_FAILED;
     }
-    HIP_TRY(pool, hipMemcpyAsync(qd, q, q_len * 4, hipMemcpyHostToDevice, pool->stream), "upload q");
     for (uint64_t done = 0; done < rows; done += block_cap) {
         const uint64_t n = std::min(block_cap, rows - done);
         itak_batch_item item{slot, uint32_t(n)};

@@ -652,7 +652,8 @@ class HipCompute:
         c = self._cache
         _check(c._h, c._lib.itak_compute_attention(
             c._h, c.slot, req.layer, _ptr(q), q.size, _ptr(k), k.size, _ptr(v), v.size,
-            cfg.q_heads, cache.position(), self._softcap, _ptr(out)), step)
+            cfg.q_heads, cache.position(), self._softcap, cfg.rope_freq_base_swa, _ptr(out)),
+            step)
         return out
 
     def _need_cache(self) -> KvCache:

@@ -631,3 +631,20 @@ def attention_step(cache: KvCache, layer: int, q, k, v, num_q_heads: int, start_
     if rc != 0:
         _raise(err)
     return out
+
+
+def compute_attention(cache: KvCache, layer: int, q, k, v, num_q_heads: int, start_position: int,
+                      rope_freq_base_swa: float, params: AttentionParams = AttentionParams(),
+                      threads: int = 1) -> np.ndarray:
+    """The body of CpuCompute::attention (cpu.rs:586-646): on a sliding-window layer every
+    row's Q and K heads are rotated with the interleaved RoPE at the SWA base and the row's
+    own position (rope_row, cpu.rs:398-418); global layers pass through. Then the per-row
+    append-then-attend loop."""
+    d = cache.head_dim()
+    q = np.ascontiguousarray(q, dtype=np.float32).reshape(-1, num_q_heads * d)
+    k = np.ascontiguousarray(k, dtype=np.float32).reshape(-1, cache.num_kv_heads() * d)
+    if cache.layer_kind(layer).window() is not None:
+        q = attention_prep(q, num_q_heads, d, start_position, None, 0.0, rope_freq_base_swa)
+        k = attention_prep(k, cache.num_kv_heads(), d, start_position, None, 0.0, rope_freq_base_swa)
+    return attention_step(cache, layer, q, k, v, num_q_heads, start_position, params, threads)
+

@@ -583,14 +583,15 @@ def test_snapshots_of_a_hybrid_cache_round_trip_and_match_the_oracles_bytes(elem
 
 @pytest.mark.parametrize("elem", ["f32", "f16"])
 def test_compute_attention_on_a_hybrid_model_takes_any_number_of_rows(elem):
-    # cpu.rs:586-646 on the reference model's kind of pattern: the host-pointer call appends
-    # and attends row by row in the reference, so a prompt longer than the device ring's
-    # headroom (and longer than the window) must come out the same, and decoding on from it
-    # too.
+    # cpu.rs:586-646 on the reference model's kind of pattern: the host-pointer call rotates
+    # Q and K on the sliding-window layers (interleaved RoPE at the SWA base, each row at its
+    # position; global layers are NoPE), then appends and attends row by row in the
+    # reference, so a prompt longer than the device ring's headroom (and longer than the
+    # window) must come out the same, and decoding on from it too.
     rng = np.random.default_rng(41)
     SW, G = P().LayerKind.SlidingWindow, P().LayerKind.Global
     cfg = P().GlimmerConfig(layers=[SW, SW, G], q_heads=8, kv_heads=2, key_length=16,
-                            value_length=16, sliding_window=20)
+                            value_length=16, sliding_window=20, rope_freq_base_swa=10000.0)
     ref = oracle.KvCache.new([oracle.LayerKind.windowed(20), oracle.LayerKind.windowed(20),
                               oracle.LayerKind.Global], cfg.kv_heads, cfg.key_length,
                              store_f16=(elem == "f16"))
@@ -602,8 +603,8 @@ def test_compute_attention_on_a_hybrid_model_takes_any_number_of_rows(elem):
             k = normal(rng, rows, cfg.k_width())
             v = normal(rng, rows, cfg.v_width())
             got = hc.attention(P().AttentionRequest(q, k, v, layer, kind, cfg), cache)
-            want = oracle.attention_step(ref, layer, q, k, v, cfg.q_heads, cache.position(),
-                                         threads=8)
+            want = oracle.compute_attention(ref, layer, q, k, v, cfg.q_heads, cache.position(),
+                                            cfg.rope_freq_base_swa, threads=8)
             if elem == "f32":
                 assert rel_err(got, want) <= 1e-5, (rows, layer)
             else:
@@ -619,10 +620,28 @@ def test_compute_attention_on_a_hybrid_model_takes_any_number_of_rows(elem):
     for layer, kind in enumerate(cfg.layers):
         q, k, v = normal(rng, 4, cfg.q_width()), normal(rng, 4, cfg.k_width()), normal(rng, 4, cfg.v_width())
         hc.attention(P().AttentionRequest(q, k, v, layer, kind, cfg), cache)
-        oracle.attention_step(ref, layer, q, k, v, cfg.q_heads, 223, threads=8)
+        oracle.compute_attention(ref, layer, q, k, v, cfg.q_heads, 223, cfg.rope_freq_base_swa,
+                                 threads=8)
     hc.cache_rewind(cp, 225)
     ref.rewind_to(rcp, 225)
     hc.cache_release(cp)
     ref.release(rcp)
     for layer in range(3):
         assert view_snapshot(dev, layer) == view_snapshot(ref, layer)
+
+
+def test_compute_attention_refuses_a_bad_swa_base_on_sliding_layers_only():
+    # rope_interleaved's refusals (crates/torch-math/src/rope_interleaved.rs:72-99) surface
+    # under the attention step; a global layer never looks at the base.
+    SW, G = P().LayerKind.SlidingWindow, P().LayerKind.Global
+    cfg = P().GlimmerConfig(layers=[SW, G], q_heads=4, kv_heads=2, key_length=8, value_length=8,
+                            sliding_window=6, rope_freq_base_swa=1.0)
+    hc = P().HipCompute.new(elem="f32", capacity_rows=32)
+    cache = P().PositionCache()
+    q, k, v = np.ones(32, np.float32), np.ones(16, np.float32), np.ones(16, np.float32)
+    with pytest.raises(P().StepFailed) as e:
+        hc.attention(P().AttentionRequest(q, k, v, 0, SW, cfg), cache)
+    assert e.value.step == "attention" and "rope: base must be finite and > 1" in e.value.detail
+    assert hc.kv_cache().next_position(0) == 0
+    out = hc.attention(P().AttentionRequest(q, k, v, 1, G, cfg), cache)
+    assert np.allclose(out, 1.0)
