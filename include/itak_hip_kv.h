@@ -171,6 +171,13 @@ typedef struct itak_itkv_header {
     uint64_t fingerprint_len;
     uint64_t fingerprint_offset; /* decode: byte offset of the UTF-8 fingerprint in the buffer */
     uint64_t encoded_len;        /* decode: bytes consumed, trailing checksum included */
+    /* decode: the format version read and the element type of the rows. Version 1 is the
+       reference's (f32 rows). Version 2 is this library's: one more u32 after the layer count
+       carries the element type (ITAK_ELEM_*), and the rows are of that type; it exists so that
+       an f16 cache can be snapshotted in its own bytes (half the size, nothing to convert).
+       The reference's reader refuses version 2 by name. */
+    uint32_t version;
+    uint32_t elem;
 } itak_itkv_header;
 
 /* One layer of an ITKV snapshot: its 28-byte header (snapshot.rs:24-26) and where its
@@ -318,8 +325,16 @@ itak_status itak_itkv_decode(const void *bytes, uint64_t len, itak_itkv_header *
 itak_status itak_kv_capture_itkv(itak_pool *pool, uint32_t slot, const char *fingerprint,
                                  uint64_t fingerprint_len, void *out, uint64_t capacity,
                                  uint64_t *written);
+/* The same capture of an f16 pool in the pool's own bytes: ITKV version 2 with f16 rows,
+   half the size of the version 1 encoding and bit-identical on restore. Refused
+   (ITAK_UNSUPPORTED) on an f32 pool: a narrowing capture would drop precision the cache
+   holds. No counterpart in the reference, whose format has no element-type field. */
+itak_status itak_kv_capture_itkv_f16(itak_pool *pool, uint32_t slot, const char *fingerprint,
+                                     uint64_t fingerprint_len, void *out, uint64_t capacity,
+                                     uint64_t *written);
 /* KvSnapshot::from_bytes followed by restore_checked (snapshot.rs:351-371) into a fresh
-   slot: the snapshot's geometry must be the pool's, and, when expected_fingerprint is not
+   slot (either format version; f16 rows go into an f16 pool as they are and are refused by
+   an f32 pool): the snapshot's geometry must be the pool's, and, when expected_fingerprint is not
    NULL, its fingerprint the expected one. The rows are gathered from `bytes` in place when
    the device can read them there (pinned host or device memory, 4-byte aligned payload),
    otherwise staged. An f32 snapshot into an f16 pool converts exactly as append does. */
@@ -409,11 +424,14 @@ itak_status itak_store_restore_prefix(itak_store *store, itak_pool *pool, uint32
                                       const char *fingerprint, uint64_t fingerprint_len,
                                       uint64_t now, uint64_t *matched);
 /* ResidentSession::capture_and_store_prefix (session.rs:5056-5094): the slot must stand at
-   exactly token_count positions; its rows are captured as ITKV v1 and put under `tokens`. */
+   exactly token_count positions; its rows are captured and put under `tokens`. elem =
+   ITAK_ELEM_F32 writes the reference's ITKV version 1 (an entry the reference's store serves
+   too); ITAK_ELEM_F16 (f16 pools) writes version 2, half the bytes on disk and over the
+   host link, which the reference's store refuses by name and walks past. */
 itak_status itak_store_capture_and_put(itak_store *store, itak_pool *pool, uint32_t slot,
                                        const uint32_t *tokens, uint64_t token_count,
                                        const char *fingerprint, uint64_t fingerprint_len,
-                                       uint64_t now);
+                                       uint32_t elem, uint64_t now);
 
 /* ---- attention over one slot, host pointers ---------------------------------------- */
 

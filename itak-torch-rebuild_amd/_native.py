@@ -81,7 +81,7 @@ class ItkvHeader(C.Structure):
     _fields_ = [("token_count", C.c_uint64), ("num_kv_heads", C.c_uint64),
                 ("head_dim", C.c_uint64), ("layer_count", C.c_uint64),
                 ("fingerprint_len", C.c_uint64), ("fingerprint_offset", C.c_uint64),
-                ("encoded_len", C.c_uint64)]
+                ("encoded_len", C.c_uint64), ("version", C.c_uint32), ("elem", C.c_uint32)]
 
 
 class ItkvLayer(C.Structure):
@@ -139,6 +139,7 @@ PROTOTYPES = {
                                 _P, _P, _P, _P, _u64, C.POINTER(_u64)]),
     "itak_itkv_decode": (_i32, [_P, _u64, C.POINTER(ItkvHeader), C.POINTER(ItkvLayer), _u64]),
     "itak_kv_capture_itkv": (_i32, [_P, _u32, C.c_char_p, _u64, _P, _u64, C.POINTER(_u64)]),
+    "itak_kv_capture_itkv_f16": (_i32, [_P, _u32, C.c_char_p, _u64, _P, _u64, C.POINTER(_u64)]),
     "itak_kv_restore_itkv": (_i32, [_P, _u32, _P, _u64, C.c_char_p, _u64]),
     "itak_kv_stats": (_i32, [_P, _u32, C.POINTER(LayerStatsRaw)]),
     "itak_kv_read_rows": (_i32, [_P, _u32, _u64, _u64, _u64, _P, _P, _P]),
@@ -177,7 +178,7 @@ PROTOTYPES = {
                                  C.c_char_p, _u64, _u64, C.POINTER(PrefixHit)]),
     "itak_store_restore_prefix": (_i32, [_P, _P, _u32, _P, _u64, C.c_char_p, _u64, _u64,
                                          C.POINTER(_u64)]),
-    "itak_store_capture_and_put": (_i32, [_P, _P, _u32, _P, _u64, C.c_char_p, _u64, _u64]),
+    "itak_store_capture_and_put": (_i32, [_P, _P, _u32, _P, _u64, C.c_char_p, _u64, _u32, _u64]),
     "itak_convert_f32_to_f16_device": (_i32, [_P, _P, _P, _u64]),
     "itak_probe_copy_device": (_i32, [_P, _P, _P, _u64]),
     "itak_probe_empty_launch": (_i32, [_P]),

@@ -1,5 +1,6 @@
-// The ITKV v1 snapshot wire format (crates/itak-kv/src/snapshot.rs:13-29) and the FNV-1a
-// hashes of crates/itak-kv/src/hash.rs, host side. Nothing here touches the device: the
+// The ITKV snapshot wire format (v1: crates/itak-kv/src/snapshot.rs:13-29; v2: the same with
+// an element-type word after the layer count and rows of that type, see kItkvVersionF16) and
+// the FNV-1a hashes of crates/itak-kv/src/hash.rs, host side. Nothing here touches the device: the
 // format fixes a byte-serial checksum over the whole file, so encoding and decoding are
 // host work; the rows themselves move between the encoded buffer and the device planes
 // through the gather / readback kernels.
@@ -16,6 +17,12 @@ constexpr uint64_t kFnvOffset = 0xcbf29ce484222325ull;     // hash.rs:14
 constexpr uint64_t kFnvPrime = 0x00000100000001b3ull;      // hash.rs:16
 constexpr uint64_t kFnvAltOffset = 0x84222325cbf29ce4ull;  // hash.rs:21
 constexpr uint32_t kItkvVersion = 1;                       // snapshot.rs:53
+// Version 2 is this library's own: v1 "carries no storage-format field; its rows are f32 by
+// definition" (bench/prefix-f16-guard-2026-11-07.md:46-70 names a format field in a later
+// version as the way to snapshots of f16 caches). v2 = v1 with one more u32 after the layer
+// count, the element type of the rows (0 = f32, 1 = f16 bits), and the rows in that type. A
+// v1 reader refuses it by name (UnsupportedVersion), never misreads it.
+constexpr uint32_t kItkvVersionTyped = 2;
 constexpr uint64_t kItkvLayerHeaderLen = 28;               // snapshot.rs:51
 
 uint64_t fnv1a64(const uint8_t *bytes, uint64_t count, uint64_t basis);           // hash.rs:24-31
@@ -46,6 +53,9 @@ struct ItkvHeader {
     uint64_t fingerprint_len = 0;
     uint64_t fingerprint_offset = 0;
     uint64_t encoded_len = 0;
+    uint32_t version = kItkvVersion;
+    uint32_t elem = 0;  // 0 = f32 rows, 1 = f16 rows (version 2 only)
+    uint64_t elem_bytes() const { return elem ? 2 : 4; }
 };
 
 // KvSnapshot::validate (snapshot.rs:187-236). `blocks` is the number of layer blocks the

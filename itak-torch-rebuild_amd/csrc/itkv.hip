@@ -188,9 +188,11 @@ bool itkv_decode(const uint8_t *bytes, uint64_t len, ItkvHeader &h, std::vector<
         return refuse(err, ITAK_KV_BAD_MAGIC, 0, 0, "snapshot: bad magic");
     uint32_t version = 0;
     if (!r.u32(&version)) return false;
-    if (version != kItkvVersion)
+    if (version != kItkvVersion && version != kItkvVersionTyped)
         return refuse(err, ITAK_KV_UNSUPPORTED_VERSION, version, 0,
                       "snapshot: unsupported format version %u", version);
+    h.version = version;
+    h.elem = 0;
     uint32_t fp_len = 0;
     if (!r.u32(&fp_len)) return false;
     h.fingerprint_offset = r.at;
@@ -204,6 +206,11 @@ bool itkv_decode(const uint8_t *bytes, uint64_t len, ItkvHeader &h, std::vector<
     h.num_kv_heads = heads;
     h.head_dim = dim;
     h.layer_count = layer_count;
+    if (version == kItkvVersionTyped) {
+        if (!r.u32(&h.elem)) return false;
+        if (h.elem > 1)
+            return inconsistent(err, "element type tag %u is not a known type", h.elem);
+    }
     // The count is bounded by the bytes that remain before it sizes anything
     // (snapshot.rs:448-462).
     if (layer_count > r.remaining() / kItkvLayerHeaderLen)
@@ -239,7 +246,7 @@ bool itkv_decode(const uint8_t *bytes, uint64_t len, ItkvHeader &h, std::vector<
         uint64_t bytes_per_side = 0;
         if (!checked_mul(layers[i].rows, row, &floats[i]))
             return inconsistent(err, "layer row count overflows the row width");
-        if (!checked_mul(floats[i], 4, &bytes_per_side))
+        if (!checked_mul(floats[i], h.elem_bytes(), &bytes_per_side))
             return inconsistent(err, "float count overflows the byte count");
         layers[i].keys_offset = r.at;
         if (!r.take(bytes_per_side)) return false;
@@ -263,7 +270,8 @@ bool itkv_decode(const uint8_t *bytes, uint64_t len, ItkvHeader &h, std::vector<
 }
 
 uint64_t itkv_header_len(const ItkvHeader &h) {
-    return 4 + 4 + 4 + h.fingerprint_len + 8 + 4 + 4 + 4 + h.layer_count * kItkvLayerHeaderLen;
+    return 4 + 4 + 4 + h.fingerprint_len + 8 + 4 + 4 + 4 + (h.version == kItkvVersionTyped ? 4 : 0) +
+           h.layer_count * kItkvLayerHeaderLen;
 }
 
 bool itkv_encoded_len(const ItkvHeader &h, const ItkvLayer *layers, uint64_t *out) {
@@ -271,7 +279,8 @@ bool itkv_encoded_len(const ItkvHeader &h, const ItkvLayer *layers, uint64_t *ou
     if (!checked_mul(h.num_kv_heads, h.head_dim, &row)) return false;
     for (uint64_t i = 0; i < h.layer_count; ++i) {
         uint64_t floats = 0, bytes = 0;
-        if (!checked_mul(layers[i].rows, row, &floats) || !checked_mul(floats, 8, &bytes) ||
+        if (!checked_mul(layers[i].rows, row, &floats) ||
+            !checked_mul(floats, 2 * h.elem_bytes(), &bytes) ||
             __builtin_add_overflow(total, bytes, &total))
             return false;
     }
@@ -285,7 +294,7 @@ void itkv_write_header(uint8_t *out, const ItkvHeader &h, const char *fingerprin
     uint8_t *p = out;
     memcpy(p, "ITKV", 4);
     p += 4;
-    put_u32(p, kItkvVersion);
+    put_u32(p, h.version);
     put_u32(p, uint32_t(h.fingerprint_len));
     if (h.fingerprint_len) memcpy(p, fingerprint, h.fingerprint_len);
     p += h.fingerprint_len;
@@ -293,6 +302,7 @@ void itkv_write_header(uint8_t *out, const ItkvHeader &h, const char *fingerprin
     put_u32(p, uint32_t(h.num_kv_heads));
     put_u32(p, uint32_t(h.head_dim));
     put_u32(p, uint32_t(h.layer_count));
+    if (h.version == kItkvVersionTyped) put_u32(p, h.elem);
     for (uint64_t i = 0; i < h.layer_count; ++i) {
         *p++ = layers[i].kind == ITAK_LAYER_GLOBAL ? 0 : 1;
         *p++ = 0;
@@ -306,9 +316,9 @@ void itkv_write_header(uint8_t *out, const ItkvHeader &h, const char *fingerprin
     const uint64_t row = h.num_kv_heads * h.head_dim;
     for (uint64_t i = 0; i < h.layer_count; ++i) {
         layers[i].keys_offset = at;
-        at += layers[i].rows * row * 4;
+        at += layers[i].rows * row * h.elem_bytes();
         layers[i].values_offset = at;
-        at += layers[i].rows * row * 4;
+        at += layers[i].rows * row * h.elem_bytes();
     }
 }
 

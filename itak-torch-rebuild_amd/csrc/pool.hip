@@ -1133,6 +1133,9 @@ itak_status itak_itkv_encode(const itak_itkv_header *header, const char *fingerp
     if (st != ITAK_OK) return st;
     if (!written) return invalid_argument(e, "written is null");
     if (header->fingerprint_len && !fingerprint) return invalid_argument(e, "fingerprint is null");
+    if (header->version > 1 || header->elem != 0)
+        return unsupported(e, "itak_itkv_encode writes version 1 (f32 rows); version 2 comes from "
+                              "itak_kv_capture_itkv_f16");
     if (header->num_kv_heads > UINT32_MAX || header->head_dim > UINT32_MAX ||
         header->layer_count > UINT32_MAX || header->fingerprint_len > UINT32_MAX)
         return invalid_argument(e, "a header field does not fit the 32-bit wire field");
@@ -1167,8 +1170,9 @@ itak_status itak_itkv_decode(const void *bytes, uint64_t len, itak_itkv_header *
     ItkvError err;
     if (!itkv_decode(static_cast<const uint8_t *>(bytes), len, h, ls, err))
         return set_itkv_error(e, err);
-    *header = itak_itkv_header{h.token_count,     h.num_kv_heads,       h.head_dim, h.layer_count,
-                               h.fingerprint_len, h.fingerprint_offset, h.encoded_len};
+    *header = itak_itkv_header{h.token_count,     h.num_kv_heads,       h.head_dim,      h.layer_count,
+                               h.fingerprint_len, h.fingerprint_offset, h.encoded_len,   h.version,
+                               h.elem};
     if (layers_capacity < ls.size())
         return invalid_argument(e, "layers_capacity is smaller than the snapshot's layer count");
     for (size_t i = 0; i < ls.size(); ++i)
@@ -1177,9 +1181,29 @@ itak_status itak_itkv_decode(const void *bytes, uint64_t len, itak_itkv_header *
     return ITAK_OK;
 }
 
+static itak_status capture_itkv(itak_pool *pool, uint32_t slot, const char *fingerprint,
+                                uint64_t fingerprint_len, bool f16_rows, void *out,
+                                uint64_t capacity, uint64_t *written);
+
 itak_status itak_kv_capture_itkv(itak_pool *pool, uint32_t slot, const char *fingerprint,
                                  uint64_t fingerprint_len, void *out, uint64_t capacity,
                                  uint64_t *written) {
+    return capture_itkv(pool, slot, fingerprint, fingerprint_len, false, out, capacity, written);
+}
+
+itak_status itak_kv_capture_itkv_f16(itak_pool *pool, uint32_t slot, const char *fingerprint,
+                                     uint64_t fingerprint_len, void *out, uint64_t capacity,
+                                     uint64_t *written) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (!pool->elem_f16)
+        return unsupported(pool->err,
+                           "an f16 snapshot of an f32 pool would drop precision the cache holds");
+    return capture_itkv(pool, slot, fingerprint, fingerprint_len, true, out, capacity, written);
+}
+
+static itak_status capture_itkv(itak_pool *pool, uint32_t slot, const char *fingerprint,
+                                uint64_t fingerprint_len, bool f16_rows, void *out,
+                                uint64_t capacity, uint64_t *written) {
     if (!pool) return ITAK_INVALID_ARGUMENT;
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
@@ -1201,6 +1225,11 @@ itak_status itak_kv_capture_itkv(itak_pool *pool, uint32_t slot, const char *fin
     h.head_dim = pool->g.head_dim;
     h.layer_count = pool->cfg.layer_count;
     h.fingerprint_len = fingerprint_len;
+    if (f16_rows) {
+        h.version = kItkvVersionTyped;
+        h.elem = ITAK_ELEM_F16;
+    }
+    const uint64_t out_elem = h.elem_bytes();
     // snapshot.rs:264-295: every row of a global layer, the last `window` rows of a windowed
     // one, oldest first.
     std::vector<ItkvLayer> ls(h.layer_count);
@@ -1238,7 +1267,7 @@ itak_status itak_kv_capture_itkv(itak_pool *pool, uint32_t slot, const char *fin
                                      pool->stream),
                     "launch row readback");
             const void *ksrc = kd, *vsrc = vd;
-            if (pool->elem_f16) {
+            if (pool->elem_f16 && !f16_rows) {
                 float *kw = reinterpret_cast<float *>(pool->stage + 2 * raw);
                 float *vw = reinterpret_cast<float *>(pool->stage + 2 * raw + wide);
                 HIP_TRY(pool,
@@ -1251,12 +1280,12 @@ itak_status itak_kv_capture_itkv(itak_pool *pool, uint32_t slot, const char *fin
                 vsrc = vw;
             }
             HIP_TRY(pool,
-                    hipMemcpyAsync(bytes + ls[layer].keys_offset + first * pool->row * 4, ksrc,
-                                   elems * 4, hipMemcpyDeviceToHost, pool->stream),
+                    hipMemcpyAsync(bytes + ls[layer].keys_offset + first * pool->row * out_elem,
+                                   ksrc, elems * out_elem, hipMemcpyDeviceToHost, pool->stream),
                     "download keys");
             HIP_TRY(pool,
-                    hipMemcpyAsync(bytes + ls[layer].values_offset + first * pool->row * 4, vsrc,
-                                   elems * 4, hipMemcpyDeviceToHost, pool->stream),
+                    hipMemcpyAsync(bytes + ls[layer].values_offset + first * pool->row * out_elem,
+                                   vsrc, elems * out_elem, hipMemcpyDeviceToHost, pool->stream),
                     "download values");
             // The staging buffer is reused by the next chunk.
             HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after readback");
@@ -1311,7 +1340,7 @@ itak_status itak_kv_restore_itkv(itak_pool *pool, uint32_t slot, const void *byt
         layers[i] = itak_snapshot_layer{ls[i].first_position, ls[i].rows, b8 + ls[i].keys_offset,
                                         b8 + ls[i].values_offset};
     return itak_kv_restore_snapshot(pool, slot, h.token_count, layers.data(), layers.size(),
-                                    ITAK_ELEM_F32);
+                                    h.elem ? ITAK_ELEM_F16 : ITAK_ELEM_F32);
 }
 
 itak_status itak_kv_stats(itak_pool *pool, uint32_t slot, itak_layer_stats *out) {

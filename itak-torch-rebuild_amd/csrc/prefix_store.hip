@@ -794,8 +794,13 @@ itak_status itak_store_restore_prefix(itak_store *store, itak_pool *pool, uint32
 itak_status itak_store_capture_and_put(itak_store *store, itak_pool *pool, uint32_t slot,
                                        const uint32_t *tokens, uint64_t token_count,
                                        const char *fingerprint, uint64_t fingerprint_len,
-                                       uint64_t now) {
+                                       uint32_t elem, uint64_t now) {
     if (!store || !pool) return ITAK_INVALID_ARGUMENT;
+    if (elem != ITAK_ELEM_F32 && elem != ITAK_ELEM_F16)
+        return fail(store->err, ITAK_INVALID_ARGUMENT, nullptr, elem, 0,
+                    "elem is neither ITAK_ELEM_F32 nor ITAK_ELEM_F16");
+    // f32 rows are the reference's version 1; f16 rows this library's version 2.
+    auto capture = elem == ITAK_ELEM_F16 ? itak_kv_capture_itkv_f16 : itak_kv_capture_itkv;
     uint64_t position = 0;
     itak_status status = itak_kv_next_position(pool, slot, 0, &position);
     if (status != ITAK_OK) return fail(store->err, status, nullptr, 0, 0, "%s", itak_last_error(pool));
@@ -806,11 +811,11 @@ itak_status itak_store_capture_and_put(itak_store *store, itak_pool *pool, uint3
                     "file one sequence's KV under another's key",
                     ULL(position), ULL(token_count));
     uint64_t bytes = 0;
-    status = itak_kv_capture_itkv(pool, slot, fingerprint, fingerprint_len, nullptr, 0, &bytes);
+    status = capture(pool, slot, fingerprint, fingerprint_len, nullptr, 0, &bytes);
     if (status == ITAK_OK) status = ensure_stage(store, bytes) == ITAK_OK ? ITAK_OK : store->err.code;
     if (status == ITAK_OK)
-        status = itak_kv_capture_itkv(pool, slot, fingerprint, fingerprint_len, store->stage,
-                                      store->stage_bytes, &bytes);
+        status = capture(pool, slot, fingerprint, fingerprint_len, store->stage, store->stage_bytes,
+                         &bytes);
     if (status != ITAK_OK) {
         if (store->err.code != status)
             return fail(store->err, status, "prefix_store", 0, 0, "%s", itak_last_error(pool));

@@ -121,7 +121,9 @@ def _header(geometry: KvGeometry, token_count: int, fingerprint: bytes, blocks: 
 
 @dataclass
 class KvSnapshot:
-    """itak_kv::KvSnapshot (snapshot.rs:163-174)."""
+    """itak_kv::KvSnapshot (snapshot.rs:163-174): rows as f32, whatever they were encoded as.
+    `to_bytes` writes the reference's version 1; bytes of version 2 (f16 rows, this library's
+    own, from `capture_bytes(..., elem="f16")`) decode into the same f32 rows exactly."""
     geometry: KvGeometry
     model_fingerprint: str
     token_count: int
@@ -184,8 +186,9 @@ class KvSnapshot:
             L = layers[i]
             kinds.append(LayerKind.Global if L.kind == N.LAYER_GLOBAL else LayerKind.windowed(int(L.window)))
             n = int(L.rows) * row
-            keys = np.frombuffer(data, dtype="<f4", count=n, offset=int(L.keys_offset)).copy()
-            vals = np.frombuffer(data, dtype="<f4", count=n, offset=int(L.values_offset)).copy()
+            wire = "<f2" if h.elem == N.ELEM_F16 else "<f4"
+            keys = np.frombuffer(data, dtype=wire, count=n, offset=int(L.keys_offset)).astype(np.float32)
+            vals = np.frombuffer(data, dtype=wire, count=n, offset=int(L.values_offset)).astype(np.float32)
             blocks.append(LayerSnapshot(int(L.first_position), keys, vals))
         fp = bytes(data[int(h.fingerprint_offset):int(h.fingerprint_offset + h.fingerprint_len)])
         return KvSnapshot(KvGeometry(kinds, int(h.num_kv_heads), int(h.head_dim)), fp.decode(),
@@ -211,16 +214,18 @@ class KvSnapshot:
         return restore_bytes(pool, self.to_bytes(), expected_fingerprint)
 
 
-def capture_bytes(cache: KvCache, model_fingerprint: str) -> bytes:
-    """KvSnapshot::capture + to_bytes in one pass: device rows straight into ITKV v1 bytes."""
+def capture_bytes(cache: KvCache, model_fingerprint: str, elem: str = "f32") -> bytes:
+    """KvSnapshot::capture + to_bytes in one pass: device rows straight into ITKV bytes.
+    elem="f32" is the reference's version 1; elem="f16" (f16 pools only) writes version 2,
+    the pool's own halves: half the size, bit-identical on restore."""
     lib = N.load()
+    fn = {"f32": lib.itak_kv_capture_itkv, "f16": lib.itak_kv_capture_itkv_f16}[elem]
     fp = model_fingerprint.encode()
     written = C.c_uint64()
     h = cache.pool._h
-    _check_kv(h, lib.itak_kv_capture_itkv(h, cache.slot, fp, len(fp), None, 0, C.byref(written)))
+    _check_kv(h, fn(h, cache.slot, fp, len(fp), None, 0, C.byref(written)))
     out = np.empty(written.value, dtype=np.uint8)
-    _check_kv(h, lib.itak_kv_capture_itkv(h, cache.slot, fp, len(fp), out.ctypes.data, out.size,
-                                          C.byref(written)))
+    _check_kv(h, fn(h, cache.slot, fp, len(fp), out.ctypes.data, out.size, C.byref(written)))
     return out.tobytes()
 
 

@@ -227,10 +227,11 @@ class PrefixStore:
         return int(matched.value)
 
     def capture_and_put(self, cache: KvCache, tokens: Sequence[int], fingerprint: str,
-                        now: Optional[int] = None) -> None:
-        """capture_and_store_prefix (session.rs:5056-5094)."""
+                        now: Optional[int] = None, elem: str = "f32") -> None:
+        """capture_and_store_prefix (session.rs:5056-5094). elem="f16" files an f16 pool's
+        rows as they are (ITKV version 2) instead of widened to the reference's version 1."""
         t = _tokens(tokens)
         fp = fingerprint.encode()
         self._check(self._lib.itak_store_capture_and_put(
             self._h, cache.pool._h, cache.slot, t.ctypes.data if t.size else None, t.size, fp,
-            len(fp), now_unix() if now is None else now))
+            len(fp), {"f32": N.ELEM_F32, "f16": N.ELEM_F16}[elem], now_unix() if now is None else now))

@@ -306,3 +306,42 @@ class _Reader:  # snapshot.rs:520-604
         if byte_count > USIZE_MAX:
             raise _inconsistent("float count overflows the byte count")
         return np.frombuffer(self.take(byte_count), dtype="<f4").copy()
+
+
+# ---- version 2 (typed rows): not the reference's, this build's own extension ---------------
+# v1 with one more u32 after the layer count, the element type of the rows (0 = f32,
+# 1 = f16 bits), and the rows in that type. Restated here independently of the library so
+# that its encoder and decoder have something to be held to; `KvSnapshot.from_bytes` above
+# stays the reference's reader and refuses version 2 by name.
+
+TYPED_FORMAT_VERSION = 2
+
+
+def to_bytes_f16(snapshot: KvSnapshot) -> bytes:
+    """Version 2 with f16 rows. The snapshot's f32 values must be exactly representable in
+    f16 (they are when captured from an f16-storing cache)."""
+    snapshot.validate()
+    out = bytearray()
+    out += MAGIC
+    out += struct.pack("<I", TYPED_FORMAT_VERSION)
+    fingerprint = snapshot.model_fingerprint.encode("utf-8")
+    out += struct.pack("<I", len(fingerprint))
+    out += fingerprint
+    out += struct.pack("<Q", snapshot.token_count)
+    out += struct.pack("<III", snapshot.geometry.num_kv_heads, snapshot.geometry.head_dim,
+                       len(snapshot.geometry.layers))
+    out += struct.pack("<I", 1)
+    row = snapshot.geometry.row_floats()
+    for kind, layer in zip(snapshot.geometry.layers, snapshot.layers):
+        w = kind.window()
+        out += bytes([0 if w is None else 1, 0, 0, 0])
+        out += struct.pack("<QQQ", 0 if w is None else w, layer.first_position, layer.rows(row))
+    for layer in snapshot.layers:
+        for side in (layer.keys, layer.values):
+            halves = np.asarray(side, dtype=np.float32).astype("<f2")
+            assert np.array_equal(halves.astype(np.float32), np.asarray(side, dtype=np.float32)), \
+                "rows are not f16 values"
+            out += halves.tobytes()
+    out += struct.pack("<Q", checksum(bytes(out)))
+    return bytes(out)
+

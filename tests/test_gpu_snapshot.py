@@ -158,3 +158,92 @@ def test_a_long_snapshot_round_trips_and_decodes_continue_identically():
         outs.append(out.cpu().numpy().tobytes())
     assert outs[0] == outs[1]
     pool.close()
+
+
+# ---- version 2: an f16 pool snapshotted in its own bytes (no counterpart in the reference) --
+
+
+@pytest.mark.parametrize("pattern,kv_heads,head_dim,tokens", [
+    (["G", "G"], 4, 128, 300), (["W40", "G", "W40"], 4, 128, 133), (["W8"], 2, 20, 5),
+])
+def test_f16_snapshots_are_half_the_size_and_restore_the_same_bits(pattern, kv_heads, head_dim, tokens):
+    kinds = [P().LayerKind.Global if p == "G" else P().LayerKind.windowed(int(p[1:])) for p in pattern]
+    okinds = [oracle.LayerKind.Global if p == "G" else oracle.LayerKind.windowed(int(p[1:]))
+              for p in pattern]
+    rng = np.random.default_rng(tokens)
+    pool = P().KvPool(kinds, kv_heads, head_dim, elem="f16", max_slots=3, capacity_rows=tokens + 40)
+    cache = pool.acquire()
+    ref = oracle.KvCache.new(okinds, kv_heads, head_dim, store_f16=True)
+    width = kv_heads * head_dim
+    for layer in range(len(kinds)):
+        k, v = normal(rng, tokens, width), normal(rng, tokens, width)
+        for p in range(tokens):
+            cache.append(layer, k[p], v[p], p)
+            ref.append(layer, k[p], v[p], p)
+    v1 = P().capture_bytes(cache, "m")
+    v2 = P().capture_bytes(cache, "m", elem="f16")
+    # The layout, restated independently: v1 plus an element-type word, rows as halves.
+    assert v2 == okv.to_bytes_f16(okv.KvSnapshot.capture(ref, "m"))
+    payload = sum(ref.stored_len(layer) for layer in range(len(kinds))) * width * 2
+    assert len(v1) - len(v2) == payload * 2 - 4
+    # The reference's reader refuses it by name; the library reads the same f32 rows from both.
+    with pytest.raises(okv.KvError) as e:
+        okv.KvSnapshot.from_bytes(v2)
+    assert e.value.variant == "UnsupportedVersion" and e.value.fields["version"] == 2
+    a, b = P().KvSnapshot.from_bytes(v1), P().KvSnapshot.from_bytes(v2)
+    assert a.geometry == b.geometry and a.token_count == b.token_count
+    for la, lb in zip(a.layers, b.layers):
+        assert la.first_position == lb.first_position
+        assert la.keys.tobytes() == lb.keys.tobytes() and la.values.tobytes() == lb.values.tobytes()
+    # Restored from either version, the slot holds the captured slot's bits.
+    r1 = P().restore_bytes(pool, v1, "m")
+    r2 = P().restore_bytes(pool, v2, "m")
+    for layer in range(len(kinds)):
+        want = cache.view(layer).rows()
+        for other in (r1, r2):
+            got = other.view(layer).rows()
+            assert all(np.asarray(x).tobytes() == np.asarray(y).tobytes() for x, y in zip(got, want))
+    pool.close()
+
+
+def test_f16_snapshots_stay_with_f16_pools_and_go_through_the_store(tmp_path):
+    rng = np.random.default_rng(2)
+    f32_pool = P().KvPool(1, 2, 8, elem="f32", max_slots=2)
+    c32 = f32_pool.acquire()
+    c32.append(0, normal(rng, 16), normal(rng, 16), 0)
+    with pytest.raises(P().KvError) as e:  # a narrowing capture is refused
+        P().capture_bytes(c32, "m", elem="f16")
+    assert "would drop precision" in e.value.message
+    f16_pool = P().KvPool(1, 2, 8, elem="f16", max_slots=3)
+    c16 = f16_pool.acquire()
+    tokens = [5, 6, 7]
+    for p in range(3):
+        c16.append(0, normal(rng, 16), normal(rng, 16), p)
+    v2 = P().capture_bytes(c16, "m", elem="f16")
+    with pytest.raises(P().KvError) as e:  # f16 rows are never widened into an f32 pool
+        P().restore_bytes(f32_pool, v2, "m")
+    assert "f16 snapshot restores only into an f16 pool" in e.value.message
+    # The prefix store files and serves the typed snapshot like any other.
+    store = P().PrefixStore.open(str(tmp_path), 1 << 20)
+    store.put(tokens, v2, 10)
+    fresh = f16_pool.acquire()
+    assert store.restore_prefix(fresh, tokens + [8], "m", now=11) == 3
+    assert np.asarray(fresh.view(0).rows()[1]).tobytes() == np.asarray(c16.view(0).rows()[1]).tobytes()
+    # The session flow's write half in the pool's own bytes, then the oracle's store (the
+    # reference's reader) walks past the typed entry by name.
+    store.capture_and_put(c16, tokens, "m", now=12, elem="f16")
+    assert store.stats().entries == 1
+    assert (tmp_path / store.entries()[0].file_name).read_bytes().endswith(v2)
+    import oracle.prefix_store as ops
+    theirs = ops.PrefixStore.open(ops.StoreConfig(str(tmp_path), 1 << 20))
+    assert theirs.lookup(tokens, None, None, 13) is None
+    assert any("unsupported format version 2" in r for r in theirs.refusals)
+    # A truncated typed snapshot is refused by name like a version 1 one.
+    with pytest.raises(P().KvError) as e:
+        P().KvSnapshot.from_bytes(v2[:-3])
+    assert e.value.variant == "Truncated"
+    bad = bytearray(v2); bad[4 + 4 + 4 + 1 + 8 + 12] = 9   # the element-type word
+    with pytest.raises(P().KvError) as e:
+        P().KvSnapshot.from_bytes(bytes(bad))
+    assert e.value.variant in ("InconsistentSnapshot", "ChecksumMismatch")
+    f32_pool.close(); f16_pool.close()
