@@ -164,6 +164,38 @@ def cache_maintenance(args, pkg, torch, dev, stream, timed):
     t_pin16 = restore_from(pin_k16, pin_v16, True)
     t_pin32 = restore_from(pin_k32, pin_v32, False)
     gbs = 2 * dst_bytes / t_dev / 1e9  # reads the f16 source and writes the planes
+
+    # The same prefix through the prefix store (entry file in the page cache): lookup with
+    # its trust checks, the payload read into the store's pinned buffer, the byte-serial
+    # FNV-1a checksum of the format, then the gather. ITKV version 1 (f32 rows, the
+    # reference's) against version 2 (the pool's own f16 rows).
+    import shutil
+    import tempfile
+    store_ms = {}
+    root = tempfile.mkdtemp(prefix="itak-bench-store-")
+    try:
+        token_ids = list(range(1, tokens + 1))
+        restore_from(dev_k, dev_v, True)  # leaves the slot empty; fill it once more
+        cache.restore_snapshot_ptrs(tokens, [(0, tokens, dev_k[l].data_ptr(), dev_v[l].data_ptr())
+                                             for l in range(layers)], src_f16=True)
+        for elem in ("f32", "f16"):
+            store = pkg.PrefixStore.open(os.path.join(root, elem), 1 << 40)
+            t0 = time.perf_counter()
+            store.capture_and_put(cache, token_ids, "bench-model", now=1, elem=elem)
+            put_s = time.perf_counter() - t0
+            other = pool  # restore into the same pool: free the slot first
+            entry_bytes = store.stats().total_bytes
+            pool.truncate([cache], [0])
+            t0 = time.perf_counter()
+            matched = store.restore_prefix(cache, token_ids + [7], "bench-model", now=2)
+            pool.synchronize()
+            restore_s = time.perf_counter() - t0
+            assert matched == tokens
+            store_ms[elem] = {"entry_bytes": entry_bytes, "capture_and_put_ms": round(put_s * 1e3, 1),
+                              "lookup_and_restore_ms": round(restore_s * 1e3, 1)}
+            store.close()
+    finally:
+        shutil.rmtree(root, ignore_errors=True)
     result = {
         "metric": "prefix-snapshot restore GB/s (48 layers x 8192 rows, source in HBM, bytes read + written)",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -177,6 +209,7 @@ def cache_maintenance(args, pkg, torch, dev, stream, timed):
             "f32_rows_ms": round(t_pin32 * 1e3, 3),
             "f32_rows_GBps_over_link": round(2 * dst_bytes / t_pin32 / 1e9, 2),
         },
+        "through_the_prefix_store": store_ms,
         "roofline": {"bound": "hbm", "kernel": "kv_restore_rows + kv_restore_v_blocked (all layers, "
                                                "two launches)",
                      "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
