@@ -1,0 +1,167 @@
+"""Random sequences of cache operations on the device against the same sequences on the CPU
+oracle: steps of random length on hybrid patterns, speculative rounds (checkpoint, block,
+rewind, release), plain truncates, snapshots restored into fresh slots and continued, attention
+at arbitrary positions. After every operation the visible rows, the positions and the attention
+outputs must agree (rows bit for bit; outputs within 1e-5 relative on f32 KV, 2e-3 absolute on
+f16 KV). The seeds are fixed: a failure names its seed and step."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import oracle.itak_kv as okv
+from helpers import max_abs, normal, pkg, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def P():
+    return pkg()
+
+
+def view_bytes(cache, layer):
+    pos, keys, vals = cache.view(layer).rows()
+    keys, vals = np.asarray(keys), np.asarray(vals)
+    if keys.dtype == np.uint16:
+        keys, vals = keys.view(np.float16).astype(np.float32), vals.view(np.float16).astype(np.float32)
+    return (np.asarray(pos, dtype=np.int64).tobytes(), np.ascontiguousarray(keys).tobytes(),
+            np.ascontiguousarray(vals).tobytes())
+
+
+def random_case(seed):
+    rng = np.random.default_rng(seed)
+    elem = ["f32", "f16"][seed % 2]
+    d = int(rng.choice([8, 16, 64, 128] if elem == "f32" else [16, 20, 64, 128, 128, 128]))
+    kvh = int(rng.choice([1, 2, 4]))
+    group = int(rng.choice([1, 2, 4, 8]))
+    layers = int(rng.integers(1, 4))
+    headroom = int(rng.choice([1, 5, 16, 40]))
+    windows = [None if rng.random() < 0.4 else int(rng.integers(2, 48)) for _ in range(layers)]
+    return rng, elem, d, kvh, group, windows, headroom
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_operation_sequences_match_the_oracle(seed):
+    rng, elem, d, kvh, group, windows, headroom = random_case(seed)
+    q_heads = kvh * group
+    kinds = [P().LayerKind.Global if w is None else P().LayerKind.windowed(w) for w in windows]
+    okinds = [oracle.LayerKind.Global if w is None else oracle.LayerKind.windowed(w) for w in windows]
+    pool = P().KvPool(kinds, kvh, d, elem=elem, max_slots=5, capacity_rows=400,
+                      ring_headroom=headroom)
+    f16 = elem == "f16"
+    cache = pool.acquire()
+    ref = oracle.KvCache.new(okinds, kvh, d, store_f16=f16)
+    windowed = [w for w in windows if w is not None]
+    smallest = min(windowed) if windowed else None
+    softcap = float(rng.choice([0.0, 0.0, 15.0]))
+
+    def close(got, want, what):
+        err = max_abs(got, want) if f16 else rel_err(got, want)
+        assert err <= (2e-3 if f16 else 1e-5), (seed, what, err)
+
+    # Every third seed a second slot rides along in the same launches with its own row counts
+    # (a ragged batch); it is never rewound, so its rings only ever move forward.
+    rider = (pool.acquire(), oracle.KvCache.new(okinds, kvh, d, store_f16=f16)) if seed % 3 == 0 else None
+
+    def step(dev, cpu, rows, what):
+        pairs = [(dev, cpu, rows)]
+        if rider is not None and rider[0].next_position(0) < 330:
+            pairs.append((rider[0], rider[1], int(rng.integers(1, max_rows + 1))))
+        bases = [c.next_position(0) for c, _, _ in pairs]
+        total = sum(r for _, _, r in pairs)
+        for layer in range(len(kinds)):
+            q, k, v = normal(rng, total, q_heads * d), normal(rng, total, kvh * d), normal(rng, total, kvh * d)
+            qd, kd, vd = (torch.from_numpy(x).cuda() for x in (q, k, v))
+            out = torch.empty_like(qd)
+            pool.attention_step_device(layer, [(c, r) for c, _, r in pairs], qd.data_ptr(),
+                                       kd.data_ptr(), vd.data_ptr(), out.data_ptr(), q_heads,
+                                       softcap=softcap)
+            pool.synchronize()
+            got, first = out.cpu().numpy(), 0
+            for (c, o, r), base in zip(pairs, bases):
+                rows_of = slice(first, first + r)
+                want = oracle.attention_step(o, layer, q[rows_of], k[rows_of], v[rows_of], q_heads,
+                                             base, oracle.AttentionParams(softcap=softcap), threads=4)
+                close(got[rows_of].reshape(-1), want, (what, layer, r, base))
+                first += r
+        if len(pairs) > 1:
+            same_views(rider[0], rider[1], (what, "rider"))
+
+    def same_views(dev, cpu, what):
+        for layer in range(len(kinds)):
+            assert dev.next_position(layer) == cpu.next_position(layer), (seed, what, layer)
+            assert view_bytes(dev, layer) == view_bytes(cpu, layer), (seed, what, layer)
+
+    max_rows = headroom if windowed else 40
+    high = 0        # one past the highest position ever written into this slot's rings
+    pending = None  # (oracle checkpoint, position before, rows) of the step just taken
+    for op_index in range(int(rng.integers(12, 22))):
+        position = cache.next_position(0)
+        if position > 330:
+            break
+        op = str(rng.choice(["step", "step", "step", "round", "truncate", "snapshot", "attend"]))
+        what = (op_index, op)
+        if op == "truncate" and pending is not None:
+            # The device's truncate keeps no state; the oracle reaches the same cache by
+            # rewinding the checkpoint it took before the step.
+            rcp, before, rows = pending
+            room = (headroom - (high - position)) if windowed else rows
+            drop = int(rng.integers(0, max(0, min(rows, room)) + 1))
+            pool.truncate([cache.slot], [position - drop])
+            ref.rewind_to(rcp, position - drop)
+            ref.release(rcp)
+            pending = None
+            same_views(cache, ref, what)
+            continue
+        if pending is not None:
+            ref.release(pending[0])
+            pending = None
+        if op in ("step", "truncate") or position == 0:
+            rows = int(rng.integers(1, max_rows + 1))
+            if smallest is None or rows <= smallest:
+                pending = (ref.checkpoint(rows), position, rows)
+            step(cache, ref, rows, what)
+            high = max(high, position + rows)
+        elif op == "round":
+            depth = int(rng.integers(1, min(8, max_rows, smallest or 8) + 1))
+            cp, rcp = cache.checkpoint(depth), ref.checkpoint(depth)
+            assert cp.bases() == rcp.bases(), (seed, what)
+            step(cache, ref, depth, what)
+            high = max(high, position + depth)
+            keep = int(rng.integers(0, depth + 1))
+            cache.rewind_to(cp, position + keep)
+            ref.rewind_to(rcp, position + keep)
+            same_views(cache, ref, (what, "first rewind"))
+            if rng.random() < 0.3 and keep > 0:  # a second rewind under the same checkpoint
+                cache.rewind_to(cp, position)
+                ref.rewind_to(rcp, position)
+            cache.release(cp)
+            ref.release(rcp)
+        elif op == "snapshot":
+            data = P().capture_bytes(cache, "fp")
+            assert data == okv.KvSnapshot.capture(ref, "fp").to_bytes(), (seed, what)
+            restored = P().restore_bytes(pool, data, "fp")
+            ref2 = okv.KvSnapshot.from_bytes(data).restore(store_f16=f16)
+            same_views(restored, ref2, what)
+            if rng.random() < 0.5:  # go on with the restored pair
+                cache.release_slot()
+                cache, ref, high = restored, ref2, position
+            else:
+                restored.release_slot()
+        else:  # attention at arbitrary positions, nothing appended
+            layer = int(rng.integers(0, len(kinds)))
+            w = windows[layer]
+            oldest = 0 if w is None else max(0, position - w)
+            newest = position + (2 if w is None else min(2, w - 1))
+            n = int(rng.integers(1, 6))
+            positions = [int(p) for p in rng.integers(oldest, newest, size=n)]
+            q = normal(rng, n, q_heads * d)
+            got = P().gqa_attention(q, n, q_heads, positions, cache.view(layer),
+                                    P().AttentionParams(softcap=softcap))
+            want = oracle.gqa_attention(q, n, q_heads, positions, ref.view(layer),
+                                        oracle.AttentionParams(softcap=softcap))
+            close(got, want, (what, layer, positions))
+        same_views(cache, ref, what)
+    if pending is not None:
+        ref.release(pending[0])
+    pool.close()
