@@ -11,6 +11,8 @@
 #include <string>
 #include <vector>
 
+struct itak_pool;
+
 namespace itak {
 
 constexpr uint64_t kFnvOffset = 0xcbf29ce484222325ull;     // hash.rs:14
@@ -64,8 +66,10 @@ bool itkv_validate(const ItkvHeader &h, const ItkvLayer *layers, uint64_t blocks
                    const uint64_t *key_floats, const uint64_t *value_floats, ItkvError &err);
 
 // KvSnapshot::from_bytes (snapshot.rs:405-509): strict; fills offsets instead of copying rows.
+// `known_sum`, when given, is the checksum of bytes[0, len-8) the caller already computed (while
+// the bytes were still arriving, say); the decoder then compares instead of walking them again.
 bool itkv_decode(const uint8_t *bytes, uint64_t len, ItkvHeader &h, std::vector<ItkvLayer> &layers,
-                 ItkvError &err);
+                 ItkvError &err, const uint64_t *known_sum = nullptr);
 
 // Bytes of everything before the row payload, and of the whole encoding (payload and the
 // trailing checksum included), for a header whose layers carry `rows` rows each.
@@ -74,5 +78,20 @@ bool itkv_encoded_len(const ItkvHeader &h, const ItkvLayer *layers, uint64_t *ou
 // Writes magic .. layer headers (snapshot.rs:383-403) and fills the payload offsets.
 void itkv_write_header(uint8_t *out, const ItkvHeader &h, const char *fingerprint,
                        ItkvLayer *layers);
+
+// Installs an encoding that itkv_decode has already accepted into a fresh slot: `h` and
+// `layers` are the decoder's outputs for `bytes`. The geometry and fingerprint checks of
+// restore_checked (snapshot.rs:351-371) run; the bytes are not walked a second time. For the
+// prefix store, which verifies an entry in its own private buffer and installs from there.
+int32_t restore_decoded_itkv(itak_pool *pool, uint32_t slot, const uint8_t *bytes,
+                             const ItkvHeader &h, const std::vector<ItkvLayer> &layers,
+                             const char *expected_fingerprint, uint64_t expected_fingerprint_len);
+
+// itak_kv_capture_itkv / itak_kv_capture_itkv_f16 with the 8 trailer bytes left zero: for a
+// caller that runs the byte-serial checksum itself while it does something else with the bytes
+// (the prefix store writes them to disk meanwhile).
+int32_t capture_itkv_unsummed(itak_pool *pool, uint32_t slot, const char *fingerprint,
+                              uint64_t fingerprint_len, bool f16_rows, void *out, uint64_t capacity,
+                              uint64_t *written);
 
 }  // namespace itak

@@ -180,7 +180,7 @@ bool itkv_validate(const ItkvHeader &h, const ItkvLayer *layers, uint64_t blocks
 }
 
 bool itkv_decode(const uint8_t *bytes, uint64_t len, ItkvHeader &h, std::vector<ItkvLayer> &layers,
-                 ItkvError &err) {
+                 ItkvError &err, const uint64_t *known_sum) {
     Reader r{bytes, len, 0, err};
     const uint8_t *magic = r.take(4);
     if (!magic) return false;
@@ -257,7 +257,7 @@ bool itkv_decode(const uint8_t *bytes, uint64_t len, ItkvHeader &h, std::vector<
     if (!r.u64(&stored)) return false;
     if (r.remaining() != 0)
         return inconsistent(err, "%llu trailing bytes after the checksum", ULL(r.remaining()));
-    const uint64_t computed = fnv1a64(bytes, len - 8, kFnvOffset);
+    const uint64_t computed = known_sum ? *known_sum : fnv1a64(bytes, len - 8, kFnvOffset);
     if (stored != computed)
         return refuse(err, ITAK_KV_CHECKSUM_MISMATCH, stored, computed,
                       "snapshot checksum mismatch: stored 0x%016llx, computed 0x%016llx",

@@ -589,6 +589,63 @@ std::vector<ItkvLayer> to_internal(const itak_itkv_layer *layers, uint64_t n) {
 
 // ======================================================================== public ABI
 
+namespace itak {
+
+int32_t restore_decoded_itkv(itak_pool *pool, uint32_t slot, const uint8_t *b8, const ItkvHeader &h,
+                             const std::vector<ItkvLayer> &ls, const char *expected_fingerprint,
+                             uint64_t expected_fingerprint_len) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (!find_slot(pool, slot)) return invalid_argument(pool->err, "slot is not in use");
+    // restore_checked (snapshot.rs:351-371): geometry first, then the fingerprint.
+    bool same = h.layer_count == pool->cfg.layer_count && h.num_kv_heads == pool->g.kv_heads &&
+                h.head_dim == pool->g.head_dim;
+    for (size_t i = 0; same && i < ls.size(); ++i)
+        same = pool->layers[i].windowed
+                   ? (ls[i].kind == ITAK_LAYER_WINDOWED && ls[i].window == pool->layers[i].window)
+                   : ls[i].kind == ITAK_LAYER_GLOBAL;
+    if (!same)
+        return set_error(pool->err, ITAK_KV_GEOMETRY_MISMATCH, "snapshot", 0, 0, 0, 0,
+                         "geometry mismatch: snapshot geometry (%llu layers, %llu KV heads, head "
+                         "dim %llu) differs from the required geometry (%llu layers, %llu KV "
+                         "heads, head dim %llu)",
+                         ULL(h.layer_count), ULL(h.num_kv_heads), ULL(h.head_dim),
+                         ULL(pool->cfg.layer_count), ULL(pool->g.kv_heads), ULL(pool->g.head_dim));
+    if (expected_fingerprint &&
+        (expected_fingerprint_len != h.fingerprint_len ||
+         memcmp(expected_fingerprint, b8 + h.fingerprint_offset, h.fingerprint_len) != 0))
+        return set_error(pool->err, ITAK_KV_FINGERPRINT_MISMATCH, "snapshot", 0, 0, 0, 0,
+                         "model fingerprint mismatch: need %.*s, snapshot carries %.*s",
+                         int(std::min<uint64_t>(expected_fingerprint_len, 400)), expected_fingerprint,
+                         int(std::min<uint64_t>(h.fingerprint_len, 400)),
+                         reinterpret_cast<const char *>(b8 + h.fingerprint_offset));
+    std::vector<itak_snapshot_layer> layers(ls.size());
+    for (size_t i = 0; i < ls.size(); ++i)
+        layers[i] = itak_snapshot_layer{ls[i].first_position, ls[i].rows, b8 + ls[i].keys_offset,
+                                        b8 + ls[i].values_offset};
+    return itak_kv_restore_snapshot(pool, slot, h.token_count, layers.data(), layers.size(),
+                                    h.elem ? ITAK_ELEM_F16 : ITAK_ELEM_F32);
+}
+
+}  // namespace itak
+
+static itak_status capture_itkv(itak_pool *pool, uint32_t slot, const char *fingerprint,
+                                uint64_t fingerprint_len, bool f16_rows, void *out,
+                                uint64_t capacity, uint64_t *written, bool with_checksum);
+
+namespace itak {
+
+int32_t capture_itkv_unsummed(itak_pool *pool, uint32_t slot, const char *fingerprint,
+                              uint64_t fingerprint_len, bool f16_rows, void *out, uint64_t capacity,
+                              uint64_t *written) {
+    if (pool && f16_rows && !pool->elem_f16)
+        return unsupported(pool->err,
+                           "an f16 snapshot of an f32 pool would drop precision the cache holds");
+    return capture_itkv(pool, slot, fingerprint, fingerprint_len, f16_rows, out, capacity, written,
+                        false);
+}
+
+}  // namespace itak
+
 extern "C" {
 
 uint32_t itak_abi_version(void) { return 1; }
@@ -1183,7 +1240,7 @@ itak_status itak_itkv_decode(const void *bytes, uint64_t len, itak_itkv_header *
 
 static itak_status capture_itkv(itak_pool *pool, uint32_t slot, const char *fingerprint,
                                 uint64_t fingerprint_len, bool f16_rows, void *out,
-                                uint64_t capacity, uint64_t *written);
+                                uint64_t capacity, uint64_t *written, bool with_checksum = true);
 
 itak_status itak_kv_capture_itkv(itak_pool *pool, uint32_t slot, const char *fingerprint,
                                  uint64_t fingerprint_len, void *out, uint64_t capacity,
@@ -1203,7 +1260,7 @@ itak_status itak_kv_capture_itkv_f16(itak_pool *pool, uint32_t slot, const char 
 
 static itak_status capture_itkv(itak_pool *pool, uint32_t slot, const char *fingerprint,
                                 uint64_t fingerprint_len, bool f16_rows, void *out,
-                                uint64_t capacity, uint64_t *written) {
+                                uint64_t capacity, uint64_t *written, bool with_checksum) {
     if (!pool) return ITAK_INVALID_ARGUMENT;
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
@@ -1291,7 +1348,7 @@ static itak_status capture_itkv(itak_pool *pool, uint32_t slot, const char *fing
             HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after readback");
         }
     }
-    const uint64_t sum = fnv1a64(bytes, total - 8, kFnvOffset);
+    const uint64_t sum = with_checksum ? fnv1a64(bytes, total - 8, kFnvOffset) : 0;
     for (int b = 0; b < 8; ++b) bytes[total - 8 + b] = uint8_t(sum >> (8 * b));
     return ITAK_OK;
 }
@@ -1313,34 +1370,7 @@ itak_status itak_kv_restore_itkv(itak_pool *pool, uint32_t slot, const void *byt
     ItkvError err;
     const uint8_t *b8 = static_cast<const uint8_t *>(bytes);
     if (!itkv_decode(b8, len, h, ls, err)) return set_itkv_error(pool->err, err);
-    // restore_checked (snapshot.rs:351-371): geometry first, then the fingerprint.
-    bool same = h.layer_count == pool->cfg.layer_count && h.num_kv_heads == pool->g.kv_heads &&
-                h.head_dim == pool->g.head_dim;
-    for (size_t i = 0; same && i < ls.size(); ++i)
-        same = pool->layers[i].windowed
-                   ? (ls[i].kind == ITAK_LAYER_WINDOWED && ls[i].window == pool->layers[i].window)
-                   : ls[i].kind == ITAK_LAYER_GLOBAL;
-    if (!same)
-        return set_error(pool->err, ITAK_KV_GEOMETRY_MISMATCH, "snapshot", 0, 0, 0, 0,
-                         "geometry mismatch: snapshot geometry (%llu layers, %llu KV heads, head "
-                         "dim %llu) differs from the required geometry (%llu layers, %llu KV "
-                         "heads, head dim %llu)",
-                         ULL(h.layer_count), ULL(h.num_kv_heads), ULL(h.head_dim),
-                         ULL(pool->cfg.layer_count), ULL(pool->g.kv_heads), ULL(pool->g.head_dim));
-    if (expected_fingerprint &&
-        (expected_fingerprint_len != h.fingerprint_len ||
-         memcmp(expected_fingerprint, b8 + h.fingerprint_offset, h.fingerprint_len) != 0))
-        return set_error(pool->err, ITAK_KV_FINGERPRINT_MISMATCH, "snapshot", 0, 0, 0, 0,
-                         "model fingerprint mismatch: need %.*s, snapshot carries %.*s",
-                         int(std::min<uint64_t>(expected_fingerprint_len, 400)), expected_fingerprint,
-                         int(std::min<uint64_t>(h.fingerprint_len, 400)),
-                         reinterpret_cast<const char *>(b8 + h.fingerprint_offset));
-    std::vector<itak_snapshot_layer> layers(ls.size());
-    for (size_t i = 0; i < ls.size(); ++i)
-        layers[i] = itak_snapshot_layer{ls[i].first_position, ls[i].rows, b8 + ls[i].keys_offset,
-                                        b8 + ls[i].values_offset};
-    return itak_kv_restore_snapshot(pool, slot, h.token_count, layers.data(), layers.size(),
-                                    h.elem ? ITAK_ELEM_F16 : ITAK_ELEM_F32);
+    return restore_decoded_itkv(pool, slot, b8, h, ls, expected_fingerprint, expected_fingerprint_len);
 }
 
 itak_status itak_kv_stats(itak_pool *pool, uint32_t slot, itak_layer_stats *out) {

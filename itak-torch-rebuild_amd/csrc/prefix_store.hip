@@ -25,7 +25,9 @@
 #include <unistd.h>
 
 #include <algorithm>
+#include <atomic>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "itkv.h"
@@ -74,6 +76,9 @@ struct itak_store {
     uint8_t *stage = nullptr;
     uint64_t stage_bytes = 0;
     bool stage_pinned = false;
+    // What the decoder made of the payload in `stage` when the last candidate was verified.
+    ItkvHeader stage_header;
+    std::vector<ItkvLayer> stage_layers;
 };
 
 namespace {
@@ -178,6 +183,65 @@ int64_t read_at(int fd, void *out, uint64_t len, uint64_t offset) {
         done += uint64_t(n);
     }
     return int64_t(done);
+}
+
+// Reads [offset, offset + len) of the file into `out` on a second thread while this one runs
+// the byte-serial checksum over the first `sum_len` bytes behind it, so a large payload costs
+// the slower of the two instead of their sum. Returns the bytes read (short at end of file),
+// -1 with errno set on a read error.
+int64_t read_at_with_checksum(int fd, uint8_t *out, uint64_t len, uint64_t offset, uint64_t sum_len,
+                              uint64_t *sum) {
+    constexpr uint64_t kPiece = 4u << 20;
+    *sum = kFnvOffset;
+    if (len <= 2 * kPiece) {
+        const int64_t got = read_at(fd, out, len, offset);
+        if (got >= 0) *sum = fnv1a64(out, std::min<uint64_t>(sum_len, uint64_t(got)), kFnvOffset);
+        return got;
+    }
+    std::atomic<uint64_t> arrived{0};
+    std::atomic<int> state{0};  // 0 reading, 1 done (possibly short), 2 failed
+    int read_errno = 0;
+    auto read_pieces = [&] {
+        uint64_t done = 0;
+        while (done < len) {
+            const uint64_t want = std::min(kPiece, len - done);
+            const int64_t got = read_at(fd, out + done, want, offset + done);
+            if (got < 0) {
+                read_errno = errno;
+                state.store(2, std::memory_order_release);
+                return;
+            }
+            done += uint64_t(got);
+            arrived.store(done, std::memory_order_release);
+            if (uint64_t(got) < want) break;
+        }
+        state.store(1, std::memory_order_release);
+    };
+    std::thread reader;
+    try {
+        reader = std::thread(read_pieces);
+    } catch (...) {  // no thread to be had: read, then sum
+        read_pieces();
+    }
+    uint64_t summed = 0, running = kFnvOffset;
+    for (;;) {
+        const int st = state.load(std::memory_order_acquire);
+        const uint64_t have = std::min(arrived.load(std::memory_order_acquire), sum_len);
+        if (have > summed) {
+            running = fnv1a64(out + summed, have - summed, running);
+            summed = have;
+            continue;
+        }
+        if (st != 0) break;
+        std::this_thread::yield();
+    }
+    if (reader.joinable()) reader.join();
+    if (state.load() == 2) {
+        errno = read_errno;
+        return -1;
+    }
+    *sum = running;
+    return int64_t(arrived.load());
 }
 
 bool write_all(int fd, const void *src, uint64_t len) {
@@ -476,12 +540,15 @@ itak_status verify_candidate(itak_store *s, StoreError &why, const Entry &meta,
         why = s->err;
         return status;
     }
-    if (read_at(fd, s->stage, payload, tokens_end) != int64_t(payload))
+    uint64_t sum = 0;
+    if (read_at_with_checksum(fd, s->stage, payload, tokens_end, payload >= 8 ? payload - 8 : 0,
+                              &sum) != int64_t(payload))
         return io_error(why, errno, "read entry %s", meta.file_name.c_str());
-    ItkvHeader h;
-    std::vector<ItkvLayer> layers;
+    ItkvHeader &h = s->stage_header;
+    std::vector<ItkvLayer> &layers = s->stage_layers;
     ItkvError decode_error;
-    if (!itkv_decode(s->stage, payload, h, layers, decode_error)) return from_itkv(why, decode_error);
+    if (!itkv_decode(s->stage, payload, h, layers, decode_error, payload >= 8 ? &sum : nullptr))
+        return from_itkv(why, decode_error);
     if (h.token_count != p.token_count)
         return fail(why, ITAK_KV_SNAPSHOT_TOKEN_MISMATCH, nullptr, p.token_count, h.token_count,
                     "entry preamble covers %llu tokens but its snapshot covers %llu",
@@ -618,9 +685,13 @@ itak_status itak_store_entries(itak_store *store, itak_store_entry *out, uint64_
     return ITAK_OK;
 }
 
-itak_status itak_store_put(itak_store *store, const uint32_t *tokens, uint64_t token_count,
-                           const void *snapshot, uint64_t snapshot_len, uint64_t now) {  // store.rs:236-300
-    if (!store) return ITAK_INVALID_ARGUMENT;
+// store.rs:236-300. `own_capture` says the bytes were written a moment ago by this library's
+// own capture into the store's buffer with the trailer still to come: the strict decode below
+// checks the structure only, and the byte-serial checksum (~1 GB/s) then runs once, on a second
+// thread, while this one writes the file.
+static itak_status put_entry(itak_store *store, const uint32_t *tokens, uint64_t token_count,
+                             void *snapshot, uint64_t snapshot_len, uint64_t now,
+                             bool own_capture) {
     StoreError &e = store->err;
     if (token_count == 0) return fail(e, ITAK_KV_EMPTY_PREFIX, nullptr, 0, 0, "empty token prefix refused");
     if (!tokens || !snapshot) return fail(e, ITAK_INVALID_ARGUMENT, nullptr, 0, 0, "tokens or snapshot is null");
@@ -629,8 +700,13 @@ itak_status itak_store_put(itak_store *store, const uint32_t *tokens, uint64_t t
     ItkvHeader h;
     std::vector<ItkvLayer> layers;
     ItkvError decode_error;
-    const uint8_t *payload = static_cast<const uint8_t *>(snapshot);
-    if (!itkv_decode(payload, snapshot_len, h, layers, decode_error)) return from_itkv(e, decode_error);
+    uint8_t *payload = static_cast<uint8_t *>(snapshot);
+    uint64_t trailer = 0;
+    if (own_capture && snapshot_len >= 8)
+        for (int b = 0; b < 8; ++b) trailer |= uint64_t(payload[snapshot_len - 8 + b]) << (8 * b);
+    if (!itkv_decode(payload, snapshot_len, h, layers, decode_error,
+                     own_capture && snapshot_len >= 8 ? &trailer : nullptr))
+        return from_itkv(e, decode_error);
     if (h.token_count != token_count)
         return fail(e, ITAK_KV_TOKEN_COUNT_MISMATCH, nullptr, h.token_count, token_count,
                     "snapshot covers %llu tokens but was offered under %llu token ids",
@@ -664,9 +740,34 @@ itak_status itak_store_put(itak_store *store, const uint32_t *tokens, uint64_t t
     std::vector<uint8_t> ids(token_count * 4);
     for (uint64_t i = 0; i < token_count; ++i)
         for (int b = 0; b < 4; ++b) ids[4 * i + b] = uint8_t(tokens[i] >> (8 * b));
-    const bool written = write_all(fd, head, kPreambleLen) && write_all(fd, ids.data(), ids.size()) &&
-                         write_all(fd, payload, snapshot_len) && fsync(fd) == 0;
-    const int write_errno = errno;
+    const bool sum_here = own_capture && snapshot_len >= 8;
+    const uint64_t body_len = sum_here ? snapshot_len - 8 : snapshot_len;
+    uint64_t sum = 0;
+    std::thread summer;
+    bool summed = false;
+    if (sum_here) {
+        try {
+            summer = std::thread([&] { sum = fnv1a64(payload, body_len, kFnvOffset); });
+        } catch (...) {  // no thread to be had: the checksum runs here, before the write
+            sum = fnv1a64(payload, body_len, kFnvOffset);
+            summed = true;
+        }
+    }
+    bool written = write_all(fd, head, kPreambleLen) && write_all(fd, ids.data(), ids.size()) &&
+                   write_all(fd, payload, body_len);
+    int write_errno = errno;
+    if (sum_here) {
+        if (!summed) summer.join();
+        for (int b = 0; b < 8; ++b) payload[body_len + b] = uint8_t(sum >> (8 * b));
+        if (written) {
+            written = write_all(fd, payload + body_len, 8);
+            write_errno = errno;
+        }
+    }
+    if (written && fsync(fd) != 0) {
+        written = false;
+        write_errno = errno;
+    }
     close(fd);
     if (!written) {
         (void)unlink(temp_path.c_str());
@@ -688,6 +789,12 @@ itak_status itak_store_put(itak_store *store, const uint32_t *tokens, uint64_t t
     meta.created_unix = meta.last_used_unix = now;
     store->entries.push_back(meta);
     return evict_except(store, file_name);
+}
+
+itak_status itak_store_put(itak_store *store, const uint32_t *tokens, uint64_t token_count,
+                           const void *snapshot, uint64_t snapshot_len, uint64_t now) {
+    if (!store) return ITAK_INVALID_ARGUMENT;
+    return put_entry(store, tokens, token_count, const_cast<void *>(snapshot), snapshot_len, now, false);
 }
 
 itak_status itak_store_lookup(itak_store *store, const uint32_t *query, uint64_t query_len,
@@ -775,8 +882,10 @@ itak_status itak_store_restore_prefix(itak_store *store, itak_pool *pool, uint32
         return ITAK_OK;
     }
     if (hit.token_count == 0) return ITAK_OK;
-    status = itak_kv_restore_itkv(pool, slot, hit.snapshot, hit.snapshot_len, fingerprint,
-                                  fingerprint_len);
+    // The hit's bytes lie verified in the store's own buffer: install from there without
+    // walking the checksum a second time.
+    status = restore_decoded_itkv(pool, slot, store->stage, store->stage_header, store->stage_layers,
+                                  fingerprint, fingerprint_len);
     if (status == ITAK_HIP_ERROR)
         return fail(store->err, status, "prefix_restore", 0, 0, "%s", itak_last_error(pool));
     if (status != ITAK_OK) {
@@ -813,15 +922,15 @@ itak_status itak_store_capture_and_put(itak_store *store, itak_pool *pool, uint3
     uint64_t bytes = 0;
     status = capture(pool, slot, fingerprint, fingerprint_len, nullptr, 0, &bytes);
     if (status == ITAK_OK) status = ensure_stage(store, bytes) == ITAK_OK ? ITAK_OK : store->err.code;
-    if (status == ITAK_OK)
-        status = capture(pool, slot, fingerprint, fingerprint_len, store->stage, store->stage_bytes,
-                         &bytes);
+    if (status == ITAK_OK)  // the trailer is left for put_entry, which sums while it writes
+        status = capture_itkv_unsummed(pool, slot, fingerprint, fingerprint_len,
+                                       elem == ITAK_ELEM_F16, store->stage, store->stage_bytes, &bytes);
     if (status != ITAK_OK) {
         if (store->err.code != status)
             return fail(store->err, status, "prefix_store", 0, 0, "%s", itak_last_error(pool));
         return status;
     }
-    return itak_store_put(store, tokens, token_count, store->stage, bytes, now);
+    return put_entry(store, tokens, token_count, store->stage, bytes, now, true);
 }
 
 }  // extern "C"

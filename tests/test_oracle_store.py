@@ -339,3 +339,43 @@ def test_library_and_oracle_write_identical_files_and_serve_each_other(tmp_path)
             assert a[0] == b[0] and list(a[1]) == list(b[1]) and a[2] == b[2]
     for name in names_o:  # both restamped the same entries in place
         assert (tmp_path / "o" / name).read_bytes() == (tmp_path / "l" / name).read_bytes()
+
+
+def test_a_payload_read_in_pieces_is_served_whole_and_a_flip_in_any_piece_is_refused(tmp_path):
+    """A payload larger than a few MB is read by a second thread while the checksum follows
+    it: what comes out is what went in, and one flipped bit in the first, a middle or the
+    last piece is still caught by name. (Library side only: the oracle's byte loop over
+    20 MB is what this path exists to avoid.)"""
+    rng = np.random.default_rng(3)
+    kvh, d, rows = 4, 128, 5000
+    geometry = P().KvGeometry([P().LayerKind.Global], kvh, d)
+    keys = rng.standard_normal(rows * kvh * d, dtype=np.float32)
+    values = rng.standard_normal(rows * kvh * d, dtype=np.float32)
+    snap = P().KvSnapshot(geometry, "big", rows, [P().LayerSnapshot(0, keys, values)])
+    data = snap.to_bytes()
+    assert len(data) > 20_000_000
+    tokens = [int(t) for t in rng.integers(0, 1 << 20, size=rows)]
+    short = tokens[:7]
+    small = P().KvSnapshot(geometry, "big", 7, [P().LayerSnapshot(0, keys[:7 * kvh * d],
+                                                                  values[:7 * kvh * d])])
+    store = P().PrefixStore.open(str(tmp_path), 1 << 30)
+    store.put(short, small.to_bytes(), 1)
+    store.put(tokens, data, 2)
+    hit = store.lookup(tokens + [5], geometry, "big", 3)
+    assert hit.token_count == rows and hit.snapshot_bytes == data
+    path = tmp_path / hit.file_name
+    whole = path.read_bytes()
+    payload_at = len(whole) - len(data)
+    for offset in (payload_at + 100, payload_at + len(data) // 2, len(whole) - 9):
+        flipped = bytearray(whole)
+        flipped[offset] ^= 0x01
+        path.write_bytes(bytes(flipped))
+        store.refusals.clear()
+        assert store.lookup(tokens + [5], geometry, "big", 4).token_count == 7
+        assert any("snapshot checksum mismatch" in r for r in store.refusals), offset
+    path.write_bytes(whole[:-3_000_000])  # the file ends inside a later piece
+    store.refusals.clear()
+    assert store.lookup(tokens + [5], geometry, "big", 5).token_count == 7
+    assert any("entry payload: truncated, needs" in r for r in store.refusals)
+    path.write_bytes(whole)
+    assert store.lookup(tokens + [5], geometry, "big", 6).snapshot_bytes == data
