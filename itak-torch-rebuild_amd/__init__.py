@@ -29,6 +29,7 @@ from .itak_kv import (  # noqa: F401
     SNAPSHOT_FORMAT_VERSION,
     capture_bytes,
     checksum,
+    checksum_blocks,
     prefix_discriminator,
     prefix_hash,
     restore_bytes,
@@ -51,7 +52,7 @@ __all__ = [
     "GlimmerConfig", "HipCompute", "KvCache", "KvPool", "LayerKind", "LayerStats",
     "PositionCache", "StepFailed", "gqa_attention", "kv_head_for_query_head",
     "KvError", "KvGeometry", "KvSnapshot", "LayerSnapshot", "SNAPSHOT_FORMAT_VERSION",
-    "capture_bytes", "checksum", "prefix_discriminator", "prefix_hash", "restore_bytes",
+    "capture_bytes", "checksum", "checksum_blocks", "prefix_discriminator", "prefix_hash", "restore_bytes",
     "EntryMeta", "PrefixHit", "PrefixStore", "StoreConfig", "StoreStats", "max_bytes_from",
     "now_unix", "prefix_store_enabled", "prefix_store_enabled_from",
 ]

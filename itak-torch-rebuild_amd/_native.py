@@ -134,6 +134,7 @@ PROTOTYPES = {
     "itak_kv_prefix_hash": (_u64, [_P, _u64]),
     "itak_kv_prefix_discriminator": (_u64, [_P, _u64]),
     "itak_kv_checksum": (_u64, [_P, _u64]),
+    "itak_kv_checksum_blocks": (_u64, [_P, _u64]),
     "itak_itkv_validate": (_i32, [C.POINTER(ItkvHeader), C.POINTER(ItkvLayer), _u64, _P, _P]),
     "itak_itkv_encode": (_i32, [C.POINTER(ItkvHeader), C.c_char_p, C.POINTER(ItkvLayer), _u64, _P,
                                 _P, _P, _P, _P, _u64, C.POINTER(_u64)]),

@@ -8,7 +8,10 @@
 
 #include <stdint.h>
 
+#include <algorithm>
+#include <atomic>
 #include <string>
+#include <thread>
 #include <vector>
 
 struct itak_pool;
@@ -21,14 +24,54 @@ constexpr uint64_t kFnvAltOffset = 0x84222325cbf29ce4ull;  // hash.rs:21
 constexpr uint32_t kItkvVersion = 1;                       // snapshot.rs:53
 // Version 2 is this library's own: v1 "carries no storage-format field; its rows are f32 by
 // definition" (bench/prefix-f16-guard-2026-11-07.md:46-70 names a format field in a later
-// version as the way to snapshots of f16 caches). v2 = v1 with one more u32 after the layer
-// count, the element type of the rows (0 = f32, 1 = f16 bits), and the rows in that type. A
-// v1 reader refuses it by name (UnsupportedVersion), never misreads it.
+// version as the way to snapshots of f16 caches). v2 differs from v1 in two places: one more
+// u32 after the layer count, the element type of the rows (0 = f32, 1 = f16 bits), with the
+// rows in that type; and the trailer, which is FNV-1a over the FNV-1a sums of consecutive
+// 1 MiB blocks of the bytes before it (fnv1a64_blocks) instead of over the bytes themselves,
+// so that host threads can share the walk. A v1 reader refuses it by name (UnsupportedVersion),
+// never misreads it.
 constexpr uint32_t kItkvVersionTyped = 2;
+constexpr uint64_t kItkvSumBlock = 1u << 20;
 constexpr uint64_t kItkvLayerHeaderLen = 28;               // snapshot.rs:51
 
 uint64_t fnv1a64(const uint8_t *bytes, uint64_t count, uint64_t basis);           // hash.rs:24-31
 uint64_t fnv1a64_tokens(const uint32_t *tokens, uint64_t count, uint64_t basis);  // hash.rs:35-41
+
+// Host threads this library may use for one call (the caller's included): 8, or what the
+// ITAK_HOST_THREADS environment variable says (1..64), never more than the machine has.
+unsigned host_threads();
+
+// f(k) for every k in [0, count), shared among host_threads() threads; returns when all are
+// done. f must not throw.
+template <class F>
+void for_each_index(uint64_t count, F f) {
+    std::atomic<uint64_t> next{0};
+    auto work = [&] {
+        for (uint64_t k; (k = next.fetch_add(1, std::memory_order_relaxed)) < count;) f(k);
+    };
+    std::vector<std::thread> helpers;
+    const uint64_t want = std::min<uint64_t>(host_threads(), count);
+    for (uint64_t i = 1; i < want; ++i) {
+        try {
+            helpers.emplace_back(work);
+        } catch (...) {  // no more threads to be had: the ones there share the rest
+            break;
+        }
+    }
+    work();
+    for (std::thread &t : helpers) t.join();
+}
+
+// Version 2's trailer. sums[k] = FNV-1a of block k (kItkvSumBlock bytes, the last one shorter);
+// the result is FNV-1a over the sums written little-endian one after another. No bytes: the
+// offset basis. fnv1a64_of_sums is the second half alone, for a caller that made the block
+// sums itself.
+uint64_t fnv1a64_blocks(const uint8_t *bytes, uint64_t count);
+uint64_t fnv1a64_of_sums(const uint64_t *sums, uint64_t blocks);
+// The trailer a snapshot of `version` carries for the `count` bytes before it.
+inline uint64_t itkv_trailer(uint32_t version, const uint8_t *bytes, uint64_t count) {
+    return version == kItkvVersionTyped ? fnv1a64_blocks(bytes, count) : fnv1a64(bytes, count, kFnvOffset);
+}
 
 // A refusal of itak_kv::KvError (crates/itak-kv/src/error.rs:13-124); `message` is its
 // Display text (error.rs:141-188).

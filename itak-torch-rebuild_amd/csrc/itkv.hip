@@ -5,6 +5,7 @@
 
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "../../include/itak_hip_kv.h"
@@ -30,6 +31,40 @@ uint64_t fnv1a64_tokens(const uint32_t *tokens, uint64_t count, uint64_t basis) 
         }
     }
     return hash;
+}
+
+unsigned host_threads() {
+    static const unsigned threads = [] {
+        unsigned limit = 8;
+        if (const char *text = getenv("ITAK_HOST_THREADS")) {
+            char *end = nullptr;
+            const long asked = strtol(text, &end, 10);
+            if (end != text && *end == 0 && asked >= 1 && asked <= 64) limit = unsigned(asked);
+        }
+        const unsigned machine = std::thread::hardware_concurrency();
+        return std::max(1u, machine ? std::min(machine, limit) : limit);
+    }();
+    return threads;
+}
+
+uint64_t fnv1a64_of_sums(const uint64_t *sums, uint64_t blocks) {
+    uint64_t hash = kFnvOffset;
+    for (uint64_t k = 0; k < blocks; ++k)
+        for (int b = 0; b < 8; ++b) {
+            hash ^= (sums[k] >> (8 * b)) & 0xffu;
+            hash *= kFnvPrime;
+        }
+    return hash;
+}
+
+uint64_t fnv1a64_blocks(const uint8_t *bytes, uint64_t count) {
+    const uint64_t blocks = count / kItkvSumBlock + (count % kItkvSumBlock ? 1 : 0);
+    std::vector<uint64_t> sums(blocks);
+    for_each_index(blocks, [&](uint64_t k) {
+        const uint64_t at = k * kItkvSumBlock;
+        sums[k] = fnv1a64(bytes + at, std::min(kItkvSumBlock, count - at), kFnvOffset);
+    });
+    return fnv1a64_of_sums(sums.data(), blocks);
 }
 
 namespace {
@@ -257,7 +292,7 @@ bool itkv_decode(const uint8_t *bytes, uint64_t len, ItkvHeader &h, std::vector<
     if (!r.u64(&stored)) return false;
     if (r.remaining() != 0)
         return inconsistent(err, "%llu trailing bytes after the checksum", ULL(r.remaining()));
-    const uint64_t computed = known_sum ? *known_sum : fnv1a64(bytes, len - 8, kFnvOffset);
+    const uint64_t computed = known_sum ? *known_sum : itkv_trailer(h.version, bytes, len - 8);
     if (stored != computed)
         return refuse(err, ITAK_KV_CHECKSUM_MISMATCH, stored, computed,
                       "snapshot checksum mismatch: stored 0x%016llx, computed 0x%016llx",

@@ -1166,6 +1166,9 @@ uint64_t itak_kv_prefix_discriminator(const uint32_t *tokens, uint64_t count) { 
 uint64_t itak_kv_checksum(const void *bytes, uint64_t count) {  // hash.rs:59-61
     return fnv1a64(static_cast<const uint8_t *>(bytes), bytes ? count : 0, kFnvOffset);
 }
+uint64_t itak_kv_checksum_blocks(const void *bytes, uint64_t count) {
+    return fnv1a64_blocks(static_cast<const uint8_t *>(bytes), bytes ? count : 0);
+}
 
 itak_status itak_itkv_validate(const itak_itkv_header *header, const itak_itkv_layer *layers,
                                uint64_t blocks, const uint64_t *key_floats,
@@ -1348,7 +1351,7 @@ static itak_status capture_itkv(itak_pool *pool, uint32_t slot, const char *fing
             HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after readback");
         }
     }
-    const uint64_t sum = with_checksum ? fnv1a64(bytes, total - 8, kFnvOffset) : 0;
+    const uint64_t sum = with_checksum ? itkv_trailer(h.version, bytes, total - 8) : 0;
     for (int b = 0; b < 8; ++b) bytes[total - 8 + b] = uint8_t(sum >> (8 * b));
     return ITAK_OK;
 }

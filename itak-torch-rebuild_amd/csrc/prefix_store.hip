@@ -244,6 +244,35 @@ int64_t read_at_with_checksum(int fd, uint8_t *out, uint64_t len, uint64_t offse
     return int64_t(arrived.load());
 }
 
+// The same for a version 2 payload, whose trailer is a sum of block sums: host threads each
+// read whole blocks of the file and sum what they read, so neither the copy out of the page
+// cache nor the walk is serial.
+int64_t read_blocks_with_checksum(int fd, uint8_t *out, uint64_t len, uint64_t offset,
+                                  uint64_t sum_len, uint64_t *sum) {
+    const uint64_t blocks = len / kItkvSumBlock + (len % kItkvSumBlock ? 1 : 0);
+    const uint64_t summed_blocks = sum_len / kItkvSumBlock + (sum_len % kItkvSumBlock ? 1 : 0);
+    std::vector<uint64_t> sums(summed_blocks);
+    std::atomic<uint64_t> arrived{0};
+    std::atomic<int> read_errno{0};
+    for_each_index(blocks, [&](uint64_t k) {
+        const uint64_t at = k * kItkvSumBlock, want = std::min(kItkvSumBlock, len - at);
+        const int64_t got = read_at(fd, out + at, want, offset + at);
+        if (got < 0) {
+            read_errno.store(errno ? errno : EIO, std::memory_order_relaxed);
+            return;
+        }
+        arrived.fetch_add(uint64_t(got), std::memory_order_relaxed);
+        if (uint64_t(got) == want && k < summed_blocks)
+            sums[k] = fnv1a64(out + at, std::min(want, sum_len - at), kFnvOffset);
+    });
+    if (read_errno.load()) {
+        errno = read_errno.load();
+        return -1;
+    }
+    *sum = fnv1a64_of_sums(sums.data(), summed_blocks);
+    return int64_t(arrived.load());
+}
+
 bool write_all(int fd, const void *src, uint64_t len) {
     const uint8_t *p = static_cast<const uint8_t *>(src);
     uint64_t done = 0;
@@ -540,9 +569,19 @@ itak_status verify_candidate(itak_store *s, StoreError &why, const Entry &meta,
         why = s->err;
         return status;
     }
+    // Magic and version lead the payload (snapshot.rs:13-16); the version says how the trailer
+    // is summed, and so how the bytes are best brought in. Anything the decoder will refuse
+    // anyway takes the version 1 way.
+    uint8_t lead[8] = {0};
+    const bool typed = payload >= 8 && read_at(fd, lead, 8, tokens_end) == 8 &&
+                       (uint32_t(lead[4]) | uint32_t(lead[5]) << 8 | uint32_t(lead[6]) << 16 |
+                        uint32_t(lead[7]) << 24) == kItkvVersionTyped;
     uint64_t sum = 0;
-    if (read_at_with_checksum(fd, s->stage, payload, tokens_end, payload >= 8 ? payload - 8 : 0,
-                              &sum) != int64_t(payload))
+    const uint64_t sum_len = payload >= 8 ? payload - 8 : 0;
+    const int64_t arrived =
+        typed ? read_blocks_with_checksum(fd, s->stage, payload, tokens_end, sum_len, &sum)
+              : read_at_with_checksum(fd, s->stage, payload, tokens_end, sum_len, &sum);
+    if (arrived != int64_t(payload))
         return io_error(why, errno, "read entry %s", meta.file_name.c_str());
     ItkvHeader &h = s->stage_header;
     std::vector<ItkvLayer> &layers = s->stage_layers;
@@ -747,9 +786,9 @@ static itak_status put_entry(itak_store *store, const uint32_t *tokens, uint64_t
     bool summed = false;
     if (sum_here) {
         try {
-            summer = std::thread([&] { sum = fnv1a64(payload, body_len, kFnvOffset); });
+            summer = std::thread([&] { sum = itkv_trailer(h.version, payload, body_len); });
         } catch (...) {  // no thread to be had: the checksum runs here, before the write
-            sum = fnv1a64(payload, body_len, kFnvOffset);
+            sum = itkv_trailer(h.version, payload, body_len);
             summed = true;
         }
     }

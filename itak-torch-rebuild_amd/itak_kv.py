@@ -78,6 +78,13 @@ def checksum(data: bytes) -> int:  # hash.rs:59-61
     return int(N.load().itak_kv_checksum(buf.ctypes.data if buf.size else None, buf.size))
 
 
+def checksum_blocks(data: bytes) -> int:
+    """The trailer of snapshot version 2 (this library's own): FNV-1a over the FNV-1a sums of
+    consecutive 1 MiB blocks, which host threads share."""
+    buf = np.frombuffer(data, dtype=np.uint8)
+    return int(N.load().itak_kv_checksum_blocks(buf.ctypes.data if buf.size else None, buf.size))
+
+
 @dataclass
 class KvGeometry:
     """itak_kv::KvGeometry (snapshot.rs:57-138)."""

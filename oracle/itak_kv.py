@@ -310,14 +310,25 @@ class _Reader:  # snapshot.rs:520-604
 
 # ---- version 2 (typed rows): not the reference's, this build's own extension ---------------
 # v1 with one more u32 after the layer count, the element type of the rows (0 = f32,
-# 1 = f16 bits), and the rows in that type. Restated here independently of the library so
-# that its encoder and decoder have something to be held to; `KvSnapshot.from_bytes` above
-# stays the reference's reader and refuses version 2 by name.
+# 1 = f16 bits), the rows in that type, and a trailer that is FNV-1a over the FNV-1a sums of
+# consecutive 1 MiB blocks of the bytes before it (each sum as 8 little-endian bytes) instead
+# of over the bytes themselves. Restated here independently of the library so that its
+# encoder and decoder have something to be held to; `KvSnapshot.from_bytes` above stays the
+# reference's reader and refuses version 2 by name.
 
 TYPED_FORMAT_VERSION = 2
+SUM_BLOCK = 1 << 20
 
 
-def to_bytes_f16(snapshot: KvSnapshot) -> bytes:
+def block_checksum(data: bytes, block_sum=checksum) -> int:
+    """`block_sum` is FNV-1a 64 from the offset basis (hash.rs:59-61); the pure-Python one
+    above by default, any faster restatement of it for inputs of many blocks."""
+    sums = b"".join(struct.pack("<Q", block_sum(data[at:at + SUM_BLOCK]))
+                    for at in range(0, len(data), SUM_BLOCK))
+    return checksum(sums)
+
+
+def to_bytes_f16(snapshot: KvSnapshot, block_sum=checksum) -> bytes:
     """Version 2 with f16 rows. The snapshot's f32 values must be exactly representable in
     f16 (they are when captured from an f16-storing cache)."""
     snapshot.validate()
@@ -342,6 +353,6 @@ def to_bytes_f16(snapshot: KvSnapshot) -> bytes:
             assert np.array_equal(halves.astype(np.float32), np.asarray(side, dtype=np.float32)), \
                 "rows are not f16 values"
             out += halves.tobytes()
-    out += struct.pack("<Q", checksum(bytes(out)))
+    out += struct.pack("<Q", block_checksum(bytes(out), block_sum))
     return bytes(out)
 

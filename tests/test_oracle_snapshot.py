@@ -286,3 +286,60 @@ def test_library_validate_matches_the_oracle_on_in_memory_snapshots():
                           for i in range(52)], 2, 128)
     assert (g.bytes_per_token(), g.stored_bytes_for(4096), g.stored_bytes_for(131_072)) == \
         (106_496, 272_629_760, 3_653_238_784)
+
+
+# ---- version 2 on the host (this library's own format; no counterpart in the reference) ----
+
+def _fast_sum(data):  # FNV-1a 64 from the offset basis, the oracle's C restatement
+    return oracle.checksum(bytes(data))
+
+
+def test_block_checksum_is_the_sum_of_block_sums_at_every_boundary():
+    P = pkg()
+    rng = np.random.default_rng(2)
+    B = okv.SUM_BLOCK
+    assert P.checksum_blocks(b"") == okv.FNV_OFFSET == okv.block_checksum(b"")
+    for size in (1, 77, B - 1, B, B + 1, 2 * B, 3 * B + 5):
+        data = rng.integers(0, 256, size=size, dtype=np.uint8).tobytes()
+        want = okv.block_checksum(data, _fast_sum)
+        assert P.checksum_blocks(data) == want, size
+        if size <= B:  # one block: the sum of one sum, not the plain checksum
+            assert want == okv.checksum(struct.pack("<Q", _fast_sum(data)))
+            assert want != _fast_sum(data)
+    # Two blocks swapped, and a byte moved across a block edge, change it.
+    data = bytearray(rng.integers(0, 256, size=2 * B, dtype=np.uint8).tobytes())
+    swapped = bytes(data[B:]) + bytes(data[:B])
+    assert P.checksum_blocks(bytes(data)) != P.checksum_blocks(swapped)
+    assert _fast_sum(bytes(data[:77])) == okv.checksum(bytes(data[:77]))  # the C sum is the Python sum
+
+
+def test_a_version_2_snapshot_of_several_blocks_decodes_and_a_flip_in_any_block_is_refused():
+    P = pkg()
+    rng = np.random.default_rng(4)
+    kvh, d, rows = 2, 64, 2600  # 2600 x 128 halves x 2 sides: 1.3 MB, two blocks
+    geometry = okv.KvGeometry([oracle.LayerKind.Global, oracle.LayerKind.windowed(2600)], kvh, d)
+    layers = []
+    for _ in range(2):
+        k = rng.standard_normal(rows * kvh * d, dtype=np.float32).astype(np.float16).astype(np.float32)
+        v = rng.standard_normal(rows * kvh * d, dtype=np.float32).astype(np.float16).astype(np.float32)
+        layers.append(okv.LayerSnapshot(0, k, v))
+    snap = okv.KvSnapshot(geometry, "typed", rows, layers)
+    v2 = okv.to_bytes_f16(snap, _fast_sum)
+    assert len(v2) > 2 * okv.SUM_BLOCK
+    decoded = P.KvSnapshot.from_bytes(v2)
+    assert decoded.token_count == rows and decoded.model_fingerprint == "typed"
+    for got, want in zip(decoded.layers, layers):
+        assert got.keys.tobytes() == want.keys.tobytes()
+        assert got.values.tobytes() == want.values.tobytes()
+    assert P.KvSnapshot.from_bytes(snap.to_bytes()).layers[1].values.tobytes() == layers[1].values.tobytes()
+    for offset in (50, okv.SUM_BLOCK + 3, len(v2) - 9):
+        bad = bytearray(v2)
+        bad[offset] ^= 0x10
+        with pytest.raises(P.KvError) as e:
+            P.KvSnapshot.from_bytes(bytes(bad))
+        assert e.value.variant == "ChecksumMismatch", offset
+    # The version 1 trailer on version 2 bytes is refused: the two sums are different functions.
+    forged = v2[:-8] + struct.pack("<Q", _fast_sum(v2[:-8]))
+    with pytest.raises(P.KvError) as e:
+        P.KvSnapshot.from_bytes(forged)
+    assert e.value.variant == "ChecksumMismatch"

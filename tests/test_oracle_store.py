@@ -341,25 +341,33 @@ def test_library_and_oracle_write_identical_files_and_serve_each_other(tmp_path)
         assert (tmp_path / "o" / name).read_bytes() == (tmp_path / "l" / name).read_bytes()
 
 
-def test_a_payload_read_in_pieces_is_served_whole_and_a_flip_in_any_piece_is_refused(tmp_path):
-    """A payload larger than a few MB is read by a second thread while the checksum follows
-    it: what comes out is what went in, and one flipped bit in the first, a middle or the
-    last piece is still caught by name. (Library side only: the oracle's byte loop over
-    20 MB is what this path exists to avoid.)"""
+@pytest.mark.parametrize("version", [1, 2])
+def test_a_payload_read_in_pieces_is_served_whole_and_a_flip_in_any_piece_is_refused(tmp_path, version):
+    """A payload larger than a few MB is not read and then summed: version 1 is read by a
+    second thread while the byte-serial checksum follows it, version 2 (block sums) by several
+    threads that each sum what they read. What comes out is what went in, and one flipped bit
+    in the first, a middle or the last piece is still caught by name. (Library side only: the
+    oracle's byte loop over 20 MB is what this path exists to avoid.)"""
     rng = np.random.default_rng(3)
-    kvh, d, rows = 4, 128, 5000
+    kvh, d, rows = 4, 128, 5000 * version
     geometry = P().KvGeometry([P().LayerKind.Global], kvh, d)
-    keys = rng.standard_normal(rows * kvh * d, dtype=np.float32)
-    values = rng.standard_normal(rows * kvh * d, dtype=np.float32)
-    snap = P().KvSnapshot(geometry, "big", rows, [P().LayerSnapshot(0, keys, values)])
-    data = snap.to_bytes()
+    keys = rng.standard_normal(rows * kvh * d, dtype=np.float32).astype(np.float16).astype(np.float32)
+    values = rng.standard_normal(rows * kvh * d, dtype=np.float32).astype(np.float16).astype(np.float32)
+
+    def encode(n):
+        if version == 1:
+            return P().KvSnapshot(geometry, "big", n, [P().LayerSnapshot(0, keys[:n * kvh * d],
+                                                                         values[:n * kvh * d])]).to_bytes()
+        snap = okv.KvSnapshot(okv.KvGeometry([oracle.LayerKind.Global], kvh, d), "big", n,
+                              [okv.LayerSnapshot(0, keys[:n * kvh * d], values[:n * kvh * d])])
+        return okv.to_bytes_f16(snap, lambda block: oracle.checksum(bytes(block)))
+
+    data = encode(rows)
     assert len(data) > 20_000_000
     tokens = [int(t) for t in rng.integers(0, 1 << 20, size=rows)]
     short = tokens[:7]
-    small = P().KvSnapshot(geometry, "big", 7, [P().LayerSnapshot(0, keys[:7 * kvh * d],
-                                                                  values[:7 * kvh * d])])
     store = P().PrefixStore.open(str(tmp_path), 1 << 30)
-    store.put(short, small.to_bytes(), 1)
+    store.put(short, encode(7), 1)
     store.put(tokens, data, 2)
     hit = store.lookup(tokens + [5], geometry, "big", 3)
     assert hit.token_count == rows and hit.snapshot_bytes == data
