@@ -12,6 +12,9 @@ Prints one JSON line: decode-attention KV GB/s over the algorithmic KV bytes
 (2 * 4097 * 4 * 128 * 2 B per layer), with the roofline figures of the attention launches and
 the CPU oracle timed on the host cores beside it.
 
+`--prep` adds a second timing of the same step preceded by the model's Q/K preparation
+(per-head RMSNorm, RoPE) and followed by its sigmoid gate (`with_prep` in the JSON line).
+
 `--workload ragged|verify|prefill` measures the other configurations (continuous batching
 over 16 ragged slots, the speculative verify block, the chunked causal prefill) with the
 same JSON shape; `--workload hybrid` a decode step over the reference model's own layer
@@ -276,6 +279,9 @@ def main():
                                            "restore", "append"], default="decode")
     ap.add_argument("--softcap", type=float, default=0.0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--prep", action="store_true",
+                    help="also time the step with the fused Q/K preparation (per-head RMSNorm + "
+                         "RoPE) before it and the sigmoid gate after it, reported as 'with_prep'")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)",
@@ -396,6 +402,42 @@ def main():
     attn_s = timed(g_attn.replay, args.steps)[0] / (args.steps * layers)
     pool.truncate(caches, lengths)
 
+    with_prep = None
+    if args.prep and wl != "prefill":
+        # The model's own sequence around the step (muse-glimmer/src/model.rs:445-464): raw
+        # projections -> per-head RMSNorm -> interleaved RoPE on sliding-window layers (global
+        # layers carry no rotation) -> append + attention -> out * sigmoid(gate).
+        qw, kw = torch.rand(D, device=dev) + 0.5, torch.rand(D, device=dev) + 0.5
+        gate = torch.randn(layers, total_rows, Q_HEADS * D, device=dev)
+
+        def prep_step():
+            for layer in range(layers):
+                qp, kp, vp, op = ptrs[layer]
+                pool.attention_prep_step_device(
+                    layer, items, qp, kp, vp, op, Q_HEADS, q_norm_ptr=qw.data_ptr(),
+                    k_norm_ptr=kw.data_ptr(), eps=1e-6,
+                    rope_base=1e4 if pattern[layer].is_windowed else 0.0, interleaved=True,
+                    gate_ptr=gate[layer].data_ptr(), softcap=args.softcap)
+            pool.truncate(caches, lengths)
+
+        for _ in range(max(args.warmup, 1)):
+            prep_step()
+        g_prep = capture(torch, pool, stream, prep_step)
+        for _ in range(max(args.warmup, 1)):
+            g_prep.replay()
+        prep_s = timed(g_prep.replay, args.steps)[0] / args.steps
+        folded = rows * (Q_HEADS // KV_HEADS) <= 16
+        with_prep = {
+            "us_per_layer": round(prep_s / layers * 1e6, 3),
+            "added_us_per_layer": round((prep_s - step_s) / layers * 1e6, 3),
+            "launches_added_per_layer": 0 if folded else 1,
+            "what": ("RMSNorm + RoPE of Q and of the new K row inside the split-K kernel, the gate "
+                     "in the kernel that writes the output: the step's own two launches"
+                     if folded else
+                     "attn_prep_kernel (RMSNorm + RoPE of Q and K, one launch) before the fused "
+                     "append + attention; the gate in the merge kernel"),
+        }
+
     if wl == "prefill":
         metric, unit = "prefill attention TFLOP/s (2048-row chunk over 30720 prefix)", "TFLOP/s"
         value = flops_layer * layers / step_s / 1e12
@@ -458,6 +500,8 @@ def main():
         "device_probes": probe,
         "roofline": roofline,
     }
+    if with_prep is not None:
+        result["with_prep"] = with_prep
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(4096, 2 * 4097 * KV_HEADS * D * 2, 48)
     print(json.dumps(result))

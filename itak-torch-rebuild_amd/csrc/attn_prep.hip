@@ -100,12 +100,6 @@ __global__ __launch_bounds__(kPrepWaves * 64) void attn_prep_kernel(PrepArgs a) 
     }
 }
 
-__device__ __forceinline__ float sigmoid_ref(float x) {  // cpu.rs:162-169
-    if (x >= 0.0f) return 1.0f / (1.0f + expf(-x));
-    const float e = expf(x);
-    return e / (1.0f + e);
-}
-
 __global__ __launch_bounds__(256) void attn_gate_kernel(float *__restrict__ out,
                                                         const float *__restrict__ gate,
                                                         uint64_t count) {

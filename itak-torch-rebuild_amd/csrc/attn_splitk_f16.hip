@@ -237,9 +237,93 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
 // bookkeeping the epilogue needs is computed in the shadow of the loads.
 // RING = the layer is windowed: blocks start at the window, live in a ring, and the mask has a
 // lower edge. Global layers run the instantiation without any of it.
-template <int NQ, int WAVES, int N, bool RING>
-__global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams p, AttnBatchT<N> b,
-                                                                     uint32_t total_partials) {
+// ---- preparation folded into the step (PREP instantiations) -----------------------------
+// The reference's model norms and rotates Q and K between their projections and attention
+// (per-head RMSNorm, crates/torch-math/src/norm.rs:40-51; RoPE, rope_interleaved.rs:103-114 /
+// rope.rs:99-114; order of calls crates/muse-glimmer/src/model.rs:445-451). A decode step is a
+// few thousand elements, so as a launch of its own that work costs a launch; here every
+// workgroup prepares the 16 query vectors it stages anyway, and the workgroup that appends
+// the new K rows prepares those. A 128-channel head row lies across 32 consecutive lanes, four
+// channels each (c4 = 4 * (lane % 32)), which is how Q and the new rows are loaded.
+//
+// Arithmetic: the angle position * base^(-2i/rot) is formed and reduced to [-pi, pi] in f64
+// (an f32 angle is off by 8e-3 rad at position 100,000); norm, sine, cosine and rotation are
+// f32. The results feed f16 storage and f16 MFMA operands, so they differ from the
+// reference's f64 chain by parts in 1e7 before that rounding: at most one f16 step after it.
+struct PrepTrig {
+    float c[4], s[4];  // per pair held by this lane: 2 (interleaved) or 4 (half split)
+};
+
+__device__ __forceinline__ void prep_trig(PrepTrig &t, double position, const double (&freq)[4],
+                                          int pairs) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (i >= pairs) break;
+        // The angle in turns, reduced to [-1/2, 1/2] exactly in f64; the sine and cosine
+        // instructions take turns. Their error (about 1e-6 absolute) is a five-hundredth of
+        // the f16 step the results are rounded to.
+        const double turns = position * freq[i] * 0.15915494309189535;
+        const float frac = float(turns - rint(turns));
+        t.s[i] = __builtin_amdgcn_sinf(frac);
+        t.c[i] = __builtin_amdgcn_cosf(frac);
+    }
+}
+
+// Sum over the 32 lanes that share a head row: four DPP steps inside each row of 16 lanes
+// (neighbour, other pair, mirrored half, mirrored row), then the row 16 lanes away.
+template <int CTRL>
+__device__ __forceinline__ float dpp_lane(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float row_sum32(float v) {
+    v += dpp_lane<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_lane<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_lane<0x141>(v);  // row_half_mirror
+    v += dpp_lane<0x140>(v);  // row_mirror
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(a[0]) + __uint_as_float(a[1]);
+}
+
+// x = channels c4 .. c4+3 of a head row, w = the norm weight's same channels.
+__device__ __forceinline__ float4 prep_chunk(float4 x, bool norm, float4 w, float eps, uint32_t c4,
+                                             uint32_t lane, uint32_t rot, bool interleaved,
+                                             const PrepTrig &t) {
+    if (norm) {
+        const float ss = row_sum32(x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w);
+        const float inv = __builtin_amdgcn_rsqf(ss * (1.0f / kD) + eps);
+        x = make_float4(x.x * inv * w.x, x.y * inv * w.y, x.z * inv * w.z, x.w * inv * w.w);
+    }
+    if (rot == 0) return x;
+    if (interleaved) {  // pairs (c4, c4+1) and (c4+2, c4+3)
+        float4 y = x;
+        if (c4 < rot) {
+            y.x = x.x * t.c[0] - x.y * t.s[0];
+            y.y = x.x * t.s[0] + x.y * t.c[0];
+        }
+        if (c4 + 2 < rot) {
+            y.z = x.z * t.c[1] - x.w * t.s[1];
+            y.w = x.z * t.s[1] + x.w * t.c[1];
+        }
+        return y;
+    }
+    // Half split: channel c < rot/2 turns with channel c + rot/2, four lanes-of-four apart.
+    const uint32_t half = rot >> 1;
+    const bool low = c4 < half, turn = c4 < rot;
+    const uint32_t partner = (lane & 32u) | (((lane & 31u) + (low ? half / 4 : 32u - half / 4)) & 31u);
+    const float4 o = make_float4(__shfl(x.x, partner), __shfl(x.y, partner), __shfl(x.z, partner),
+                                 __shfl(x.w, partner));
+    if (!turn) return x;
+    if (low)
+        return make_float4(x.x * t.c[0] - o.x * t.s[0], x.y * t.c[1] - o.y * t.s[1],
+                           x.z * t.c[2] - o.z * t.s[2], x.w * t.c[3] - o.w * t.s[3]);
+    return make_float4(o.x * t.s[0] + x.x * t.c[0], o.y * t.s[1] + x.y * t.c[1],
+                       o.z * t.s[2] + x.z * t.c[2], o.w * t.s[3] + x.w * t.c[3]);
+}
+
+template <int NQ, int WAVES, int N, bool RING, bool PREP>
+__device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const AttnBatchT<N> &b,
+                                                     uint32_t total_partials,
+                                                     [[maybe_unused]] const FoldedParams &fold) {
     extern __shared__ float lds[];
     float *sm_m = lds;                          // [WAVES][NQ*16]
     float *sm_l = sm_m + WAVES * NQ * 16;       // [WAVES][NQ*16]
@@ -267,6 +351,9 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
                      "s"(b.item[0].keys_per_split), "s"(b.item[0].block0), "s"(b.item[0].ws0),
                      "s"(b.item[0].splits_magic), "s"(b.item[0].kv_lo), "s"(p.window),
                      "s"(p.ring_blocks));
+    if (N == 1 && PREP)
+        asm volatile("" ::"s"(fold.prep_q_weight), "s"(fold.prep_k_weight), "s"(fold.prep_eps),
+                     "s"(fold.prep_rot), "s"(fold.prep_interleaved), "s"(fold.prep_freq_step), "s"(fold.gate));
     const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
     const uint32_t local = blockIdx.x - item.block0;
     const uint32_t kv_head = item.splits > 1 ? __umulhi(local, item.splits_magic) : local;
@@ -324,6 +411,14 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
             p.q + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + c4);
     }
 
+    // PREP: the norm weights of this lane's four channels (Q's and K's), issued with Q.
+    const uint32_t pc4 = (tid & 31u) * 4;
+    [[maybe_unused]] float4 wq = make_float4(1.f, 1.f, 1.f, 1.f), wk = wq;
+    if constexpr (PREP) {
+        if (fold.prep_q_weight) wq = *reinterpret_cast<const float4 *>(fold.prep_q_weight + pc4);
+        if (fold.prep_k_weight) wk = *reinterpret_cast<const float4 *>(fold.prep_k_weight + pc4);
+    }
+
     // ---- 3. the wavefront's first block (a wavefront without one loads the split's first
     // block and ignores it).
     BlockOperands buf_a;
@@ -351,6 +446,26 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
     const float softcap = p.softcap;
     const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
     const float qscale = softcap > 0.0f ? p.scale : p.scale * kLog2e;
+    // PREP: this lane's pairs and their rotation at the step's first position, still in the
+    // shadow of the loads (nothing here depends on what they bring).
+    [[maybe_unused]] PrepTrig trig0;
+    [[maybe_unused]] double freq[4] = {0.0, 0.0, 0.0, 0.0};
+    [[maybe_unused]] int trig_pairs = 0;
+    const uint32_t prot = PREP ? fold.prep_rot : 0;
+    const bool pinter = PREP && fold.prep_interleaved != 0;
+    if constexpr (PREP) {
+        if (prot) {
+            const uint32_t half = prot >> 1;
+            // First pair index of this lane: interleaved pairs are (2i, 2i+1); half-split pair i
+            // joins channels i and i + rot/2.
+            const uint32_t pair0 = pinter ? pc4 >> 1 : (pc4 < half ? pc4 : pc4 - half);
+            trig_pairs = pinter ? 2 : 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (i < trig_pairs) freq[i] = exp2(double(pair0 + i) * fold.prep_freq_step);
+            prep_trig(trig0, double(item.pos0), freq, trig_pairs);
+        }
+    }
     ITAK_MARK(3)
 
     // ---- 5. stage Q^T (scaled, f16) and the new rows (f16, also stored to the planes).
@@ -358,7 +473,13 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
     for (int u = 0; u < QL; ++u) {
         const uint32_t f = tid + u * WAVES * 64;
         const uint32_t j = f >> 5, c4 = (f & 31) * 4;
-        const float4 a = qld[u];
+        float4 a = qld[u];
+        if constexpr (PREP) {
+            const uint32_t jr = min(j, nvec - 1), row = (jr * magic) >> 16;
+            PrepTrig t = trig0;
+            if (prot && row != 0) prep_trig(t, double(item.pos0 + row), freq, trig_pairs);
+            a = prep_chunk(a, fold.prep_q_weight != nullptr, wq, fold.prep_eps, c4, lane, prot, pinter, t);
+        }
         half4 h{static_cast<_Float16>(a.x * qscale), static_cast<_Float16>(a.y * qscale),
                 static_cast<_Float16>(a.z * qscale), static_cast<_Float16>(a.w * qscale)};
         if (j >= nvec) h = half4{0, 0, 0, 0};
@@ -369,8 +490,15 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
         for (int u = 0; u < NL; ++u) {
             const uint32_t f = tid + u * WAVES * 64;
             const uint32_t r = f >> 6, side = (f >> 5) & 1, c4 = (f & 31) * 4;
+            float4 a = nreg[u];
+            if constexpr (PREP) {  // lanes 0..31 of a wavefront hold a K row, 32..63 its V row
+                PrepTrig t = trig0;
+                if (prot && r != 0 && r < item.rows) prep_trig(t, double(item.pos0 + r), freq, trig_pairs);
+                const float4 k = prep_chunk(a, fold.prep_k_weight != nullptr, wk, fold.prep_eps, c4, lane, prot,
+                                            pinter, t);
+                if (side == 0) a = k;
+            }
             if (r >= item.rows) continue;
-            const float4 a = nreg[u];
             const uint16_t h0 = f32_to_f16_bits(a.x), h1 = f32_to_f16_bits(a.y);
             const uint16_t h2 = f32_to_f16_bits(a.z), h3 = f32_to_f16_bits(a.w);
             uint2 packed{uint32_t(h0) | (uint32_t(h1) << 16), uint32_t(h2) | (uint32_t(h3) << 16)};
@@ -507,6 +635,12 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
 #pragma unroll
             for (int w = 1; w < WAVES; ++w) acc += ow[x][w] * wgt[w];
             acc *= post;
+            if (PREP && final_out && fold.gate) {
+                const float4 gt = *reinterpret_cast<const float4 *>(
+                    fold.gate + uint64_t(colout[qt]) * kD + (wave * kDtPerWave + x) * 16 + g * 4);
+                acc = floatx4{acc[0] * sigmoid_fast(gt.x), acc[1] * sigmoid_fast(gt.y),
+                              acc[2] * sigmoid_fast(gt.z), acc[3] * sigmoid_fast(gt.w)};
+            }
             *reinterpret_cast<floatx4 *>(dst + (wave * kDtPerWave + x) * 16 + g * 4) = acc;
         }
         if (!final_out && wave == 0 && g == 0)
@@ -514,6 +648,20 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
     }
     ITAK_MARK(9)
     ITAK_MARK_END
+}
+
+template <int NQ, int WAVES, int N, bool RING>
+__global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams p, AttnBatchT<N> b,
+                                                                     uint32_t total_partials) {
+    attn_splitk_f16_body<NQ, WAVES, N, RING, false>(p, b, total_partials, FoldedParams{});
+}
+// The 16-vector variants with the preparation and the gate folded in.
+template <int WAVES, int N, bool RING>
+__global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_prep_kernel(AttnParams p,
+                                                                          AttnBatchT<N> b,
+                                                                          uint32_t total_partials,
+                                                                          FoldedParams f) {
+    attn_splitk_f16_body<1, WAVES, N, RING, true>(p, b, total_partials, f);
 }
 
 }  // namespace
@@ -547,22 +695,30 @@ static size_t variant_lds(int nq, int waves) {
     return (size_t(2) * waves * nq * 16 + size_t(waves) * nq * 8 * 64 * 4) * 4 +
            size_t(nq) * 16 * kQStride * 2 + size_t(2) * kMaxNewRows * kNewStride * 2;
 }
-template <int NQ, int W>
+template <int NQ, int W, bool PREP = false>
 static hipError_t grant_lds(size_t lds) {
     static size_t granted = 64 * 1024;
     if (lds <= granted) return hipSuccess;
     // The attribute is per kernel function: set it on each batch-size instantiation.
-    const void *kernels[] = {
+    const void *plain[] = {
         reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 1, false>),
         reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 8, false>),
         reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 64, false>),
         reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 1, true>),
         reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 8, true>),
         reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 64, true>)};
+    const void *prepping[] = {
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<W, 1, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<W, 8, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<W, 64, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<W, 1, true>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<W, 8, true>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<W, 64, true>)};
+    const void *const *kernels = PREP ? prepping : plain;
     hipError_t e = hipSuccess;
-    for (const void *k : kernels)
+    for (int k = 0; k < 6; ++k)
         if (e == hipSuccess)
-            e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+            e = hipFuncSetAttribute(kernels[k], hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
     if (e == hipSuccess) granted = lds;
     return e;
 }
@@ -636,10 +792,13 @@ uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads)
 }
 
 hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
-                                  uint32_t max_rows, hipStream_t stream) {
+                                  uint32_t max_rows, hipStream_t stream,
+                                  const FoldedParams *folded) {
     (void)max_rows;
     if (b.total_blocks == 0) return hipSuccess;
     const Variant v = pick_variant(p.g, b, p.group);
+    const bool prep = folded && folded->prep_on;
+    if (prep && v.nq != 1) return hipErrorInvalidValue;
 #define ITAK_LAUNCH(NQ, W)                                                                \
     do {                                                                                  \
         const size_t lds = variant_lds(NQ, W);                                            \
@@ -652,17 +811,32 @@ hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint3
             attn_splitk_f16_kernel<NQ, W, N, false><<<b.total_blocks, W * 64, lds, stream>>>( \
                 p, AttnBatchT<N>(b), total_partials);                                     \
     } while (0)
-#define ITAK_LAUNCH_NQ()               \
-    do {                               \
-        switch (v.index) {             \
-            case 0: ITAK_LAUNCH(1, 4); break; \
-            case 1: ITAK_LAUNCH(1, 8); break; \
-            case 2: ITAK_LAUNCH(2, 4); break; \
-            default: ITAK_LAUNCH(4, 4); break; \
-        }                              \
+#define ITAK_LAUNCH_PREP(W)                                                               \
+    do {                                                                                  \
+        const size_t lds = variant_lds(1, W);                                             \
+        hipError_t e = grant_lds<1, W, true>(lds);                                        \
+        if (e != hipSuccess) return e;                                                    \
+        if (p.ring_blocks)                                                                \
+            attn_splitk_f16_prep_kernel<W, N, true><<<b.total_blocks, W * 64, lds, stream>>>( \
+                p, AttnBatchT<N>(b), total_partials, *folded);                            \
+        else                                                                              \
+            attn_splitk_f16_prep_kernel<W, N, false><<<b.total_blocks, W * 64, lds, stream>>>( \
+                p, AttnBatchT<N>(b), total_partials, *folded);                            \
+    } while (0)
+#define ITAK_LAUNCH_NQ()                                  \
+    do {                                                  \
+        switch (v.index + (prep ? 4 : 0)) {               \
+            case 0: ITAK_LAUNCH(1, 4); break;             \
+            case 1: ITAK_LAUNCH(1, 8); break;             \
+            case 2: ITAK_LAUNCH(2, 4); break;             \
+            case 3: ITAK_LAUNCH(4, 4); break;             \
+            case 4: ITAK_LAUNCH_PREP(4); break;           \
+            default: ITAK_LAUNCH_PREP(8); break;          \
+        }                                                 \
     } while (0)
     ITAK_DISPATCH_BATCH(b.n, ITAK_LAUNCH_NQ());
 #undef ITAK_LAUNCH_NQ
+#undef ITAK_LAUNCH_PREP
 #undef ITAK_LAUNCH
     return hipGetLastError();
 }
@@ -680,7 +854,8 @@ template <int N>
 __global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(AttnParams p,
                                                                        AttnBatchT<N> b,
                                                                        uint32_t total_partials,
-                                                                       int base2) {
+                                                                       int base2,
+                                                                       const float *gate) {
     __shared__ float w_s[1024];
     __shared__ float red[8];
     __shared__ float4 part[kCombineThreads];
@@ -737,7 +912,7 @@ __global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(AttnParam
         for (uint32_t d = tid; d < D; d += kCombineThreads) {
             float acc = 0.0f;
             for (uint32_t s = 0; s < S; ++s) acc = fmaf(ws_acc[uint64_t(s) * D + d], w_s[s], acc);
-            dst[d] = acc * inv;
+            dst[d] = acc * inv * (gate ? sigmoid_fast(gate[(dst - p.out) + d]) : 1.0f);
         }
         return;
     }
@@ -781,8 +956,13 @@ __global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(AttnParam
             sum.z += y.z;
             sum.w += y.w;
         }
-        *reinterpret_cast<float4 *>(dst + tid * 4) =
-            make_float4(sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv);
+        float4 o = make_float4(sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv);
+        if (gate) {
+            const float4 gt = *reinterpret_cast<const float4 *>(gate + (dst - p.out) + tid * 4);
+            o = make_float4(o.x * sigmoid_fast(gt.x), o.y * sigmoid_fast(gt.y),
+                            o.z * sigmoid_fast(gt.z), o.w * sigmoid_fast(gt.w));
+        }
+        *reinterpret_cast<float4 *>(dst + tid * 4) = o;
     }
 }
 
@@ -791,9 +971,10 @@ __global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(AttnParam
 // A thread issues every load of its first 8 splits, accumulators and (m, l) pairs alike,
 // before it waits for anything, folds them with its own running maximum, and the eight
 // split lanes meet once in LDS. One memory round trip and one barrier.
-template <int N, bool BASE2>
-__global__ __launch_bounds__(256) void attn_combine128_kernel(AttnParams p, AttnBatchT<N> b,
-                                                              uint32_t total_partials) {
+template <int N, bool BASE2, bool GATE>
+__device__ __forceinline__ void attn_combine128_body(const AttnParams &p, const AttnBatchT<N> &b,
+                                                     uint32_t total_partials,
+                                                     [[maybe_unused]] const float *gate) {
     __shared__ float4 part[256];
     __shared__ float part_m[8], part_l[8];
     const uint32_t tid = threadIdx.x;
@@ -804,6 +985,7 @@ __global__ __launch_bounds__(256) void attn_combine128_kernel(AttnParams p, Attn
         asm volatile("" ::"s"(p.out), "s"(p.ws), "s"(p.q_heads), "s"(total_partials),
                      "s"(b.base_row), "s"(b.item[0].q_row0), "s"(b.item[0].splits),
                      "s"(b.item[0].ws0));
+    if (N == 1 && GATE) asm volatile("" ::"s"(gate));
     const AttnItem item = b.item[b.find_by_row(grow)];
     const uint32_t S = item.splits;
     if (S == 1) return;
@@ -812,6 +994,11 @@ __global__ __launch_bounds__(256) void attn_combine128_kernel(AttnParams p, Attn
     const uint32_t c = tid & 31, sl = tid >> 5;
     const float *ws_acc = p.ws + ps0 * 128 + c * 4;
     const float2 *ws_ml = reinterpret_cast<const float2 *>(p.ws + uint64_t(total_partials) * 128) + ps0;
+    // The gate of the 32 threads that write the output, fetched with the partials.
+    [[maybe_unused]] float4 gt = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (GATE && tid < 32)
+        gt = *reinterpret_cast<const float4 *>(
+            gate + (uint64_t(item.q_row0 + row) * p.q_heads + head) * 128 + tid * 4);
     ITAK_MARK(1)
 
     float m_run = -INFINITY, l_run = 0.0f;
@@ -874,21 +1061,42 @@ __global__ __launch_bounds__(256) void attn_combine128_kernel(AttnParams p, Attn
         }
         const float inv = 1.0f / L;
         float *dst = p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * 128;
-        *reinterpret_cast<float4 *>(dst + tid * 4) =
-            make_float4(sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv);
+        float4 o = make_float4(sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv);
+        if (GATE)
+            o = make_float4(o.x * sigmoid_fast(gt.x), o.y * sigmoid_fast(gt.y),
+                            o.z * sigmoid_fast(gt.z), o.w * sigmoid_fast(gt.w));
+        *reinterpret_cast<float4 *>(dst + tid * 4) = o;
     }
     ITAK_MARK(9)
     ITAK_MARK_END2
 }
+template <int N, bool BASE2>
+__global__ __launch_bounds__(256) void attn_combine128_kernel(AttnParams p, AttnBatchT<N> b,
+                                                              uint32_t total_partials) {
+    attn_combine128_body<N, BASE2, false>(p, b, total_partials, nullptr);
+}
+// The same merge whose writers multiply by sigmoid(gate) (cpu.rs:657-673).
+template <int N, bool BASE2>
+__global__ __launch_bounds__(256) void attn_combine128_gate_kernel(AttnParams p, AttnBatchT<N> b,
+                                                                   uint32_t total_partials,
+                                                                   const float *gate) {
+    attn_combine128_body<N, BASE2, true>(p, b, total_partials, gate);
+}
 
 hipError_t launch_attn_combine(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
-                               uint32_t total_rows, int base2, hipStream_t stream) {
+                               uint32_t total_rows, int base2, hipStream_t stream, const float *gate) {
     bool any = false;
     for (uint32_t i = 0; i < b.n; ++i) any = any || b.item[i].splits > 1;
     if (!any || total_rows == 0) return hipSuccess;
     if (p.g.head_dim == 128) {
         const dim3 grid(p.q_heads, total_rows);
-        if (base2)
+        if (gate && base2)
+            ITAK_DISPATCH_BATCH(b.n, (attn_combine128_gate_kernel<N, true><<<grid, 256, 0, stream>>>(
+                                         p, AttnBatchT<N>(b), total_partials, gate)));
+        else if (gate)
+            ITAK_DISPATCH_BATCH(b.n, (attn_combine128_gate_kernel<N, false><<<grid, 256, 0, stream>>>(
+                                         p, AttnBatchT<N>(b), total_partials, gate)));
+        else if (base2)
             ITAK_DISPATCH_BATCH(b.n, (attn_combine128_kernel<N, true><<<grid, 256, 0, stream>>>(
                                          p, AttnBatchT<N>(b), total_partials)));
         else
@@ -898,7 +1106,7 @@ hipError_t launch_attn_combine(const AttnParams &p, const AttnBatch &b, uint32_t
     }
     ITAK_DISPATCH_BATCH(b.n, (attn_combine_kernel<N><<<total_rows * p.q_heads, kCombineThreads, 0,
                                                       stream>>>(p, AttnBatchT<N>(b), total_partials,
-                                                                base2)));
+                                                                base2, gate)));
     return hipGetLastError();
 }
 

@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <math.h>
 #include <stdint.h>
 
 namespace itak {
@@ -278,6 +279,34 @@ struct AttnParams {
     uint32_t window;        // attention window of the layer (cache.rs:36-48); 0 = global
     uint32_t ring_blocks;   // 32-row blocks of the layer's storage ring; 0 = rows are positions
 };
+// What the reference's model does around the step (muse-glimmer/src/model.rs:445-464),
+// folded into the step's own launches instead of running as launches of their own. `gate`
+// (out *= sigmoid(gate), cpu.rs:657-673) is applied by whichever kernel writes the final
+// output; `prep_on` makes the split-K kernel norm and rotate the raw Q rows and new K rows it
+// reads (its 16-vector variants only). A separate kernel argument, so that launches without
+// any of it carry and fetch nothing more.
+struct FoldedParams {
+    const float *gate;          // [sum rows][q_heads*head_dim] or null
+    uint32_t prep_on;
+    uint32_t prep_interleaved;  // 1: pairs (2i, 2i+1); 0: pairs (i, i + prep_rot/2)
+    uint32_t prep_rot;          // rotary_dim; 0 = no rotation
+    float prep_eps;
+    const float *prep_q_weight; // [head_dim] or null: no norm
+    const float *prep_k_weight;
+    double prep_freq_step;      // pair i turns at position * 2^(i * prep_freq_step) radians
+};
+// sigmoid for the writers of f16-KV attention output, whose bar is 2e-3: one exponential
+// and one reciprocal instruction, a few ulp, the same limits at both ends (0 and 1) as the
+// reference's two-branch form (cpu.rs:162-169).
+__device__ __forceinline__ float sigmoid_fast(float x) {
+    return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
+}
+// sigmoid as the reference writes it (cpu.rs:162-169).
+__device__ __forceinline__ float sigmoid_ref(float x) {
+    if (x >= 0.0f) return 1.0f / (1.0f + expf(-x));
+    const float e = expf(x);
+    return e / (1.0f + e);
+}
 // The oldest position a query at `pos` sees (attention.rs:77-85 and the view's oldest row).
 __host__ __device__ inline uint32_t lowest_visible(uint32_t pos, uint32_t window, uint32_t kv_lo) {
     const uint32_t lo = (window != 0 && pos + 1 > window) ? pos + 1 - window : 0;
@@ -297,8 +326,11 @@ uint32_t attn_generic_tile(uint32_t head_dim);
 // Partials are in log2 domain (combine with base2 = 1).
 bool attn_splitk_f16_supports(const PoolGeom &g, uint32_t group, uint32_t max_rows);
 uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads);
+// `folded` with prep_on set selects the variants that prepare Q and the new K rows themselves
+// and gate what they write (every item must then be a 16-vector step); otherwise it is ignored.
 hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
-                                  uint32_t max_rows, hipStream_t stream);
+                                  uint32_t max_rows, hipStream_t stream,
+                                  const FoldedParams *folded = nullptr);
 // MFMA block path (speculative blocks and prefill chunks): same pools, any number of rows,
 // group dividing 16; K/V staged through LDS, split over the context when the launch would
 // otherwise not fill the device. Partials are in log2 domain (combine with base2 = 1).
@@ -307,8 +339,11 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
                                uint32_t window);
 hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                    hipStream_t stream);
-// Merge of split partials; total_rows = query rows of the batch.
+// Merge of split partials; total_rows = query rows of the batch. With `gate` the merged rows
+// are multiplied by sigmoid(gate) as they are written (items with one split are not touched:
+// their writer was the attention kernel).
 hipError_t launch_attn_combine(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
-                               uint32_t total_rows, int base2, hipStream_t stream);
+                               uint32_t total_rows, int base2, hipStream_t stream,
+                               const float *gate = nullptr);
 
 }  // namespace itak

@@ -311,7 +311,8 @@ bool takes_splitk_f16(const itak_pool *pool, const PlanInput *in, uint32_t n, ui
 itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, uint32_t n,
                           const float *q_dev, float *out_dev, const uint32_t *q_pos_dev,
                           uint64_t q_heads, float scale, float softcap,
-                          const float *k_new = nullptr, const float *v_new = nullptr) {
+                          const float *k_new = nullptr, const float *v_new = nullptr,
+                          const FoldedParams *folded = nullptr) {
     const uint32_t group = uint32_t(q_heads / pool->g.kv_heads);
     uint32_t max_rows = 0;
     for (uint32_t i = 0; i < n; ++i) max_rows = std::max(max_rows, in[i].rows);
@@ -398,8 +399,18 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         p.group_magic = (65536u + group - 1) / group;
         p.scale = scale;
         p.softcap = softcap;
+        // The gate is applied by whoever writes the output: the merge for items of several
+        // splits; for items of one split the split-K kernel, which only its preparing
+        // variants can; otherwise a launch of its own over the chunk's rows.
+        const float *gate = folded ? folded->gate : nullptr;
+        const bool prepares = folded && folded->prep_on && mfma;
+        bool merged_only = mfma || prefill;
+        for (uint32_t i = 0; i < count; ++i) merged_only = merged_only && b.item[i].splits > 1;
+        const bool gate_folded = gate && (prepares || (mfma && merged_only));
         if (mfma) {
-            HIP_TRY(pool, launch_attn_splitk_f16(p, b, partials, max_rows, pool->stream),
+            HIP_TRY(pool,
+                    launch_attn_splitk_f16(p, b, partials, max_rows, pool->stream,
+                                           prepares ? folded : nullptr),
                     "launch split-K attention");
         } else if (prefill) {
             HIP_TRY(pool, launch_attn_prefill_f16(p, b, partials, pool->stream),
@@ -409,8 +420,14 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
                     "launch attention");
         }
         HIP_TRY(pool, launch_attn_combine(p, b, partials, total_rows, (mfma || prefill) ? 1 : 0,
-                                          pool->stream),
+                                          pool->stream, gate_folded ? gate : nullptr),
                 "launch split merge");
+        if (gate && !gate_folded) {
+            const uint64_t q_width = q_heads * pool->g.head_dim;
+            const uint64_t at = uint64_t(q_row0 - total_rows) * q_width;
+            HIP_TRY(pool, launch_attn_gate(out_dev + at, gate + at, total_rows * q_width, pool->stream),
+                    "launch attention gate");
+        }
     }
     return ITAK_OK;
 }
@@ -1686,7 +1703,7 @@ static itak_status step_on_device(itak_pool *pool, uint64_t layer, const itak_ba
                                   uint32_t item_count, const std::vector<PlanInput> &plan,
                                   const float *q_dev, const float *k_dev, const float *v_dev,
                                   float *out_dev, uint64_t num_q_heads, float scale,
-                                  float softcap) {
+                                  float softcap, const FoldedParams *folded = nullptr) {
     // Rows of zero-row items contribute nothing; q/k/v rows are numbered by walking the
     // items in order, so such items may simply be dropped.
     std::vector<PlanInput> active;
@@ -1698,12 +1715,12 @@ static itak_status step_on_device(itak_pool *pool, uint64_t layer, const itak_ba
         for (uint32_t i = 0; i < item_count; ++i)
             advance(pool->slots[items[i].slot], layer, items[i].rows);
         return run_attention(pool, layer, active.data(), uint32_t(active.size()), q_dev, out_dev,
-                             nullptr, num_q_heads, scale, softcap, k_dev, v_dev);
+                             nullptr, num_q_heads, scale, softcap, k_dev, v_dev, folded);
     }
     itak_status st = run_append(pool, layer, items, item_count, k_dev, v_dev);
     if (st != ITAK_OK) return st;
     return run_attention(pool, layer, active.data(), uint32_t(active.size()), q_dev, out_dev,
-                         nullptr, num_q_heads, scale, softcap);
+                         nullptr, num_q_heads, scale, softcap, nullptr, nullptr, folded);
 }
 
 // Validates one batched step and returns the per-item plan (positions before the append).
@@ -1790,6 +1807,36 @@ itak_status itak_attention_prep_step_device(itak_pool *pool, uint64_t layer,
     for (const PlanInput &p : plan) total_rows += p.rows;
     if (total_rows == 0) return ITAK_OK;
     const uint64_t q_width = num_q_heads * D, k_width = pool->row;
+    if (std::isnan(scale)) scale = default_scale(D);
+    // Steps the split-K kernel takes have the gate applied by the kernel that writes the
+    // output, and, when every item is a 16-vector step (decode, short blocks), Q and K
+    // prepared by the split-K kernel itself: no launch but the step's own two.
+    std::vector<PlanInput> active;
+    uint32_t max_rows = 0;
+    for (const PlanInput &p : plan)
+        if (p.rows) {
+            active.push_back(p);
+            max_rows = std::max(max_rows, p.rows);
+        }
+    const bool splitk = takes_splitk_f16(pool, active.data(), uint32_t(active.size()), num_q_heads,
+                                         nullptr);
+    const uint32_t group = uint32_t(num_q_heads / pool->g.kv_heads);
+    const bool interleaved = prep->rope_interleaved != 0;
+    const bool folds = splitk && max_rows * group <= 16 && (!rotate || interleaved || rotary % 8 == 0);
+    FoldedParams folded{};
+    folded.gate = gate_dev;
+    if (folds) {
+        folded.prep_on = 1;
+        folded.prep_interleaved = interleaved ? 1 : 0;
+        folded.prep_rot = rotate ? rotary : 0;
+        folded.prep_eps = prep->eps;
+        folded.prep_q_weight = prep->q_norm_weight;
+        folded.prep_k_weight = prep->k_norm_weight;
+        // Pair i turns at position * base^(-2i/rot) = position * 2^(i * step).
+        folded.prep_freq_step = rotate ? -2.0 * std::log2(double(prep->rope_base)) / double(rotary) : 0.0;
+        return step_on_device(pool, layer, items, item_count, plan, q_dev, k_dev, v_dev, out_dev,
+                              num_q_heads, scale, softcap, &folded);
+    }
     st = ensure_prep(pool, total_rows * (q_width + k_width));
     if (st != ITAK_OK) return st;
     float *q_prep = pool->prep, *k_prep = pool->prep + total_rows * q_width;
@@ -1805,7 +1852,7 @@ itak_status itak_attention_prep_step_device(itak_pool *pool, uint64_t layer,
         a.k_weight = prep->k_norm_weight;
         a.eps = prep->eps;
         a.rope_base = rotate ? prep->rope_base : 0.0f;
-        a.interleaved = prep->rope_interleaved ? 1 : 0;
+        a.interleaved = interleaved ? 1 : 0;
         a.rotary_dim = rotary;
         a.head_dim = D;
         a.q_heads = uint32_t(num_q_heads);
@@ -1821,14 +1868,8 @@ itak_status itak_attention_prep_step_device(itak_pool *pool, uint64_t layer,
         HIP_TRY(pool, launch_attn_prep(a, pool->stream), "launch attention preparation");
         row += chunk_rows;
     }
-    if (std::isnan(scale)) scale = default_scale(D);
-    st = step_on_device(pool, layer, items, item_count, plan, q_prep, k_prep, v_dev, out_dev,
-                        num_q_heads, scale, softcap);
-    if (st != ITAK_OK) return st;
-    if (gate_dev)
-        HIP_TRY(pool, launch_attn_gate(out_dev, gate_dev, total_rows * q_width, pool->stream),
-                "launch attention gate");
-    return ITAK_OK;
+    return step_on_device(pool, layer, items, item_count, plan, q_prep, k_prep, v_dev, out_dev,
+                          num_q_heads, scale, softcap, &folded);
 }
 
 itak_status itak_attention_device(itak_pool *pool, uint64_t layer, const itak_batch_item *items,

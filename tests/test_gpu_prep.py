@@ -24,10 +24,13 @@ def dev(a):
 
 
 def run_case(elem, q_heads, kv_heads, d, ctx, rows, norm, rope_base, interleaved, rotary, gate,
-             seed=0, slots=1):
+             seed=0, slots=1, window=None):
     rng = np.random.default_rng(seed)
     width = kv_heads * d
-    pool = P().KvPool(1, kv_heads, d, elem=elem, max_slots=slots, capacity_rows=ctx + 13 * (slots - 1) + rows + 8)
+    kind = P().LayerKind.Global if window is None else P().LayerKind.windowed(window)
+    okind = oracle.LayerKind.Global if window is None else oracle.LayerKind.windowed(window)
+    pool = P().KvPool([kind], kv_heads, d, elem=elem, max_slots=slots,
+                      capacity_rows=ctx + 13 * (slots - 1) + rows + 8)
     pool.set_stream(torch.cuda.current_stream().cuda_stream)
     qw = (1.0 + 0.1 * normal(rng, d)) if norm else None
     kw = (1.0 + 0.1 * normal(rng, d)) if norm else None
@@ -35,12 +38,16 @@ def run_case(elem, q_heads, kv_heads, d, ctx, rows, norm, rope_base, interleaved
     caches, refs, qs, ks, vs, gs = [], [], [], [], [], []
     for s in range(slots):
         cache = pool.acquire()
-        ref = oracle.KvCache.new([oracle.LayerKind.Global], kv_heads, d, store_f16=(elem == "f16"))
+        ref = oracle.KvCache.new([okind], kv_heads, d, store_f16=(elem == "f16"))
         n0 = ctx + 13 * s
         k0 = oracle.attention_prep(normal(rng, n0, width), kv_heads, d, 0, kw, eps, rope_base,
                                    interleaved, rotary or None)
         v0 = normal(rng, n0, width)
-        if n0:
+        if n0 and window is not None:  # what a prefill leaves in the ring: the last `window` rows
+            first = max(0, n0 - window)
+            cache.restore_bulk(0, first, k0[first:], v0[first:])
+            ref.restore_bulk(0, first, k0[first:], v0[first:])
+        elif n0:
             k0d, v0d = dev(k0), dev(v0)
             pool.append_device(0, [(cache, n0)], k0d.data_ptr(), v0d.data_ptr())
             torch.cuda.synchronize()
@@ -72,7 +79,7 @@ def run_case(elem, q_heads, kv_heads, d, ctx, rows, norm, rope_base, interleaved
         else:
             assert max_abs(mine, want) <= 2e-3
         # The appended rows: prepared keys, untouched values.
-        _, gk, gv = caches[s].read_rows(0, n0, rows)
+        _, gk, gv = caches[s].read_rows(0, caches[s].stored_len(0) - rows, rows)
         if elem == "f32":
             assert max_abs(gk.reshape(rows, width), kp) <= 1e-6
             assert gv.reshape(rows, width).tobytes() == vs[s].tobytes()
@@ -123,6 +130,47 @@ def test_long_positions_need_the_f64_angle_law():
 def test_blocks_pairings_partial_rotary_and_nope(rows, interleaved, rotary, norm, rope_base):
     run_case("f16", 32, 4, 128, ctx=150, rows=rows, norm=norm, rope_base=rope_base,
              interleaved=interleaved, rotary=rotary, gate=(rows < 100), seed=rows)
+
+
+@pytest.mark.parametrize("q_heads,rows,interleaved,rotary,norm,rope_base,ctx,window", [
+    (32, 2, True, 0, True, 1e6, 150, None),     # 16 vectors, two positions in one tile
+    (32, 2, False, 0, True, 1e4, 150, None),    # half split over the whole head
+    (32, 2, False, 64, True, 1e4, 150, None),   # half split, partial rotary
+    (32, 1, True, 32, False, 5e5, 150, None),   # partial interleaved, no norm
+    (16, 4, True, 0, True, 1e6, 700, None),     # group 4, four rows
+    (4, 8, False, 0, True, 1e4, 40, None),      # group 1, eight rows, single split
+    (32, 1, True, 0, True, 1e6, 9, None),       # one split: the split kernel writes and gates the output
+    (32, 1, False, 0, False, 0.0, 300, None),   # nothing to prepare: the gate alone
+    (32, 1, True, 0, True, 1e4, 5000, 1024),    # sliding-window layer, ring wrapped
+    (32, 2, True, 0, True, 1e4, 1500, 1024),
+])
+def test_steps_of_up_to_16_vectors_prepare_inside_the_attention_launch(q_heads, rows, interleaved,
+                                                                       rotary, norm, rope_base, ctx,
+                                                                       window):
+    run_case("f16", q_heads, 4, 128, ctx=ctx, rows=rows, norm=norm, rope_base=rope_base,
+             interleaved=interleaved, rotary=rotary, gate=True, seed=ctx + rows, window=window)
+
+
+def test_folded_preparation_at_a_long_position_keeps_the_f16_bar():
+    # Position ~100,000: the angle must be formed and reduced in f64 inside the kernel too.
+    rng = np.random.default_rng(9)
+    d, kv_heads, q_heads, pos = 128, 4, 32, 100_000
+    pool = P().KvPool(1, kv_heads, d, elem="f16", capacity_rows=pos + 4)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    cache = pool.acquire()
+    zeros = torch.zeros(pos, kv_heads * d, device="cuda")
+    pool.append_device(0, [(cache, pos)], zeros.data_ptr(), zeros.data_ptr())
+    q, k, v = normal(rng, 1, q_heads * d), normal(rng, 1, kv_heads * d), normal(rng, 1, kv_heads * d)
+    out = torch.empty(1, q_heads * d, device="cuda")
+    qd, kd, vd = dev(q), dev(k), dev(v)
+    pool.attention_prep_step_device(0, [(cache, 1)], qd.data_ptr(), kd.data_ptr(), vd.data_ptr(),
+                                    out.data_ptr(), q_heads, rope_base=1e4, interleaved=True)
+    torch.cuda.synchronize()
+    _, gk, _ = cache.read_rows(0, pos, 1)
+    want = oracle.f32_to_f16_array(oracle.attention_prep(k, kv_heads, d, pos, None, 1e-6, 1e4, True))
+    ulp = np.abs(gk.reshape(-1).view(np.int16).astype(np.int32) - want.reshape(-1).view(np.int16).astype(np.int32))
+    assert ulp.max() <= 1
+    pool.close()
 
 
 def test_several_slots_each_at_its_own_position():
