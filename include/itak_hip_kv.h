@@ -509,10 +509,15 @@ typedef struct itak_prep_params {
 /* itak_attention_step_device preceded by the fused preparation of the resident chain
    (crates/wgpu-compute/src/kernels/k9_attn_prep.rs:1-60: the Q and K norms, the rotations
    and the append as one dispatch) and followed by the attention gate
-   (CpuCompute::attn_gate, cpu.rs:657-673): q_dev and k_dev are the raw projections; norms
-   and rotation run as one launch, the append is part of the attention launch, and with
-   gate_dev != NULL ([sum rows][q_heads*head_dim]) out = attention * sigmoid(gate). Numerics
-   are those of the reference's CPU path (f64 norm, f64 angles), not of its f32 shader. */
+   (CpuCompute::attn_gate, cpu.rs:657-673): q_dev and k_dev are the raw projections, and with
+   gate_dev != NULL ([sum rows][q_heads*head_dim]) out = attention * sigmoid(gate).
+   On f16 pools with head_dim 128, steps of up to 16 query vectors per KV head (rows x group:
+   decode, short blocks) add no launch to the plain step's two: the attention kernel norms and
+   rotates the Q rows it stages and the new K row it appends (f64 angle, f32 arithmetic:
+   within one f16 step of the reference's f64 chain in the stored K), and the kernel that
+   writes the output applies the gate. Other shapes run norms and rotation as one launch
+   before the step, with the numerics of the reference's CPU path (f64 norm, f64 angles),
+   not of its f32 shader; f32 pools hold prepared K rows within 1e-6 of that path. */
 itak_status itak_attention_prep_step_device(itak_pool *pool, uint64_t layer,
                                             const itak_batch_item *items, uint32_t item_count,
                                             const float *q_dev, const float *k_dev,
