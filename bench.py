@@ -426,7 +426,7 @@ def main():
         for _ in range(max(args.warmup, 1)):
             g_prep.replay()
         prep_s = timed(g_prep.replay, args.steps)[0] / args.steps
-        folded = rows * (Q_HEADS // KV_HEADS) <= 16
+        folded = rows * (Q_HEADS // KV_HEADS) <= 64 and rows <= 8
         with_prep = {
             "us_per_layer": round(prep_s / layers * 1e6, 3),
             "added_us_per_layer": round((prep_s - step_s) / layers * 1e6, 3),

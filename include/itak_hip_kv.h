@@ -511,8 +511,8 @@ typedef struct itak_prep_params {
    and the append as one dispatch) and followed by the attention gate
    (CpuCompute::attn_gate, cpu.rs:657-673): q_dev and k_dev are the raw projections, and with
    gate_dev != NULL ([sum rows][q_heads*head_dim]) out = attention * sigmoid(gate).
-   On f16 pools with head_dim 128, steps of up to 16 query vectors per KV head (rows x group:
-   decode, short blocks) add no launch to the plain step's two: the attention kernel norms and
+   On f16 pools with head_dim 128, steps of up to 64 query vectors per KV head (rows x group:
+   decode, speculative blocks) add no launch to the plain step's two: the attention kernel norms and
    rotates the Q rows it stages and the new K row it appends (f64 angle, f32 arithmetic:
    within one f16 step of the reference's f64 chain in the stored K), and the kernel that
    writes the output applies the gate. Other shapes run norms and rotation as one launch

@@ -655,13 +655,13 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_kernel(AttnParams 
                                                                      uint32_t total_partials) {
     attn_splitk_f16_body<NQ, WAVES, N, RING, false>(p, b, total_partials, FoldedParams{});
 }
-// The 16-vector variants with the preparation and the gate folded in.
-template <int WAVES, int N, bool RING>
+// The same variants with the preparation and the gate folded in.
+template <int NQ, int WAVES, int N, bool RING>
 __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_prep_kernel(AttnParams p,
                                                                           AttnBatchT<N> b,
                                                                           uint32_t total_partials,
                                                                           FoldedParams f) {
-    attn_splitk_f16_body<1, WAVES, N, RING, true>(p, b, total_partials, f);
+    attn_splitk_f16_body<NQ, WAVES, N, RING, true>(p, b, total_partials, f);
 }
 
 }  // namespace
@@ -708,12 +708,12 @@ static hipError_t grant_lds(size_t lds) {
         reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 8, true>),
         reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 64, true>)};
     const void *prepping[] = {
-        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<W, 1, false>),
-        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<W, 8, false>),
-        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<W, 64, false>),
-        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<W, 1, true>),
-        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<W, 8, true>),
-        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<W, 64, true>)};
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<NQ, W, 1, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<NQ, W, 8, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<NQ, W, 64, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<NQ, W, 1, true>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<NQ, W, 8, true>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<NQ, W, 64, true>)};
     const void *const *kernels = PREP ? prepping : plain;
     hipError_t e = hipSuccess;
     for (int k = 0; k < 6; ++k)
@@ -798,7 +798,6 @@ hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint3
     if (b.total_blocks == 0) return hipSuccess;
     const Variant v = pick_variant(p.g, b, p.group);
     const bool prep = folded && folded->prep_on;
-    if (prep && v.nq != 1) return hipErrorInvalidValue;
 #define ITAK_LAUNCH(NQ, W)                                                                \
     do {                                                                                  \
         const size_t lds = variant_lds(NQ, W);                                            \
@@ -811,17 +810,19 @@ hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint3
             attn_splitk_f16_kernel<NQ, W, N, false><<<b.total_blocks, W * 64, lds, stream>>>( \
                 p, AttnBatchT<N>(b), total_partials);                                     \
     } while (0)
-#define ITAK_LAUNCH_PREP(W)                                                               \
+#define ITAK_LAUNCH_PREP(NQ, W)                                                           \
     do {                                                                                  \
-        const size_t lds = variant_lds(1, W);                                             \
-        hipError_t e = grant_lds<1, W, true>(lds);                                        \
+        const size_t lds = variant_lds(NQ, W);                                            \
+        hipError_t e = grant_lds<NQ, W, true>(lds);                                       \
         if (e != hipSuccess) return e;                                                    \
         if (p.ring_blocks)                                                                \
-            attn_splitk_f16_prep_kernel<W, N, true><<<b.total_blocks, W * 64, lds, stream>>>( \
-                p, AttnBatchT<N>(b), total_partials, *folded);                            \
+            attn_splitk_f16_prep_kernel<NQ, W, N, true>                                   \
+                <<<b.total_blocks, W * 64, lds, stream>>>(p, AttnBatchT<N>(b), total_partials, \
+                                                          *folded);                       \
         else                                                                              \
-            attn_splitk_f16_prep_kernel<W, N, false><<<b.total_blocks, W * 64, lds, stream>>>( \
-                p, AttnBatchT<N>(b), total_partials, *folded);                            \
+            attn_splitk_f16_prep_kernel<NQ, W, N, false>                                  \
+                <<<b.total_blocks, W * 64, lds, stream>>>(p, AttnBatchT<N>(b), total_partials, \
+                                                          *folded);                       \
     } while (0)
 #define ITAK_LAUNCH_NQ()                                  \
     do {                                                  \
@@ -830,8 +831,10 @@ hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint3
             case 1: ITAK_LAUNCH(1, 8); break;             \
             case 2: ITAK_LAUNCH(2, 4); break;             \
             case 3: ITAK_LAUNCH(4, 4); break;             \
-            case 4: ITAK_LAUNCH_PREP(4); break;           \
-            default: ITAK_LAUNCH_PREP(8); break;          \
+            case 4: ITAK_LAUNCH_PREP(1, 4); break;        \
+            case 5: ITAK_LAUNCH_PREP(1, 8); break;        \
+            case 6: ITAK_LAUNCH_PREP(2, 4); break;        \
+            default: ITAK_LAUNCH_PREP(4, 4); break;       \
         }                                                 \
     } while (0)
     ITAK_DISPATCH_BATCH(b.n, ITAK_LAUNCH_NQ());

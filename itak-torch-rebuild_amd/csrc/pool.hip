@@ -1808,21 +1808,16 @@ itak_status itak_attention_prep_step_device(itak_pool *pool, uint64_t layer,
     if (total_rows == 0) return ITAK_OK;
     const uint64_t q_width = num_q_heads * D, k_width = pool->row;
     if (std::isnan(scale)) scale = default_scale(D);
-    // Steps the split-K kernel takes have the gate applied by the kernel that writes the
-    // output, and, when every item is a 16-vector step (decode, short blocks), Q and K
-    // prepared by the split-K kernel itself: no launch but the step's own two.
+    // Steps the split-K kernel takes (decode, speculative blocks: up to 64 query vectors per KV
+    // head) have Q and the new K rows prepared by that kernel and the gate applied by the
+    // kernel that writes the output: no launch but the step's own two.
     std::vector<PlanInput> active;
-    uint32_t max_rows = 0;
     for (const PlanInput &p : plan)
-        if (p.rows) {
-            active.push_back(p);
-            max_rows = std::max(max_rows, p.rows);
-        }
+        if (p.rows) active.push_back(p);
     const bool splitk = takes_splitk_f16(pool, active.data(), uint32_t(active.size()), num_q_heads,
                                          nullptr);
-    const uint32_t group = uint32_t(num_q_heads / pool->g.kv_heads);
     const bool interleaved = prep->rope_interleaved != 0;
-    const bool folds = splitk && max_rows * group <= 16 && (!rotate || interleaved || rotary % 8 == 0);
+    const bool folds = splitk && (!rotate || interleaved || rotary % 8 == 0);
     FoldedParams folded{};
     folded.gate = gate_dev;
     if (folds) {
