@@ -91,6 +91,10 @@ struct itak_pool {
     uint64_t ws_floats = 0;
     float *prep = nullptr;  // prepared Q and K rows of a prep step
     uint64_t prep_floats = 0;
+    // Pinned host memory for the host-pointer attention call: its small inputs are packed here
+    // and go up in one copy; its kernels write the output here directly.
+    unsigned char *hstage = nullptr;
+    uint64_t hstage_bytes = 0;
     mutable ErrorState err;
 };
 
@@ -273,6 +277,19 @@ itak_status ensure_prep(itak_pool *pool, uint64_t floats) {
                 "allocate prep scratch");
         pool->prep_floats = want;
     }
+    return ITAK_OK;
+}
+
+itak_status ensure_hstage(itak_pool *pool, uint64_t bytes) {
+    if (bytes <= pool->hstage_bytes) return ITAK_OK;
+    HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize before growing pinned staging");
+    if (pool->hstage) HIP_TRY(pool, hipHostFree(pool->hstage), "free pinned staging");
+    pool->hstage = nullptr;
+    pool->hstage_bytes = 0;
+    const uint64_t want = std::max<uint64_t>(bytes + bytes / 2, 1u << 18);
+    HIP_TRY(pool, hipHostMalloc(reinterpret_cast<void **>(&pool->hstage), want, hipHostMallocDefault),
+            "allocate pinned staging");
+    pool->hstage_bytes = want;
     return ITAK_OK;
 }
 
@@ -814,6 +831,7 @@ void itak_pool_destroy(itak_pool *pool) {
     if (pool->stage) (void)hipFree(pool->stage);
     if (pool->ws) (void)hipFree(pool->ws);
     if (pool->prep) (void)hipFree(pool->prep);
+    if (pool->hstage) (void)hipHostFree(pool->hstage);
     delete pool;
 }
 
@@ -1964,27 +1982,31 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
     itak_status st = ensure_stage(pool, 2 * q_bytes + 2 * kv_bytes);
     if (st != ITAK_OK) return st;
     float *qd = reinterpret_cast<float *>(pool->stage);
-    float *od = reinterpret_cast<float *>(pool->stage + q_bytes);
-    float *kd = reinterpret_cast<float *>(pool->stage + 2 * q_bytes);
-    float *vd = reinterpret_cast<float *>(pool->stage + 2 * q_bytes + kv_bytes);
-    HIP_TRY(pool, hipMemcpyAsync(kd, k, k_len * 4, hipMemcpyHostToDevice, pool->stream), "upload k");
-    HIP_TRY(pool, hipMemcpyAsync(vd, v, v_len * 4, hipMemcpyHostToDevice, pool->stream), "upload v");
-    HIP_TRY(pool, hipMemcpyAsync(qd, q, q_len * 4, hipMemcpyHostToDevice, pool->stream), "upload q");
-    if (rotate) {  // in place on the staged rows, row i at position appended + i
-        PrepArgs a{};
-        a.q_in = a.q_out = qd;
-        a.k_in = a.k_out = kd;
-        a.rope_base = rope_freq_base_swa;
-        a.interleaved = 1;
-        a.rotary_dim = pool->g.head_dim;
-        a.head_dim = pool->g.head_dim;
-        a.q_heads = uint32_t(num_q_heads);
-        a.kv_heads = pool->g.kv_heads;
-        a.total_rows = uint32_t(rows);
-        a.n = 1;
-        a.row0[0] = 0;
-        a.pos0[0] = uint32_t(appended);
-        HIP_TRY(pool, launch_attn_prep(a, pool->stream), "launch rope");
+    float *kd = reinterpret_cast<float *>(pool->stage + q_bytes);
+    float *vd = reinterpret_cast<float *>(pool->stage + q_bytes + kv_bytes);
+    float *od = reinterpret_cast<float *>(pool->stage + q_bytes + 2 * kv_bytes);
+    // A call is dominated by its trips over the host link, not by its kernels. Small inputs
+    // (a decode row, a speculative block) are packed into pinned memory and go up in one copy,
+    // and the kernel that writes the output writes it into pinned memory directly; large ones
+    // (a prefill chunk) are copied as they lie.
+    const uint64_t in_bytes = q_bytes + 2 * kv_bytes;
+    const bool packed = in_bytes <= (1u << 20);
+    float *out_pinned = nullptr;
+    if (packed) {
+        st = ensure_hstage(pool, in_bytes + q_bytes);
+        if (st != ITAK_OK) return st;
+        memcpy(pool->hstage, q, q_len * 4);
+        memcpy(pool->hstage + q_bytes, k, k_len * 4);
+        memcpy(pool->hstage + q_bytes + kv_bytes, v, v_len * 4);
+        HIP_TRY(pool, hipMemcpyAsync(qd, pool->hstage, in_bytes, hipMemcpyHostToDevice, pool->stream),
+                "upload q, k, v");
+        void *mapped = nullptr;
+        HIP_TRY(pool, hipHostGetDevicePointer(&mapped, pool->hstage + in_bytes, 0), "map pinned output");
+        out_pinned = static_cast<float *>(mapped);
+    } else {
+        HIP_TRY(pool, hipMemcpyAsync(kd, k, k_len * 4, hipMemcpyHostToDevice, pool->stream), "upload k");
+        HIP_TRY(pool, hipMemcpyAsync(vd, v, v_len * 4, hipMemcpyHostToDevice, pool->stream), "upload v");
+        HIP_TRY(pool, hipMemcpyAsync(qd, q, q_len * 4, hipMemcpyHostToDevice, pool->stream), "upload q");
     }
     // The reference appends and attends row by row (cpu.rs:586-646). Here a block is appended
     // whole and attended under the causal mask, which is the same thing on a global layer; on
@@ -1992,9 +2014,36 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
     // several blocks.
     const LayerInfo &L = pool->layers[layer];
     const uint64_t block_cap = L.windowed ? L.ring - L.window : std::max<uint64_t>(rows, 1);
+    // The rotation of a sliding-window layer (row i at position appended + i): inside the
+    // attention launch where the split-K kernel takes the block, else in place on the staged
+    // rows beforehand.
+    FoldedParams folded{};
+    folded.prep_on = 1;
+    folded.prep_interleaved = 1;
+    folded.prep_rot = pool->g.head_dim;
+    folded.prep_freq_step = rotate ? -2.0 * std::log2(double(rope_freq_base_swa)) / double(pool->g.head_dim) : 0.0;
+    auto rotate_block = [&](uint64_t done, uint64_t n, bool with_q) -> itak_status {
+        PrepArgs a{};
+        a.q_in = a.q_out = qd + done * q_width;
+        a.k_in = a.k_out = kd + done * pool->row;
+        a.rope_base = rope_freq_base_swa;
+        a.interleaved = 1;
+        a.rotary_dim = pool->g.head_dim;
+        a.head_dim = pool->g.head_dim;
+        a.q_heads = with_q ? uint32_t(num_q_heads) : 0;
+        a.kv_heads = pool->g.kv_heads;
+        a.total_rows = uint32_t(n);
+        a.n = 1;
+        a.row0[0] = 0;
+        a.pos0[0] = uint32_t(appended + done);
+        HIP_TRY(pool, launch_attn_prep(a, pool->stream), "launch rope");
+        return ITAK_OK;
+    };
     if (refusal != ITAK_OK) {
         for (uint64_t done = 0; done < ok_rows; done += block_cap) {
-            itak_batch_item item{slot, uint32_t(std::min(block_cap, ok_rows - done))};
+            const uint64_t n = std::min(block_cap, ok_rows - done);
+            if (rotate && (st = rotate_block(done, n, false)) != ITAK_OK) return st;
+            itak_batch_item item{slot, uint32_t(n)};
             st = run_append(pool, layer, &item, 1, kd + done * pool->row, vd + done * pool->row);
             if (st != ITAK_OK) return st;
         }
@@ -2003,22 +2052,27 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
         pool->err.info.code = ITAK_STEP_FAILED;
         return ITAK_STEP_FAILED;
     }
+    float *out_dev = out_pinned ? out_pinned : od;
     for (uint64_t done = 0; done < rows; done += block_cap) {
         const uint64_t n = std::min(block_cap, rows - done);
         itak_batch_item item{slot, uint32_t(n)};
-        st = run_append(pool, layer, &item, 1, kd + done * pool->row, vd + done * pool->row);
-        if (st != ITAK_OK) return st;
         const uint64_t base = appended + done;
         const uint64_t lo = (L.window && base + 1 > L.window) ? base + 1 - L.window : 0;
-        PlanInput pi{slot, uint32_t(n), uint32_t(base), uint32_t(base + n), uint32_t(lo)};
-        st = run_attention(pool, layer, &pi, 1, qd + done * q_width, od + done * q_width, nullptr,
-                           num_q_heads, default_scale(pool->g.head_dim),
-                           softcap);  // AttentionParams::new(), cpu.rs:584
+        std::vector<PlanInput> plan{
+            PlanInput{slot, uint32_t(n), uint32_t(base), uint32_t(base + n), uint32_t(lo)}};
+        const bool folds = rotate && takes_splitk_f16(pool, plan.data(), 1, num_q_heads, nullptr);
+        if (rotate && !folds && (st = rotate_block(done, n, true)) != ITAK_OK) return st;
+        st = step_on_device(pool, layer, &item, 1, plan, qd + done * q_width, kd + done * pool->row,
+                            vd + done * pool->row, out_dev + done * q_width, num_q_heads,
+                            default_scale(pool->g.head_dim),  // AttentionParams::new(), cpu.rs:584
+                            softcap, folds ? &folded : nullptr);
         if (st != ITAK_OK) return st;
     }
-    HIP_TRY(pool, hipMemcpyAsync(out, od, q_len * 4, hipMemcpyDeviceToHost, pool->stream),
-            "download attention output");
+    if (!out_pinned)
+        HIP_TRY(pool, hipMemcpyAsync(out, od, q_len * 4, hipMemcpyDeviceToHost, pool->stream),
+                "download attention output");
     HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after attention");
+    if (out_pinned) memcpy(out, pool->hstage + in_bytes, q_len * 4);
     return ITAK_OK;
 }
 
