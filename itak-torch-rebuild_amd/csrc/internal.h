@@ -139,6 +139,11 @@ hipError_t launch_read_rows(const void *layer_base, int elem_f16, const PoolGeom
 hipError_t launch_convert_f16(const float *src, uint16_t *dst, uint64_t count, hipStream_t stream);
 // f16 bits -> f32, exact (the widening a snapshot capture of an f16 pool needs).
 hipError_t launch_widen_f16(const uint16_t *src, float *dst, uint64_t count, hipStream_t stream);
+// Host-pointer calls: `bytes` (rounded up to 16) from pinned host memory into device memory by
+// a kernel, and a word in pinned host memory set to `value` once everything before it on the
+// stream has finished.
+hipError_t launch_stage_in(const void *pinned, void *dst, uint64_t bytes, hipStream_t stream);
+hipError_t launch_signal_done(uint32_t *pinned_word, uint32_t value, hipStream_t stream);
 hipError_t launch_probe_copy(const void *src, void *dst, uint64_t bytes, hipStream_t stream);
 hipError_t launch_probe_empty(hipStream_t stream);
 

@@ -375,6 +375,34 @@ hipError_t launch_widen_f16(const uint16_t *src, float *dst, uint64_t count, hip
     return hipGetLastError();
 }
 
+// ------------------------------------------------- host-pointer call: in and done
+// The small inputs of a host-pointer call lie packed in pinned host memory. One launch reads
+// them over the host link into device memory (a copy engine's command costs more than this
+// launch at 20 KB), and a one-thread launch at the end of the call's work writes the call's
+// number into pinned memory, where the host is watching for it: finding out from the runtime
+// that a stream has drained costs several microseconds more than seeing a word change.
+__global__ __launch_bounds__(256) void stage_in_kernel(const uint4 *__restrict__ pinned,
+                                                       uint4 *__restrict__ dst, uint32_t n) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) dst[i] = pinned[i];
+}
+__global__ void signal_done_kernel(uint32_t *pinned_word, uint32_t value) {
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(pinned_word, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+}
+hipError_t launch_stage_in(const void *pinned, void *dst, uint64_t bytes, hipStream_t stream) {
+    const uint32_t n = uint32_t((bytes + 15) / 16);
+    if (n == 0) return hipSuccess;
+    stage_in_kernel<<<(n + 255) / 256, 256, 0, stream>>>(static_cast<const uint4 *>(pinned),
+                                                         static_cast<uint4 *>(dst), n);
+    return hipGetLastError();
+}
+hipError_t launch_signal_done(uint32_t *pinned_word, uint32_t value, hipStream_t stream) {
+    signal_done_kernel<<<1, 64, 0, stream>>>(pinned_word, value);
+    return hipGetLastError();
+}
+
 // ------------------------------------------------------------- measurement aids
 // A plain streaming copy of known size (the yardstick the FETCH_SIZE / WRITE_SIZE counters
 // are scaled by) and an empty kernel (the per-launch floor of a stream of dependent

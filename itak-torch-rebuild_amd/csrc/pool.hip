@@ -11,6 +11,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <ctime>
 #include <string>
 #include <vector>
 
@@ -95,6 +96,7 @@ struct itak_pool {
     // and go up in one copy; its kernels write the output here directly.
     unsigned char *hstage = nullptr;
     uint64_t hstage_bytes = 0;
+    uint32_t call_number = 0;  // what the last host-pointer call asked to be told when done
     mutable ErrorState err;
 };
 
@@ -1992,17 +1994,23 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
     const uint64_t in_bytes = q_bytes + 2 * kv_bytes;
     const bool packed = in_bytes <= (1u << 20);
     float *out_pinned = nullptr;
+    uint32_t *done_word = nullptr;  // in pinned memory, after the output
     if (packed) {
-        st = ensure_hstage(pool, in_bytes + q_bytes);
+        st = ensure_hstage(pool, in_bytes + q_bytes + 256);
         if (st != ITAK_OK) return st;
         memcpy(pool->hstage, q, q_len * 4);
         memcpy(pool->hstage + q_bytes, k, k_len * 4);
         memcpy(pool->hstage + q_bytes + kv_bytes, v, v_len * 4);
-        HIP_TRY(pool, hipMemcpyAsync(qd, pool->hstage, in_bytes, hipMemcpyHostToDevice, pool->stream),
-                "upload q, k, v");
         void *mapped = nullptr;
-        HIP_TRY(pool, hipHostGetDevicePointer(&mapped, pool->hstage + in_bytes, 0), "map pinned output");
-        out_pinned = static_cast<float *>(mapped);
+        HIP_TRY(pool, hipHostGetDevicePointer(&mapped, pool->hstage, 0), "map pinned staging");
+        unsigned char *pinned_dev = static_cast<unsigned char *>(mapped);
+        if (in_bytes <= (64u << 10))
+            HIP_TRY(pool, launch_stage_in(pinned_dev, qd, in_bytes, pool->stream), "launch stage-in");
+        else
+            HIP_TRY(pool, hipMemcpyAsync(qd, pool->hstage, in_bytes, hipMemcpyHostToDevice, pool->stream),
+                    "upload q, k, v");
+        out_pinned = reinterpret_cast<float *>(pinned_dev + in_bytes);
+        done_word = reinterpret_cast<uint32_t *>(pinned_dev + in_bytes + q_bytes);
     } else {
         HIP_TRY(pool, hipMemcpyAsync(kd, k, k_len * 4, hipMemcpyHostToDevice, pool->stream), "upload k");
         HIP_TRY(pool, hipMemcpyAsync(vd, v, v_len * 4, hipMemcpyHostToDevice, pool->stream), "upload v");
@@ -2068,11 +2076,34 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
                             softcap, folds ? &folded : nullptr);
         if (st != ITAK_OK) return st;
     }
-    if (!out_pinned)
+    if (!out_pinned) {
         HIP_TRY(pool, hipMemcpyAsync(out, od, q_len * 4, hipMemcpyDeviceToHost, pool->stream),
                 "download attention output");
-    HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after attention");
-    if (out_pinned) memcpy(out, pool->hstage + in_bytes, q_len * 4);
+        HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after attention");
+        return ITAK_OK;
+    }
+    // The last launch of the call writes the call's number where the host can see it; the host
+    // watches that word for a short while before it asks the runtime (which also reports a
+    // failed launch, and is what a call that takes longer falls back to).
+    const uint32_t number = ++pool->call_number ? pool->call_number : ++pool->call_number;
+    HIP_TRY(pool, launch_signal_done(done_word, number, pool->stream), "launch completion signal");
+    const volatile uint32_t *seen =
+        reinterpret_cast<const volatile uint32_t *>(pool->hstage + in_bytes + q_bytes);
+    timespec t0{};
+    clock_gettime(CLOCK_MONOTONIC, &t0);
+    bool arrived = false;
+    for (uint32_t spin = 0; !arrived; ++spin) {
+        arrived = __atomic_load_n(seen, __ATOMIC_ACQUIRE) == number;
+        if (arrived || (spin & 63u) != 63u) {
+            __builtin_ia32_pause();
+            continue;
+        }
+        timespec t1{};
+        clock_gettime(CLOCK_MONOTONIC, &t1);
+        if ((t1.tv_sec - t0.tv_sec) * 1000000000ll + (t1.tv_nsec - t0.tv_nsec) > 300000) break;
+    }
+    if (!arrived) HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after attention");
+    memcpy(out, pool->hstage + in_bytes, q_len * 4);
     return ITAK_OK;
 }
 
