@@ -402,6 +402,41 @@ def main():
     attn_s = timed(g_attn.replay, args.steps)[0] / (args.steps * layers)
     pool.truncate(caches, lengths)
 
+    host_call = None
+    if wl == "decode":
+        # The same layer step through the host-pointer entry point (what a Compute::attention
+        # call with host slices costs): inputs and output cross the host link and the call
+        # waits for its result. A secondary figure, never `value`.
+        import ctypes as C
+
+        lib = pkg._native.load()
+        hq = q[0, :1].cpu().numpy().copy()
+        hk = k_new[0, :1].cpu().numpy().copy()
+        hv = v_new[0, :1].cpu().numpy().copy()
+        ho = np.empty_like(hq)
+        pos = lengths[0]
+        calls = 0
+
+        def host_step():
+            st = lib.itak_compute_attention(pool._h, caches[0].slot, 0, hq.ctypes.data, hq.size,
+                                            hk.ctypes.data, hk.size, hv.ctypes.data, hv.size,
+                                            Q_HEADS, pos, C.c_float(args.softcap), C.c_float(0.0),
+                                            ho.ctypes.data)
+            assert st == 0, lib.itak_last_error(pool._h)
+            pool.truncate(caches[:1], lengths[:1])
+
+        for _ in range(20):
+            host_step()
+        t0 = time.perf_counter()
+        for _ in range(200):
+            host_step()
+        per_call = (time.perf_counter() - t0) / 200
+        host_call = {
+            "entry_point": "itak_compute_attention (host q/k/v in, host output out, one layer)",
+            "us_per_layer": round(per_call * 1e6, 2),
+            "kv_GBps": round(kv_bytes_layer / per_call / 1e9, 1),
+        }
+
     with_prep = None
     if args.prep and wl != "prefill":
         # The model's own sequence around the step (muse-glimmer/src/model.rs:445-464): raw
@@ -502,6 +537,8 @@ def main():
     }
     if with_prep is not None:
         result["with_prep"] = with_prep
+    if host_call is not None:
+        result["host_pointer_call"] = host_call
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(4096, 2 * 4097 * KV_HEADS * D * 2, 48)
     print(json.dumps(result))
