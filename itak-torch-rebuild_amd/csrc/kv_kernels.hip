@@ -171,55 +171,71 @@ __global__ __launch_bounds__(256) void kv_restore_rows(D *__restrict__ pool_base
     }
 }
 
-// Blocked value planes: one workgroup moves one (32-row block, kv head): coalesced reads of
-// the 32 source rows into LDS (converted), then each thread writes 8 consecutive rows of
-// one channel as one 16-byte store, so both sides of the transpose are full-width.
-// Requires first_row % 32 == 0. grid = (row blocks, kv_heads, layer entry).
-template <typename S>
-__global__ __launch_bounds__(256) void kv_restore_v_blocked(uint16_t *__restrict__ pool_base,
-                                                            PoolGeom g, RestoreBatch b) {
-    extern __shared__ uint16_t tile[];  // [32][head_dim + 8]
+// Blocked planes, both sides in one launch: a workgroup moves one (32-row block, kv head) of
+// keys and of values. The 32 source rows of each side are read coalesced into LDS (converted):
+// whole 256- or 512-byte runs, which is what a source in pinned host memory needs to keep the
+// host link at its rate (a variant whose threads fetch their key piece directly, 64-byte
+// runs, gains 4 % from HBM and loses 12 % over the link). The key block then leaves as the
+// 8 KiB of 16-byte pieces the MFMA kernels read (piece (tile t, channel chunk c, row i) at
+// ((t*(D/8) + c)*16 + i)*8, k_offset above) and the value block transposed, every thread
+// storing 16 contiguous bytes. Requires first_row % 32 == 0; rows of the last block past the source are written as
+// zeros, which is what a fresh layer holds there. grid = (row blocks, kv_heads, layer entry).
+// HD = the head_dim the index arithmetic is compiled for (shifts instead of divisions: at
+// 128 bytes moved per thread the divisions by a run-time head_dim cost more than the copy);
+// 0 = any head_dim, read from the geometry.
+template <typename S, int HD>
+__global__ __launch_bounds__(256) void kv_restore_blocked(uint16_t *__restrict__ pool_base,
+                                                          PoolGeom g, RestoreBatch b) {
+    extern __shared__ uint16_t tile[];  // [2][32][head_dim + 8]: keys, values
     const RestoreLayer L = b.layer[blockIdx.z];
     const uint32_t head = blockIdx.y;
-    const uint32_t D = g.head_dim;
+    const uint32_t D = HD ? uint32_t(HD) : g.head_dim;
     const uint32_t stride = D + 8;
-    const S *src = static_cast<const S *>(L.values);
-    uint16_t *plane = pool_base + L.layer * g.layer_stride + b.slot * g.slot_stride +
-                      g.side_stride + head * g.head_stride;
+    uint16_t *ktile = tile, *vtile = tile + kVBlock * stride;
+    uint16_t *kplane = pool_base + L.layer * g.layer_stride + b.slot * g.slot_stride +
+                       head * g.head_stride;
+    uint16_t *vplane = kplane + g.side_stride;
     const uint32_t nblocks = (L.rows + kVBlock - 1) / kVBlock;
+    constexpr int VEC = 16 / sizeof(S);
+    const uint32_t chunks = D / VEC;
     for (uint32_t blk = blockIdx.x; blk < nblocks; blk += gridDim.x) {
         const uint32_t row0 = blk * kVBlock;
-        constexpr int VEC = 16 / sizeof(S);
-        const uint32_t chunks = D / VEC;
-        for (uint32_t i = threadIdx.x; i < kVBlock * chunks; i += 256) {
-            const uint32_t r = i / chunks, c = (i % chunks) * VEC;
-            uint16_t *t = tile + r * stride + c;
+        for (uint32_t i = threadIdx.x; i < 2 * kVBlock * chunks; i += 256) {
+            const uint32_t side = i / (kVBlock * chunks), j = i % (kVBlock * chunks);
+            const uint32_t r = j / chunks, c = (j % chunks) * VEC;
+            uint16_t *t = (side ? vtile : ktile) + r * stride + c;
             if (row0 + r < L.rows) {
-                const S *s = src + (uint64_t(row0 + r) * g.kv_heads + head) * D + c;
+                const S *s = static_cast<const S *>(side ? L.values : L.keys) +
+                             (uint64_t(row0 + r) * g.kv_heads + head) * D + c;
                 if constexpr (sizeof(S) == 4) {
                     store4(t, *reinterpret_cast<const float4 *>(s));
                 } else {
                     *reinterpret_cast<uint4 *>(t) = *reinterpret_cast<const uint4 *>(s);
                 }
             } else {
-                // Rows past the snapshot stay zero, as a fresh layer holds them.
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) t[e] = 0;
             }
         }
         __syncthreads();
-        uint16_t *dst_blk = plane + uint64_t(L.first_row / kVBlock + blk) * (kVBlock * D);
+        const uint64_t block_at = uint64_t(L.first_row / kVBlock + blk) * (kVBlock * D);
+        for (uint32_t piece = threadIdx.x; piece < kVBlock * (D / 8); piece += 256) {
+            const uint32_t i = piece % 16, tc = piece / 16, c = tc % (D / 8), t = tc / (D / 8);
+            const uint32_t key = (i >> 2) * 8 + t * 4 + (i & 3);
+            *reinterpret_cast<uint4 *>(kplane + block_at + uint64_t(piece) * 8) =
+                *reinterpret_cast<const uint4 *>(ktile + key * stride + c * 8);
+        }
         for (uint32_t i = threadIdx.x; i < D * (kVBlock / 8); i += 256) {
             const uint32_t d = i / (kVBlock / 8), r8 = (i % (kVBlock / 8)) * 8;
             uint16_t v[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = tile[(r8 + e) * stride + d];
+            for (int e = 0; e < 8; ++e) v[e] = vtile[(r8 + e) * stride + d];
             uint4 packed;
             packed.x = v[0] | (uint32_t(v[1]) << 16);
             packed.y = v[2] | (uint32_t(v[3]) << 16);
             packed.z = v[4] | (uint32_t(v[5]) << 16);
             packed.w = v[6] | (uint32_t(v[7]) << 16);
-            *reinterpret_cast<uint4 *>(dst_blk + d * kVBlock + r8) = packed;
+            *reinterpret_cast<uint4 *>(vplane + block_at + d * kVBlock + r8) = packed;
         }
         __syncthreads();
     }
@@ -271,11 +287,26 @@ hipError_t launch_restore(void *pool_base, int dst_f16, int src_f16, const PoolG
                 static_cast<float *>(pool_base), g, b);
         return hipGetLastError();
     }
+    if (g.v_block != 0) {  // blocked planes: keys and values of a block in one workgroup
+        uint32_t nblocks = (b.max_rows + kVBlock - 1) / kVBlock;
+        if (nblocks > 2048) nblocks = 2048;
+        dim3 grid(nblocks, g.kv_heads, b.n);
+        const size_t lds = size_t(2) * kVBlock * (g.head_dim + 8) * sizeof(uint16_t);
+        uint16_t *base = static_cast<uint16_t *>(pool_base);
+        if (g.head_dim == 128 && src_f16)
+            kv_restore_blocked<uint16_t, 128><<<grid, 256, lds, stream>>>(base, g, b);
+        else if (g.head_dim == 128)
+            kv_restore_blocked<float, 128><<<grid, 256, lds, stream>>>(base, g, b);
+        else if (src_f16)
+            kv_restore_blocked<uint16_t, 0><<<grid, 256, lds, stream>>>(base, g, b);
+        else
+            kv_restore_blocked<float, 0><<<grid, 256, lds, stream>>>(base, g, b);
+        return hipGetLastError();
+    }
     const uint64_t per_layer = uint64_t(b.max_rows) * g.kv_heads * (g.head_dim / vec);
     uint32_t bx = uint32_t((per_layer + 255) / 256);
     if (bx > 2048) bx = 2048;
-    const uint32_t row_sides = g.v_block != 0 ? 1 : 2;  // keys only when values are blocked
-    dim3 grid(bx, row_sides, b.n);
+    dim3 grid(bx, 2, b.n);
     if (src_f16)
         kv_restore_rows<uint16_t, uint16_t><<<grid, 256, 0, stream>>>(
             static_cast<uint16_t *>(pool_base), g, b, 0);
@@ -285,18 +316,6 @@ hipError_t launch_restore(void *pool_base, int dst_f16, int src_f16, const PoolG
     else
         kv_restore_rows<float, float><<<grid, 256, 0, stream>>>(static_cast<float *>(pool_base), g,
                                                                b, 0);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess || g.v_block == 0) return e;
-    uint32_t nblocks = (b.max_rows + kVBlock - 1) / kVBlock;
-    if (nblocks > 1024) nblocks = 1024;
-    dim3 vgrid(nblocks, g.kv_heads, b.n);
-    const size_t lds = size_t(kVBlock) * (g.head_dim + 8) * sizeof(uint16_t);
-    if (src_f16)
-        kv_restore_v_blocked<uint16_t><<<vgrid, 256, lds, stream>>>(
-            static_cast<uint16_t *>(pool_base), g, b);
-    else
-        kv_restore_v_blocked<float><<<vgrid, 256, lds, stream>>>(
-            static_cast<uint16_t *>(pool_base), g, b);
     return hipGetLastError();
 }
 
