@@ -113,3 +113,35 @@ def test_device_and_oracle_stores_serve_each_other(tmp_path):
     files = sorted(p.name for p in (tmp_path / "dev").iterdir())
     assert files == sorted(p.name for p in (tmp_path / "ora").iterdir())
     pool.close()
+
+
+@pytest.mark.parametrize("elem", ["f32", "f16"])
+def test_an_entry_filed_from_a_slot_carries_the_trailer_an_independent_sum_gives(tmp_path, elem):
+    """The store sums a captured payload while it writes it. What lands on disk must be what a
+    capture into memory gives, trailer included, and the trailer what the oracle's restatement
+    of the checksum (byte-serial for version 1, sum of block sums for version 2) computes."""
+    import struct
+
+    rng = np.random.default_rng(21)
+    kvh, d, n = 4, 128, 1500  # 1500 x 512 x 2 sides: 6.1 MB of f32 rows, 3.1 MB of f16 rows
+    pool = P().KvPool([P().LayerKind.Global, P().LayerKind.windowed(256)], kvh, d, elem="f16",
+                      max_slots=2, capacity_rows=n + 8)
+    cache = pool.acquire()
+    k, v = normal(rng, n, kvh * d), normal(rng, n, kvh * d)
+    cache.restore_bulk(0, 0, k, v)
+    cache.restore_bulk(1, n - 256, k[n - 256:], v[n - 256:])
+    tokens = [int(t) for t in rng.integers(0, 1 << 20, size=n)]
+    store = P().PrefixStore.open(str(tmp_path), 1 << 30)
+    store.capture_and_put(cache, tokens, "m", now=5, elem=elem)
+    entry = (tmp_path / store.entries()[0].file_name).read_bytes()
+    payload = entry[72 + 4 * n:]
+    assert payload == P().capture_bytes(cache, "m", elem=elem)
+    stored = struct.unpack("<Q", payload[-8:])[0]
+    fast = lambda block: oracle.checksum(bytes(block))
+    want = fast(payload[:-8]) if elem == "f32" else okv.block_checksum(payload[:-8], fast)
+    assert stored == want
+    fresh = pool.acquire()
+    assert store.restore_prefix(fresh, tokens, "m", now=6) == n
+    for layer in range(2):
+        assert view_bytes(fresh, layer) == view_bytes(cache, layer)
+    pool.close()
