@@ -581,8 +581,8 @@ def test_snapshots_of_a_hybrid_cache_round_trip_and_match_the_oracles_bytes(elem
 # ---------------------------------------------------------------- Compute::attention mirror
 
 
-@pytest.mark.parametrize("elem", ["f32", "f16"])
-def test_compute_attention_on_a_hybrid_model_takes_any_number_of_rows(elem):
+@pytest.mark.parametrize("elem,d", [("f32", 16), ("f16", 16), ("f16", 128)])
+def test_compute_attention_on_a_hybrid_model_takes_any_number_of_rows(elem, d):
     # cpu.rs:586-646 on the reference model's kind of pattern: the host-pointer call rotates
     # Q and K on the sliding-window layers (interleaved RoPE at the SWA base, each row at its
     # position; global layers are NoPE), then appends and attends row by row in the
@@ -590,14 +590,16 @@ def test_compute_attention_on_a_hybrid_model_takes_any_number_of_rows(elem):
     # window) must come out the same, and decoding on from it too.
     rng = np.random.default_rng(41)
     SW, G = P().LayerKind.SlidingWindow, P().LayerKind.Global
-    cfg = P().GlimmerConfig(layers=[SW, SW, G], q_heads=8, kv_heads=2, key_length=16,
-                            value_length=16, sliding_window=20, rope_freq_base_swa=10000.0)
+    # (head_dim 128 on an f16 pool is the MFMA path: single rows and short blocks rotate inside
+    # the attention launch, long blocks by a launch of their own before the block kernel.)
+    cfg = P().GlimmerConfig(layers=[SW, SW, G], q_heads=8, kv_heads=2, key_length=d,
+                            value_length=d, sliding_window=20, rope_freq_base_swa=10000.0)
     ref = oracle.KvCache.new([oracle.LayerKind.windowed(20), oracle.LayerKind.windowed(20),
                               oracle.LayerKind.Global], cfg.kv_heads, cfg.key_length,
                              store_f16=(elem == "f16"))
     hc = P().HipCompute.new(elem=elem, capacity_rows=512)
     cache = P().PositionCache()
-    for rows in (150, 1, 1, 70, 1):
+    for rows in (150, 1, 1, 65, 5, 1):
         for layer, kind in enumerate(cfg.layers):
             q = normal(rng, rows, cfg.q_width())
             k = normal(rng, rows, cfg.k_width())
