@@ -146,7 +146,7 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
                                               uint32_t lo_max, float softcap, float inv_cap) {
     const uint32_t key_base = kb * kBlockKeys + g * 8;  // first of this lane's 8 keys
     const bool tail = (kb + 1) * kBlockKeys > kv_len || (RING && kb * kBlockKeys < lo_min);
-    if (tail) {
+    auto zero_tail = [&] {
         // Rows past the stored length, and ring rows older than anything the block's queries
         // see, may hold stale data: keep them out of P.V even as 0*x.
 #pragma unroll
@@ -155,7 +155,10 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
             for (int e = 0; e < 8; ++e)
                 if (key_base + e >= kv_len || (RING && key_base + e < lo_min))
                     b.v[dt][e] = _Float16(0.0f);
-    }
+    };
+    if (NQ <= 2 && tail) zero_tail();
+    [[maybe_unused]] half8 pbs[NQ > 2 ? NQ : 1];
+    [[maybe_unused]] float alphas[NQ > 2 ? NQ : 1];
     const bool need_mask =
         (kb + 1) * kBlockKeys > pos0 + 1 || (RING && kb * kBlockKeys < lo_max);
 #pragma unroll
@@ -197,7 +200,13 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
 #pragma unroll
         for (int e = 1; e < 8; ++e) mx = fmaxf(mx, sc[e]);
         mx = column_max(mx);
-        const float m_new = FIRST ? mx : fmaxf(st.m[qt], mx);
+        // 64 vectors: the column's reference follows the block maximum only when that runs
+        // more than kSlack ahead of it (P stays below 2^kSlack, far inside f16 and f32 range;
+        // every term of numerator and denominator carries the same factor, so the softmax is
+        // the same). Rescaling the 32 accumulators of a tile, which live in accumulation
+        // registers there and cost three instructions an element, then leaves the common path.
+        constexpr float kSlack = NQ > 2 ? 8.0f : 0.0f;
+        const float m_new = FIRST ? mx : (mx > st.m[qt] + kSlack ? mx : st.m[qt]);
         const bool dead = m_new == -INFINITY;  // nothing visible to this column so far
         float p[8];
         float sum = 0.0f;
@@ -209,15 +218,21 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
         half8 pb;
 #pragma unroll
         for (int e = 0; e < 8; ++e) pb[e] = static_cast<_Float16>(p[e]);
-        if constexpr (FIRST) {
-            st.l[qt] = sum;
+        const float alpha = (FIRST || dead) ? 1.0f : fast_exp2(st.m[qt] - m_new);
+        st.l[qt] = FIRST ? sum : st.l[qt] * alpha + sum;
+        st.m[qt] = m_new;
+        if constexpr (NQ > 2) {
+            // 64 vectors: P.V of all tiles after the scores of all tiles, so that the value
+            // operands (fetched after the keys, with no block of lead) are not needed before
+            // four tiles of score MFMAs and softmax have run.
+            pbs[qt] = pb;
+            alphas[qt] = alpha;
+        } else if constexpr (FIRST) {
 #pragma unroll
             for (int dt = 0; dt < 8; ++dt)
                 st.o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
                     b.v[dt], pb, floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
         } else {
-            const float alpha = dead ? 1.0f : fast_exp2(st.m[qt] - m_new);
-            st.l[qt] = st.l[qt] * alpha + sum;
 #pragma unroll
             for (int dt = 0; dt < 8; ++dt) {
                 st.o[qt][dt] *= alpha;
@@ -225,7 +240,29 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
                     __builtin_amdgcn_mfma_f32_16x16x32_f16(b.v[dt], pb, st.o[qt][dt], 0, 0, 0);
             }
         }
-        st.m[qt] = m_new;
+    }
+    if constexpr (NQ > 2) {
+        if (tail) zero_tail();
+        if constexpr (!FIRST) {
+#pragma unroll
+            for (int qt = 0; qt < NQ; ++qt)
+                if (__builtin_amdgcn_ballot_w64(alphas[qt] != 1.0f) != 0) {  // some reference moved
+#pragma unroll
+                    for (int dt = 0; dt < 8; ++dt) st.o[qt][dt] *= alphas[qt];
+                }
+        }
+#pragma unroll
+        for (int qt = 0; qt < NQ; ++qt)
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) {
+                if constexpr (FIRST) {
+                    st.o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        b.v[dt], pbs[qt], floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+                } else {
+                    st.o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b.v[dt], pbs[qt],
+                                                                          st.o[qt][dt], 0, 0, 0);
+                }
+            }
     }
 }
 
