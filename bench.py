@@ -42,7 +42,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # HBM bytes per layer (all launches of the layer's attention) measured with rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE and scaled by the same counters on the probe copy of known size
 # (profiles/*_traffic.md hold the runs and the scaling factors). Missing = not measured.
-MEASURED_TRAFFIC = {"decode": 9_961_044, "ragged": 216_851_725, "prefill": 290_273_442}
+MEASURED_TRAFFIC = {"decode": 9_962_081, "ragged": 216_870_262, "prefill": 290_264_395}
 
 
 def rope_on_device(x, base):
