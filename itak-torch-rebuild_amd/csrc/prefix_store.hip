@@ -581,8 +581,11 @@ itak_status verify_candidate(itak_store *s, StoreError &why, const Entry &meta,
     const int64_t arrived =
         typed ? read_blocks_with_checksum(fd, s->stage, payload, tokens_end, sum_len, &sum)
               : read_at_with_checksum(fd, s->stage, payload, tokens_end, sum_len, &sum);
-    if (arrived != int64_t(payload))
-        return io_error(why, errno, "read entry %s", meta.file_name.c_str());
+    if (arrived < 0) return io_error(why, errno, "read entry %s", meta.file_name.c_str());
+    if (uint64_t(arrived) != payload)  // the file shrank after it was measured
+        return fail(why, ITAK_KV_TRUNCATED, "entry payload", payload, uint64_t(arrived),
+                    "entry payload: truncated, needs %llu bytes, has %llu", ULL(payload),
+                    ULL(uint64_t(arrived)));
     ItkvHeader &h = s->stage_header;
     std::vector<ItkvLayer> &layers = s->stage_layers;
     ItkvError decode_error;
