@@ -282,6 +282,7 @@ itak_status ensure_prep(itak_pool *pool, uint64_t floats) {
     return ITAK_OK;
 }
 
+constexpr uint64_t kHostWord = 256;  // bytes at the head of the pinned staging kept for the completion word
 itak_status ensure_hstage(itak_pool *pool, uint64_t bytes) {
     if (bytes <= pool->hstage_bytes) return ITAK_OK;
     HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize before growing pinned staging");
@@ -291,6 +292,7 @@ itak_status ensure_hstage(itak_pool *pool, uint64_t bytes) {
     const uint64_t want = std::max<uint64_t>(bytes + bytes / 2, 1u << 18);
     HIP_TRY(pool, hipHostMalloc(reinterpret_cast<void **>(&pool->hstage), want, hipHostMallocDefault),
             "allocate pinned staging");
+    memset(pool->hstage, 0, want);  // the completion word of a call must not start out matching
     pool->hstage_bytes = want;
     return ITAK_OK;
 }
@@ -1996,21 +1998,25 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
     float *out_pinned = nullptr;
     uint32_t *done_word = nullptr;  // in pinned memory, after the output
     if (packed) {
-        st = ensure_hstage(pool, in_bytes + q_bytes + 256);
+        // Layout: [completion word, 256 bytes] [q | k | v] [output]. The word sits at a fixed
+        // place, so it only ever holds call numbers, which only grow.
+        st = ensure_hstage(pool, kHostWord + in_bytes + q_bytes);
         if (st != ITAK_OK) return st;
-        memcpy(pool->hstage, q, q_len * 4);
-        memcpy(pool->hstage + q_bytes, k, k_len * 4);
-        memcpy(pool->hstage + q_bytes + kv_bytes, v, v_len * 4);
+        unsigned char *hin = pool->hstage + kHostWord;
+        memcpy(hin, q, q_len * 4);
+        memcpy(hin + q_bytes, k, k_len * 4);
+        memcpy(hin + q_bytes + kv_bytes, v, v_len * 4);
         void *mapped = nullptr;
         HIP_TRY(pool, hipHostGetDevicePointer(&mapped, pool->hstage, 0), "map pinned staging");
         unsigned char *pinned_dev = static_cast<unsigned char *>(mapped);
         if (in_bytes <= (64u << 10))
-            HIP_TRY(pool, launch_stage_in(pinned_dev, qd, in_bytes, pool->stream), "launch stage-in");
+            HIP_TRY(pool, launch_stage_in(pinned_dev + kHostWord, qd, in_bytes, pool->stream),
+                    "launch stage-in");
         else
-            HIP_TRY(pool, hipMemcpyAsync(qd, pool->hstage, in_bytes, hipMemcpyHostToDevice, pool->stream),
+            HIP_TRY(pool, hipMemcpyAsync(qd, hin, in_bytes, hipMemcpyHostToDevice, pool->stream),
                     "upload q, k, v");
-        out_pinned = reinterpret_cast<float *>(pinned_dev + in_bytes);
-        done_word = reinterpret_cast<uint32_t *>(pinned_dev + in_bytes + q_bytes);
+        out_pinned = reinterpret_cast<float *>(pinned_dev + kHostWord + in_bytes);
+        done_word = reinterpret_cast<uint32_t *>(pinned_dev);
     } else {
         HIP_TRY(pool, hipMemcpyAsync(kd, k, k_len * 4, hipMemcpyHostToDevice, pool->stream), "upload k");
         HIP_TRY(pool, hipMemcpyAsync(vd, v, v_len * 4, hipMemcpyHostToDevice, pool->stream), "upload v");
@@ -2088,7 +2094,7 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
     const uint32_t number = ++pool->call_number ? pool->call_number : ++pool->call_number;
     HIP_TRY(pool, launch_signal_done(done_word, number, pool->stream), "launch completion signal");
     const volatile uint32_t *seen =
-        reinterpret_cast<const volatile uint32_t *>(pool->hstage + in_bytes + q_bytes);
+        reinterpret_cast<const volatile uint32_t *>(pool->hstage);
     timespec t0{};
     clock_gettime(CLOCK_MONOTONIC, &t0);
     bool arrived = false;
@@ -2103,7 +2109,7 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
         if ((t1.tv_sec - t0.tv_sec) * 1000000000ll + (t1.tv_nsec - t0.tv_nsec) > 300000) break;
     }
     if (!arrived) HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize after attention");
-    memcpy(out, pool->hstage + in_bytes, q_len * 4);
+    memcpy(out, pool->hstage + kHostWord + in_bytes, q_len * 4);
     return ITAK_OK;
 }
 
