@@ -4,7 +4,8 @@ and gate as one device step, against the oracle's composition of the reference's
 
 Bars: prepared K rows in an f32 cache within 1e-6 of the oracle's (the reference pins its own
 fused kernel against the unfused chain at 1e-5, crates/wgpu-compute/tests/fused_kernels.rs:
-408-431), V rows exact; outputs within 1e-5 relative on f32 KV and 2e-3 max-abs on f16 KV."""
+408-431), in an f16 cache within one f16 step or 1e-6, V rows exact; outputs within 1e-5
+relative on f32 KV and 2e-3 max-abs on f16 KV."""
 import numpy as np
 import pytest
 import torch
@@ -84,11 +85,16 @@ def run_case(elem, q_heads, kv_heads, d, ctx, rows, norm, rope_base, interleaved
             assert max_abs(gk.reshape(rows, width), kp) <= 1e-6
             assert gv.reshape(rows, width).tobytes() == vs[s].tobytes()
         else:
-            # A prepared key that differs from the oracle's in its last f32 bit can round to
-            # the neighbouring half: one f16 ulp at most.
+            # A prepared key that differs from the oracle's in its last f32 bits can round to
+            # the neighbouring half: one f16 step at most, except where the rotation cancelled
+            # (|x*cos - y*sin| far below |x|), whose result carries the absolute error of the
+            # f32 products, a few 1e-7, which near zero is more than one of f16's small steps.
+            want_bits = oracle.f32_to_f16_array(kp)
             ulp = np.abs(gk.reshape(rows, width).view(np.int16).astype(np.int32)
-                         - oracle.f32_to_f16_array(kp).view(np.int16).astype(np.int32))
-            assert ulp.max() <= 1
+                         - want_bits.view(np.int16).astype(np.int32))
+            far = np.abs(gk.reshape(rows, width).view(np.float16).astype(np.float64)
+                         - want_bits.view(np.float16).astype(np.float64))
+            assert np.all((ulp <= 1) | (far <= 1e-6))
             assert np.array_equal(gv.reshape(rows, width), oracle.f32_to_f16_array(vs[s]))
         assert caches[s].next_position(0) == n0 + rows
     pool.close()
@@ -169,7 +175,9 @@ def test_folded_preparation_at_a_long_position_keeps_the_f16_bar():
     _, gk, _ = cache.read_rows(0, pos, 1)
     want = oracle.f32_to_f16_array(oracle.attention_prep(k, kv_heads, d, pos, None, 1e-6, 1e4, True))
     ulp = np.abs(gk.reshape(-1).view(np.int16).astype(np.int32) - want.reshape(-1).view(np.int16).astype(np.int32))
-    assert ulp.max() <= 1
+    far = np.abs(gk.reshape(-1).view(np.float16).astype(np.float64)
+                 - want.reshape(-1).view(np.float16).astype(np.float64))
+    assert np.all((ulp <= 1) | (far <= 1e-6))
     pool.close()
 
 
