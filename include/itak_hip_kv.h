@@ -514,7 +514,8 @@ typedef struct itak_prep_params {
    On f16 pools with head_dim 128, steps of up to 64 query vectors per KV head (rows x group:
    decode, speculative blocks) add no launch to the plain step's two: the attention kernel norms and
    rotates the Q rows it stages and the new K row it appends (f64 angle, f32 arithmetic:
-   within one f16 step of the reference's f64 chain in the stored K), and the kernel that
+   within one f16 step, or 1e-6 where a rotation cancels, of the reference's f64 chain in the
+   stored K), and the kernel that
    writes the output applies the gate. Other shapes run norms and rotation as one launch
    before the step, with the numerics of the reference's CPU path (f64 norm, f64 angles),
    not of its f32 shader; f32 pools hold prepared K rows within 1e-6 of that path. */
