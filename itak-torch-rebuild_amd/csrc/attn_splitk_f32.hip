@@ -1,0 +1,327 @@
+// GQA flash-decode for gfx950 over f32 KV (the reference's own storage type), head_dim 128,
+// up to 16 query vectors per KV head (rows x group: decode steps and short blocks): split over
+// the context like the f16 kernel, products on v_mfma_f32_16x16x4_f32 (f32 in, f32 out: the
+// 1e-5 bar of f32 pools holds), K and V read straight from their row-major planes with 16-byte
+// loads, no LDS in the loop; a step's new rows are appended by the same launch. Everything
+// else (other head dims, more vectors, explicit query positions) stays on the generic kernel.
+//
+// One workgroup of four wavefronts owns (item, kv head, split = a run of 32-key blocks); each
+// wavefront walks its own blocks with a private online softmax, the four merge once through
+// LDS. The MFMA takes one float per lane and operand: A[i][k] from lane i + 16k, B[k][j] from
+// lane j + 16k, and returns rows 4g .. 4g+3 of column j to lane j + 16g. A dot product does
+// not care in which order its terms are taken, so the channels (for K.Q^T) and the keys (for
+// V^T.P^T) are assigned to the MFMA's k index in whatever order lets every lane fetch 16
+// contiguous bytes:
+//
+//   S^T = K . Q^T   per 16-key tile t, 32 steps (s, e): lane (i, g) supplies K[key 16t + i]
+//                   [channel 16s + 4g + e], i.e. the float4 at channels 16s + 4g of its key
+//                   row covers the four e of a step group; Q^T is held the same way.
+//                   Lane (j, g) receives the scores of keys 16t + 4g + r, r = 0..3.
+//   O^T += V^T . P^T  per tile t and r = 0..3 the k index g stands for key 16t + 4g + r, whose
+//                   probability is exactly what lane (j, g) holds in score register r: P needs
+//                   no shuffle. Output tile (h, e) row i is channel 64h + 4i + e, so lane
+//                   (i, g) fetches the float4 at channels 64h + 4i of value row 16t + 4g + r.
+//
+// Semantics: gqa_attention in crates/attention/src/attention.rs:104-215, softcap as
+// crates/torch-math/src/logits.rs:26-37. Partials are in the log2 domain.
+#include "internal.h"
+#include "mfma_common.h"
+
+#include <math.h>
+
+#include <algorithm>
+
+namespace itak {
+
+namespace {
+
+constexpr int kWavesF32 = 4;
+
+__device__ __forceinline__ float lanes4_max(float v) {  // over lanes l, l^16, l^32, l^48
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(c[0]), __uint_as_float(c[1]));
+}
+__device__ __forceinline__ float lanes4_sum(float v) {
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(c[0]) + __uint_as_float(c[1]);
+}
+
+template <int N, bool RING>
+__global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnParams p,
+                                                                         AttnBatchT<N> b,
+                                                                         uint32_t total_partials) {
+    __shared__ float sm_m[kWavesF32][16], sm_l[kWavesF32][16];
+    __shared__ float sm_o[kWavesF32][8][64][4];  // [wave][tile (h, e)][lane][row of the lane]
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = tid >> 6, lane = tid & 63;
+    const uint32_t g = lane >> 4, jl = lane & 15;
+
+    const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
+    const uint32_t local = blockIdx.x - item.block0;
+    const uint32_t kv_head = local / item.splits, split = local % item.splits;
+    const uint32_t group = p.group, nvec = item.rows * group;
+
+    const float *kplane = static_cast<const float *>(p.layer_base) + item.slot * p.g.slot_stride +
+                          kv_head * p.g.head_stride;
+    const float *vplane = kplane + p.g.side_stride;
+
+    const uint32_t nblocks = (item.kv_len + kBlockKeys - 1) / kBlockKeys;
+    const uint32_t blocks_per_split = item.keys_per_split / kBlockKeys;
+    const uint32_t kb_begin = (RING ? item_first_block(item) : 0) + split * blocks_per_split;
+    const uint32_t kb_end = min(nblocks, kb_begin + blocks_per_split);
+    const uint32_t ring = RING ? p.ring_blocks * kBlockKeys : 0;
+    const uint32_t window = RING ? p.window : 0, kv_lo = RING ? item.kv_lo : 0;
+
+    // Fused append (p.k_new set): the last `rows` positions are not in the planes yet. The
+    // workgroups whose blocks reach them copy the new rows in (f32 to f32, all threads, 16 bytes
+    // each) and meet at a barrier before anybody reads a block; where two splits both reach
+    // them both write the same bytes. No other workgroup reads these positions.
+    if (p.k_new != nullptr && kb_end * kBlockKeys > item.pos0) {
+        const uint32_t row_width = p.g.kv_heads * kD;
+        for (uint32_t f = tid; f < item.rows * 64; f += kWavesF32 * 64) {
+            const uint32_t r = f >> 6, side = (f >> 5) & 1, c4 = (f & 31) * 4;
+            const float *src = (side ? p.v_new : p.k_new) + uint64_t(item.q_row0 + r) * row_width +
+                               kv_head * kD + c4;
+            const uint32_t pos = item.pos0 + r;
+            float *dst = const_cast<float *>(side ? vplane : kplane) +
+                         uint64_t(RING ? pos % ring : pos) * kD + c4;
+            *reinterpret_cast<float4 *>(dst) = *reinterpret_cast<const float4 *>(src);
+        }
+        __syncthreads();
+    }
+
+    // This lane's query vector (column jl) and what its mask and its output need.
+    const uint32_t j = min(jl, nvec - 1);
+    const uint32_t row = j / group, head = kv_head * group + j % group;
+    const uint32_t colpos = min(item.pos0 + row, item.kv_len - 1);
+    const uint32_t collo = lowest_visible(item.pos0 + row, window, kv_lo);
+    const uint32_t lo_min = lowest_visible(item.pos0, window, kv_lo);
+    const float softcap = p.softcap;
+    const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
+    const float qscale = softcap > 0.0f ? p.scale : p.scale * kLog2e;
+
+    // Q^T as B operands: step (s, e) takes channel 16s + 4g + e of vector jl.
+    float4 qreg[8];
+    {
+        const float *qp = p.q + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + 4 * g;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            float4 a = *reinterpret_cast<const float4 *>(qp + 16 * s);
+            if (jl >= nvec) a = make_float4(0.f, 0.f, 0.f, 0.f);
+            qreg[s] = make_float4(a.x * qscale, a.y * qscale, a.z * qscale, a.w * qscale);
+        }
+    }
+
+    float m_run = -INFINITY, l_run = 0.0f;
+    floatx4 o[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[h][e] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (uint32_t kb = kb_begin + wave; kb < kb_end; kb += kWavesF32) {
+        const uint32_t key0 = kb * kBlockKeys;
+        // Rows past the stored length are fetched from the last stored row instead (the
+        // plane may end there) and masked; a position's storage row on a ring is pos % ring.
+        auto storage_row = [&](uint32_t pos) {
+            const uint32_t q = min(pos, item.kv_len - 1);
+            return RING ? q % ring : q;
+        };
+        float4 kreg[2][8], vreg[2][4][2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const float *kr = kplane + uint64_t(storage_row(key0 + 16 * t + jl)) * kD + 4 * g;
+#pragma unroll
+            for (int s = 0; s < 8; ++s) kreg[t][s] = *reinterpret_cast<const float4 *>(kr + 16 * s);
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float *vr = vplane + uint64_t(storage_row(key0 + 16 * t + 4 * g + r)) * kD + 4 * jl;
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+                    vreg[t][r][h] = *reinterpret_cast<const float4 *>(vr + 64 * h);
+            }
+
+        // Scores of keys key0 + 16t + 4g + r for this lane's vector.
+        float sc[2][4];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            floatx4 acc = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[t][s].x, qreg[s].x, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[t][s].y, qreg[s].y, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[t][s].z, qreg[s].z, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[t][s].w, qreg[s].w, acc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sc[t][r] = acc[r];
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t kp = key0 + 16 * t + 4 * g + r;
+                float v = sc[t][r];
+                if (softcap > 0.0f) v = softcap_log2(v, softcap, inv_cap);
+                if (kp > colpos || (RING && kp < collo)) v = -INFINITY;
+                sc[t][r] = v;
+                mx = fmaxf(mx, v);
+                // A row no query of the item sees (past the stored length, or older than the
+                // oldest window on a ring) may hold anything: keep it out of P.V even as 0*x.
+                if (kp >= item.kv_len || (RING && kp < lo_min)) {
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) vreg[t][r][h] = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
+        mx = lanes4_max(mx);
+        const float m_new = fmaxf(m_run, mx);
+        const bool dead = m_new == -INFINITY;
+        const float alpha = (dead || m_run == -INFINITY) ? (dead ? 1.0f : 0.0f) : fast_exp2(m_run - m_new);
+        float sum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float pe = dead ? 0.0f : fast_exp2(sc[t][r] - m_new);
+                sc[t][r] = pe;
+                sum += pe;
+            }
+        l_run = l_run * alpha + sum;
+        m_run = m_new;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[h][e] *= alpha;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const float4 a = vreg[t][r][h];
+                    o[h][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, sc[t][r], o[h][0], 0, 0, 0);
+                    o[h][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, sc[t][r], o[h][1], 0, 0, 0);
+                    o[h][2] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, sc[t][r], o[h][2], 0, 0, 0);
+                    o[h][3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, sc[t][r], o[h][3], 0, 0, 0);
+                }
+    }
+
+    // ---- merge the wavefronts through LDS: wavefront w finishes tiles 2w and 2w + 1.
+    const float l_col = lanes4_sum(l_run);
+    if (g == 0) {
+        sm_m[wave][jl] = m_run;
+        sm_l[wave][jl] = l_col;
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            *reinterpret_cast<floatx4 *>(&sm_o[wave][h * 4 + e][lane][0]) = o[h][e];
+    __syncthreads();
+
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kWavesF32; ++w) M = fmaxf(M, sm_m[w][jl]);
+    float L = 0.0f, wgt[kWavesF32];
+#pragma unroll
+    for (int w = 0; w < kWavesF32; ++w) {
+        const float mw = sm_m[w][jl];
+        wgt[w] = mw == -INFINITY ? 0.0f : fast_exp2(mw - M);
+        L = fmaf(sm_l[w][jl], wgt[w], L);
+    }
+    if (jl >= nvec) return;
+    const bool final_out = item.splits == 1;
+    const uint64_t ps = item.ws0 + (uint64_t(row) * p.q_heads + head) * item.splits + split;
+    float *dst = final_out ? p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD
+                           : p.ws + ps * kD;
+    const float post = final_out ? 1.0f / L : 1.0f;
+    // Tile (h, e), lane (jl, g), register rr holds channel 64h + 16g + 4rr + e: the four e of
+    // one (h, rr) are 16 contiguous bytes, and this wavefront owns e = 2 (wave % 2) .. +1 of
+    // h = wave / 2.
+    const uint32_t h = wave >> 1, e0 = (wave & 1) * 2;
+    floatx4 fin[2];
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+        fin[x] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int w = 0; w < kWavesF32; ++w)
+            fin[x] += *reinterpret_cast<const floatx4 *>(&sm_o[w][h * 4 + e0 + x][lane][0]) * wgt[w];
+        fin[x] *= post;
+    }
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr)
+        *reinterpret_cast<float2 *>(dst + 64 * h + 16 * g + 4 * rr + e0) =
+            make_float2(fin[0][rr], fin[1][rr]);
+    if (!final_out && wave == 0 && g == 0)
+        *reinterpret_cast<float2 *>(p.ws + uint64_t(total_partials) * kD + ps * 2) = make_float2(M, L);
+}
+
+}  // namespace
+
+bool attn_splitk_f32_supports(const PoolGeom &g, uint32_t group, uint32_t max_rows) {
+    return g.v_block == 0 && g.head_dim == kD && group >= 1 && max_rows >= 1 &&
+           max_rows * group <= 16;
+}
+
+// Fills splits / keys_per_split / block0 / ws0 (slot, rows, pos0, q_row0, kv_len, kv_lo are
+// set) and returns the number of partials. Every (item, KV head) is cut into equal runs of at
+// most T blocks, T the smallest run for which the batch is at most two workgroups per
+// compute unit, and never shorter than one block per wavefront.
+uint32_t attn_splitk_f32_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads) {
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        (void)hipGetLastError();
+    const uint64_t capacity = uint64_t(2) * uint64_t(cus > 0 ? cus : 256);
+    uint64_t blocks = 0;
+    for (uint32_t i = 0; i < b.n; ++i) blocks += uint64_t(g.kv_heads) * item_block_count(b.item[i]);
+    uint64_t T = std::max<uint64_t>((blocks + capacity - 1) / capacity, uint64_t(kWavesF32));
+    for (;; ++T) {
+        uint64_t groups = 0;
+        for (uint32_t i = 0; i < b.n; ++i) {
+            const uint64_t nb = item_block_count(b.item[i]);
+            groups += uint64_t(g.kv_heads) * std::max<uint64_t>((nb + T - 1) / T, 1);
+        }
+        if (groups <= capacity || T >= blocks) break;
+    }
+    uint32_t block0 = 0, ws0 = 0;
+    for (uint32_t i = 0; i < b.n; ++i) {
+        AttnItem &it = b.item[i];
+        const uint32_t nblocks = item_block_count(it);
+        it.splits = std::max<uint32_t>(uint32_t((nblocks + T - 1) / T), 1);
+        const uint32_t bps = std::max<uint32_t>((nblocks + it.splits - 1) / it.splits, 1);
+        it.splits = std::max<uint32_t>((nblocks + bps - 1) / bps, 1);
+        it.keys_per_split = bps * kBlockKeys;
+        it.splits_magic = 0;
+        it.block0 = block0;
+        it.ws0 = ws0;
+        block0 += g.kv_heads * it.splits;
+        if (it.splits > 1) ws0 += it.rows * q_heads * it.splits;
+    }
+    b.total_blocks = block0;
+    b.rows_per_block = 0;
+    return ws0;
+}
+
+hipError_t launch_attn_splitk_f32(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                                  hipStream_t stream) {
+    if (b.total_blocks == 0) return hipSuccess;
+    if (p.ring_blocks)
+        ITAK_DISPATCH_BATCH(b.n, (attn_splitk_f32_kernel<N, true><<<b.total_blocks, kWavesF32 * 64, 0, stream>>>(
+                                     p, AttnBatchT<N>(b), total_partials)));
+    else
+        ITAK_DISPATCH_BATCH(b.n, (attn_splitk_f32_kernel<N, false><<<b.total_blocks, kWavesF32 * 64, 0, stream>>>(
+                                     p, AttnBatchT<N>(b), total_partials)));
+    return hipGetLastError();
+}
+
+}  // namespace itak

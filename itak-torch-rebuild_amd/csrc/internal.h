@@ -336,6 +336,12 @@ uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads)
 hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                   uint32_t max_rows, hipStream_t stream,
                                   const FoldedParams *folded = nullptr);
+// f32 MFMA split-K path: f32 pools (row-major planes), head_dim 128, rows*group <= 16, implied
+// query positions. Partials are in log2 domain (combine with base2 = 1).
+bool attn_splitk_f32_supports(const PoolGeom &g, uint32_t group, uint32_t max_rows);
+uint32_t attn_splitk_f32_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads);
+hipError_t launch_attn_splitk_f32(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                                  hipStream_t stream);
 // MFMA block path (speculative blocks and prefill chunks): same pools, any number of rows,
 // group dividing 16; K/V staged through LDS, split over the context when the launch would
 // otherwise not fill the device. Partials are in log2 domain (combine with base2 = 1).

@@ -341,9 +341,12 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
     // Blocks of many rows (prefill chunks) on the same pools take the MFMA prefill kernel.
     const bool prefill = !mfma && pool->elem_f16 && q_pos_dev == nullptr &&
                          attn_prefill_f16_supports(pool->g, group);
+    // Decode steps and short blocks on f32 pools of head_dim 128: the f32 MFMA split-K kernel.
+    const bool f32fast = !pool->elem_f16 && q_pos_dev == nullptr &&
+                         attn_splitk_f32_supports(pool->g, group, max_rows);
     const uint32_t rpb =
-        (mfma || prefill) ? 0 : attn_generic_rows_per_block(group, pool->g.head_dim);
-    if (!mfma && !prefill && rpb == 0)
+        (mfma || prefill || f32fast) ? 0 : attn_generic_rows_per_block(group, pool->g.head_dim);
+    if (!mfma && !prefill && !f32fast && rpb == 0)
         return unsupported(pool->err, "head_dim above 256 or GQA group too wide");
     const uint32_t tile = attn_generic_tile(pool->g.head_dim);
     constexpr uint64_t kTargetBlocks = 1024;  // about four workgroups per CU
@@ -374,6 +377,8 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
             partials = attn_splitk_f16_plan(geom, b, uint32_t(q_heads));
         } else if (prefill) {
             partials = attn_prefill_f16_plan(geom, b, group, uint32_t(q_heads), window);
+        } else if (f32fast) {
+            partials = attn_splitk_f32_plan(geom, b, uint32_t(q_heads));
         } else {
             b.rows_per_block = rpb;
             uint64_t key_work = 0;
@@ -413,8 +418,8 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         p.out = out_dev;
         p.q_pos = q_pos_dev;
         p.ws = pool->ws;
-        p.k_new = mfma ? k_new : nullptr;
-        p.v_new = mfma ? v_new : nullptr;
+        p.k_new = (mfma || f32fast) ? k_new : nullptr;
+        p.v_new = (mfma || f32fast) ? v_new : nullptr;
         p.q_heads = uint32_t(q_heads);
         p.group = group;
         p.group_magic = (65536u + group - 1) / group;
@@ -436,11 +441,14 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         } else if (prefill) {
             HIP_TRY(pool, launch_attn_prefill_f16(p, b, partials, pool->stream),
                     "launch block attention");
+        } else if (f32fast) {
+            HIP_TRY(pool, launch_attn_splitk_f32(p, b, partials, pool->stream),
+                    "launch f32 split-K attention");
         } else {
             HIP_TRY(pool, launch_attn_generic(pool->elem_f16, p, b, partials, pool->stream),
                     "launch attention");
         }
-        HIP_TRY(pool, launch_attn_combine(p, b, partials, total_rows, (mfma || prefill) ? 1 : 0,
+        HIP_TRY(pool, launch_attn_combine(p, b, partials, total_rows, (mfma || prefill || f32fast) ? 1 : 0,
                                           pool->stream, gate_folded ? gate : nullptr),
                 "launch split merge");
         if (gate && !gate_folded) {
@@ -1731,8 +1739,12 @@ static itak_status step_on_device(itak_pool *pool, uint64_t layer, const itak_ba
     std::vector<PlanInput> active;
     for (const PlanInput &p : plan)
         if (p.rows) active.push_back(p);
-    const bool fuse = takes_splitk_f16(pool, active.data(), uint32_t(active.size()), num_q_heads,
-                                       nullptr);
+    uint32_t most_rows = 0;
+    for (const PlanInput &p : active) most_rows = std::max(most_rows, p.rows);
+    const bool fuse =
+        takes_splitk_f16(pool, active.data(), uint32_t(active.size()), num_q_heads, nullptr) ||
+        (!pool->elem_f16 && !active.empty() &&
+         attn_splitk_f32_supports(pool->g, uint32_t(num_q_heads / pool->g.kv_heads), most_rows));
     if (fuse) {
         for (uint32_t i = 0; i < item_count; ++i)
             advance(pool->slots[items[i].slot], layer, items[i].rows);
