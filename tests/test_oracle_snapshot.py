@@ -343,3 +343,72 @@ def test_a_version_2_snapshot_of_several_blocks_decodes_and_a_flip_in_any_block_
     with pytest.raises(P.KvError) as e:
         P.KvSnapshot.from_bytes(forged)
     assert e.value.variant == "ChecksumMismatch"
+
+
+def _mutated(good, rng):
+    """One seeded corruption of encoded bytes: flips, cuts, insertions and extreme field values,
+    half of them with the trailer recomputed so that the checks behind the checksum are reached."""
+    b = bytearray(good)
+    extremes = (0, 1, 2, 3, 0x80000000, 0xFFFFFFFF, 1 << 32, 1 << 61, 1 << 62, (1 << 63) - 1, (1 << 64) - 1)
+    for _ in range(int(rng.integers(1, 4))):
+        kind = int(rng.integers(0, 6))
+        if kind == 0 and b:
+            b[int(rng.integers(0, len(b)))] ^= 1 << int(rng.integers(0, 8))
+        elif kind == 1:
+            del b[int(rng.integers(0, len(b) + 1)):]
+        elif kind == 2 and len(b) >= 16:
+            width = 8 if rng.integers(0, 2) else 4
+            at = int(rng.integers(0, min(len(b) - 8, 200) - width + 1)) & ~3
+            b[at:at + width] = int(extremes[int(rng.integers(0, len(extremes)))] % (1 << (8 * width))).to_bytes(width, "little")
+        elif kind == 3:
+            b += rng.integers(0, 256, size=int(rng.integers(1, 40)), dtype=np.uint8).tobytes()
+        elif kind == 4 and len(b) > 12:
+            at = int(rng.integers(0, len(b) - 4))
+            del b[at:at + int(rng.integers(1, 33))]
+        elif kind == 5 and len(b) >= 16:
+            b[int(rng.integers(0, min(len(b) - 8, 200)))] = int(rng.integers(0, 256))
+    if rng.integers(0, 2) and len(b) >= 8:
+        b[-8:] = struct.pack("<Q", okv.checksum(bytes(b[:-8])))
+    return bytes(b)
+
+
+def test_seeded_corruptions_get_the_same_verdict_from_library_and_oracle():
+    """600 corrupted snapshots: the library accepts exactly what the oracle accepts, with the same
+    contents, and refuses the rest under the same variant, message and fields."""
+    P = pkg()
+    rng = np.random.default_rng(20)
+    seeds = [okv.KvSnapshot.capture(filled_cache(n), fp).to_bytes()
+             for n, fp in ((1, ""), (3, "m"), (5, "model-a"), (9, "längere-Kennung"))]
+    accepted = refused = 0
+    variants = set()
+    for case in range(600):
+        data = _mutated(seeds[case % len(seeds)], rng)
+        if len(data) >= 8 and data[:4] == b"ITKV" and struct.unpack_from("<I", data, 4)[0] == 2:
+            # The library's own typed format: the reference's reader refuses the version by
+            # name, the library goes on to read it (and refuses these bytes for other reasons).
+            assert oracle_refusal(data).variant == "UnsupportedVersion"
+            library_refusal(data)
+            continue
+        try:
+            want = okv.KvSnapshot.from_bytes(data)
+        except okv.KvError as e:
+            got = library_refusal(data)
+            assert (got.variant, got.message) == (e.variant, e.message), (case, data[:64])
+            for key in ("expected", "actual", "stored", "computed", "version"):
+                if key in e.fields:
+                    assert got.fields[key] == e.fields[key], (case, key)
+            refused += 1
+            variants.add(e.variant)
+            continue
+        got = P.KvSnapshot.from_bytes(data)
+        assert got.token_count == want.token_count and got.model_fingerprint == want.model_fingerprint
+        assert (got.geometry.num_kv_heads, got.geometry.head_dim) == (want.geometry.num_kv_heads, want.geometry.head_dim)
+        assert [(k.is_windowed, k.window_size) for k in got.geometry.layers] == \
+               [(k.is_windowed, k.window_size) for k in want.geometry.layers]
+        assert len(got.layers) == len(want.layers)
+        for x, y in zip(got.layers, want.layers):
+            assert x.first_position == y.first_position
+            assert np.asarray(x.keys).tobytes() == np.asarray(y.keys).tobytes()
+            assert np.asarray(x.values).tobytes() == np.asarray(y.values).tobytes()
+        accepted += 1
+    assert accepted >= 10 and refused >= 400 and len(variants) >= 4, (accepted, refused, variants)

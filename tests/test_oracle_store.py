@@ -387,3 +387,84 @@ def test_a_payload_read_in_pieces_is_served_whole_and_a_flip_in_any_piece_is_ref
     assert any("entry payload: truncated, needs" in r for r in store.refusals)
     path.write_bytes(whole)
     assert store.lookup(tokens + [5], geometry, "big", 6).snapshot_bytes == data
+
+
+def _corrupt(data, rng):
+    """A seeded corruption of an entry file: a flipped bit, a cut, stray bytes, or an extreme
+    value over a field of the header or of the snapshot's own header."""
+    b = bytearray(data)
+    extremes = (0, 1, 2, 0x80000000, 0xFFFFFFFF, 1 << 32, 1 << 61, (1 << 63) - 1, (1 << 64) - 1)
+    for _ in range(int(rng.integers(1, 3))):
+        kind = int(rng.integers(0, 5))
+        if kind == 0 and b:
+            b[int(rng.integers(0, len(b)))] ^= 1 << int(rng.integers(0, 8))
+        elif kind == 1:
+            del b[int(rng.integers(0, len(b) + 1)):]
+        elif kind == 2 and len(b) >= 16:
+            width = 8 if rng.integers(0, 2) else 4
+            at = int(rng.integers(0, min(len(b), 240) - width + 1)) & ~3
+            b[at:at + width] = int(extremes[int(rng.integers(0, len(extremes)))] % (1 << (8 * width))).to_bytes(width, "little")
+        elif kind == 3:
+            b += rng.integers(0, 256, size=int(rng.integers(1, 24)), dtype=np.uint8).tobytes()
+        elif kind == 4 and len(b) > 12:
+            at = int(rng.integers(0, len(b) - 4))
+            del b[at:at + int(rng.integers(1, 17))]
+    return bytes(b)
+
+
+def test_corrupted_directories_are_indexed_refused_and_served_alike_by_library_and_oracle(tmp_path):
+    """60 directories of honest entries, some then corrupted on disk (240 files in all): the
+    library's store and the oracle's index the same entries, refuse the same files in the same
+    words, serve the same prefixes with the same bytes, and leave the same files behind."""
+    import shutil
+    o, l = OracleSide(), LibrarySide()
+    rng = np.random.default_rng(31)
+    served = refused = 0
+
+    def meta(store):
+        return [(e.file_name, e.prefix_hash, e.token_count, e.bytes, e.created_unix, e.last_used_unix)
+                for e in store.entries()]
+
+    def said(store, root, but=()):  # the refusal lines, the directory's own path taken out
+        return sorted(r.replace(str(root), "<root>") for r in store.refusals
+                      if not any(name in r for name in but))
+
+    def typed(store):
+        # A corruption that writes 2 over the snapshot's version makes it the library's own typed
+        # format: the reference's reader refuses the version by name, the library reads on and
+        # refuses what follows. Both refuse; only the words differ, and are left out below.
+        return [r.split()[4].rstrip(":") for r in store.refusals if r.endswith("unsupported format version 2")]
+
+    for case in range(60):
+        a, b = tmp_path / f"o{case}", tmp_path / f"l{case}"
+        writer = o.open(a, 1 << 30)
+        base = [int(t) for t in rng.integers(0, 9, size=2)]
+        prefixes = [base, base + [int(rng.integers(0, 9))], base + [7, 7, int(rng.integers(0, 9))],
+                    [int(t) for t in rng.integers(10, 20, size=int(rng.integers(1, 6)))]]
+        for now, tokens in enumerate(prefixes, start=1):
+            o.put(writer, tokens, snapshot_for(tokens, "m"), now)
+        for name in sorted(os.listdir(a)):
+            if rng.integers(0, 2):
+                (a / name).write_bytes(_corrupt((a / name).read_bytes(), rng))
+        if case % 7 == 0:
+            (a / "stray.itkv").write_bytes(rng.integers(0, 256, size=int(rng.integers(0, 90)), dtype=np.uint8).tobytes())
+        shutil.copytree(a, b)
+        so, sl = o.open(a, 1 << 30), l.open(b, 1 << 30)
+        assert meta(so) == meta(sl), case
+        assert said(so, a, typed(so)) == said(sl, b, typed(so)), case
+        assert len(so.refusals) == len(sl.refusals), case
+        for now, tokens in enumerate(prefixes + [base + [7, 7, 7, 7]], start=10):
+            query = tokens + [3]
+            want, got = o.lookup(so, query, None, None, now), l.lookup(sl, query, None, None, now)
+            assert (want is None) == (got is None), (case, tokens)
+            if want is not None:
+                assert want[0] == got[0] and list(want[1]) == list(got[1]) and want[2] == got[2], (case, tokens)
+                served += 1
+        assert said(so, a, typed(so)) == said(sl, b, typed(so)), case
+        assert len(so.refusals) == len(sl.refusals), case
+        refused += len(so.refusals)
+        assert meta(so) == meta(sl), case
+        assert sorted(os.listdir(a)) == sorted(os.listdir(b))
+        for name in os.listdir(a):
+            assert (a / name).read_bytes() == (b / name).read_bytes(), (case, name)
+    assert served >= 100 and refused >= 60, (served, refused)
