@@ -21,7 +21,8 @@ same JSON shape; `--workload hybrid` a decode step over the reference model's ow
 pattern (three sliding-window layers of 2048 to one global layer, crates/attention/src/
 cache.rs:66-84) at context 32768; `--workload restore|append` measures the cache-maintenance kernels (the
 48-layer prefix-snapshot gather of configs[4]; the append of a 2048-row chunk). They are
-secondary measurements, the default line is the contract.
+secondary measurements, the default line is the contract. `--kv f32` runs the decode or ragged
+workload on an f32 cache, the reference's own storage (twice the bytes per row).
 """
 from __future__ import annotations
 
@@ -59,9 +60,11 @@ def rope_on_device(x, base):
     return torch.cat([(a * c - b * s).float(), (a * s + b * c).float()], dim=-1)
 
 
-def cpu_baseline(ctx: int, kv_bytes_per_layer: int, layers: int, budget_s: float = 12.0):
+def cpu_baseline(ctx: int, kv_bytes_per_layer: int, layers: int, budget_s: float = 12.0,
+                 store_f16: bool = True):
     """The CPU oracle (a port of the reference's single-threaded Rust path) on the decode
-    step: append one row at position ctx, attend over ctx + 1 positions, f16-rounded KV."""
+    step: append one row at position ctx, attend over ctx + 1 positions, f16-rounded KV (or f32
+    rows, as the reference stores them, with store_f16=False)."""
     import numpy as np
 
     import oracle
@@ -71,7 +74,7 @@ def cpu_baseline(ctx: int, kv_bytes_per_layer: int, layers: int, budget_s: float
     k = k.reshape(ctx + 1, ROW)
     v = rng.standard_normal((ctx + 1, ROW), dtype=np.float32)
     q = rng.standard_normal((1, Q_HEADS * D), dtype=np.float32)
-    cache = oracle.KvCache.new([oracle.LayerKind.Global], KV_HEADS, D, store_f16=True)
+    cache = oracle.KvCache.new([oracle.LayerKind.Global], KV_HEADS, D, store_f16=store_f16)
     cache.restore_bulk(0, 0, k[:ctx], v[:ctx])
     done, spent = 0, 0.0
     while spent < budget_s or done < 4:
@@ -90,7 +93,7 @@ def cpu_baseline(ctx: int, kv_bytes_per_layer: int, layers: int, budget_s: float
         "kind": "port",
         "us_per_token": round(per_layer * layers * 1e6, 1),
         "sample": f"{done} layer-steps of the decode step (append + attend over {ctx + 1} "
-                  f"positions, 32 Q / 4 KV heads, d=128, f16-rounded KV), single thread; the "
+                  f"positions, 32 Q / 4 KV heads, d=128, {'f16-rounded' if store_f16 else 'f32'} KV), single thread; the "
                   f"per-token figure is x{layers} layers",
     }
 
@@ -277,6 +280,9 @@ def main():
     ap.add_argument("--workload", choices=["decode", "ragged", "verify", "prefill", "hybrid",
                                            "restore", "append"], default="decode")
     ap.add_argument("--softcap", type=float, default=0.0)
+    ap.add_argument("--kv", choices=["f16", "f32"], default="f16",
+                    help="element type of the cache: f16 (the metric's) or f32, the reference's "
+                         "own storage (decode and ragged workloads only; a secondary figure)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--prep", action="store_true",
                     help="also time the step with the fused Q/K preparation (per-head RMSNorm + "
@@ -301,6 +307,10 @@ def main():
 
     # ---- workload shapes -------------------------------------------------------------
     wl = args.workload
+    if args.kv == "f32" and wl not in ("decode", "ragged"):
+        print("--kv f32 is measured on the decode and ragged workloads only", file=sys.stderr)
+        sys.exit(2)
+    elem_bytes = 4 if args.kv == "f32" else 2
     if wl in ("restore", "append"):
         print(json.dumps(cache_maintenance(args, pkg, torch, dev, stream, timed)))
         return
@@ -335,10 +345,12 @@ def main():
     # Rows a layer's attention reads per slot: everything stored, or the window.
     visible = [[min(n + rows, window + rows - 1) if kind.is_windowed else n + rows for n in lengths]
                for kind in pattern]
-    kv_bytes_layer = sum(sum(2 * r * KV_HEADS * D * 2 for r in per) for per in visible) // layers
+    kv_bytes_layer = sum(sum(2 * r * KV_HEADS * D * elem_bytes for r in per) for per in visible) // layers
     flops_layer = sum(4 * D * Q_HEADS * (rows * n + rows * (rows + 1) // 2) for n in lengths)
 
-    pool = pkg.KvPool(pattern, KV_HEADS, D, elem="f16", max_slots=slots,
+    if args.kv == "f32":
+        name = name.replace("f16 KV", "f32 KV (the reference's storage; the metric is quoted on f16)")
+    pool = pkg.KvPool(pattern, KV_HEADS, D, elem=args.kv, max_slots=slots,
                       capacity_rows=max_len + rows + 8, scrub_on_truncate=False)
     pool.set_stream(stream.cuda_stream)
     caches = [pool.acquire() for _ in range(slots)]
@@ -493,13 +505,13 @@ def main():
         value = kv_bytes_layer * layers / step_s / 1e9
         roofline = {
             "bound": "hbm",
-            "kernel": "attn_splitk_f16_kernel + attn_combine128_kernel (the two launches of "
-                      "one layer's attention)",
+            "kernel": f"attn_splitk_{args.kv}_kernel + attn_combine128_kernel (the two launches "
+                      "of one layer's attention)",
             "achieved": round(kv_bytes_layer / attn_s / 1e9, 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(kv_bytes_layer / attn_s / 1e9 / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC.get(wl),
+            "traffic": MEASURED_TRAFFIC.get(wl) if args.kv == "f16" else None,
             "us_per_launch": round(attn_s * 1e6, 3),
             "bytes_per_launch": kv_bytes_layer,
         }
@@ -515,7 +527,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f16",
+        "dtype": args.kv,
         "data": "synthetic",
         "config": {
             "workload": name,
@@ -523,7 +535,8 @@ def main():
             "layers_per_step": layers,
             "kv_bytes_per_step": kv_bytes_layer * layers,
             "softcap": args.softcap,
-            "arithmetic": "f16 KV and MFMA operands, f32 scores, softmax and accumulation",
+            "arithmetic": ("f16 KV and MFMA operands, f32 scores, softmax and accumulation"
+                           if args.kv == "f16" else "f32 KV, f32 MFMA operands and accumulation"),
         },
         "us_per_token": round(step_s * 1e6 * ((52 if wl == "hybrid" else 48) / layers), 2),
         "pct_of_hbm_peak": round(100.0 * kv_bytes_layer * layers / step_s / 1e9 / HBM_PEAK_GBS, 2),
@@ -539,7 +552,8 @@ def main():
     if host_call is not None:
         result["host_pointer_call"] = host_call
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(4096, 2 * 4097 * KV_HEADS * D * 2, 48)
+        result["cpu_baseline"] = cpu_baseline(4096, 2 * 4097 * KV_HEADS * D * elem_bytes, 48,
+                                              store_f16=args.kv == "f16")
     print(json.dumps(result))
     pool.close()
 
