@@ -258,7 +258,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
                         x[qt][e >> 2][e & 3] =
-                            softcap_log2(x[qt][e >> 2][e & 3], softcap, inv_cap) - ref[qt];
+                            softcap_log2(x[qt][e >> 2][e & 3], softcap, inv_cap, ref[qt]);
             }
             if (RING && kb < low_masked_end) {
 #pragma unroll

@@ -19,13 +19,18 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// cap * tanh(x / cap) * log2(e), via exp2; x is a scaled score in natural units.
-__device__ __forceinline__ float softcap_log2(float x, float cap, float inv_cap) {
-    const float y = x * inv_cap;
-    // tanh(y) = 1 - 2 / (exp(2y) + 1); exp2 saturates to inf/0 at the tails, giving +-1.
-    const float e = fast_exp2(y * (2.0f * kLog2e));
-    const float t = 1.0f - 2.0f / (e + 1.0f);
-    return cap * kLog2e * t;
+// cap * tanh(x / cap) * log2(e); x is a scaled score in natural units.
+// tanh(y) = 1 - 2 / (exp(2y) + 1) with the hardware's exp2 and reciprocal (each within one
+// unit in the last place; exp2 saturates to inf / 0 at the tails, giving +-1): a multiply, an
+// add and a fused multiply-add around two transcendental instructions. An IEEE division
+// here costs four times as much vector work, on every score of a block.
+// `shift` is subtracted from the result inside the same fused multiply-add (a caller that keeps
+// scores relative to a reference passes the reference).
+__device__ __forceinline__ float softcap_log2(float x, float cap, float inv_cap, float shift = 0.0f) {
+    const float e = fast_exp2(x * (inv_cap * (2.0f * kLog2e)));
+    const float r = __builtin_amdgcn_rcpf(e + 1.0f);
+    const float c = cap * kLog2e;
+    return __builtin_fmaf(r, -2.0f * c, c - shift);
 }
 
 }  // namespace itak
