@@ -19,7 +19,8 @@ the CPU oracle timed on the host cores beside it.
 over 16 ragged slots, the speculative verify block, the chunked causal prefill) with the
 same JSON shape; `--workload hybrid` a decode step over the reference model's own layer
 pattern (three sliding-window layers of 2048 to one global layer, crates/attention/src/
-cache.rs:66-84) at context 32768; `--workload restore|append` measures the cache-maintenance kernels (the
+cache.rs:66-84) at context 32768; `--workload prefill_windowed` a 2048-row prefill chunk on
+sliding-window layers; `--workload restore|append` measures the cache-maintenance kernels (the
 48-layer prefix-snapshot gather of configs[4]; the append of a 2048-row chunk). They are
 secondary measurements, the default line is the contract. `--kv f32` runs the decode or ragged
 workload on an f32 cache, the reference's own storage (twice the bytes per row).
@@ -278,7 +279,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", choices=["decode", "ragged", "verify", "prefill", "hybrid",
-                                           "restore", "append"], default="decode")
+                                           "prefill_windowed", "restore", "append"],
+                    default="decode")
     ap.add_argument("--softcap", type=float, default=0.0)
     ap.add_argument("--kv", choices=["f16", "f32"], default="f16",
                     help="element type of the cache: f16 (the metric's) or f32, the reference's "
@@ -332,6 +334,11 @@ def main():
         name = ("hybrid decode step: sliding-window layers (window 2048) and global layers 3:1, "
                 "the pattern of the reference's 52-layer model, batch 1, context 32768, 30B-class "
                 "heads, f16 KV, 8 layers cycled (6 windowed, 2 global)")
+    elif wl == "prefill_windowed":
+        layers, slots, rows, lengths = 4, 1, 2048, [30720]
+        name = ("chunked causal prefill on sliding-window layers (window 2048, three of four layers "
+                "of the reference's model): 2048-row chunk at position 30720, each row over its "
+                "last 2048 keys, 30B-class heads, f16 KV, f32 accumulate, 4 layers cycled")
     else:
         layers, slots, rows, lengths = 4, 1, 2048, [30720]
         name = ("configs[4]: chunked causal prefill, 2048-row chunk over a 30720-token prefix, "
@@ -339,6 +346,8 @@ def main():
     max_len = max(lengths)
     window = 2048
     pattern = [pkg.LayerKind.Global] * layers
+    if wl == "prefill_windowed":
+        pattern = [pkg.LayerKind.windowed(window)] * layers
     if wl == "hybrid":  # glimmer_layer_pattern: every fourth layer global
         pattern = [pkg.LayerKind.Global if (i + 1) % 4 == 0 else pkg.LayerKind.windowed(window)
                    for i in range(layers)]
@@ -347,11 +356,15 @@ def main():
                for kind in pattern]
     kv_bytes_layer = sum(sum(2 * r * KV_HEADS * D * elem_bytes for r in per) for per in visible) // layers
     flops_layer = sum(4 * D * Q_HEADS * (rows * n + rows * (rows + 1) // 2) for n in lengths)
+    if wl == "prefill_windowed":  # row i at position n + i sees min(window, n + i + 1) keys
+        flops_layer = sum(4 * D * Q_HEADS * sum(min(window, n + i + 1) for i in range(rows))
+                          for n in lengths)
 
     if args.kv == "f32":
         name = name.replace("f16 KV", "f32 KV (the reference's storage; the metric is quoted on f16)")
     pool = pkg.KvPool(pattern, KV_HEADS, D, elem=args.kv, max_slots=slots,
-                      capacity_rows=max_len + rows + 8, scrub_on_truncate=False)
+                      capacity_rows=max_len + rows + 8, scrub_on_truncate=False,
+                      ring_headroom=rows if wl == "prefill_windowed" else 0)
     pool.set_stream(stream.cuda_stream)
     caches = [pool.acquire() for _ in range(slots)]
 
@@ -360,7 +373,7 @@ def main():
     q = torch.randn(layers, total_rows, Q_HEADS * D, device=dev)
     k_new = torch.randn(layers, total_rows, ROW, device=dev)
     v_new = torch.randn(layers, total_rows, ROW, device=dev)
-    if wl == "prefill":  # f16-valued Q/K/V
+    if wl.startswith("prefill"):  # f16-valued Q/K/V
         q, k_new, v_new = q.half().float(), k_new.half().float(), v_new.half().float()
     out = torch.empty_like(q)
     for layer in range(layers):
@@ -412,6 +425,20 @@ def main():
         g_attn.replay()
     attn_s = timed(g_attn.replay, args.steps)[0] / (args.steps * layers)
     pool.truncate(caches, lengths)
+    if wl == "prefill_windowed":
+        # On a sliding-window layer a chunk attended after its append sees only what the ring
+        # still promises (the last `window` rows: the chunk's first rows would see almost
+        # nothing), so the attention launch is timed as the step minus its append.
+        def append_only():
+            for layer in range(layers):
+                pool.append_device(layer, items, ptrs[layer][1], ptrs[layer][2])
+            pool.truncate(caches, lengths)
+
+        g_append = capture(torch, pool, stream, append_only)
+        for _ in range(max(args.warmup, 1)):
+            g_append.replay()
+        append_s = timed(g_append.replay, args.steps)[0] / args.steps
+        attn_s = (step_s - append_s) / layers
 
     host_call = None
     if wl == "decode":
@@ -449,7 +476,7 @@ def main():
         }
 
     with_prep = None
-    if args.prep and wl != "prefill":
+    if args.prep and not wl.startswith("prefill"):
         # The model's own sequence around the step (muse-glimmer/src/model.rs:445-464): raw
         # projections -> per-head RMSNorm -> interleaved RoPE on sliding-window layers (global
         # layers carry no rotation) -> append + attention -> out * sigmoid(gate).
@@ -484,12 +511,15 @@ def main():
                      "append + attention; the gate in the merge kernel"),
         }
 
-    if wl == "prefill":
+    if wl.startswith("prefill"):
         metric, unit = "prefill attention TFLOP/s (2048-row chunk over 30720 prefix)", "TFLOP/s"
+        if wl == "prefill_windowed":
+            metric = "prefill attention TFLOP/s (2048-row chunk, window 2048)"
         value = flops_layer * layers / step_s / 1e12
         roofline = {
             "bound": "mfma",
-            "kernel": "attn_prefill_f16_kernel (one launch per layer)",
+            "kernel": "attn_prefill_f16_kernel (one launch per layer)" +
+                      (": the step's time less its append's" if wl == "prefill_windowed" else ""),
             "achieved": round(flops_layer / attn_s / 1e12, 2),
             "peak": MFMA_F16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
