@@ -63,7 +63,8 @@ __device__ __forceinline__ float column_sum4(float v) {
 // The direct-to-LDS load is issued from inline assembly: the compiler then neither tracks it
 // (it would make every LDS read wait for all of them) nor needs to, because the only consumer
 // is ordered by the explicit s_waitcnt vmcnt + s_barrier at the top of each iteration.
-constexpr int kStages = 4;
+constexpr int kStages = 4;      // blocks of the LDS ring: three in flight while one is read
+constexpr int kDeepStages = 8;  // for short runs of blocks, one workgroup per compute unit
 constexpr int kStageBytes = 2 * kBlockElems * 2;  // one key block + one value block
 
 __device__ __forceinline__ void lds_dma16(const void *src, uint32_t lds_addr) {
@@ -80,7 +81,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 
 // RING = the layer is windowed (blocks start at the window, live in a ring, the mask has a
 // lower edge); global layers run the instantiation without any of it.
-template <int N, bool SOFTCAP, int kTiles, bool RING>
+template <int N, bool SOFTCAP, int kTiles, bool RING, int STAGES>
 __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnParams p,
                                                                            AttnBatchT<N> b,
                                                                            uint32_t total_partials) {
@@ -155,7 +156,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
         // number of loads in flight stays the same in every iteration.
         const uint64_t off = uint64_t(RING ? next_sb : min(kb, nblocks - 1)) * kBlockVec;
         if (RING && kb + 1 < nblocks) next_sb = next_sb + 1 == ring_blocks ? 0 : next_sb + 1;
-        const uint32_t dst = dma_base + (kb % kStages) * kStageBytes;
+        const uint32_t dst = dma_base + (kb % STAGES) * kStageBytes;
         lds_dma16(kg + off, dst);
         lds_dma16(kg + off + 256, dst + 4096);
         lds_dma16(vg + off, dst + 8192);
@@ -163,9 +164,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     };
     const bool any_block = kb_begin < nblocks;  // a split past the rows' horizon has none
     if (any_block) {
-        issue_block(kb_begin);
-        issue_block(kb_begin + 1);
-        issue_block(kb_begin + 2);
+#pragma unroll
+        for (int ahead = 0; ahead < STAGES - 1; ++ahead) issue_block(kb_begin + ahead);
     }
 
     const float softcap = p.softcap;
@@ -214,10 +214,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
         // This thread's pieces of block kb have landed (the 8 loads of the next two blocks
         // may still fly); after the barrier everybody's have, and everybody is done with
         // block kb - 1, whose stage the loads for block kb + 3 may now overwrite.
-        wait_vmcnt<8>();
+        wait_vmcnt<4 * (STAGES - 2)>();
         __builtin_amdgcn_s_barrier();
-        issue_block(kb + 3);
-        const uint16_t *lds_k = lds_ring + (kb % kStages) * (kStageBytes / 2);
+        issue_block(kb + STAGES - 1);
+        const uint16_t *lds_k = lds_ring + (kb % STAGES) * (kStageBytes / 2);
         const uint16_t *lds_v = lds_k + kBlockElems;
 
         if (kb < wave_blocks && (!RING || kb >= wave_first)) {
@@ -410,12 +410,21 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
         (void)hipGetLastError();
-    const uint64_t target = uint64_t(2) * uint64_t(cus > 0 ? cus : 256);
+    const uint64_t per_cu = uint64_t(cus > 0 ? cus : 256);
     uint64_t unit_blocks = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         const uint64_t units = uint64_t(g.kv_heads) * ((b.item[i].rows + rows_per_group - 1) / rows_per_group);
         unit_blocks += units * unit_block_count(b.item[i], rows_per_group, window);
     }
+    // Two workgroups per compute unit hide each other's waits when their runs are long. When
+    // the whole launch is 8 to 40 blocks per compute unit, a run is over before that pays:
+    // then one workgroup per compute unit with twice the blocks in flight (the deep ring), so
+    // that its handful of blocks arrive behind one another after a single memory latency
+    // (measured: 64 rows at context 4096 30.8 -> 27.1 us, 256 rows 52.6 -> 48.4 us, 16 rows at
+    // context 30720 36.3 -> 31.6 us; above the range it loses, below it nothing changes).
+    const bool deep = unit_blocks >= 8 * per_cu && unit_blocks <= 40 * per_cu;
+    b.deep_ring = deep ? 1 : 0;
+    const uint64_t target = deep ? per_cu : 2 * per_cu;
     const uint64_t T = std::max<uint64_t>((unit_blocks + target - 1) / target, 8);
     uint32_t block0 = 0, ws0 = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
@@ -438,17 +447,25 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
     return ws0;
 }
 
+template <int N, bool SOFTCAP, int TILES, bool RING, int STAGES>
+static hipError_t launch_prefill_ring(const AttnParams &p, const AttnBatch &b,
+                                      uint32_t total_partials, hipStream_t stream) {
+    constexpr size_t lds = size_t(STAGES) * kStageBytes;
+    static const hipError_t granted = hipFuncSetAttribute(
+        reinterpret_cast<const void *>(&attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING, STAGES>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+    if (granted != hipSuccess) return granted;
+    attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING, STAGES>
+        <<<b.total_blocks, kWaves * 64, lds, stream>>>(p, AttnBatchT<N>(b), total_partials);
+    return hipGetLastError();
+}
+
 template <int N, bool SOFTCAP, int TILES, bool RING>
 static hipError_t launch_prefill(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                  hipStream_t stream) {
-    constexpr size_t lds = size_t(kStages) * kStageBytes;
-    static const hipError_t granted = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(&attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING>),
-        hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
-    if (granted != hipSuccess) return granted;
-    attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING><<<b.total_blocks, kWaves * 64, lds, stream>>>(
-        p, AttnBatchT<N>(b), total_partials);
-    return hipGetLastError();
+    return b.deep_ring
+               ? launch_prefill_ring<N, SOFTCAP, TILES, RING, kDeepStages>(p, b, total_partials, stream)
+               : launch_prefill_ring<N, SOFTCAP, TILES, RING, kStages>(p, b, total_partials, stream);
 }
 
 hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,

@@ -204,7 +204,7 @@ struct AttnBatch {
     uint32_t n;
     uint32_t total_blocks;
     uint32_t rows_per_block;
-    uint32_t pad;
+    uint32_t deep_ring;  // host side only: the block kernel's plan asks for its deeper LDS ring
     AttnItem item[kMaxBatchItems];
 };
 // The kernel argument form of AttnBatch, sized to the batch: kernel arguments are

@@ -276,7 +276,11 @@ def test_speculative_round_trip_rewind_restores_the_exact_continuation():
     assert "not this cache's live checkpoint" in e.value.detail
 
 
-@pytest.mark.parametrize("rows,ctx,softcap", [(9, 3000, 0.0), (40, 5000, 0.0), (130, 2100, 25.0)])
+@pytest.mark.parametrize("rows,ctx,softcap", [
+    (9, 3000, 0.0), (40, 5000, 0.0),
+    # 8 to 40 key blocks per compute unit in all: the block kernel's deep-ring instantiation.
+    (130, 2100, 25.0), (64, 4096, 0.0), (48, 6000, 0.0),
+])
 def test_mid_size_blocks_split_over_the_context(rows, ctx, softcap):
     # Blocks too long for the decode kernel and too short to fill the device by rows alone:
     # the block kernel cuts the context into splits and the merge launch joins them.

@@ -464,6 +464,7 @@ def run_steps(pool, cache, ref, rng, q_heads, steps, elem, softcap=0.0):
     ("f16", 128, 32, 4, 128, [100, 1, 64, 33, 128, 7, 1, 128, 90], 128),  # block kernel
     ("f16", 300, 8, 8, 128, [256, 256, 17, 256, 1, 200], 256),            # MHA, two tiles per wavefront
     ("f16", 96, 16, 2, 64, [1, 5, 40, 1, 1, 64], 64),                     # generic f16 path
+    ("f16", 1500, 32, 4, 128, [256] * 7 + [1, 256], 256),  # block kernel, deep ring, through a wrap
 ])
 def test_steps_on_a_windowed_layer_match_the_oracle(elem, window, q_heads, kvh, d, steps, headroom):
     pool, cache, ref, rng = pair(window, kvh, d, elem, seed=window + d, headroom=headroom)
