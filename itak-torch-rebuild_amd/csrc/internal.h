@@ -88,6 +88,10 @@ struct AppendBatch {
     uint32_t n;
     uint32_t total_rows;
     uint32_t ring;      // storage rows of a windowed layer's ring (position p lives in row p % ring); 0 = row p
+    // The launch moves total_rows source rows: rows [0, gap_at) and, when gap_rows != 0, the
+    // rows from gap_at + gap_rows on (the rows in between go another way).
+    uint32_t gap_at;
+    uint32_t gap_rows;
     uint32_t pad;
     AppendItem item[kMaxBatchItems];
 };

@@ -34,7 +34,8 @@ __global__ __launch_bounds__(256) void kv_append_kernel(T *__restrict__ layer_ba
     const uint64_t per_row = 2ull * g.kv_heads * chunks;
     const uint64_t idx = blockIdx.x * 256ull + threadIdx.x;
     if (idx >= per_row * b.total_rows) return;
-    const uint32_t row = uint32_t(idx / per_row);
+    uint32_t row = uint32_t(idx / per_row);  // among the rows this launch moves, then in the source
+    if (b.gap_rows && row >= b.gap_at) row += b.gap_rows;
     uint32_t rem = uint32_t(idx % per_row);
     const uint32_t side = rem / (g.kv_heads * chunks);
     rem -= side * g.kv_heads * chunks;

@@ -502,6 +502,47 @@ itak_status run_append(itak_pool *pool, uint64_t layer, const itak_batch_item *i
         advance(pool->slots[slot], layer, rows);
         return ITAK_OK;
     }
+    // The same on a ring whose length is a whole number of blocks: the rows before the first
+    // block boundary and those after the last one go through the row kernel in one launch,
+    // the whole blocks between them through the gather, in two pieces where they wrap. Nothing
+    // beyond the run is written: on a ring the rows behind it are older positions that a
+    // rewind may still need.
+    if (n == 1 && L.windowed && pool->elem_f16 && pool->gw.v_block != 0 &&
+        L.ring % kVBlock == 0 && items[0].rows >= kChunkRows && items[0].rows <= L.ring) {
+        const uint32_t slot = items[0].slot, rows = items[0].rows;
+        const uint32_t pos0 = uint32_t(pool->slots[slot].appended[layer]);
+        const uint32_t head_rows = (kVBlock - pos0 % kVBlock) % kVBlock;
+        const uint32_t body = (rows - head_rows) / kVBlock * kVBlock;
+        const uint32_t tail_rows = rows - head_rows - body;
+        if (head_rows + tail_rows) {
+            AppendBatch b{};
+            b.ring = uint32_t(L.ring);
+            b.total_rows = head_rows + tail_rows;
+            b.gap_at = head_rows;
+            b.gap_rows = body;
+            if (head_rows) b.item[b.n++] = AppendItem{slot, head_rows, pos0, 0};
+            if (tail_rows)
+                b.item[b.n++] = AppendItem{slot, tail_rows, pos0 + head_rows + body, head_rows + body};
+            HIP_TRY(pool, launch_append(layer_base(pool, layer), 1, pool->gw, b, k_dev, v_dev,
+                                        pool->stream),
+                    "launch append");
+        }
+        const uint32_t at = uint32_t((pos0 + head_rows) % L.ring);
+        const uint32_t first_piece = std::min<uint32_t>(body, uint32_t(L.ring) - at);
+        RestoreBatch rb{};
+        rb.slot = slot;
+        rb.max_rows = std::max(first_piece, body - first_piece);
+        const float *ks = k_dev + uint64_t(head_rows) * pool->row, *vs = v_dev + uint64_t(head_rows) * pool->row;
+        rb.layer[rb.n++] = RestoreLayer{ks, vs, L.index, first_piece, at, 0};
+        if (body > first_piece)
+            rb.layer[rb.n++] = RestoreLayer{ks + uint64_t(first_piece) * pool->row,
+                                            vs + uint64_t(first_piece) * pool->row, L.index,
+                                            body - first_piece, 0, 0};
+        HIP_TRY(pool, launch_restore(pool->base_w, 1, 0, pool->gw, rb, pool->stream),
+                "launch chunk append");
+        advance(pool->slots[slot], layer, rows);
+        return ITAK_OK;
+    }
     uint32_t src_row = 0;
     for (uint32_t first = 0; first < n; first += kMaxBatchItems) {
         const uint32_t count = std::min<uint32_t>(kMaxBatchItems, n - first);

@@ -648,3 +648,48 @@ def test_compute_attention_refuses_a_bad_swa_base_on_sliding_layers_only():
     assert hc.kv_cache().next_position(0) == 0
     out = hc.attention(P().AttentionRequest(q, k, v, 1, G, cfg), cache)
     assert np.allclose(out, 1.0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kvh,d", [(4, 128), (2, 64)])
+def test_chunk_appends_into_a_ring_land_where_row_appends_would(kvh, d):
+    """Chunks of 128 rows and more go into a ring as whole 32-row blocks (in two pieces where
+    they wrap) with the rows before the first block boundary and after the last one beside them:
+    after every chunk the view holds exactly what the oracle's row-by-row appends leave, and a
+    rewind into the chunk still finds the rows the chunk must not have touched."""
+    import torch
+    window, headroom = 200, 320
+    pool, cache, ref, rng = pair(window, kvh, d, "f16", headroom=headroom)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    for rows in (128, 129, 31, 320, 1, 160, 255, 128, 7, 300, 192):  # starts at 0, 128, 257, 288, ...
+        base = cache.next_position(0)
+        k, v = normal(rng, rows, kvh * d), normal(rng, rows, kvh * d)
+        kd, vd = torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda()
+        pool.append_device(0, [(cache, rows)], kd.data_ptr(), vd.data_ptr())
+        pool.synchronize()
+        for i in range(rows):
+            ref.append(0, k[i], v[i], base + i)
+        assert cache.next_position(0) == ref.next_position(0) == base + rows
+        assert view_snapshot(cache, 0) == view_snapshot(ref, 0), (rows, base)
+    # A truncate into the last chunk keeps every row of the window before the cut: the chunk's
+    # whole-block stores wrote nothing outside its own rows.
+    end = cache.next_position(0)
+    cut = end - 100
+    pool.truncate([cache], [cut])
+    def values_of(rows):  # f16 storage compared as the values it holds
+        rows = np.asarray(rows)
+        if rows.dtype == np.uint16:
+            rows = rows.view(np.float16)
+        return rows.astype(np.float32).reshape(window, -1)
+
+    pos, keys, _ = ref.view(0).rows()
+    got_pos, got_k, _ = cache.view(0).rows()
+    got_pos = list(np.asarray(got_pos, dtype=np.int64))
+    assert got_pos == list(range(cut - window, cut))
+    ref_pos = list(np.asarray(pos, dtype=np.int64))
+    # The oracle's view (uncut) and the cut view overlap on positions [end - window, cut).
+    lo = end - window
+    a = values_of(got_k)[lo - (cut - window):]
+    b = values_of(keys)[: cut - lo]
+    assert ref_pos[0] == lo and a.tobytes() == b.tobytes()
+    pool.close()
