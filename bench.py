@@ -44,7 +44,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # HBM bytes per layer (all launches of the layer's attention) measured with rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE and scaled by the same counters on the probe copy of known size
 # (profiles/*_traffic.md hold the runs and the scaling factors). Missing = not measured.
-MEASURED_TRAFFIC = {"decode": 9_962_081, "ragged": 216_870_262, "prefill": 290_264_395}
+MEASURED_TRAFFIC = {"decode": 9_958_468, "ragged": 216_836_109, "prefill": 290_168_799}
 
 
 def rope_on_device(x, base):
