@@ -511,15 +511,18 @@ class KvCache:
         if rc != 0:
             _raise(err)
         self._h = h
+        # Kept on the object: at interpreter shutdown module globals may be gone before a
+        # cache that is still alive is collected.
+        self._free = lib().orc_cache_free
 
     @staticmethod
     def new(pattern, num_kv_heads, head_dim, store_f16=False) -> "KvCache":
         return KvCache(pattern, num_kv_heads, head_dim, store_f16)
 
     def __del__(self):
-        h = getattr(self, "_h", None)
-        if h:
-            lib().orc_cache_free(h)
+        h, free = getattr(self, "_h", None), getattr(self, "_free", None)
+        if h and free:
+            free(h)
             self._h = None
 
     def layer_count(self) -> int:
