@@ -381,10 +381,19 @@ bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group) {
 
 // Up to 64 query vectors per KV head (speculative blocks) take one 16-vector tile per
 // wavefront, so that all four wavefronts of the workgroup have columns; more take two.
+// So do blocks of up to 256 vectors over at most 256 key blocks (a draft tree of 16 to 32
+// tokens at a context up to 8192): the launch has to split the context anyway, and with
+// twice the row tiles it needs half the splits, half the partials to write and merge
+// (measured at context 4096: 16 rows 20.6 -> 17.7 us, 32 rows 24.0 -> 21.2 us; at context
+// 30720 the second pass over the keys costs more than the partials saved).
 static int tiles_for(const AttnBatch &b, uint32_t group) {
-    uint32_t nvec = 0;
-    for (uint32_t i = 0; i < b.n; ++i) nvec = std::max(nvec, b.item[i].rows * group);
-    return nvec <= uint32_t(kWaves * 16) ? 1 : kMaxTiles;
+    uint32_t nvec = 0, nblocks = 0;
+    for (uint32_t i = 0; i < b.n; ++i) {
+        nvec = std::max(nvec, b.item[i].rows * group);
+        nblocks = std::max(nblocks, item_block_count(b.item[i]));
+    }
+    if (nvec <= uint32_t(kWaves * 16)) return 1;
+    return nvec <= 256 && nblocks <= 256 ? 1 : kMaxTiles;
 }
 
 // Fills splits / keys_per_split / block0 / ws0 for a batch (slot, rows, pos0, q_row0, kv_len
