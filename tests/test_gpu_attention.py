@@ -307,3 +307,41 @@ def test_mid_size_blocks_split_over_the_context(rows, ctx, softcap):
                                  oracle.AttentionParams(softcap=softcap), threads=8)
     assert max_abs(out.cpu().numpy().reshape(-1), want) <= 2e-3
     pool.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(8))
+def test_random_blocks_match_the_oracle_across_groups_windows_and_softcap(seed):
+    """Seeded blocks of 9 to 200 rows over contexts of 64 to 6000 positions, GQA groups 8, 4, 1
+    and 2, every fourth on a sliding-window layer, every third with a softcap: whichever way the
+    block kernel cuts them (one or two tiles per wavefront, split or not, either LDS ring), the
+    output is the oracle's within the f16-KV bar."""
+    import torch
+
+    rng = np.random.default_rng(5000 + seed)
+    group, kvh = [(8, 4), (4, 2), (1, 8), (2, 4)][seed % 4]
+    qh, d = kvh * group, 128
+    ctx, rows = int(rng.integers(64, 6000)), int(rng.integers(9, 200))
+    softcap = 20.0 if seed % 3 == 0 else 0.0
+    window = int(rng.integers(200, 1500)) if seed % 4 == 3 else 0
+    n = ctx + rows
+    k, v, q = normal(rng, n, kvh * d), normal(rng, n, kvh * d), normal(rng, rows, qh * d)
+    kind = P().LayerKind.windowed(window) if window else P().LayerKind.Global
+    okind = oracle.LayerKind.windowed(window) if window else oracle.LayerKind.Global
+    pool = P().KvPool([kind], kvh, d, elem="f16", capacity_rows=n + 8,
+                      ring_headroom=rows if window else 0)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    cache = pool.acquire()
+    ref = oracle.KvCache.new([okind], kvh, d, store_f16=True)
+    first = max(0, ctx - window) if window else 0
+    cache.restore_bulk(0, first, k[first:ctx], v[first:ctx])
+    ref.restore_bulk(0, first, k[first:ctx], v[first:ctx])
+    qd, kd, vd = (torch.from_numpy(np.ascontiguousarray(x)).cuda() for x in (q, k[ctx:], v[ctx:]))
+    out = torch.empty_like(qd)
+    pool.attention_step_device(0, [(cache, rows)], qd.data_ptr(), kd.data_ptr(), vd.data_ptr(),
+                               out.data_ptr(), qh, softcap=softcap)
+    pool.synchronize()
+    want = oracle.attention_step(ref, 0, q, k[ctx:], v[ctx:], qh, ctx,
+                                 oracle.AttentionParams(softcap=softcap), threads=8)
+    assert max_abs(out.cpu().numpy().reshape(-1), want) <= 2e-3, (group, ctx, rows, softcap, window)
+    pool.close()
