@@ -532,6 +532,8 @@ def main():
         metric, unit = "decode-attn KV GB/s (all layers, ctx 4096)", "GB/s"
         if wl != "decode":
             metric = f"decode-attn KV GB/s ({wl})"
+        if args.kv == "f32":
+            metric += " on an f32 cache"
         value = kv_bytes_layer * layers / step_s / 1e9
         roofline = {
             "bound": "hbm",
