@@ -44,7 +44,9 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # HBM bytes per layer (all launches of the layer's attention) measured with rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE and scaled by the same counters on the probe copy of known size
 # (profiles/*_traffic.md hold the runs and the scaling factors). Missing = not measured.
-MEASURED_TRAFFIC = {"decode": 9_958_468, "ragged": 216_836_109, "prefill": 290_168_799}
+MEASURED_TRAFFIC = {"decode": 9_958_451, "ragged": 216_836_265, "prefill": 290_164_626,
+                    "verify": 87_329_078}
+MEASURED_TRAFFIC_F32 = {"decode": 18_240_005}  # the same workload on an f32 cache (--kv f32)
 
 
 def rope_on_device(x, base):
@@ -543,7 +545,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(kv_bytes_layer / attn_s / 1e9 / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC.get(wl) if args.kv == "f16" else None,
+            "traffic": (MEASURED_TRAFFIC if args.kv == "f16" else MEASURED_TRAFFIC_F32).get(wl),
             "us_per_launch": round(attn_s * 1e6, 3),
             "bytes_per_launch": kv_bytes_layer,
         }
