@@ -288,6 +288,9 @@ def main():
                     help="element type of the cache: f16 (the metric's) or f32, the reference's "
                          "own storage (decode and ragged workloads only; a secondary figure)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--merge-in-launch", action="store_true",
+                    help="merge split partials inside the attention launch (workgroups exchange "
+                         "them through a buffer) instead of with a launch of its own")
     ap.add_argument("--prep", action="store_true",
                     help="also time the step with the fused Q/K preparation (per-head RMSNorm + "
                          "RoPE) before it and the sigmoid gate after it, reported as 'with_prep'")
@@ -366,7 +369,8 @@ def main():
         name = name.replace("f16 KV", "f32 KV (the reference's storage; the metric is quoted on f16)")
     pool = pkg.KvPool(pattern, KV_HEADS, D, elem=args.kv, max_slots=slots,
                       capacity_rows=max_len + rows + 8, scrub_on_truncate=False,
-                      ring_headroom=rows if wl == "prefill_windowed" else 0)
+                      ring_headroom=rows if wl == "prefill_windowed" else 0,
+                      merge_in_launch=args.merge_in_launch)
     pool.set_stream(stream.cuda_stream)
     caches = [pool.acquire() for _ in range(slots)]
 

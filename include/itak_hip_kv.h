@@ -93,7 +93,15 @@ enum { ITAK_LAYER_GLOBAL = 0, ITAK_LAYER_WINDOWED = 1 };
 enum {
     /* Zero the rows a truncate / rewind drops, so the raw device bytes (not only the
        visible rows) equal those of a cache that never held them. */
-    ITAK_POOL_SCRUB_ON_TRUNCATE = 1u
+    ITAK_POOL_SCRUB_ON_TRUNCATE = 1u,
+    /* Merge split partials inside the attention launch instead of with a launch of their own
+       (decode steps and speculative blocks of f16 pools at head_dim 128): the workgroups of a KV
+       head exchange their partials through a buffer while the launch runs, each polling for the
+       others' words (itak_pool_set_merge_spin_limit bounds the wait). One launch per layer
+       instead of two; results agree with the default form to rounding. On an MI355X the
+       exchange costs what the second launch costs (a round trip through memory between
+       compute dies, then the stores that hand the buffer back), so it is not the default. */
+    ITAK_POOL_MERGE_IN_LAUNCH = 2u
 };
 
 typedef struct itak_pool itak_pool;
@@ -217,6 +225,12 @@ void itak_pool_destroy(itak_pool *pool);
    buffers are already large enough (run the same step once uncaptured first). */
 itak_status itak_pool_set_stream(itak_pool *pool, void *hip_stream);
 itak_status itak_pool_synchronize(itak_pool *pool);
+/* No counterpart in the reference. Workgroups of a launch that merges its own splits
+   (ITAK_POOL_MERGE_IN_LAUNCH) wait for each other's partials by polling; `polls` bounds that
+   wait (default 131072, about a microsecond each). A workgroup that runs out writes NaN outputs and is reported by the next
+   itak_pool_synchronize as ITAK_STEP_FAILED. 0 makes every wait a single look: for tests of
+   that report. */
+itak_status itak_pool_set_merge_spin_limit(itak_pool *pool, uint32_t polls);
 /* Bytes of device memory the pool holds for KV rows. */
 uint64_t itak_pool_device_bytes(const itak_pool *pool);
 

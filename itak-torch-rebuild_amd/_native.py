@@ -29,6 +29,7 @@ KV_ERROR_FIRST, KV_ERROR_LAST = 21, 35
 ELEM_F32, ELEM_F16 = 0, 1
 LAYER_GLOBAL, LAYER_WINDOWED = 0, 1
 POOL_SCRUB_ON_TRUNCATE = 1
+POOL_MERGE_IN_LAUNCH = 2
 
 
 class PoolConfig(C.Structure):
@@ -117,6 +118,7 @@ PROTOTYPES = {
     "itak_pool_destroy": (None, [_P]),
     "itak_pool_set_stream": (_i32, [_P, _P]),
     "itak_pool_synchronize": (_i32, [_P]),
+    "itak_pool_set_merge_spin_limit": (_i32, [_P, _u32]),
     "itak_pool_device_bytes": (_u64, [_P]),
     "itak_slot_acquire": (_i32, [_P, C.POINTER(_u32)]),
     "itak_slot_release": (_i32, [_P, _u32]),

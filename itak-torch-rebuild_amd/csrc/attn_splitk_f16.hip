@@ -25,6 +25,7 @@
 // cap*tanh(s/cap) of crates/torch-math/src/logits.rs:26-37 applied to the scaled scores.
 #include "internal.h"
 #include "mfma_common.h"
+#include "split_exchange.h"
 
 #include <math.h>
 
@@ -308,10 +309,6 @@ __device__ __forceinline__ void prep_trig(PrepTrig &t, double position, const do
 
 // Sum over the 32 lanes that share a head row: four DPP steps inside each row of 16 lanes
 // (neighbour, other pair, mirrored half, mirrored row), then the row 16 lanes away.
-template <int CTRL>
-__device__ __forceinline__ float dpp_lane(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
-}
 __device__ __forceinline__ float row_sum32(float v) {
     v += dpp_lane<0xB1>(v);   // quad_perm [1,0,3,2]
     v += dpp_lane<0x4E>(v);   // quad_perm [2,3,0,1]
@@ -356,6 +353,7 @@ __device__ __forceinline__ float4 prep_chunk(float4 x, bool norm, float4 w, floa
     return make_float4(o.x * t.s[0] + x.x * t.c[0], o.y * t.s[1] + x.y * t.c[1],
                        o.z * t.s[2] + x.z * t.c[2], o.w * t.s[3] + x.w * t.c[3]);
 }
+
 
 template <int NQ, int WAVES, int N, bool RING, bool PREP>
 __device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const AttnBatchT<N> &b,
@@ -637,6 +635,10 @@ __device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const 
     // Every LDS read of the merge is issued before the first one is used.
     constexpr int kDtPerWave = 8 / WAVES;  // channel tiles each wavefront finishes
     const bool final_out = item.splits == 1;
+    // The merge inside the launch: this group's run of the exchange buffer (p.ws).
+    const bool exchanges = p.exchange != 0 && !final_out;
+    ExchangeGroup xg;
+    if (exchanges) xg.init(p.ws, item, kv_head, split, nvec);
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
         const uint32_t j = qt * 16 + jl;
@@ -663,6 +665,17 @@ __device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const 
             L = fmaf(lw[w], wgt[w], L);
         }
         if (j >= nvec) continue;
+        if (exchanges) {
+            // Publish this wavefront's channel tiles of vector j to the slices' owners.
+#pragma unroll
+            for (int x = 0; x < kDtPerWave; ++x) {
+                floatx4 acc = ow[x][0] * wgt[0];
+#pragma unroll
+                for (int w = 1; w < WAVES; ++w) acc += ow[x][w] * wgt[w];
+                xg.publish(j, wave * kDtPerWave + x, g, acc, M, L);
+            }
+            continue;
+        }
         float *dst = final_out ? p.out + uint64_t(colout[qt]) * kD
                                : ws_acc + uint64_t(colps[qt]) * kD;
         const float post = final_out ? __builtin_amdgcn_rcpf(L) : 1.0f;
@@ -684,6 +697,12 @@ __device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const 
             *reinterpret_cast<float2 *>(ws_ml + uint64_t(colps[qt]) * 2) = make_float2(M, L);
     }
     ITAK_MARK(9)
+    if (exchanges) {
+        const float *gate = nullptr;
+        if constexpr (PREP) gate = fold.gate;
+        xg.template finish<WAVES * 64, kExchangePerThread, 1>(reinterpret_cast<unsigned long long *>(sm_o), p, item, kv_head,
+                                       group, magic, gate);
+    }
     ITAK_MARK_END
 }
 
@@ -828,6 +847,39 @@ uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads)
     return ws0;
 }
 
+// Decides whether a planned batch can merge its splits inside the split-K launch, and if so
+// re-bases every item's ws0 on the exchange buffer (in records of kExchangeWords words, after
+// the header). Returns the 64-bit words the buffer must hold, 0 when the batch keeps its merge
+// launch: nothing is split, or some workgroup would have more words to gather than its
+// threads and its merge area take.
+uint64_t attn_splitk_f16_plan_exchange(const PoolGeom &g, AttnBatch &b, uint32_t q_heads) {
+    const uint32_t group = q_heads / g.kv_heads;
+    const Variant v = pick_variant(g, b, group);
+    const uint64_t threads = uint64_t(v.waves) * 64;
+    bool any = false;
+    for (uint32_t i = 0; i < b.n; ++i) {
+        const AttnItem &it = b.item[i];
+        if (it.splits <= 1) continue;
+        any = true;
+        const uint64_t slices = uint64_t(it.rows) * group * 4;
+        const uint64_t max_local = (slices + it.splits - 1) / it.splits;
+        if (max_local * it.splits * kExchangeWords > threads * kExchangePerThread) return 0;
+        if (slices + it.splits >= 65536) return 0;  // the kernel divides by multiplication
+    }
+    if (!any) return 0;
+    uint64_t records = 0;
+    for (uint32_t i = 0; i < b.n; ++i) {
+        AttnItem &it = b.item[i];
+        if (it.splits <= 1) continue;
+        const uint64_t slices = uint64_t(it.rows) * group * 4;
+        const uint64_t max_local = (slices + it.splits - 1) / it.splits;
+        if (records > 0xffffffffull) return 0;
+        it.ws0 = uint32_t(records);
+        records += uint64_t(g.kv_heads) * it.splits * max_local * it.splits;
+    }
+    return kExchangeHeaderWords + records * kExchangeWords;
+}
+
 hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                   uint32_t max_rows, hipStream_t stream,
                                   const FoldedParams *folded) {
@@ -835,6 +887,7 @@ hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint3
     if (b.total_blocks == 0) return hipSuccess;
     const Variant v = pick_variant(p.g, b, p.group);
     const bool prep = folded && folded->prep_on;
+    if (!prep && v.index == 0 && attn_decode_f16_takes(p, b)) return launch_attn_decode_f16(p, b, total_partials, stream);
 #define ITAK_LAUNCH(NQ, W)                                                                \
     do {                                                                                  \
         const size_t lds = variant_lds(NQ, W);                                            \

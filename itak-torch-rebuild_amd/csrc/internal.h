@@ -287,6 +287,11 @@ struct AttnParams {
     float softcap;
     uint32_t window;        // attention window of the layer (cache.rs:36-48); 0 = global
     uint32_t ring_blocks;   // 32-row blocks of the layer's storage ring; 0 = rows are positions
+    // Split-K f16 kernel only: merge the splits inside the launch. `ws` is then the exchange
+    // buffer (every word empty between launches) and item.ws0 counts its records; a consumer
+    // gives up after spin_limit polls.
+    uint32_t exchange;
+    uint32_t spin_limit;
 };
 // What the reference's model does around the step (muse-glimmer/src/model.rs:445-464),
 // folded into the step's own launches instead of running as launches of their own. `gate`
@@ -335,11 +340,25 @@ uint32_t attn_generic_tile(uint32_t head_dim);
 // Partials are in log2 domain (combine with base2 = 1).
 bool attn_splitk_f16_supports(const PoolGeom &g, uint32_t group, uint32_t max_rows);
 uint32_t attn_splitk_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads);
+// After attn_splitk_f16_plan: whether the batch can merge its splits inside the split-K launch
+// (AttnParams::exchange). Returns the 64-bit words the exchange buffer must hold and re-bases
+// the items' ws0 on it, or 0 (items untouched) when the batch keeps the merge launch.
+uint64_t attn_splitk_f16_plan_exchange(const PoolGeom &g, AttnBatch &b, uint32_t q_heads);
+// Sets `count` 64-bit words to `value` (the exchange buffer's empty pattern, at set-up).
+hipError_t launch_fill_words(unsigned long long *dst, uint64_t count, unsigned long long value,
+                             hipStream_t stream);
+constexpr unsigned long long kExchangeEmptyWord = 0xffffffffffffffffull;
 // `folded` with prep_on set selects the variants that prepare Q and the new K rows themselves
 // and gate what they write (every item must then be a 16-vector step); otherwise it is ignored.
 hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                   uint32_t max_rows, hipStream_t stream,
                                   const FoldedParams *folded = nullptr);
+// The latency-shaped form of the same path for decode steps (attn_decode_f16.hip): every item
+// one new row, at most one block per wavefront, splits merged inside the launch. `takes` is
+// asked after the batch has been planned and AttnParams::exchange set.
+bool attn_decode_f16_takes(const AttnParams &p, const AttnBatch &b);
+hipError_t launch_attn_decode_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                                  hipStream_t stream);
 // f32 MFMA split-K path: f32 pools (row-major planes), head_dim 128, rows*group <= 16, implied
 // query positions. Partials are in log2 domain (combine with base2 = 1).
 bool attn_splitk_f32_supports(const PoolGeom &g, uint32_t group, uint32_t max_rows);

@@ -423,6 +423,23 @@ hipError_t launch_signal_done(uint32_t *pinned_word, uint32_t value, hipStream_t
     return hipGetLastError();
 }
 
+// ------------------------------------------------------------- word fill
+// Sets 64-bit words to one value: the empty pattern of the split-K exchange buffer. A kernel,
+// not a memset, so that a stream under capture can carry it.
+__global__ __launch_bounds__(256) void fill_words_kernel(unsigned long long *dst, uint64_t n,
+                                                         unsigned long long value) {
+    for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < n; i += gridDim.x * 256ull)
+        dst[i] = value;
+}
+hipError_t launch_fill_words(unsigned long long *dst, uint64_t count, unsigned long long value,
+                             hipStream_t stream) {
+    if (count == 0) return hipSuccess;
+    uint64_t blocks = (count + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    fill_words_kernel<<<uint32_t(blocks), 256, 0, stream>>>(dst, count, value);
+    return hipGetLastError();
+}
+
 // ------------------------------------------------------------- measurement aids
 // A plain streaming copy of known size (the yardstick the FETCH_SIZE / WRITE_SIZE counters
 // are scaled by) and an empty kernel (the per-launch floor of a stream of dependent

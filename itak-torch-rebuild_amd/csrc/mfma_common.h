@@ -19,6 +19,12 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// The value of another lane of the same 16-lane row, chosen by a DPP control word.
+template <int CTRL>
+__device__ __forceinline__ float dpp_lane(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
 // cap * tanh(x / cap) * log2(e); x is a scaled score in natural units.
 // tanh(y) = 1 - 2 / (exp(2y) + 1) with the hardware's exp2 and reciprocal (each within one
 // unit in the last place; exp2 saturates to inf / 0 at the tails, giving +-1): a multiply, an

@@ -92,6 +92,13 @@ struct itak_pool {
     uint64_t ws_floats = 0;
     float *prep = nullptr;  // prepared Q and K rows of a prep step
     uint64_t prep_floats = 0;
+    // Exchange buffer of split-K launches that merge their splits themselves: 64-bit words,
+    // every one holding the empty pattern whenever no such launch is running; word 0 counts
+    // the consumers that gave up waiting (checked by itak_pool_synchronize).
+    unsigned long long *xws = nullptr;
+    uint64_t xws_words = 0;
+    uint32_t spin_limit = 1u << 17;  // polls a consumer makes (about a microsecond each)
+    bool merge_in_launch = false;
     // Pinned host memory for the host-pointer attention call: its small inputs are packed here
     // and go up in one copy; its kernels write the output here directly.
     unsigned char *hstage = nullptr;
@@ -268,6 +275,29 @@ itak_status ensure_workspace(itak_pool *pool, uint64_t floats) {
     return ITAK_OK;
 }
 
+// (Re)fills the exchange buffer with the empty pattern and zeroes its give-up counter.
+itak_status clean_exchange(itak_pool *pool) {
+    HIP_TRY(pool, launch_fill_words(pool->xws, pool->xws_words, kExchangeEmptyWord, pool->stream),
+            "fill the split exchange buffer");
+    HIP_TRY(pool, launch_fill_words(pool->xws, 1, 0, pool->stream), "zero the give-up counter");
+    return ITAK_OK;
+}
+
+itak_status ensure_exchange(itak_pool *pool, uint64_t words) {
+    if (words > pool->xws_words) {
+        HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize before growing the exchange buffer");
+        if (pool->xws) HIP_TRY(pool, hipFree(pool->xws), "free the exchange buffer");
+        pool->xws = nullptr;
+        pool->xws_words = 0;
+        const uint64_t want = std::max<uint64_t>(words + words / 2, 1u << 17);
+        HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&pool->xws), want * 8),
+                "allocate the split exchange buffer");
+        pool->xws_words = want;
+        return clean_exchange(pool);
+    }
+    return ITAK_OK;
+}
+
 itak_status ensure_prep(itak_pool *pool, uint64_t floats) {
     if (floats > pool->prep_floats) {
         HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize before growing prep scratch");
@@ -407,7 +437,16 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
             }
             b.total_blocks = block0;
         }
-        itak_status st = ensure_workspace(pool, uint64_t(partials) * (pool->g.head_dim + 2));
+        // Split-K launches merge their splits themselves where the plan allows it (the gate,
+        // when there is one, must then be applied by that kernel: its preparing variants).
+        const float *gate = folded ? folded->gate : nullptr;
+        const bool prepares = folded && folded->prep_on && mfma;
+        uint64_t exchange_words = 0;
+        if (mfma && pool->merge_in_launch && (!gate || prepares))
+            exchange_words = attn_splitk_f16_plan_exchange(geom, b, uint32_t(q_heads));
+        itak_status st = exchange_words
+                             ? ensure_exchange(pool, exchange_words)
+                             : ensure_workspace(pool, uint64_t(partials) * (pool->g.head_dim + 2));
         if (st != ITAK_OK) return st;
         AttnParams p{};
         p.layer_base = layer_base(pool, layer);
@@ -417,7 +456,9 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         p.q = q_dev;
         p.out = out_dev;
         p.q_pos = q_pos_dev;
-        p.ws = pool->ws;
+        p.ws = exchange_words ? reinterpret_cast<float *>(pool->xws) : pool->ws;
+        p.exchange = exchange_words ? 1 : 0;
+        p.spin_limit = pool->spin_limit;
         p.k_new = (mfma || f32fast) ? k_new : nullptr;
         p.v_new = (mfma || f32fast) ? v_new : nullptr;
         p.q_heads = uint32_t(q_heads);
@@ -428,8 +469,6 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         // The gate is applied by whoever writes the output: the merge for items of several
         // splits; for items of one split the split-K kernel, which only its preparing
         // variants can; otherwise a launch of its own over the chunk's rows.
-        const float *gate = folded ? folded->gate : nullptr;
-        const bool prepares = folded && folded->prep_on && mfma;
         bool merged_only = mfma || prefill;
         for (uint32_t i = 0; i < count; ++i) merged_only = merged_only && b.item[i].splits > 1;
         const bool gate_folded = gate && (prepares || (mfma && merged_only));
@@ -448,9 +487,10 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
             HIP_TRY(pool, launch_attn_generic(pool->elem_f16, p, b, partials, pool->stream),
                     "launch attention");
         }
-        HIP_TRY(pool, launch_attn_combine(p, b, partials, total_rows, (mfma || prefill || f32fast) ? 1 : 0,
-                                          pool->stream, gate_folded ? gate : nullptr),
-                "launch split merge");
+        if (!exchange_words)
+            HIP_TRY(pool, launch_attn_combine(p, b, partials, total_rows, (mfma || prefill || f32fast) ? 1 : 0,
+                                              pool->stream, gate_folded ? gate : nullptr),
+                    "launch split merge");
         if (gate && !gate_folded) {
             const uint64_t q_width = q_heads * pool->g.head_dim;
             const uint64_t at = uint64_t(q_row0 - total_rows) * q_width;
@@ -873,6 +913,7 @@ itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out) {
         return hip_error(e, he, "zero KV pool");
     }
     pool->slots.resize(config->max_slots);
+    pool->merge_in_launch = (config->flags & ITAK_POOL_MERGE_IN_LAUNCH) != 0;
     *out = pool;
     return ITAK_OK;
 }
@@ -884,6 +925,7 @@ void itak_pool_destroy(itak_pool *pool) {
     if (pool->stage) (void)hipFree(pool->stage);
     if (pool->ws) (void)hipFree(pool->ws);
     if (pool->prep) (void)hipFree(pool->prep);
+    if (pool->xws) (void)hipFree(pool->xws);
     if (pool->hstage) (void)hipHostFree(pool->hstage);
     delete pool;
 }
@@ -897,6 +939,28 @@ itak_status itak_pool_set_stream(itak_pool *pool, void *hip_stream) {
 itak_status itak_pool_synchronize(itak_pool *pool) {
     if (!pool) return ITAK_INVALID_ARGUMENT;
     HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize");
+    if (pool->xws) {
+        // Consumers of an in-launch merge that gave up waiting counted themselves here; their
+        // outputs are NaN and the buffer may hold words nobody took, so it is made clean again.
+        uint32_t gave_up = 0;
+        HIP_TRY(pool, hipMemcpy(&gave_up, pool->xws, sizeof(gave_up), hipMemcpyDeviceToHost),
+                "read the split merge's give-up counter");
+        if (gave_up) {
+            itak_status st = clean_exchange(pool);
+            if (st != ITAK_OK) return st;
+            HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize");
+            return set_error(pool->err, ITAK_STEP_FAILED, "attention", gave_up, 0, 0, 0,
+                             "attention: %u workgroups of a split merge gave up waiting for their "
+                             "group; the outputs of that step are NaN",
+                             gave_up);
+        }
+    }
+    return ITAK_OK;
+}
+
+itak_status itak_pool_set_merge_spin_limit(itak_pool *pool, uint32_t polls) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    pool->spin_limit = polls;
     return ITAK_OK;
 }
 

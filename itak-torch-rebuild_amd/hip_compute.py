@@ -180,7 +180,8 @@ class KvPool:
 
     def __init__(self, pattern: Union[int, Sequence[LayerKind]], num_kv_heads: int, head_dim: int,
                  *, elem: str = "f16", max_slots: int = 1, capacity_rows: int = 4096,
-                 device: int = 0, scrub_on_truncate: bool = True, ring_headroom: int = 0):
+                 device: int = 0, scrub_on_truncate: bool = True, ring_headroom: int = 0,
+                 merge_in_launch: bool = False):
         if isinstance(pattern, int):
             pattern = [LayerKind.Global] * pattern
         self.pattern = list(pattern)
@@ -200,7 +201,8 @@ class KvPool:
         cfg.max_slots = max_slots
         cfg.capacity_rows = capacity_rows
         cfg.device = device
-        cfg.flags = N.POOL_SCRUB_ON_TRUNCATE if scrub_on_truncate else 0
+        cfg.flags = (N.POOL_SCRUB_ON_TRUNCATE if scrub_on_truncate else 0) | \
+                    (N.POOL_MERGE_IN_LAUNCH if merge_in_launch else 0)
         cfg.ring_headroom = ring_headroom
         handle = C.c_void_p()
         self._h = None
@@ -232,6 +234,10 @@ class KvPool:
 
     def synchronize(self) -> None:
         _check(self._h, self._lib.itak_pool_synchronize(self._h))
+
+    def set_merge_spin_limit(self, polls: int) -> None:
+        """Bound on the polls a workgroup of an in-launch split merge waits for its group."""
+        _check(self._h, self._lib.itak_pool_set_merge_spin_limit(self._h, polls))
 
     def acquire(self) -> "KvCache":
         slot = C.c_uint32()

@@ -85,7 +85,7 @@ def test_config2_30b_class_decode_step_all_layers(softcap):
         pool.attention_step_device(layer, [(cache, 1)], qd.data_ptr(), kd[ctx:].data_ptr(),
                                    vd[ctx:].data_ptr(), out.data_ptr(), Q_HEADS, softcap=softcap)
         torch.cuda.synchronize()
-        if layer % 6 == 0 or layer == layers - 1:  # the oracle checks 9 of the 48 layers
+        if True:  # every layer is checked against the oracle
             ref = oracle_cache(1, KV_HEADS, D, True)
             ref.restore_bulk(0, 0, k[:ctx], v[:ctx])
             want = oracle.attention_step(ref, 0, q, k[ctx:], v[ctx:], Q_HEADS, ctx,
