@@ -506,6 +506,22 @@ itak_status itak_attention_step_device(itak_pool *pool, uint64_t layer,
                                        const float *q_dev, const float *k_dev, const float *v_dev,
                                        float *out_dev, uint64_t num_q_heads, float scale,
                                        float softcap);
+/* itak_attention_step_device for callers that cannot allocate device memory (code under HIP
+   graph capture, tight serving loops, harnesses that forbid it). No counterpart in the
+   reference. Same arguments, results and refusals; but where that call takes the split
+   workspace of its launches from buffers the pool allocates and grows, this one takes it from
+   a static array of 16 MiB in the library's device image (8 MiB of exchange words for launches
+   that merge their own splits, 8 MiB of split partials for the others) and calls no
+   hipMalloc, hipFree or other allocating routine. A step whose launches would need more
+   (8 MiB of partials = rows x q_heads x splits x 520 bytes summed over the slots) is
+   refused with ITAK_CAPACITY_EXCEEDED before anything is changed. Every call on a device
+   shares that device's array, whichever pool makes it: calls that overlap on one device (two
+   pools on two streams) race on it, and so must be ordered by the caller. */
+itak_status itak_attention_step_device_noalloc(itak_pool *pool, uint64_t layer,
+                                               const itak_batch_item *items, uint32_t item_count,
+                                               const float *q_dev, const float *k_dev,
+                                               const float *v_dev, float *out_dev,
+                                               uint64_t num_q_heads, float scale, float softcap);
 /* What Q and K go through between their projections and attention in the reference's
    model (crates/muse-glimmer/src/model.rs:445-451, crates/cpu-compute/src/cpu.rs:598-622):
    a per-head RMSNorm under one [head_dim] weight each (torch_math::rms_norm,

@@ -161,6 +161,8 @@ PROTOTYPES = {
     "itak_compute_cache_release": (_i32, [_P, _u32, C.POINTER(CheckpointRaw)]),
     "itak_attention_step_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P, _P, _P,
                                           _u64, _f32, _f32]),
+    "itak_attention_step_device_noalloc": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P, _P,
+                                                  _P, _u64, _f32, _f32]),
     "itak_attention_prep_step_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P, _P, _P,
                                                _P, _u64, _f32, _f32, C.POINTER(PrepParams)]),
     "itak_attention_device": (_i32, [_P, _u64, C.POINTER(BatchItem), _u32, _P, _P, _u64, _f32,

@@ -7,6 +7,8 @@
 #include "itkv.h"
 
 #include <algorithm>
+#include <atomic>
+#include <mutex>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -16,6 +18,11 @@
 #include <vector>
 
 using namespace itak;
+
+// Split workspace of itak_attention_step_device_noalloc: see the notes at g_scratch_of_device.
+// Host code never passes this name to a kernel or a memory call: it is a host-side handle,
+// the device address comes from hipGetSymbolAddress.
+static __device__ __align__(256) unsigned char scratch[16ull << 20];
 
 namespace {
 
@@ -57,7 +64,20 @@ struct ErrorState {
 };
 
 thread_local ErrorState g_create_error;
-uint64_t g_next_cache_id = 1;  // cache.rs:32
+
+// ---- the split workspace of the allocation-free entry point --------------------------------
+// itak_attention_step_device_noalloc may not allocate, so its split workspace is this array:
+// every device the library runs on holds a copy until the process ends. The first part holds
+// exchange words for launches that merge their own splits (all empty between launches, like
+// the pool's own exchange buffer); the rest takes the partials of launches that leave the
+// merge to a second launch. In host code the array's name is only a handle: the address the
+// kernels get is looked up once per device (bind_scratch) and kept here.
+constexpr uint64_t kScratchBytes = sizeof(scratch);
+constexpr uint64_t kScratchExchangeBytes = 8ull << 20;
+constexpr int kMaxDevices = 64;
+unsigned char *g_scratch_of_device[kMaxDevices];
+std::mutex g_scratch_mutex;
+std::atomic<uint64_t> g_next_cache_id{1};  // cache.rs:32
 
 }  // namespace
 
@@ -98,6 +118,11 @@ struct itak_pool {
     unsigned long long *xws = nullptr;
     uint64_t xws_words = 0;
     uint32_t spin_limit = 1u << 17;  // polls a consumer makes (about a microsecond each)
+    // This device's copy of the static split workspace, and whether the call in progress must
+    // use it instead of the pool's own buffers (itak_attention_step_device_noalloc).
+    unsigned char *scratch_dev = nullptr;
+    bool no_alloc_call = false;
+    bool scratch_exchange_used = false;  // its give-up counter is then looked at too
     bool merge_in_launch = false;
     // Pinned host memory for the host-pointer attention call: its small inputs are packed here
     // and go up in one copy; its kernels write the output here directly.
@@ -329,6 +354,34 @@ itak_status ensure_hstage(itak_pool *pool, uint64_t bytes) {
 
 uint64_t align_up(uint64_t x, uint64_t a) { return (x + a - 1) / a * a; }
 
+// The address of this device's copy of `scratch`, looked up on first use with the device
+// current; the exchange part is filled with the empty pattern then (a kernel on the null
+// stream, waited for). Later calls return the kept address.
+hipError_t bind_scratch(int device, unsigned char **out) {
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_of_device[device]) {
+        unsigned char *ptr = nullptr;
+        hipError_t e = hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!ptr) return hipErrorInvalidSymbol;
+        e = launch_fill_words(reinterpret_cast<unsigned long long *>(ptr), kScratchExchangeBytes / 8,
+                              kExchangeEmptyWord, nullptr);
+        if (e == hipSuccess) e = launch_fill_words(reinterpret_cast<unsigned long long *>(ptr), 1, 0, nullptr);
+        if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+        if (e != hipSuccess) return e;
+        g_scratch_of_device[device] = ptr;
+    }
+    *out = g_scratch_of_device[device];
+    return hipSuccess;
+}
+
+// What the launches of one attention call need beyond their inputs and outputs.
+struct WorkspaceNeed {
+    uint64_t partial_floats = 0;   // split partials for a merge launch
+    uint64_t exchange_words = 0;   // exchange words of launches that merge their own splits
+};
+
 // One item's query rows against its slot; fills the split plan.
 struct PlanInput {
     uint32_t slot;
@@ -363,7 +416,7 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
                           const float *q_dev, float *out_dev, const uint32_t *q_pos_dev,
                           uint64_t q_heads, float scale, float softcap,
                           const float *k_new = nullptr, const float *v_new = nullptr,
-                          const FoldedParams *folded = nullptr) {
+                          const FoldedParams *folded = nullptr, WorkspaceNeed *need_only = nullptr) {
     const uint32_t group = uint32_t(q_heads / pool->g.kv_heads);
     uint32_t max_rows = 0;
     for (uint32_t i = 0; i < n; ++i) max_rows = std::max(max_rows, in[i].rows);
@@ -444,10 +497,24 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         uint64_t exchange_words = 0;
         if (mfma && pool->merge_in_launch && (!gate || prepares))
             exchange_words = attn_splitk_f16_plan_exchange(geom, b, uint32_t(q_heads));
-        itak_status st = exchange_words
-                             ? ensure_exchange(pool, exchange_words)
-                             : ensure_workspace(pool, uint64_t(partials) * (pool->g.head_dim + 2));
-        if (st != ITAK_OK) return st;
+        const uint64_t partial_floats = uint64_t(partials) * (pool->g.head_dim + 2);
+        if (need_only) {  // planning only: nothing is allocated, launched or changed
+            need_only->exchange_words = std::max(need_only->exchange_words, exchange_words);
+            if (!exchange_words)
+                need_only->partial_floats = std::max(need_only->partial_floats, partial_floats);
+            continue;
+        }
+        float *ws = nullptr;
+        if (pool->no_alloc_call) {
+            // The caller has checked the need against the static workspace's two parts.
+            ws = reinterpret_cast<float *>(exchange_words ? pool->scratch_dev
+                                                          : pool->scratch_dev + kScratchExchangeBytes);
+        } else {
+            itak_status st = exchange_words ? ensure_exchange(pool, exchange_words)
+                                            : ensure_workspace(pool, partial_floats);
+            if (st != ITAK_OK) return st;
+            ws = exchange_words ? reinterpret_cast<float *>(pool->xws) : pool->ws;
+        }
         AttnParams p{};
         p.layer_base = layer_base(pool, layer);
         p.g = geom;
@@ -456,7 +523,7 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         p.q = q_dev;
         p.out = out_dev;
         p.q_pos = q_pos_dev;
-        p.ws = exchange_words ? reinterpret_cast<float *>(pool->xws) : pool->ws;
+        p.ws = ws;
         p.exchange = exchange_words ? 1 : 0;
         p.spin_limit = pool->spin_limit;
         p.k_new = (mfma || f32fast) ? k_new : nullptr;
@@ -914,6 +981,12 @@ itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out) {
     }
     pool->slots.resize(config->max_slots);
     pool->merge_in_launch = (config->flags & ITAK_POOL_MERGE_IN_LAUNCH) != 0;
+    he = bind_scratch(config->device, &pool->scratch_dev);
+    if (he != hipSuccess) {
+        (void)hipFree(pool->base);
+        delete pool;
+        return hip_error(e, he, "look up the static split workspace");
+    }
     *out = pool;
     return ITAK_OK;
 }
@@ -939,22 +1012,32 @@ itak_status itak_pool_set_stream(itak_pool *pool, void *hip_stream) {
 itak_status itak_pool_synchronize(itak_pool *pool) {
     if (!pool) return ITAK_INVALID_ARGUMENT;
     HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize");
-    if (pool->xws) {
-        // Consumers of an in-launch merge that gave up waiting counted themselves here; their
-        // outputs are NaN and the buffer may hold words nobody took, so it is made clean again.
+    // Consumers of an in-launch merge that gave up waiting counted themselves in their
+    // buffer's first word; their outputs are NaN and the buffer may hold words nobody took,
+    // so it is made clean again.
+    unsigned long long *buffers[2] = {pool->xws,
+                                      pool->scratch_exchange_used
+                                          ? reinterpret_cast<unsigned long long *>(pool->scratch_dev)
+                                          : nullptr};
+    const uint64_t words[2] = {pool->xws_words, kScratchExchangeBytes / 8};
+    uint32_t total = 0;
+    for (int i = 0; i < 2; ++i) {
+        if (!buffers[i]) continue;
         uint32_t gave_up = 0;
-        HIP_TRY(pool, hipMemcpy(&gave_up, pool->xws, sizeof(gave_up), hipMemcpyDeviceToHost),
+        HIP_TRY(pool, hipMemcpy(&gave_up, buffers[i], sizeof(gave_up), hipMemcpyDeviceToHost),
                 "read the split merge's give-up counter");
-        if (gave_up) {
-            itak_status st = clean_exchange(pool);
-            if (st != ITAK_OK) return st;
-            HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize");
-            return set_error(pool->err, ITAK_STEP_FAILED, "attention", gave_up, 0, 0, 0,
-                             "attention: %u workgroups of a split merge gave up waiting for their "
-                             "group; the outputs of that step are NaN",
-                             gave_up);
-        }
+        if (!gave_up) continue;
+        total += gave_up;
+        HIP_TRY(pool, launch_fill_words(buffers[i], words[i], kExchangeEmptyWord, pool->stream),
+                "fill the split exchange buffer");
+        HIP_TRY(pool, launch_fill_words(buffers[i], 1, 0, pool->stream), "zero the give-up counter");
+        HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize");
     }
+    if (total)
+        return set_error(pool->err, ITAK_STEP_FAILED, "attention", total, 0, 0, 0,
+                         "attention: %u workgroups of a split merge gave up waiting for their "
+                         "group; the outputs of that step are NaN",
+                         total);
     return ITAK_OK;
 }
 
@@ -1838,7 +1921,8 @@ static itak_status step_on_device(itak_pool *pool, uint64_t layer, const itak_ba
                                   uint32_t item_count, const std::vector<PlanInput> &plan,
                                   const float *q_dev, const float *k_dev, const float *v_dev,
                                   float *out_dev, uint64_t num_q_heads, float scale,
-                                  float softcap, const FoldedParams *folded = nullptr) {
+                                  float softcap, const FoldedParams *folded = nullptr,
+                                  bool no_alloc = false) {
     // Rows of zero-row items contribute nothing; q/k/v rows are numbered by walking the
     // items in order, so such items may simply be dropped.
     std::vector<PlanInput> active;
@@ -1850,6 +1934,38 @@ static itak_status step_on_device(itak_pool *pool, uint64_t layer, const itak_ba
         takes_splitk_f16(pool, active.data(), uint32_t(active.size()), num_q_heads, nullptr) ||
         (!pool->elem_f16 && !active.empty() &&
          attn_splitk_f32_supports(pool->g, uint32_t(num_q_heads / pool->g.kv_heads), most_rows));
+    // The allocation-free form plans first and refuses, before anything changes, a step whose
+    // launches need more workspace than the static array has.
+    struct NoAllocScope {
+        itak_pool *pool;
+        bool on;
+        ~NoAllocScope() { if (on) pool->no_alloc_call = false; }
+    } scope{pool, no_alloc};
+    if (no_alloc) {
+        WorkspaceNeed need;
+        itak_status st = run_attention(pool, layer, active.data(), uint32_t(active.size()), q_dev, out_dev,
+                                       nullptr, num_q_heads, scale, softcap, nullptr, nullptr, folded,
+                                       &need);
+        if (st != ITAK_OK) return st;
+        const uint64_t partial_bytes = need.partial_floats * sizeof(float);
+        const uint64_t exchange_bytes = need.exchange_words * 8;
+        if (partial_bytes > kScratchBytes - kScratchExchangeBytes)
+            return set_error(pool->err, ITAK_CAPACITY_EXCEEDED, "split workspace", layer, partial_bytes,
+                             kScratchBytes - kScratchExchangeBytes, 0,
+                             "the step's split partials need %llu bytes of workspace and the "
+                             "allocation-free entry point holds %llu: use fewer slots or rows per "
+                             "step, or itak_attention_step_device",
+                             ULL(partial_bytes), ULL(kScratchBytes - kScratchExchangeBytes));
+        if (exchange_bytes > kScratchExchangeBytes)
+            return set_error(pool->err, ITAK_CAPACITY_EXCEEDED, "split workspace", layer, exchange_bytes,
+                             kScratchExchangeBytes, 0,
+                             "the step's split exchange needs %llu bytes of workspace and the "
+                             "allocation-free entry point holds %llu: use fewer slots or rows per "
+                             "step, or itak_attention_step_device",
+                             ULL(exchange_bytes), ULL(kScratchExchangeBytes));
+        pool->no_alloc_call = true;
+        if (need.exchange_words) pool->scratch_exchange_used = true;
+    }
     if (fuse) {
         for (uint32_t i = 0; i < item_count; ++i)
             advance(pool->slots[items[i].slot], layer, items[i].rows);
@@ -1907,6 +2023,23 @@ itak_status itak_attention_step_device(itak_pool *pool, uint64_t layer,
     if (std::isnan(scale)) scale = default_scale(pool->g.head_dim);
     return step_on_device(pool, layer, items, item_count, plan, q_dev, k_dev, v_dev, out_dev,
                           num_q_heads, scale, softcap);
+}
+
+itak_status itak_attention_step_device_noalloc(itak_pool *pool, uint64_t layer,
+                                               const itak_batch_item *items, uint32_t item_count,
+                                               const float *q_dev, const float *k_dev,
+                                               const float *v_dev, float *out_dev,
+                                               uint64_t num_q_heads, float scale, float softcap) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (item_count == 0) return ITAK_OK;
+    if (!items || !q_dev || !k_dev || !v_dev || !out_dev)
+        return invalid_argument(pool->err, "items or a device tensor is null");
+    std::vector<PlanInput> plan;
+    itak_status st = plan_step(pool, layer, items, item_count, num_q_heads, plan);
+    if (st != ITAK_OK) return st;
+    if (std::isnan(scale)) scale = default_scale(pool->g.head_dim);
+    return step_on_device(pool, layer, items, item_count, plan, q_dev, k_dev, v_dev, out_dev,
+                          num_q_heads, scale, softcap, nullptr, true);
 }
 
 itak_status itak_attention_prep_step_device(itak_pool *pool, uint64_t layer,

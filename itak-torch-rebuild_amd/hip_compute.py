@@ -261,6 +261,16 @@ class KvPool:
             self._h, layer, raw, n, q_ptr, k_ptr, v_ptr, out_ptr, num_q_heads,
             math.nan if scale is None else scale, softcap))
 
+    def attention_step_device_noalloc(self, layer: int, items, q_ptr: int, k_ptr: int, v_ptr: int,
+                                      out_ptr: int, num_q_heads: int, scale: Optional[float] = None,
+                                      softcap: float = 0.0) -> None:
+        """attention_step_device with its split workspace in the library's static device array:
+        allocates nothing; refuses steps that need more than the array holds."""
+        raw, n = self._items(items)
+        _check(self._h, self._lib.itak_attention_step_device_noalloc(
+            self._h, layer, raw, n, q_ptr, k_ptr, v_ptr, out_ptr, num_q_heads,
+            math.nan if scale is None else scale, softcap))
+
     def attention_prep_step_device(self, layer: int, items, q_ptr: int, k_ptr: int, v_ptr: int,
                                    out_ptr: int, num_q_heads: int, *, q_norm_ptr: int = 0,
                                    k_norm_ptr: int = 0, eps: float = 1e-6, rope_base: float = 0.0,
