@@ -124,7 +124,11 @@ typedef struct itak_pool_config {
        carry on a windowed layer, max_round_tokens of a checkpoint, and how far a truncate may
        go back (the chunk_cap of the reference's resident session,
        crates/wgpu-compute/src/session.rs:235-249, 5376-5428). A ring is window +
-       ring_headroom rows, rounded up to a multiple of 32. */
+       ring_headroom rows, rounded up to a multiple of 32; the bound that blocks, checkpoints
+       (max_round_tokens) and truncates meet is what the rounding leaves, ring - window of the
+       shortest such layer, so at least ring_headroom. The reference's CPU cache takes any
+       max_round_tokens up to the smallest window (cache.rs:634-651): a round longer than the
+       bound is refused here with ITAK_CAPACITY_EXCEEDED. */
     uint64_t ring_headroom;
 } itak_pool_config;
 

@@ -1137,6 +1137,7 @@ itak_status itak_kv_storage_rows(itak_pool *pool, uint64_t layer, uint64_t *out)
 
 itak_status itak_kv_stored_len(itak_pool *pool, uint32_t slot, uint64_t layer, uint64_t *out) {
     if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (!out) return invalid_argument(pool->err, "out is null");
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
     if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
@@ -1146,6 +1147,7 @@ itak_status itak_kv_stored_len(itak_pool *pool, uint32_t slot, uint64_t layer, u
 
 itak_status itak_kv_next_position(itak_pool *pool, uint32_t slot, uint64_t layer, uint64_t *out) {
     if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (!out) return invalid_argument(pool->err, "out is null");
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
     if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
@@ -1678,6 +1680,7 @@ itak_status itak_kv_read_raw(itak_pool *pool, uint32_t slot, uint64_t layer, voi
 
 itak_status itak_kv_checkpoint_active(itak_pool *pool, uint32_t slot, int32_t *out) {
     if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (!out) return invalid_argument(pool->err, "out is null");
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
     *out = s->cp.live ? 1 : 0;
@@ -1708,12 +1711,17 @@ itak_status itak_kv_checkpoint(itak_pool *pool, uint32_t slot, uint64_t max_roun
                          ULL(max_round_tokens), ULL(smallest_window));
     // The device keeps no copies of evicted rows: the ring's headroom is what lets a round be
     // undone, so a round may not be longer than it.
-    if (windowed && max_round_tokens > pool->headroom)
+    // (what the rings really hold beyond their windows: the configured headroom rounded up to
+    // whole 32-row blocks, the bound check_block_rows and check_ring_rewind use too)
+    uint64_t ring_room = ~0ull;
+    for (const LayerInfo &L : pool->layers)
+        if (L.windowed) ring_room = std::min<uint64_t>(ring_room, L.ring - L.window);
+    if (windowed && max_round_tokens > ring_room)
         return set_error(pool->err, ITAK_CAPACITY_EXCEEDED, nullptr, 0, max_round_tokens,
-                         pool->headroom, 0,
+                         ring_room, 0,
                          "a round of up to %llu tokens does not fit the %llu rows of ring headroom "
                          "of the windowed layers; build the pool with a larger ring_headroom",
-                         ULL(max_round_tokens), ULL(pool->headroom));
+                         ULL(max_round_tokens), ULL(ring_room));
     s->next_serial += 1;
     s->cp.live = true;
     s->cp.serial = s->next_serial;
@@ -1737,6 +1745,7 @@ static itak_status live_data(itak_pool *pool, Slot &s, const itak_checkpoint *cp
 itak_status itak_kv_checkpoint_bases(itak_pool *pool, uint32_t slot, const itak_checkpoint *cp,
                                      uint64_t *out) {
     if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (!out || !cp) return invalid_argument(pool->err, "cp or out is null");
     Slot *s = find_slot(pool, slot);
     if (!s) return invalid_argument(pool->err, "slot is not in use");
     itak_status st = live_data(pool, *s, cp);

@@ -72,6 +72,14 @@ static void host_checks(const char *dir) {
         CHECK(itak_kv_prefix_discriminator(tokens, 3) != itak_kv_prefix_hash(tokens, 3));
     }
     {
+        /* The discriminator's basis (hash.rs:21) and two values folded by hand. */
+        const uint32_t one[1] = {1}, two[2] = {0xdeadbeefu, 7};
+        CHECK(itak_kv_prefix_discriminator(one, 0) == 0x84222325cbf29ce4ull);
+        CHECK(itak_kv_prefix_discriminator(one, 1) == 0xb61d2746190c09b5ull);
+        CHECK(itak_kv_prefix_discriminator(two, 2) == 0x393db72d40db1afdull);
+        CHECK(itak_kv_prefix_hash(one, 1) == 0xad2aca7747985764ull);
+    }
+    {
         /* One block: the sum of one sum. */
         const uint64_t inner = itak_kv_checksum("foobar", 6);
         uint8_t le[8];

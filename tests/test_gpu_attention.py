@@ -345,3 +345,68 @@ def test_random_blocks_match_the_oracle_across_groups_windows_and_softcap(seed):
                                  oracle.AttentionParams(softcap=softcap), threads=8)
     assert max_abs(out.cpu().numpy().reshape(-1), want) <= 2e-3, (group, ctx, rows, softcap, window)
     pool.close()
+
+
+@pytest.mark.parametrize("rows", [1, 7])
+@pytest.mark.parametrize("q_scale,k_scale", [(3.0, 1.0), (1.0, 3.0), (1.5, 2.0)])
+def test_f16_operands_meet_the_bar_up_to_scores_of_deviation_three(rows, q_scale, k_scale):
+    # Q and P enter the MFMAs as f16, so the error grows with the size of the scaled scores
+    # (Q's rounding is relative). The bar of 2e-3 holds up to scores of standard deviation 3
+    # (measured on an MI355X: 3e-5 at deviation 1, the scale of the benchmark's inputs; about
+    # 1e-3 to 1.5e-3 at 3; 1.9e-3 at 4; above the bar at 6). This pins the documented limit.
+    ctx = 4096
+    worst = 0.0
+    for seed in range(2):
+        rng = np.random.default_rng(1000 + seed)
+        k = normal(rng, ctx + rows, 512) * k_scale
+        v = normal(rng, ctx + rows, 512)
+        q = normal(rng, rows, 32 * 128) * q_scale
+        pool = P().KvPool(1, 4, 128, elem="f16", capacity_rows=ctx + rows)
+        cache = pool.acquire()
+        import torch
+        pool.set_stream(torch.cuda.current_stream().cuda_stream)
+        kd, vd, qd = (torch.from_numpy(x).cuda() for x in (k, v, q))
+        out = torch.empty_like(qd)
+        pool.append_device(0, [(cache, ctx)], kd.data_ptr(), vd.data_ptr())
+        pool.attention_step_device(0, [(cache, rows)], qd.data_ptr(), kd[ctx:].data_ptr(),
+                                   vd[ctx:].data_ptr(), out.data_ptr(), 32)
+        pool.synchronize()
+        ref = oracle.KvCache.new([oracle.LayerKind.Global], 4, 128, store_f16=True)
+        ref.restore_bulk(0, 0, k[:ctx], v[:ctx])
+        want = oracle.attention_step(ref, 0, q, k[ctx:], v[ctx:], 32, ctx, threads=8)
+        worst = max(worst, max_abs(out.cpu().numpy().reshape(-1), want))
+        pool.close()
+    assert worst <= F16_ABS, worst
+
+
+def test_masked_rows_with_non_finite_values_do_not_reach_a_decode_query():
+    # The reference never reads the value row of a key a query does not see
+    # (attention.rs:160-173): rows of a windowed layer that have just left the window, and
+    # storage rows past the sequence's length, may hold anything, NaN and infinity included.
+    import torch
+    window, ctx = 64, 200
+    rng = np.random.default_rng(5)
+    k, v = normal(rng, ctx + 1, 512), normal(rng, ctx + 1, 512)
+    lo = ctx + 1 - window  # the oldest position the query at `ctx` sees
+    v[lo - 1] = np.inf     # just outside the window, in the same 32-row block as visible rows
+    v[lo - 2] = np.nan
+    q = normal(rng, 1, 32 * 128)
+    for in_launch in (False, True):
+        pool = P().KvPool([P().LayerKind.windowed(window)], 4, 128, elem="f16", capacity_rows=ctx + 8,
+                          ring_headroom=64, merge_in_launch=in_launch)
+        pool.set_stream(torch.cuda.current_stream().cuda_stream)
+        cache = pool.acquire()
+        kd, vd, qd = (torch.from_numpy(x).cuda() for x in (k, v, q))
+        out = torch.empty_like(qd)
+        for p0 in range(0, ctx, 50):  # the ring keeps the rows just outside the window too
+            pool.append_device(0, [(cache, 50)], kd[p0:].data_ptr(), vd[p0:].data_ptr())
+        pool.attention_step_device(0, [(cache, 1)], qd.data_ptr(), kd[ctx:].data_ptr(),
+                                   vd[ctx:].data_ptr(), out.data_ptr(), 32)
+        pool.synchronize()
+        ref = oracle.KvCache.new([oracle.LayerKind.windowed(window)], 4, 128, store_f16=True)
+        ref.restore_bulk(0, ctx - window, k[ctx - window:ctx], v[ctx - window:ctx])
+        want = oracle.attention_step(ref, 0, q, k[ctx:], v[ctx:], 32, ctx, threads=4)
+        got = out.cpu().numpy().reshape(-1)
+        assert np.isfinite(want).all() and np.isfinite(got).all()
+        assert max_abs(got, want) <= F16_ABS
+        pool.close()

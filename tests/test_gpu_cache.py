@@ -432,3 +432,21 @@ def test_slots_are_independent_and_reset_gives_a_fresh_cache():
     a.release_slot()
     c = pool.acquire()
     assert c.slot == a.slot and c.stored_len(0) == 0
+
+
+def test_getters_refuse_null_outputs_by_name():
+    # Nothing aborts across the boundary: a null out pointer is an InvalidArgument refusal.
+    pool = P().KvPool(1, 2, 8, elem="f32", capacity_rows=8)
+    cache = pool.acquire()
+    lib = P()._native.load()
+    cp = cache.checkpoint(1)
+    raw = P()._native.CheckpointRaw()
+    for status in (lib.itak_kv_stored_len(pool._h, cache.slot, 0, None),
+                   lib.itak_kv_next_position(pool._h, cache.slot, 0, None),
+                   lib.itak_kv_checkpoint_active(pool._h, cache.slot, None),
+                   lib.itak_kv_checkpoint_bases(pool._h, cache.slot, raw, None),
+                   lib.itak_kv_checkpoint_bases(pool._h, cache.slot, None, None)):
+        assert status == 17, status
+        assert b"null" in lib.itak_last_error(pool._h)
+    cache.release(cp)
+    pool.close()

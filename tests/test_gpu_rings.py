@@ -278,14 +278,21 @@ def test_the_rings_headroom_bounds_blocks_rounds_and_truncates():
     for _ in range(4):
         pool.append_device(0, [(cache, 32)], rows.data_ptr(), rows.data_ptr())
     assert cache.next_position(0) == 128
+    # A round may be as long as the ring can undo: ring - window = 32 rows (the configured 16
+    # rounded up to whole blocks), the same bound blocks and truncates have; 33 is refused.
     with pytest.raises(P().AttentionError) as e:
-        cache.checkpoint(17)
+        cache.checkpoint(33)
     assert e.value.variant == "CapacityExceeded" and "ring headroom" in e.value.message
     pool.truncate([cache.slot], [100])   # 28 positions back: inside the 32 spare rows
     assert cache.next_position(0) == 100
     with pytest.raises(P().AttentionError) as e:
         pool.truncate([cache.slot], [90])  # the rows up to 128 are still in the ring
     assert e.value.variant == "CapacityExceeded"
+    assert cache.next_position(0) == 100
+    cp = cache.checkpoint(32)  # exactly the bound
+    pool.append_device(0, [(cache, 32)], rows.data_ptr(), rows.data_ptr())
+    cache.rewind_to(cp, 100)
+    cache.release(cp)
     assert cache.next_position(0) == 100
     pool.close()
 

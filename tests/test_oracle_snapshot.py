@@ -59,6 +59,20 @@ def test_fnv1a_matches_the_published_vectors_and_the_reference_cases():
     assert oracle.prefix_hash([7, 8, 9, 10]) == okv.prefix_hash([7, 8, 9, 10])
 
 
+def test_prefix_discriminator_is_pinned_by_literals():
+    # The discriminator is FNV-1a 64 from the alternate basis of hash.rs:21. No tokens give the
+    # basis itself; the other two values were folded by hand (xor a byte, multiply by the prime
+    # 0x100000001b3 modulo 2^64, four little-endian bytes per token), not by the code under
+    # test: [1] and [0xDEADBEEF, 7].
+    P = pkg()
+    for fn in (okv.prefix_discriminator, P.prefix_discriminator):
+        assert fn([]) == 0x84222325CBF29CE4
+        assert fn([1]) == 0xB61D2746190C09B5
+        assert fn([0xDEADBEEF, 7]) == 0x393DB72D40DB1AFD
+    # The same fold from the standard basis, for contrast (hash.rs:44-46).
+    assert okv.prefix_hash([1]) == 0xAD2ACA7747985764 == P.prefix_hash([1])
+
+
 # ---- layout -----------------------------------------------------------------------------
 
 def test_bytes_follow_the_layout_table():
