@@ -45,6 +45,7 @@ from .prefix_store import (  # noqa: F401
     prefix_store_enabled,
     prefix_store_enabled_from,
 )
+from .resident import LayerInputCapture, ResidentTarget, SpecRoundRecord  # noqa: F401
 from . import _native  # noqa: F401
 
 __all__ = [
@@ -55,4 +56,5 @@ __all__ = [
     "capture_bytes", "checksum", "checksum_blocks", "prefix_discriminator", "prefix_hash", "restore_bytes",
     "EntryMeta", "PrefixHit", "PrefixStore", "StoreConfig", "StoreStats", "max_bytes_from",
     "now_unix", "prefix_store_enabled", "prefix_store_enabled_from",
+    "LayerInputCapture", "ResidentTarget", "SpecRoundRecord",
 ]
