@@ -1,11 +1,13 @@
 """CPU-only checks of the C ABI: the library loads, exports exactly what the header
 declares, and refuses bad construction arguments by name without touching a GPU."""
 import ctypes as C
+import os
 import subprocess
+import sys
 
 import pytest
 
-from helpers import declared_symbols, pkg
+from helpers import HEADER, ROOT, declared_symbols, pkg
 
 
 def test_library_exports_every_declared_symbol():
@@ -113,3 +115,45 @@ def test_product_sources_never_reference_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "import oracle" not in text and "itak_oracle" not in text, f
+
+
+def _rust_externs():
+    """name -> argument count of every `pub fn` in the extern block of itak-hip-sys."""
+    import re
+    path = os.path.join(ROOT, "crates", "itak-hip-sys", "src", "lib.rs")
+    text = open(path).read()
+    block = text[text.index('extern "C" {'):]
+    block = block[:block.index("\n}")]
+    out = {}
+    for name, args in re.findall(r"pub fn (itak_[a-z0-9_]+)\((.*?)\)(?: -> [^;]+)?;", block):
+        out[name] = 0 if not args.strip() else len([a for a in args.split(",") if a.strip()])
+    return out
+
+
+def _header_functions():
+    import re
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    out = {}
+    for name, args in re.findall(r"\b(itak_[a-z0-9_]+)\s*\(([^;{}]*?)\)\s*;", text, flags=re.S):
+        args = " ".join(args.split())
+        out[name] = 0 if args in ("", "void") else len(args.split(","))
+    return out
+
+
+def test_rust_binding_declares_the_header_symbol_for_symbol():
+    # crates/itak-hip-sys/src/lib.rs is written from the header by gen_bindings.py: the same
+    # functions with the same number of arguments, the ctypes table too, and the file is current.
+    N = pkg()._native
+    rust, header = _rust_externs(), _header_functions()
+    assert sorted(rust) == sorted(header) == declared_symbols()
+    assert rust == header
+    table = {name: len(proto[1]) for name, proto in N.PROTOTYPES.items()}
+    assert table == header
+    gen = os.path.join(ROOT, "crates", "itak-hip-sys", "gen_bindings.py")
+    assert subprocess.run([sys.executable, gen, "--check"]).returncode == 0
+    # Every struct the header declares has a #[repr(C)] twin.
+    import re
+    text = open(os.path.join(ROOT, "crates", "itak-hip-sys", "src", "lib.rs")).read()
+    header_text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    for name in re.findall(r"typedef\s+struct\s+(\w+)", header_text):
+        assert f"pub struct {name} " in text, name
