@@ -41,12 +41,30 @@ ROW = KV_HEADS * D
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
-# HBM bytes per layer (all launches of the layer's attention) measured with rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE and scaled by the same counters on the probe copy of known size
-# (profiles/*_traffic.md hold the runs and the scaling factors). Missing = not measured.
-MEASURED_TRAFFIC = {"decode": 9_958_451, "ragged": 216_836_265, "prefill": 290_164_626,
-                    "verify": 87_329_078}
-MEASURED_TRAFFIC_F32 = {"decode": 18_240_005}  # the same workload on an f32 cache (--kv f32)
+# HBM bytes per layer (all launches of the layer's attention) as rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE counted them in an earlier run, scaled by the same counters on the probe copy of
+# known size: (bytes, the summary under profiles/ that holds the run and the scaling factors).
+# They are not measured by this run: `traffic_source` says where each came from.
+PROFILE_TRAFFIC = {
+    ("decode", "f16"): (9_958_451, "profiles/attn_splitk_f16_decode_ctx4096_traffic.md"),
+    ("ragged", "f16"): (216_836_265, "profiles/attn_splitk_f16_ragged16_traffic.md"),
+    ("prefill", "f16"): (290_164_626, "profiles/attn_prefill_f16_chunk2048_prefix30720_traffic.md"),
+    ("verify", "f16"): (87_329_078, "profiles/attn_splitk_f16_verify_traffic.md"),
+    ("decode", "f32"): (18_240_005, "profiles/attn_splitk_f32_decode_ctx4096_traffic.md"),
+}
+
+
+def host_cpu():
+    """Model name and logical CPU count of the host the baseline is timed on."""
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return model, os.cpu_count()
 
 
 def rope_on_device(x, base):
@@ -89,11 +107,14 @@ def cpu_baseline(ctx: int, kv_bytes_per_layer: int, layers: int, budget_s: float
         cache.release(cp)
         done += 1
     per_layer = spent / done
+    model, logical = host_cpu()
     return {
         "value": round(kv_bytes_per_layer / per_layer / 1e9, 4),
         "unit": "GB/s",
         "cores": 1,
         "kind": "port",
+        "cpu_model": model,
+        "nproc": logical,
         "us_per_token": round(per_layer * layers * 1e6, 1),
         "sample": f"{done} layer-steps of the decode step (append + attend over {ctx + 1} "
                   f"positions, 32 Q / 4 KV heads, d=128, {'f16-rounded' if store_f16 else 'f32'} KV), single thread; the "
@@ -228,6 +249,102 @@ def cache_maintenance(args, pkg, torch, dev, stream, timed):
     return result
 
 
+def timeline(args, pkg, torch, np):
+    """Where a decode layer's time goes: the stage timestamps that the measurement build of the
+    library records in every wavefront (csrc/timeline.h), read after HIP-graph replays of the
+    default workload's step and printed as a table, times in ns from the attention kernel's
+    first wavefront's first instruction. The layer shown is the last of the 48."""
+    import ctypes as C
+
+    lib_path = os.path.join(os.path.dirname(pkg._native.LIB_PATH), "libitak_hip_kv_timeline.so")
+    if not os.path.exists(lib_path):
+        print("bench.py --timeline needs the measurement build: run "
+              "`python itak-torch-rebuild_amd/build.py --timeline` first", file=sys.stderr)
+        sys.exit(2)
+    pkg._native.LIB_PATH = lib_path
+    pkg._native.load()
+    raw = C.CDLL(lib_path)
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream()
+    layers, ctx = 48, 4096
+    pool = pkg.KvPool(layers, KV_HEADS, D, elem="f16", max_slots=1, capacity_rows=ctx + 8,
+                      scrub_on_truncate=False, merge_in_launch=args.merge_in_launch)
+    pool.set_stream(stream.cuda_stream)
+    cache = pool.acquire()
+    torch.manual_seed(0)
+    for layer in range(layers):
+        k = rope_on_device(torch.randn(ctx, KV_HEADS, D, device=dev), 1e6).reshape(ctx, ROW).contiguous()
+        v = torch.randn(ctx, ROW, device=dev)
+        pool.append_device(layer, [(cache, ctx)], k.data_ptr(), v.data_ptr())
+        torch.cuda.synchronize()
+    q = torch.randn(layers, 1, Q_HEADS * D, device=dev)
+    k_new, v_new = torch.randn(layers, 1, ROW, device=dev), torch.randn(layers, 1, ROW, device=dev)
+    out = torch.empty_like(q)
+
+    def step():
+        for layer in range(layers):
+            pool.attention_step_device(layer, [(cache, 1)], q[layer].data_ptr(), k_new[layer].data_ptr(),
+                                       v_new[layer].data_ptr(), out[layer].data_ptr(), Q_HEADS,
+                                       softcap=args.softcap)
+        pool.truncate([cache], [ctx])
+
+    for _ in range(3):
+        step()
+    graph = capture(torch, pool, stream, step)
+    marks, waves = 12, 8192
+    buf = np.zeros(waves * marks, dtype=np.uint64)
+    decode_rows, merge_rows = [], []
+    for _ in range(max(args.steps // 10, 8)):
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = None
+        for reader, second_half in (("itak_timeline_read_decode", False), ("itak_timeline_read_splitk", True)):
+            rc = getattr(raw, reader)(buf.ctypes.data_as(C.c_void_p), C.c_ulonglong(buf.size))
+            assert rc == 0, f"{reader} failed with HIP error {rc}"
+            t = buf.reshape(waves, marks).astype(np.int64)
+            t = t[waves // 2:] if second_half else t[:waves // 2]
+            t = t[t[:, 0] > 0]
+            if not second_half:
+                if len(t) == 0:
+                    print("no decode kernel records: the step did not take attn_decode_f16_kernel",
+                          file=sys.stderr)
+                    sys.exit(1)
+                t0 = t[:, 0].min()
+                decode_rows.append((t - t0) * 10)
+            elif len(t):
+                merge_rows.append((t - t0) * 10)
+    step_s = Timer(torch, stream)(graph.replay, 50)[0] / 50
+
+    def table(title, rows, names):
+        print(title)
+        allr = np.concatenate(rows)
+        for i, name in names:
+            col = allr[:, i]
+            col = col[col > -10**9]
+            if len(col) == 0 or col.max() <= 0 and i:
+                continue
+            print(f"  {name:44s} min {col.min():6d}  p50 {int(np.median(col)):6d}  "
+                  f"p90 {int(np.percentile(col, 90)):6d}  max {col.max():6d} ns")
+
+    print(f"decode layer timeline: batch 1, context {ctx}, 48 layers as one HIP graph, "
+          f"{'splits merged inside the launch' if args.merge_in_launch else 'merge launch'}; "
+          f"{step_s / layers * 1e6:.2f} us per layer with the timestamps compiled in")
+    table(f"attn_decode_f16_kernel ({decode_rows[0].shape[0]} wavefronts per launch)", decode_rows, [
+        (0, "first instruction"), (1, "kernel arguments in, addresses known"),
+        (2, "every load issued"), (3, "scores done (keys and queries arrived)"),
+        (4, "O^T written to LDS (values arrived)"), (5, "past the workgroup barrier"),
+        (6, "partials / exchange words issued"), (7, "every exchange word gathered"),
+        (11, "everything in flight done (stores acknowledged)")])
+    if merge_rows:
+        table(f"attn_combine128_kernel ({merge_rows[0].shape[0]} wavefronts per launch)", merge_rows, [
+            (0, "first instruction"), (1, "kernel arguments in, addresses known"),
+            (2, "every load issued"), (7, "sums done (partials arrived)"),
+            (8, "past the workgroup barrier"), (9, "output issued"),
+            (11, "everything in flight done (stores acknowledged)")])
+    pool.close()
+
+
 class Timer:
     def __init__(self, torch, stream):
         self.torch, self.stream = torch, stream
@@ -294,10 +411,20 @@ def main():
     ap.add_argument("--prep", action="store_true",
                     help="also time the step with the fused Q/K preparation (per-head RMSNorm + "
                          "RoPE) before it and the sigmoid gate after it, reported as 'with_prep'")
+    ap.add_argument("--timeline", action="store_true",
+                    help="print where a decode layer's time goes: stage timestamps from the "
+                         "measurement build of the library (python itak-torch-rebuild_amd/build.py "
+                         "--timeline), a table instead of the JSON line")
+    ap.add_argument("--only", action="store_true",
+                    help="measure the named workload alone (the default decode run otherwise "
+                         "adds short runs of the other configurations under 'workloads')")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)",
               file=sys.stderr)
+        sys.exit(2)
+    if args.kv == "f32" and args.workload not in ("decode", "ragged"):
+        print("--kv f32 is measured on the decode and ragged workloads only", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
@@ -306,21 +433,54 @@ def main():
     from __graft_entry__ import load_package
 
     pkg = load_package()
+    if args.timeline:
+        timeline(args, pkg, torch, np)
+        return
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
     stream = torch.cuda.current_stream()
     timed = Timer(torch, stream)
 
+    result = run_workload(args, pkg, torch, np, dev, stream, timed)
+    primary = (args.workload == "decode" and args.kv == "f16" and args.softcap == 0.0
+               and not args.only and not args.merge_in_launch)
+    if primary:
+        # The other configurations in short runs of their own, so that one line carries every
+        # kernel's figure; `metric`, `value` and `config` stay those of the decode step.
+        import copy
+        workloads = {"decode": summary_of(result)}
+        for wl in ("ragged", "verify", "prefill", "restore"):
+            sub = copy.copy(args)
+            sub.workload, sub.no_cpu_baseline, sub.prep = wl, True, False
+            sub.steps, sub.warmup = max(10, args.steps // 4), max(3, args.warmup // 4)
+            try:
+                torch.cuda.empty_cache()
+                workloads[wl] = summary_of(run_workload(sub, pkg, torch, np, dev, stream, timed))
+            except Exception as e:  # a secondary figure must not take the contract line down
+                workloads[wl] = {"error": f"{type(e).__name__}: {e}"}
+        result["workloads"] = workloads
+    print(json.dumps(result))
+
+
+def summary_of(result):
+    """The few figures of a workload's result that the one-line summary carries."""
+    r = result["roofline"]
+    out = {"metric": result["metric"], "value": result["value"], "unit": result["unit"],
+           "ms_per_step": result["ms_per_step"], "bound": r["bound"], "frac": r["frac"],
+           "us_per_launch": r.get("us_per_launch"), "kernel": r.get("kernel")}
+    if "step_frac" in r:
+        out["step_frac"] = r["step_frac"]
+    return out
+
+
+def run_workload(args, pkg, torch, np, dev, stream, timed):
+    """Measures one workload and returns its JSON object."""
     # ---- workload shapes -------------------------------------------------------------
     wl = args.workload
-    if args.kv == "f32" and wl not in ("decode", "ragged"):
-        print("--kv f32 is measured on the decode and ragged workloads only", file=sys.stderr)
-        sys.exit(2)
     elem_bytes = 4 if args.kv == "f32" else 2
     if wl in ("restore", "append"):
-        print(json.dumps(cache_maintenance(args, pkg, torch, dev, stream, timed)))
-        return
+        return cache_maintenance(args, pkg, torch, dev, stream, timed)
     if wl == "decode":
         layers, slots, rows, lengths = 48, 1, 1, [4096]
         name = ("configs[1]: 30B-class decode step, batch 1, 48 layers, 32 Q / 4 KV heads, "
@@ -530,9 +690,14 @@ def main():
             "peak": MFMA_F16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(flops_layer / attn_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-            "traffic": MEASURED_TRAFFIC.get(wl),
+            "traffic": PROFILE_TRAFFIC.get((wl, args.kv), (None, None))[0],
+            "traffic_source": PROFILE_TRAFFIC.get((wl, args.kv), (None, None))[1],
             "us_per_launch": round(attn_s * 1e6, 2),
             "flops_per_launch": flops_layer,
+            # The same over the whole timed step (the chunk's append launches included).
+            "step_frac": round(value / MFMA_F16_PEAK_TFLOPS, 4),
+            "timed": "the attention launch of a layer, event-timed in a graph of its own on a "
+                     "cache that already holds the chunk",
         }
     else:
         metric, unit = "decode-attn KV GB/s (all layers, ctx 4096)", "GB/s"
@@ -541,17 +706,27 @@ def main():
         if args.kv == "f32":
             metric += " on an f32 cache"
         value = kv_bytes_layer * layers / step_s / 1e9
+        # The layer's launches as the timed step runs them (fused append + attention, then the
+        # merge): achieved = algorithmic KV bytes of a layer / the step's time per layer.
+        layer_s = step_s / layers
+        lean = args.kv == "f16" and rows == 1 and wl in ("decode", "hybrid")
         roofline = {
             "bound": "hbm",
-            "kernel": f"attn_splitk_{args.kv}_kernel + attn_combine128_kernel (the two launches "
-                      "of one layer's attention)",
-            "achieved": round(kv_bytes_layer / attn_s / 1e9, 2),
+            "kernel": (("attn_decode_f16_kernel" if lean else f"attn_splitk_{args.kv}_kernel") +
+                       (" (splits merged inside the launch)" if args.merge_in_launch else
+                        " + attn_combine128_kernel (the two launches of one layer's attention)")),
+            "achieved": round(kv_bytes_layer / layer_s / 1e9, 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(kv_bytes_layer / attn_s / 1e9 / HBM_PEAK_GBS, 4),
-            "traffic": (MEASURED_TRAFFIC if args.kv == "f16" else MEASURED_TRAFFIC_F32).get(wl),
-            "us_per_launch": round(attn_s * 1e6, 3),
+            "frac": round(kv_bytes_layer / layer_s / 1e9 / HBM_PEAK_GBS, 4),
+            "traffic": PROFILE_TRAFFIC.get((wl, args.kv), (None, None))[0],
+            "traffic_source": PROFILE_TRAFFIC.get((wl, args.kv), (None, None))[1],
+            "us_per_launch": round(layer_s * 1e6, 3),
             "bytes_per_launch": kv_bytes_layer,
+            "timed": "one layer of the timed step (HIP graph replay of all layers), HIP events on "
+                     "the stream the kernels run on",
+            # The attention launches alone, on a cache that already holds the new rows.
+            "attention_only_us_per_launch": round(attn_s * 1e6, 3),
         }
 
     result = {
@@ -592,8 +767,8 @@ def main():
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(4096, 2 * 4097 * KV_HEADS * D * elem_bytes, 48,
                                               store_f16=args.kv == "f16")
-    print(json.dumps(result))
     pool.close()
+    return result
 
 
 if __name__ == "__main__":

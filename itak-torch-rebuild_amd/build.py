@@ -14,6 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libitak_hip_kv.so")
+TIMELINE_LIB_PATH = os.path.join(LIB_DIR, "libitak_hip_kv_timeline.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
 ARCH = "gfx950"
@@ -31,9 +32,10 @@ def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
-def _compile(src: str) -> str:
-    obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
-    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(src: str, timeline: bool = False) -> str:
+    obj = os.path.join(OBJ_DIR + ("_timeline" if timeline else ""), src.replace(".hip", ".o"))
+    cmd = [HIPCC, *FLAGS, *(["-DITAK_TIMELINE"] if timeline else []), "-c",
+           os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     lines = [l for l in res.stderr.splitlines() if noise not in l]
@@ -56,20 +58,25 @@ def _compile(src: str) -> str:
     return obj
 
 
-def build(verbose: bool = False) -> str:
-    os.makedirs(OBJ_DIR, exist_ok=True)
+def build(verbose: bool = False, timeline: bool = False) -> str:
+    """Builds lib/libitak_hip_kv.so; with `timeline`, lib/libitak_hip_kv_timeline.so instead: the
+    same library with stage timestamps compiled into the attention kernels (csrc/timeline.h),
+    which `bench.py --timeline` loads. The measurement build is never the one tests or
+    benchmarks of throughput run."""
+    os.makedirs(OBJ_DIR + ("_timeline" if timeline else ""), exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
     srcs = sources()
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
-        objs = list(pool.map(_compile, srcs))
-    cmd = [HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-pthread", "-o", LIB_PATH, *objs]
+        objs = list(pool.map(lambda src: _compile(src, timeline), srcs))
+    lib_path = TIMELINE_LIB_PATH if timeline else LIB_PATH
+    cmd = [HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-pthread", "-o", lib_path, *objs]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stderr}")
     if verbose:
-        print(f"built {LIB_PATH}")
-    return LIB_PATH
+        print(f"built {lib_path}")
+    return lib_path
 
 
 if __name__ == "__main__":
-    build(verbose=True)
+    build(verbose=True, timeline="--timeline" in sys.argv[1:])

@@ -26,14 +26,16 @@
 #include "internal.h"
 #include "mfma_common.h"
 #include "split_exchange.h"
+#include "timeline.h"
 
 #include <math.h>
 
-#ifndef ITAK_MARK
-#define ITAK_MARK_BEGIN
-#define ITAK_MARK(i)
-#define ITAK_MARK_END
-#endif
+
+// Timeline marks of attn_decode_f16_kernel: 0 first instruction, 1 addresses known (the kernel
+// arguments have arrived), 2 every load issued, 3 scores done (keys and queries have arrived),
+// 4 O^T written to LDS (values have arrived), 5 past the barrier, 6 partials or exchange words
+// issued, 7 every exchange word gathered (in-launch merge only), 11 everything in flight done.
+ITAK_TIMELINE_READER(itak_timeline_read_decode)
 
 namespace itak {
 
@@ -328,6 +330,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
                 *reinterpret_cast<float2 *>(p.ws + uint64_t(total_partials) * kD + uint64_t(ps) * 2) =
                     make_float2(M, L);
         }
+        ITAK_MARK(6)
         ITAK_MARK_END
         return;
     }
@@ -338,8 +341,12 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
         xg.publish(jl, wave * 2 + 1, g, acc[1], M, L);
     }
     ITAK_MARK(6)
+    unsigned long long gathered_at = 0;
     xg.template finish<kWaves * 64, kDecodeWords, kDecodeLooks>(reinterpret_cast<unsigned long long *>(sm_o), p, item, kv_head, group,
-                                    p.group_magic, nullptr);
+                                    p.group_magic, nullptr, &gathered_at);
+#ifdef ITAK_TIMELINE
+    tm_[7] = gathered_at;
+#endif
     ITAK_MARK_END
 }
 

@@ -241,9 +241,6 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                         for (int k = 0; k < 4; ++k)
                             s = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[t][k], qb[qt][k], s, 0, 0, 0);
                         x[qt][t] = s;
-#ifdef ITAK_CHAIN
-                        __builtin_amdgcn_sched_barrier(0x7f6);  // MFMAs keep their order: chains stay whole
-#endif
                     }
             }
             half8 va[8];

@@ -26,19 +26,18 @@
 #include "internal.h"
 #include "mfma_common.h"
 #include "split_exchange.h"
+#include "timeline.h"
 
 #include <math.h>
 
 #include <algorithm>
 
-// Timeline hooks: a measurement build may pre-define these to record timestamps at the
-// numbered points; the library build compiles them to nothing.
-#ifndef ITAK_MARK
-#define ITAK_MARK_BEGIN
-#define ITAK_MARK(i)
-#define ITAK_MARK_END
-#define ITAK_MARK_END2
-#endif
+// Timeline marks (timeline.h). Split-K kernel: 0 first instruction, 1 addresses known, 2 loads
+// issued, 3 bookkeeping done, 4 Q staged, 5 past the barrier, 6 blocks done, 7 O^T in LDS, 8 past
+// the barrier, 9 partials issued, 11 all done. Merge kernel (records in the buffer's second
+// half): 0 first instruction, 1 addresses known, 2 loads issued, 7 sums done, 8 past the
+// barrier, 9 output issued, 11 all done.
+ITAK_TIMELINE_READER(itak_timeline_read_splitk)
 
 namespace itak {
 
@@ -1161,7 +1160,7 @@ __device__ __forceinline__ void attn_combine128_body(const AttnParams &p, const 
         *reinterpret_cast<float4 *>(dst + tid * 4) = o;
     }
     ITAK_MARK(9)
-    ITAK_MARK_END2
+    ITAK_MARK_END_AT(ITAK_TIMELINE_WAVES / 2)
 }
 template <int N, bool BASE2>
 __global__ __launch_bounds__(256) void attn_combine128_kernel(AttnParams p, AttnBatchT<N> b,

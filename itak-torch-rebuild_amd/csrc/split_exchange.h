@@ -114,7 +114,8 @@ struct ExchangeGroup {
     template <uint32_t T, int NW, int DEPTH>
     __device__ __forceinline__ void finish(unsigned long long *sm_x, const AttnParams &p,
                                            const AttnItem &item, uint32_t kv_head, uint32_t group,
-                                           uint32_t group_magic, const float *gate) const {
+                                           uint32_t group_magic, const float *gate,
+                                           unsigned long long *gathered_at = nullptr) const {
         const uint32_t tid = threadIdx.x;
         const uint32_t S = splits;
         const uint32_t n_my = split < slices ? __umulhi(slices - split + S - 1, magic) : 0;
@@ -168,6 +169,7 @@ struct ExchangeGroup {
                 }
             }
         }
+        if (gathered_at) *gathered_at = wall_clock64();  // the timeline build's mark
         // The wavefronts are done with their own merge: its LDS now takes the gathered words.
         // What was read is given back to the buffer as empty at once, so that those stores are
         // under way while the slices are summed.
