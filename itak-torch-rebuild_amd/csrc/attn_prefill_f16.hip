@@ -35,8 +35,14 @@
 // position pos0 + r and sees keys <= its position (attention.rs:77-85 with no window).
 #include "internal.h"
 #include "mfma_common.h"
+#include "timeline.h"
 
 #include <algorithm>
+
+// Timeline marks of attn_prefill_f16_kernel: 0 first instruction, 1 addresses known, 2 first
+// blocks and Q requested, 3 Q converted (it has arrived), 4 first block multiplied, 5 last block
+// multiplied, 6 output or partials issued, 11 all done.
+ITAK_TIMELINE_READER(itak_timeline_read_prefill)
 
 namespace itak {
 
@@ -53,11 +59,12 @@ __device__ __forceinline__ float column_max4(float v) {
     const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
     return fmaxf(__uint_as_float(c[0]), __uint_as_float(c[1]));
 }
-__device__ __forceinline__ float column_sum4(float v) {
-    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
-    const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return __uint_as_float(c[0]) + __uint_as_float(c[1]);
+// The largest of three, none of them a signalling NaN (scores and -inf): one instruction, no
+// quieting of the inputs.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
 }
 
 // The direct-to-LDS load is issued from inline assembly: the compiler then neither tracks it
@@ -92,6 +99,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     const uint32_t tid = threadIdx.x;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const uint32_t g = lane >> 4, jl = lane & 15;
+    ITAK_MARK_BEGIN
+    ITAK_MARK(0)
 
     const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
     const uint32_t group = p.group;
@@ -163,48 +172,92 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
         lds_dma16(vg + off + 256, dst + 12288);
     };
     const bool any_block = kb_begin < nblocks;  // a split past the rows' horizon has none
-    if (any_block) {
-#pragma unroll
-        for (int ahead = 0; ahead < STAGES - 1; ++ahead) issue_block(kb_begin + ahead);
-    }
+    ITAK_MARK(1)
 
+    // With a softcap the score MFMA yields the argument of tanh's exponential directly
+    // (2 * log2(e) * s / cap): one multiply less on every score.
     const float softcap = p.softcap;
-    const float inv_cap = SOFTCAP ? 1.0f / softcap : 0.0f;
-    const float qscale = SOFTCAP ? p.scale : p.scale * kLog2e;
+    const float cap2 = SOFTCAP ? softcap * kLog2e : 0.0f;
+    const float qscale = SOFTCAP ? p.scale * (2.0f * kLog2e / softcap) : p.scale * kLog2e;
+    // Q^T of the wavefront's vectors. The Q loads go out first, the ring is filled behind them,
+    // and Q is converted as soon as it is in: loads return in order, so Q is not held up by
+    // three to seven blocks of keys and values, which a short run of blocks could not hide.
+    // The compiler cannot count the ring's loads (they are issued from assembly), so it would
+    // wait for everything before the first use of Q: the Q loads are issued from assembly too
+    // and waited for by count. Rows past the block's end re-read its last row and are scaled
+    // to zero columns (no branch around a load).
     half8 qb[kTiles][4];
     uint32_t colpos[kTiles], collo[kTiles];
+    {
+        floatx4 qraw[kTiles][8];
 #pragma unroll
-    for (int qt = 0; qt < kTiles; ++qt) {
-        const uint32_t j = qt * 16 + jl;
-        const uint32_t row = row_begin + j / group;
-        colpos[qt] = min(item.pos0 + row, item.kv_len - 1);
-        collo[qt] = lowest_visible(item.pos0 + row, window, kv_lo);
-        if (row < item.rows) {
+        for (int qt = 0; qt < kTiles; ++qt) {
+            const uint32_t j = qt * 16 + jl;
+            const uint32_t row = row_begin + j / group;
+            colpos[qt] = min(item.pos0 + row, item.kv_len - 1);
+            collo[qt] = lowest_visible(item.pos0 + row, window, kv_lo);
             const uint32_t head = kv_head * group + j % group;
-            const float *qp = p.q + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + g * 8;
+            const float *qp =
+                p.q + (uint64_t(item.q_row0 + min(row, item.rows - 1)) * p.q_heads + head) * kD + g * 8;
+#pragma unroll
+            for (int s = 0; s < 8; ++s)
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qraw[qt][s]) : "v"(qp + (s >> 1) * 32 + (s & 1) * 4) : "memory");
+        }
+        if (any_block) {
+#pragma unroll
+            for (int ahead = 0; ahead < STAGES - 1; ++ahead) issue_block(kb_begin + ahead);
+        }
+        ITAK_MARK(2)
+        // Everything older than the ring's loads has landed: that is Q. A workgroup without
+        // blocks issued no ring loads, so there the count to wait for is zero: a Q load still in
+        // flight would land in a register the compiler has meanwhile given to something else
+        // (an address of the epilogue's stores, for one).
+#define ITAK_Q_REGS(qt)                                                                         \
+    "+v"(qraw[qt][0]), "+v"(qraw[qt][1]), "+v"(qraw[qt][2]), "+v"(qraw[qt][3]), "+v"(qraw[qt][4]), \
+        "+v"(qraw[qt][5]), "+v"(qraw[qt][6]), "+v"(qraw[qt][7])
+        if (any_block) {
+            if constexpr (kTiles == 2)
+                asm volatile("s_waitcnt vmcnt(%16)" : ITAK_Q_REGS(0), ITAK_Q_REGS(1) : "n"(4 * (STAGES - 1)) : "memory");
+            else
+                asm volatile("s_waitcnt vmcnt(%8)" : ITAK_Q_REGS(0) : "n"(4 * (STAGES - 1)) : "memory");
+        } else {
+            if constexpr (kTiles == 2)
+                asm volatile("s_waitcnt vmcnt(0)" : ITAK_Q_REGS(0), ITAK_Q_REGS(1) : : "memory");
+            else
+                asm volatile("s_waitcnt vmcnt(0)" : ITAK_Q_REGS(0) : : "memory");
+        }
+#undef ITAK_Q_REGS
+#pragma unroll
+        for (int qt = 0; qt < kTiles; ++qt) {
+            const uint32_t row = row_begin + (qt * 16 + jl) / group;
+            const float sc = row < item.rows ? qscale : 0.0f;
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-                const float4 a = *reinterpret_cast<const float4 *>(qp + s * 32);
-                const float4 c = *reinterpret_cast<const float4 *>(qp + s * 32 + 4);
-                qb[qt][s] = half8{static_cast<_Float16>(a.x * qscale), static_cast<_Float16>(a.y * qscale),
-                                  static_cast<_Float16>(a.z * qscale), static_cast<_Float16>(a.w * qscale),
-                                  static_cast<_Float16>(c.x * qscale), static_cast<_Float16>(c.y * qscale),
-                                  static_cast<_Float16>(c.z * qscale), static_cast<_Float16>(c.w * qscale)};
+                const floatx4 a = qraw[qt][2 * s], c = qraw[qt][2 * s + 1];
+                qb[qt][s] = half8{static_cast<_Float16>(a[0] * sc), static_cast<_Float16>(a[1] * sc),
+                                  static_cast<_Float16>(a[2] * sc), static_cast<_Float16>(a[3] * sc),
+                                  static_cast<_Float16>(c[0] * sc), static_cast<_Float16>(c[1] * sc),
+                                  static_cast<_Float16>(c[2] * sc), static_cast<_Float16>(c[3] * sc)};
             }
-        } else {
-#pragma unroll
-            for (int s = 0; s < 4; ++s) qb[qt][s] = half8{0, 0, 0, 0, 0, 0, 0, 0};
         }
     }
-
-    float ref[kTiles], thr[kTiles], l[kTiles];
+    ITAK_MARK(3)
+    // The denominator goes through the matrix pipe: one more MFMA per tile and block with an
+    // all-ones A operand leaves the block's sum of P (as rounded for P.V, over all 32 keys) in
+    // every row of a 16x16 accumulator. That replaces eight additions per tile and block, and
+    // ordinary vector instructions are what this loop runs out of (they do not overlap with a
+    // SIMD's MFMAs; the extra MFMA costs a quarter of the additions' issue time).
+    float ref[kTiles], thr[kTiles];
+    floatx4 l[kTiles];
     floatx4 negref[kTiles];
+    const half8 ones = {_Float16(1.0f), _Float16(1.0f), _Float16(1.0f), _Float16(1.0f),
+                        _Float16(1.0f), _Float16(1.0f), _Float16(1.0f), _Float16(1.0f)};
     floatx4 o[kTiles][8];
 #pragma unroll
     for (int qt = 0; qt < kTiles; ++qt) {
         ref[qt] = 0.0f;
         thr[qt] = -INFINITY;
-        l[qt] = 0.0f;
+        l[qt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
         negref[qt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt) o[qt][dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -223,6 +276,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
         if (kb < wave_blocks && (!RING || kb >= wave_first)) {
             const uint32_t key_base = kb * kBlockKeys + g * 8;
             floatx4 x[kTiles][2];
+            __builtin_amdgcn_s_setprio(0);  // raised again below, for the block's second half
             {
                 half8 ka[2][4];
                 const uint16_t *kl = lds_k + (g * 16 + jl) * 8;
@@ -254,8 +308,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                 for (int qt = 0; qt < kTiles; ++qt)
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
-                        x[qt][e >> 2][e & 3] =
-                            softcap_log2(x[qt][e >> 2][e & 3], softcap, inv_cap, ref[qt]);
+                        x[qt][e >> 2][e & 3] = softcap_of_exp2_arg(x[qt][e >> 2][e & 3], cap2, ref[qt]);
             }
             if (RING && kb < low_masked_end) {
 #pragma unroll
@@ -291,10 +344,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
             bool over = false;
 #pragma unroll
             for (int qt = 0; qt < kTiles; ++qt) {
-                float mx = fmaxf(fmaxf(x[qt][0][0], x[qt][0][1]), x[qt][0][2]);
-                mx = fmaxf(fmaxf(mx, x[qt][0][3]), x[qt][1][0]);
-                mx = fmaxf(fmaxf(mx, x[qt][1][1]), x[qt][1][2]);
-                lmax[qt] = fmaxf(mx, x[qt][1][3]);
+                float mx = max3(x[qt][0][0], x[qt][0][1], x[qt][0][2]);
+                mx = max3(mx, x[qt][0][3], x[qt][1][0]);
+                mx = max3(mx, x[qt][1][1], x[qt][1][2]);
+                lmax[qt] = max3(mx, x[qt][1][3], x[qt][1][3]);
                 over = over || lmax[qt] > thr[qt];
             }
             if (__builtin_amdgcn_ballot_w64(over) != 0) {
@@ -321,6 +374,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                     }
                 }
             }
+            // From here to the block's last MFMA this wavefront goes first when the SIMD picks
+            // an instruction: the exponentials and P.V of the wavefront that is ahead then do
+            // not wait behind the score MFMAs of the one that shares its SIMD, which keeps the
+            // two half a block apart (one in the matrix pipe, one in vector work) instead of
+            // drifting into step (measured on the 2048-row chunk: +4.5 %; the other placements
+            // of the raised stretch tried, scores only or masks and maxima only, gave +3 %).
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int qt = 0; qt < kTiles; ++qt) {
                 float pe[8];
@@ -329,14 +389,15 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                 half8 pb;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) pb[e] = static_cast<_Float16>(pe[e]);
-                l[qt] += ((pe[0] + pe[1]) + (pe[2] + pe[3])) + ((pe[4] + pe[5]) + (pe[6] + pe[7]));
+                l[qt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pb, l[qt], 0, 0, 0);
 #pragma unroll
                 for (int dt = 0; dt < 8; ++dt)
                     o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[dt], pb, o[qt][dt], 0, 0, 0);
             }
         }
-
+        if (kb == kb_begin) { ITAK_MARK(4) }
     }
+    ITAK_MARK(5)
     if (any_block) wait_vmcnt<0>();  // the surplus loads of the last iterations
 
     // One split: the normalised output. Several: the partial (m, l, acc[128]) of this split
@@ -347,7 +408,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     float *const ws_ml = p.ws + uint64_t(total_partials) * kD;
 #pragma unroll
     for (int qt = 0; qt < kTiles; ++qt) {
-        const float lt = column_sum4(l[qt]);
+        const float lt = l[qt][0];
         const uint32_t j = qt * 16 + jl;
         const uint32_t row = row_begin + j / group, head = kv_head * group + j % group;
         if (row >= item.rows) continue;
@@ -367,6 +428,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                     make_float2(thr[qt] == -INFINITY ? -INFINITY : ref[qt], lt);
         }
     }
+    ITAK_MARK(6)
+    ITAK_MARK_END
 }
 
 }  // namespace
@@ -378,11 +441,12 @@ bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group) {
 
 // Up to 64 query vectors per KV head (speculative blocks) take one 16-vector tile per
 // wavefront, so that all four wavefronts of the workgroup have columns; more take two.
-// So do blocks of up to 256 vectors over at most 256 key blocks (a draft tree of 16 to 32
-// tokens at a context up to 8192): the launch has to split the context anyway, and with
-// twice the row tiles it needs half the splits, half the partials to write and merge
-// (measured at context 4096: 16 rows 20.6 -> 17.7 us, 32 rows 24.0 -> 21.2 us; at context
-// 30720 the second pass over the keys costs more than the partials saved).
+// So do blocks of up to 512 vectors over at most 256 key blocks (a draft tree of 16 to 32
+// tokens, or a 64-row chunk, at a context up to 8192): the launch has to split the context
+// anyway, and with twice the row tiles it needs half the splits, half the partials to write
+// and merge (measured at context 4096: 16 rows 20.6 -> 17.7 us, 32 rows 24.0 -> 21.2 us,
+// 64 rows 25.1 -> 23.7 us; at context 30720 the second pass over the keys costs more than
+// the partials saved).
 static int tiles_for(const AttnBatch &b, uint32_t group) {
     uint32_t nvec = 0, nblocks = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
@@ -390,7 +454,7 @@ static int tiles_for(const AttnBatch &b, uint32_t group) {
         nblocks = std::max(nblocks, item_block_count(b.item[i]));
     }
     if (nvec <= uint32_t(kWaves * 16)) return 1;
-    return nvec <= 256 && nblocks <= 256 ? 1 : kMaxTiles;
+    return nvec <= 512 && nblocks <= 256 ? 1 : kMaxTiles;
 }
 
 // Fills splits / keys_per_split / block0 / ws0 for a batch (slot, rows, pos0, q_row0, kv_len

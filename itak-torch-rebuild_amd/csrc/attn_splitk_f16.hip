@@ -1175,11 +1175,98 @@ __global__ __launch_bounds__(256) void attn_combine128_gate_kernel(AttnParams p,
     attn_combine128_body<N, BASE2, true>(p, b, total_partials, gate);
 }
 
+// The same merge for items of at most 16 splits, one wavefront per (row, Q head): lane =
+// (4 channels c, split lane sl of 2), every load of the wavefront's 16 splits issued at once,
+// the two split lanes joined by a half-wave swap. A workgroup is four such wavefronts (four
+// heads of one row) that never meet: no LDS, no barrier, and a quarter of the wavefronts of the
+// form above, whose launch of a few microseconds is mostly wavefront dispatch once a block of
+// several rows has hundreds of (row, head) pairs to merge.
+__device__ __forceinline__ float half_max(float v) {
+    const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(c[0]), __uint_as_float(c[1]));
+}
+__device__ __forceinline__ float half_sum(float v) {
+    const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(c[0]) + __uint_as_float(c[1]);
+}
+template <int N, bool BASE2, bool GATE>
+__global__ __launch_bounds__(256) void attn_combine128_wave_kernel(AttnParams p, AttnBatchT<N> b,
+                                                                   uint32_t total_partials,
+                                                                   const float *gate) {
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const uint32_t head = blockIdx.x * 4 + wave, grow = blockIdx.y;
+    if (head >= p.q_heads) return;
+    const AttnItem item = b.item[b.find_by_row(grow)];
+    const uint32_t S = item.splits;
+    if (S == 1) return;
+    const uint32_t row = grow - (item.q_row0 - b.base_row);
+    const uint64_t ps0 = item.ws0 + (uint64_t(row) * p.q_heads + head) * S;
+    const uint32_t c = lane & 31, sl = lane >> 5;
+    const float *ws_acc = p.ws + ps0 * 128 + c * 4;
+    const float2 *ws_ml = reinterpret_cast<const float2 *>(p.ws + uint64_t(total_partials) * 128) + ps0;
+    const uint64_t at = (uint64_t(item.q_row0 + row) * p.q_heads + head) * 128 + c * 4;
+    [[maybe_unused]] float4 gt = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (GATE && sl == 0) gt = *reinterpret_cast<const float4 *>(gate + at);
+    float4 x[8];
+    float2 ml[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {  // clamped, so the loads need no branch
+        const uint32_t s = min(sl + u * 2, S - 1);
+        x[u] = *reinterpret_cast<const float4 *>(ws_acc + uint64_t(s) * 128);
+        ml[u] = ws_ml[s];
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        if (sl + u * 2 >= S) ml[u].x = -INFINITY;
+        mx = fmaxf(mx, ml[u].x);
+    }
+    const float M = half_max(mx);
+    float l = 0.0f;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const float w = ml[u].x == -INFINITY ? 0.0f : (BASE2 ? fast_exp2(ml[u].x - M) : __expf(ml[u].x - M));
+        l = fmaf(ml[u].y, w, l);
+        acc.x = fmaf(x[u].x, w, acc.x);
+        acc.y = fmaf(x[u].y, w, acc.y);
+        acc.z = fmaf(x[u].z, w, acc.z);
+        acc.w = fmaf(x[u].w, w, acc.w);
+    }
+    const float inv = 1.0f / half_sum(l);
+    float4 o = make_float4(half_sum(acc.x) * inv, half_sum(acc.y) * inv, half_sum(acc.z) * inv,
+                           half_sum(acc.w) * inv);
+    if (sl == 0) {
+        if (GATE)
+            o = make_float4(o.x * sigmoid_fast(gt.x), o.y * sigmoid_fast(gt.y),
+                            o.z * sigmoid_fast(gt.z), o.w * sigmoid_fast(gt.w));
+        *reinterpret_cast<float4 *>(p.out + at) = o;
+    }
+}
+
 hipError_t launch_attn_combine(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                uint32_t total_rows, int base2, hipStream_t stream, const float *gate) {
     bool any = false;
     for (uint32_t i = 0; i < b.n; ++i) any = any || b.item[i].splits > 1;
     if (!any || total_rows == 0) return hipSuccess;
+    uint32_t most_splits = 0;
+    for (uint32_t i = 0; i < b.n; ++i) most_splits = std::max(most_splits, b.item[i].splits);
+    if (p.g.head_dim == 128 && most_splits <= 16 && uint64_t(total_rows) * p.q_heads >= 128) {
+        const dim3 grid((p.q_heads + 3) / 4, total_rows);
+        if (gate && base2)
+            ITAK_DISPATCH_BATCH(b.n, (attn_combine128_wave_kernel<N, true, true><<<grid, 256, 0, stream>>>(
+                                         p, AttnBatchT<N>(b), total_partials, gate)));
+        else if (gate)
+            ITAK_DISPATCH_BATCH(b.n, (attn_combine128_wave_kernel<N, false, true><<<grid, 256, 0, stream>>>(
+                                         p, AttnBatchT<N>(b), total_partials, gate)));
+        else if (base2)
+            ITAK_DISPATCH_BATCH(b.n, (attn_combine128_wave_kernel<N, true, false><<<grid, 256, 0, stream>>>(
+                                         p, AttnBatchT<N>(b), total_partials, nullptr)));
+        else
+            ITAK_DISPATCH_BATCH(b.n, (attn_combine128_wave_kernel<N, false, false><<<grid, 256, 0, stream>>>(
+                                         p, AttnBatchT<N>(b), total_partials, nullptr)));
+        return hipGetLastError();
+    }
     if (p.g.head_dim == 128) {
         const dim3 grid(p.q_heads, total_rows);
         if (gate && base2)

@@ -39,4 +39,11 @@ __device__ __forceinline__ float softcap_log2(float x, float cap, float inv_cap,
     return __builtin_fmaf(r, -2.0f * c, c - shift);
 }
 
+// The same for a score that arrives as the exponential's argument, a = 2 * log2(e) * x / cap
+// (the factor folded into whatever scaled x), with c = cap * log2(e).
+__device__ __forceinline__ float softcap_of_exp2_arg(float a, float c, float shift) {
+    const float r = __builtin_amdgcn_rcpf(fast_exp2(a) + 1.0f);
+    return __builtin_fmaf(r, -2.0f * c, c - shift);
+}
+
 }  // namespace itak
