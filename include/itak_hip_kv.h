@@ -83,7 +83,13 @@ enum {
     ITAK_KV_IO = 35                       /* what = context, a = errno; message as std::io::Error prints it */
 };
 
-/* Storage / source element types. */
+/* Storage / source element types. An f32 pool computes in f32 throughout. An f16 pool rounds
+   the rows it stores to f16 (round to nearest even, as the reference's f16 session does) and its
+   attention kernels feed Q and the softmax weights to the matrix pipe as f16 too (scores,
+   softmax state and accumulators stay f32): outputs are within 2e-3 (max abs) of f32 arithmetic
+   over the same rounded rows as long as the scaled scores q.k*scale have a standard deviation
+   of at most about 3 (3e-5 at unit scale, 1.5e-3 at 3, above the bar from about 4.5 on). Q and K
+   normed per head, as the reference's model norms them, stay at unit scale. */
 enum { ITAK_ELEM_F32 = 0, ITAK_ELEM_F16 = 1 };
 
 /* Layer kinds (attention::LayerKind, cache.rs:36-48). */

@@ -9,7 +9,9 @@ restore_can_continue_appending / capture_refuses_a_divergent_cache /
 decode_refuses_corruption / restore_checked_refuses_geometry_and_fingerprint and the
 forged-header regressions (snapshot.rs:606-861), the sizing figures 106,496 / 272,629,760 /
 3,653,238,784 (snapshot.rs:844-861), FNV offset basis and order sensitivity
-(hash.rs:63-87), plus a hand-assembled byte string for the layout.
+(hash.rs:63-87), plus a hand-assembled byte string for the layout; prefix_discriminator by
+literals folded by hand from the alternate offset basis (the empty input, one token, two
+tokens: tests/test_oracle_snapshot.py).
 """
 from __future__ import annotations
 
