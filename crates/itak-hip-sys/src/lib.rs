@@ -262,6 +262,8 @@ extern "C" {
     pub fn itak_attention_device(pool: *mut itak_pool, layer: u64, items: *const itak_batch_item, item_count: u32, q_dev: *const f32, out_dev: *mut f32, num_q_heads: u64, scale: f32, softcap: f32) -> itak_status;
     pub fn itak_kv_append_device(pool: *mut itak_pool, layer: u64, items: *const itak_batch_item, item_count: u32, k_dev: *const f32, v_dev: *const f32) -> itak_status;
     pub fn itak_convert_f32_to_f16_device(pool: *mut itak_pool, src_dev: *const f32, dst_dev: *mut u16, count: u64) -> itak_status;
+    pub fn itak_set_debug_enabled(enabled: i32);
+    pub fn itak_debug_enabled() -> i32;
     pub fn itak_probe_copy_device(pool: *mut itak_pool, src_dev: *const c_void, dst_dev: *mut c_void, bytes: u64) -> itak_status;
     pub fn itak_probe_empty_launch(pool: *mut itak_pool) -> itak_status;
 }

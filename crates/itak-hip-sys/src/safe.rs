@@ -115,6 +115,20 @@ fn last_error(pool: *const itak_pool, code: itak_status) -> HipKvError {
     HipKvError { code, message, what, fields: [info.a, info.b, info.c, info.d] }
 }
 
+/// `attention::diag::set_debug_enabled` (`crates/attention/src/diag.rs:17-19`): one stderr line
+/// per cache and attention event and per refusal, prefixed `[itak_hip_kv::diag]`. The
+/// environment variable `ITAK_HIP_KV_DEBUG` turns the same lines on from outside.
+pub fn set_debug_enabled(enabled: bool) {
+    // SAFETY: the switch is one atomic flag of the library.
+    unsafe { itak_set_debug_enabled(i32::from(enabled)) }
+}
+
+/// `attention::diag::debug_enabled` (`diag.rs:24-33`).
+pub fn debug_enabled() -> bool {
+    // SAFETY: reads the flag and the environment.
+    unsafe { itak_debug_enabled() != 0 }
+}
+
 impl Pool {
     /// `KvCache::new` for every slot (`cache.rs:327-371`; the same zero-dimension, window and
     /// overflow refusals).

@@ -581,6 +581,17 @@ itak_status itak_kv_append_device(itak_pool *pool, uint64_t layer, const itak_ba
 itak_status itak_convert_f32_to_f16_device(itak_pool *pool, const float *src_dev,
                                            uint16_t *dst_dev, uint64_t count);
 
+/* ---- debug channel ------------------------------------------------------------------- */
+
+/* attention::diag (crates/attention/src/diag.rs:13-33,71-79): one line per cache and
+   attention event and per refusal on stderr, prefix "[itak_hip_kv::diag] ", off by default.
+   On when this switch is set or the environment holds ITAK_HIP_KV_DEBUG with a value other
+   than "0" or empty (looked up at every event, so a running process can be switched from
+   outside through its own setenv). Host code only; nothing in a kernel or a captured graph
+   changes. itak_kv_stats returns the same state without any logging. */
+void itak_set_debug_enabled(int32_t enabled);
+int32_t itak_debug_enabled(void);
+
 /* ---- measurement aids (no counterpart in the reference) ------------------------------ */
 
 /* A plain streaming copy of `bytes` (a multiple of 16) on the pool's stream: the kernel of

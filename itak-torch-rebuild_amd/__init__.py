@@ -17,6 +17,8 @@ from .hip_compute import (  # noqa: F401
     LayerKind,
     LayerStats,
     PositionCache,
+    debug_enabled,
+    set_debug_enabled,
     StepFailed,
     gqa_attention,
     kv_head_for_query_head,

@@ -134,6 +134,32 @@ struct itak_pool {
 
 namespace {
 
+// ------------------------------------------------------------------------------ debug channel
+// attention::diag (crates/attention/src/diag.rs:13-33,71-79): off by default; the switch or
+// ITAK_HIP_KV_DEBUG in the environment (any value but "0" or empty, looked up at every event as
+// the reference looks its variable up) turns one stderr line per event on.
+std::atomic<bool> g_debug_enabled{false};
+
+bool diag_enabled() {
+    if (g_debug_enabled.load(std::memory_order_relaxed)) return true;
+    const char *v = getenv("ITAK_HIP_KV_DEBUG");
+    return v && v[0] != '\0' && !(v[0] == '0' && v[1] == '\0');
+}
+
+__attribute__((format(printf, 1, 2))) void diag_emit(const char *fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    fprintf(stderr, "[itak_hip_kv::diag] %s\n", buf);
+}
+
+#define ITAK_DIAG(...)                          \
+    do {                                        \
+        if (diag_enabled()) diag_emit(__VA_ARGS__); \
+    } while (0)
+
 // ------------------------------------------------------------------------------ errors
 
 itak_status set_error(ErrorState &e, int32_t code, const char *what, uint64_t a, uint64_t b,
@@ -151,6 +177,7 @@ itak_status set_error(ErrorState &e, int32_t code, const char *what, uint64_t a,
     vsnprintf(buf, sizeof(buf), fmt, ap);
     va_end(ap);
     e.message = buf;
+    ITAK_DIAG("refused code=%d: %s", int(code), buf);  // every refusal says why
     return code;
 }
 
@@ -515,6 +542,23 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
             if (st != ITAK_OK) return st;
             ws = exchange_words ? reinterpret_cast<float *>(pool->xws) : pool->ws;
         }
+        // The reference's line (attention.rs:147-155) plus which kernel takes the launch.
+        if (diag_enabled()) {
+            uint32_t splits = 0;
+            uint64_t view_len = 0;
+            for (uint32_t i = 0; i < count; ++i) {
+                splits = std::max(splits, b.item[i].splits);
+                view_len = std::max<uint64_t>(view_len, b.item[i].kv_len - b.item[i].kv_lo);
+            }
+            diag_emit("gqa_attention layer=%llu items=%u queries=%u q_heads=%llu kv_heads=%llu "
+                      "view_len=%llu window=%u scale=%g softcap=%g kernel=%s workgroups=%u splits=%u "
+                      "fused_append=%d merge=%s",
+                      ULL(layer), count, total_rows, ULL(q_heads), ULL(pool->g.kv_heads), ULL(view_len),
+                      window, double(scale), double(softcap),
+                      mfma ? "splitk_f16" : prefill ? "prefill_f16" : f32fast ? "splitk_f32" : "generic",
+                      b.total_blocks, splits, int(k_new != nullptr && (mfma || f32fast)),
+                      partials == 0 ? "none" : exchange_words ? "in_launch" : "launch");
+        }
         AttnParams p{};
         p.layer_base = layer_base(pool, layer);
         p.g = geom;
@@ -672,7 +716,12 @@ itak_status run_append(itak_pool *pool, uint64_t layer, const itak_batch_item *i
                               v_dev + uint64_t(chunk_row0) * pool->row, pool->stream),
                 "launch append");
     }
-    for (uint32_t i = 0; i < n; ++i) advance(pool->slots[items[i].slot], layer, items[i].rows);
+    for (uint32_t i = 0; i < n; ++i) {
+        advance(pool->slots[items[i].slot], layer, items[i].rows);
+        ITAK_DIAG("append layer=%llu slot=%u rows=%u kind=%s stored=%llu", ULL(layer), items[i].slot,
+                  items[i].rows, L.windowed ? "windowed" : "global",
+                  ULL(pool->slots[items[i].slot].appended[layer]));
+    }
     return ITAK_OK;
 }
 
@@ -987,6 +1036,11 @@ itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out) {
         delete pool;
         return hip_error(e, he, "look up the static split workspace");
     }
+    ITAK_DIAG("kv pool built layers=%u kv_heads=%llu head_dim=%llu elem=%s slots=%u capacity_rows=%llu "
+              "device_bytes=%llu",
+              config->layer_count, ULL(config->num_kv_heads), ULL(config->head_dim),
+              pool->elem_f16 ? "f16" : "f32", config->max_slots, ULL(config->capacity_rows),
+              ULL(pool->bytes));
     *out = pool;
     return ITAK_OK;
 }
@@ -1312,6 +1366,9 @@ static itak_status restore_layers(itak_pool *pool, uint32_t slot, Slot &s,
         s.appended[layer] = layers[i].first_position + layers[i].rows;  // cache.rs:568
         s.high[layer] = s.appended[layer];
         s.floor[layer] = layers[i].first_position;
+        ITAK_DIAG("bulk restore slot=%u layer=%llu first_position=%llu rows=%llu appended=%llu", slot,
+                  ULL(layer), ULL(layers[i].first_position), ULL(layers[i].rows),
+                  ULL(s.appended[layer]));
     }
     return ITAK_OK;
 }
@@ -1733,6 +1790,8 @@ itak_status itak_kv_checkpoint(itak_pool *pool, uint32_t slot, uint64_t max_roun
     // What the reference's snapshot of the evictable ring slots would hold (cache.rs:678-697):
     // reported for accounting; the device saves nothing, the rows stay in the ring's headroom.
     out->saved_bytes = windowed * max_round_tokens * 2 * pool->row * 4;
+    ITAK_DIAG("checkpoint slot=%u serial=%llu max_round_tokens=%llu saved_bytes=%llu", slot,
+              ULL(out->serial), ULL(max_round_tokens), ULL(out->saved_bytes));
     return ITAK_OK;
 }
 
@@ -1827,6 +1886,7 @@ itak_status itak_kv_rewind_to(itak_pool *pool, uint32_t slot, const itak_checkpo
     }
     st = check_ring_rewind(pool, *s, target);
     if (st != ITAK_OK) return st;
+    ITAK_DIAG("rewind slot=%u serial=%llu target=%llu", slot, ULL(cp->serial), ULL(target));
     return truncate_slots(pool, &slot, &target, 1);
 }
 
@@ -1837,6 +1897,7 @@ itak_status itak_kv_release(itak_pool *pool, uint32_t slot, const itak_checkpoin
     itak_status st = live_data(pool, *s, cp);
     if (st != ITAK_OK) return st;
     s->cp.live = false;  // cache.rs:824-833
+    ITAK_DIAG("release slot=%u serial=%llu", slot, ULL(cp->serial));
     return ITAK_OK;
 }
 
@@ -1855,6 +1916,8 @@ itak_status itak_kv_truncate(itak_pool *pool, const uint32_t *slots, const uint6
         itak_status st = check_ring_rewind(pool, *s, new_lengths[i]);
         if (st != ITAK_OK) return st;
     }
+    for (uint32_t i = 0; i < count; ++i)
+        ITAK_DIAG("truncate slot=%u new_length=%llu", slots[i], ULL(new_lengths[i]));
     return truncate_slots(pool, slots, new_lengths, count);
 }
 
@@ -2433,6 +2496,11 @@ itak_status itak_probe_copy_device(itak_pool *pool, const void *src_dev, void *d
     HIP_TRY(pool, launch_probe_copy(src_dev, dst_dev, bytes, pool->stream), "launch probe copy");
     return ITAK_OK;
 }
+
+void itak_set_debug_enabled(int32_t enabled) {
+    g_debug_enabled.store(enabled != 0, std::memory_order_relaxed);
+}
+int32_t itak_debug_enabled(void) { return diag_enabled() ? 1 : 0; }
 
 itak_status itak_probe_empty_launch(itak_pool *pool) {
     if (!pool) return ITAK_INVALID_ARGUMENT;

@@ -167,6 +167,18 @@ class LayerStats:
 
 # ------------------------------------------------------------------------------ pool
 
+def set_debug_enabled(enabled: bool) -> None:
+    """attention::diag::set_debug_enabled (crates/attention/src/diag.rs:17-19): one stderr line,
+    prefixed `[itak_hip_kv::diag]`, per cache and attention event and per refusal; the
+    environment variable ITAK_HIP_KV_DEBUG turns the same lines on from outside."""
+    N.load().itak_set_debug_enabled(1 if enabled else 0)
+
+
+def debug_enabled() -> bool:
+    """attention::diag::debug_enabled (diag.rs:24-33): the switch or the environment variable."""
+    return bool(N.load().itak_debug_enabled())
+
+
 def _as_f32(x) -> np.ndarray:
     return np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
 

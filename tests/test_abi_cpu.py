@@ -85,6 +85,34 @@ def test_construction_refusals_need_no_gpu():
     assert status == 17
 
 
+def test_debug_channel_is_off_by_default_and_says_why_a_call_was_refused(capfd):
+    # attention::diag (crates/attention/src/diag.rs:13-33 and its two tests, :108-131): silent
+    # unless switched on; a line per event with a fixed prefix when it is.
+    lib = pkg()._native.load()
+    os.environ.pop("ITAK_HIP_KV_DEBUG", None)
+    lib.itak_set_debug_enabled(0)
+    assert lib.itak_debug_enabled() == 0
+    _create(layers=0)
+    assert "[itak_hip_kv::diag]" not in capfd.readouterr().err
+    lib.itak_set_debug_enabled(1)
+    try:
+        assert lib.itak_debug_enabled() == 1
+        _create(layers=0)
+        err = capfd.readouterr().err
+        assert "[itak_hip_kv::diag] refused code=1: layer pattern must be positive, got 0" in err
+    finally:
+        lib.itak_set_debug_enabled(0)
+    # The environment variable is looked up at every event: any value but "0" or empty.
+    for value, on in (("1", True), ("yes", True), ("0", False), ("", False)):
+        os.environ["ITAK_HIP_KV_DEBUG"] = value
+        try:
+            assert lib.itak_debug_enabled() == int(on), value
+            _create(kv_heads=0)
+            assert ("refused code=1: num_kv_heads" in capfd.readouterr().err) == on, value
+        finally:
+            del os.environ["ITAK_HIP_KV_DEBUG"]
+
+
 def test_python_front_end_raises_named_errors_without_a_gpu():
     P = pkg()
     with pytest.raises(P.AttentionError) as e:

@@ -450,3 +450,41 @@ def test_getters_refuse_null_outputs_by_name():
         assert b"null" in lib.itak_last_error(pool._h)
     cache.release(cp)
     pool.close()
+
+
+def test_debug_channel_reports_cache_and_attention_events(capfd):
+    # attention::diag (crates/attention/src/diag.rs): the events the reference logs (cache built,
+    # append, checkpoint, rewind, release, gqa_attention, bulk restore) each give one line, and
+    # nothing is printed once the switch is off again.
+    import torch
+    kv_heads, d = 2, 128
+    P().set_debug_enabled(True)
+    try:
+        pool = P().KvPool(1, kv_heads, d, elem="f16", capacity_rows=64)
+        pool.set_stream(torch.cuda.current_stream().cuda_stream)
+        cache = pool.acquire()
+        for p in range(3):
+            cache.append(0, k_row(kv_heads, d, p), v_row(kv_heads, d, p), p)
+        cp = cache.checkpoint(4)
+        cache.append(0, k_row(kv_heads, d, 3), v_row(kv_heads, d, 3), 3)
+        q = normal(np.random.default_rng(0), 1, 4 * d)
+        P().gqa_attention(q, 1, 4, [3], cache.view(0))
+        cache.rewind_to(cp, 3)
+        cache.release(cp)
+        with pytest.raises(P().AttentionError):
+            cache.append(0, k_row(kv_heads, d, 9), v_row(kv_heads, d, 9), 9)
+    finally:
+        P().set_debug_enabled(False)
+    err = capfd.readouterr().err
+    lines = [l[len("[itak_hip_kv::diag] "):] for l in err.splitlines() if l.startswith("[itak_hip_kv::diag] ")]
+    assert lines[0].startswith("kv pool built layers=1 kv_heads=2 head_dim=128 elem=f16 slots=")
+    assert "append layer=0 slot=0 rows=1 kind=global stored=3" in lines
+    assert "checkpoint slot=0 serial=1 max_round_tokens=4 saved_bytes=0" in lines
+    assert any(l.startswith("gqa_attention layer=0 items=1 queries=1 q_heads=4 kv_heads=2 view_len=4 window=0")
+               for l in lines)
+    assert "rewind slot=0 serial=1 target=3" in lines
+    assert "release slot=0 serial=1" in lines
+    assert any(l.startswith("refused code=") and "position" in l for l in lines)
+    cache.append(0, k_row(kv_heads, d, 3), v_row(kv_heads, d, 3), 3)
+    assert "[itak_hip_kv::diag]" not in capfd.readouterr().err
+    pool.close()
