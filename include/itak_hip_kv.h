@@ -127,14 +127,14 @@ typedef struct itak_pool_config {
        step appends its whole block before its queries run, so the ring must still hold the
        window of the block's first row after the last row has landed; the same spare rows let
        a rewind drop positions without saved copies. It bounds the rows one device step may
-       carry on a windowed layer, max_round_tokens of a checkpoint, and how far a truncate may
-       go back (the chunk_cap of the reference's resident session,
-       crates/wgpu-compute/src/session.rs:235-249, 5376-5428). A ring is window +
-       ring_headroom rows, rounded up to a multiple of 32; the bound that blocks, checkpoints
-       (max_round_tokens) and truncates meet is what the rounding leaves, ring - window of the
-       shortest such layer, so at least ring_headroom. The reference's CPU cache takes any
-       max_round_tokens up to the smallest window (cache.rs:634-651): a round longer than the
-       bound is refused here with ITAK_CAPACITY_EXCEEDED. */
+       carry on a windowed layer and how far a truncate may go back (the chunk_cap of the
+       reference's resident session, crates/wgpu-compute/src/session.rs:235-249, 5376-5428).
+       A ring is window + ring_headroom rows, rounded up to a multiple of 32; the bound that
+       blocks and truncates meet is what the rounding leaves, ring - window of the shortest
+       such layer, so at least ring_headroom. A checkpoint takes any max_round_tokens up to
+       the smallest window, as the reference's cache does (cache.rs:634-651): a round within
+       the bound costs nothing, a longer one has the rows it may overwrite copied aside at the
+       checkpoint (one small launch, a buffer kept per slot) and copied back by a rewind. */
     uint64_t ring_headroom;
 } itak_pool_config;
 

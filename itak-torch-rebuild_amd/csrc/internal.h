@@ -140,6 +140,30 @@ hipError_t launch_read_rows(const void *layer_base, int elem_f16, const PoolGeom
                             uint32_t first_row, uint32_t rows, uint32_t ring, void *keys_out,
                             void *values_out, hipStream_t stream);
 
+// ---- ring rows aside and back (checkpoints deeper than a ring's headroom) -----------------
+// Copies rows of windowed layers between their rings and a side buffer that holds, per entry,
+// [side][saved_rows][kv_head][d] elements at saved_off: row saved_row0 + r of the buffer is
+// position pos0 + r, storage row (pos0 + r) % ring.
+struct RingRowsLayer {
+    uint32_t layer;       // index among the windowed layers
+    uint32_t ring;
+    uint32_t pos0;
+    uint32_t rows;
+    uint32_t saved_row0;
+    uint32_t saved_rows;
+    uint64_t saved_off;   // elements
+};
+struct RingRowsBatch {
+    uint32_t n;
+    uint32_t slot;
+    uint32_t max_rows;
+    uint32_t pad;
+    RingRowsLayer layer[kMaxRestoreLayers];
+};
+// to_ring = false: rings -> buffer; true: buffer -> rings.
+hipError_t launch_ring_rows(void *pool_base_w, int elem_f16, const PoolGeom &gw,
+                            const RingRowsBatch &b, void *saved, bool to_ring, hipStream_t stream);
+
 hipError_t launch_convert_f16(const float *src, uint16_t *dst, uint64_t count, hipStream_t stream);
 // f16 bits -> f32, exact (the widening a snapshot capture of an f16 pool needs).
 hipError_t launch_widen_f16(const uint16_t *src, float *dst, uint64_t count, hipStream_t stream);

@@ -344,6 +344,50 @@ __global__ __launch_bounds__(256) void kv_read_rows(const T *__restrict__ layer_
     }
 }
 
+// ------------------------------------------------------- ring rows aside and back
+// One element per thread and step: a checkpoint deeper than the headroom is taken once per
+// speculative round at most and moves a few MB.
+template <typename T, bool TO_RING>
+__global__ __launch_bounds__(256) void kv_ring_rows_kernel(T *__restrict__ pool_base_w, PoolGeom g,
+                                                           RingRowsBatch b, T *__restrict__ saved) {
+    const RingRowsLayer L = b.layer[blockIdx.z];
+    const uint32_t side = blockIdx.y;
+    const uint32_t row_elems = g.kv_heads * g.head_dim;
+    const uint64_t total = uint64_t(L.rows) * row_elems;
+    T *plane_side = pool_base_w + L.layer * g.layer_stride + b.slot * g.slot_stride +
+                    side * g.side_stride;
+    T *buf = saved + L.saved_off + (uint64_t(side) * L.saved_rows + L.saved_row0) * row_elems;
+    for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < total; i += gridDim.x * 256ull) {
+        const uint32_t row = uint32_t(i / row_elems), rem = uint32_t(i % row_elems);
+        const uint32_t head = rem / g.head_dim, d = rem % g.head_dim;
+        const uint32_t srow = (L.pos0 + row) % L.ring;
+        T *at = plane_side + head * g.head_stride + kv_offset(g, side, srow, d);
+        if (TO_RING)
+            *at = buf[i];
+        else
+            buf[i] = *at;
+    }
+}
+
+hipError_t launch_ring_rows(void *pool_base_w, int elem_f16, const PoolGeom &gw,
+                            const RingRowsBatch &b, void *saved, bool to_ring, hipStream_t stream) {
+    if (b.n == 0 || b.max_rows == 0) return hipSuccess;
+    const uint64_t total = uint64_t(b.max_rows) * gw.kv_heads * gw.head_dim;
+    uint32_t bx = uint32_t((total + 255) / 256);
+    if (bx > 1024) bx = 1024;
+    dim3 grid(bx, 2, b.n);
+#define ITAK_RING_ROWS(T, TO)                                                                  \
+    kv_ring_rows_kernel<T, TO><<<grid, 256, 0, stream>>>(static_cast<T *>(pool_base_w), gw, b, \
+                                                         static_cast<T *>(saved))
+    if (elem_f16) {
+        if (to_ring) ITAK_RING_ROWS(uint16_t, true); else ITAK_RING_ROWS(uint16_t, false);
+    } else {
+        if (to_ring) ITAK_RING_ROWS(float, true); else ITAK_RING_ROWS(float, false);
+    }
+#undef ITAK_RING_ROWS
+    return hipGetLastError();
+}
+
 hipError_t launch_read_rows(const void *layer_base, int elem_f16, const PoolGeom &g, uint32_t slot,
                             uint32_t first_row, uint32_t rows, uint32_t ring, void *keys_out,
                             void *values_out, hipStream_t stream) {

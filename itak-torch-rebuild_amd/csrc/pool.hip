@@ -26,11 +26,21 @@ static __device__ __align__(256) unsigned char scratch[16ull << 20];
 
 namespace {
 
+// One windowed layer's rows set aside by a checkpoint whose round is longer than the ring's
+// headroom (the saved slots of cache.rs:678-697): `rows` positions from the layer's base on.
+struct RingSave {
+    uint32_t layer = 0;      // pool layer
+    uint32_t rows = 0;
+    uint64_t saved_off = 0;  // elements into the slot's side buffer
+    uint64_t high0 = 0;      // the layer's high-water mark when the checkpoint was taken
+};
+
 struct LiveCheckpoint {
     bool live = false;
     uint64_t serial = 0;
     uint64_t max_round_tokens = 0;
     std::vector<uint64_t> bases;
+    std::vector<RingSave> ring_saves;  // empty when the headroom covers the round
 };
 
 struct Slot {
@@ -124,6 +134,10 @@ struct itak_pool {
     bool no_alloc_call = false;
     bool scratch_exchange_used = false;  // its give-up counter is then looked at too
     bool merge_in_launch = false;
+    // Per slot: the side buffer of a deep checkpoint's ring rows, kept for the next one
+    // (cache.rs:620-625: allocated once per cache, not once per round).
+    std::vector<void *> ring_saved;
+    std::vector<uint64_t> ring_saved_bytes;
     // Pinned host memory for the host-pointer attention call: its small inputs are packed here
     // and go up in one copy; its kernels write the output here directly.
     unsigned char *hstage = nullptr;
@@ -1029,6 +1043,8 @@ itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out) {
         return hip_error(e, he, "zero KV pool");
     }
     pool->slots.resize(config->max_slots);
+    pool->ring_saved.assign(config->max_slots, nullptr);
+    pool->ring_saved_bytes.assign(config->max_slots, 0);
     pool->merge_in_launch = (config->flags & ITAK_POOL_MERGE_IN_LAUNCH) != 0;
     he = bind_scratch(config->device, &pool->scratch_dev);
     if (he != hipSuccess) {
@@ -1053,6 +1069,8 @@ void itak_pool_destroy(itak_pool *pool) {
     if (pool->ws) (void)hipFree(pool->ws);
     if (pool->prep) (void)hipFree(pool->prep);
     if (pool->xws) (void)hipFree(pool->xws);
+    for (void *buf : pool->ring_saved)
+        if (buf) (void)hipFree(buf);
     if (pool->hstage) (void)hipHostFree(pool->hstage);
     delete pool;
 }
@@ -1735,6 +1753,62 @@ itak_status itak_kv_read_raw(itak_pool *pool, uint32_t slot, uint64_t layer, voi
     return read_rows_common(pool, slot, layer, 0, rows, 0, keys_out, values_out);
 }
 
+// Moves ring rows of the layers in `saves` between their rings and the slot's side buffer:
+// positions [from, to) of each layer that fall inside what its save covers.
+static itak_status move_ring_rows(itak_pool *pool, uint32_t slot, const Slot &s,
+                                  const std::vector<RingSave> &saves, const uint64_t *bases,
+                                  uint64_t from, const uint64_t *to_per_layer, bool to_ring) {
+    RingRowsBatch b{};
+    b.slot = slot;
+    auto flush = [&]() -> itak_status {
+        if (b.n == 0) return ITAK_OK;
+        hipError_t e = launch_ring_rows(pool->base_w, pool->elem_f16, pool->gw, b,
+                                        pool->ring_saved[slot], to_ring, pool->stream);
+        b.n = 0;
+        b.max_rows = 0;
+        return e == hipSuccess ? ITAK_OK : hip_error(pool->err, e, "launch ring row copy");
+    };
+    (void)s;
+    for (const RingSave &rs : saves) {
+        const uint64_t base = bases[rs.layer];
+        const uint64_t lo = std::max(from, base);
+        const uint64_t hi = std::min<uint64_t>(to_per_layer[rs.layer], base + rs.rows);
+        if (hi <= lo) continue;
+        const LayerInfo &L = pool->layers[rs.layer];
+        RingRowsLayer &R = b.layer[b.n++];
+        R.layer = L.index;
+        R.ring = L.ring;
+        R.pos0 = uint32_t(lo);
+        R.rows = uint32_t(hi - lo);
+        R.saved_row0 = uint32_t(lo - base);
+        R.saved_rows = rs.rows;
+        R.saved_off = rs.saved_off;
+        b.max_rows = std::max(b.max_rows, R.rows);
+        if (b.n == kMaxRestoreLayers) {
+            itak_status st = flush();
+            if (st != ITAK_OK) return st;
+        }
+    }
+    return flush();
+}
+
+// The checkpoint's copy of the rows a deep round may overwrite (cache.rs:678-697).
+static itak_status save_ring_rows(itak_pool *pool, uint32_t slot, const Slot &s,
+                                  const std::vector<RingSave> &saves, uint64_t elems) {
+    const uint64_t bytes = elems * pool->elem_bytes;
+    if (bytes > pool->ring_saved_bytes[slot]) {
+        HIP_TRY(pool, hipStreamSynchronize(pool->stream), "synchronize before growing the checkpoint buffer");
+        if (pool->ring_saved[slot]) HIP_TRY(pool, hipFree(pool->ring_saved[slot]), "free the checkpoint buffer");
+        pool->ring_saved[slot] = nullptr;
+        pool->ring_saved_bytes[slot] = 0;
+        HIP_TRY(pool, hipMalloc(&pool->ring_saved[slot], bytes), "allocate the checkpoint buffer");
+        pool->ring_saved_bytes[slot] = bytes;
+    }
+    std::vector<uint64_t> to(pool->layers.size());
+    for (const RingSave &rs : saves) to[rs.layer] = s.appended[rs.layer] + rs.rows;
+    return move_ring_rows(pool, slot, s, saves, s.appended.data(), 0, to.data(), false);
+}
+
 itak_status itak_kv_checkpoint_active(itak_pool *pool, uint32_t slot, int32_t *out) {
     if (!pool) return ITAK_INVALID_ARGUMENT;
     if (!out) return invalid_argument(pool->err, "out is null");
@@ -1766,29 +1840,39 @@ itak_status itak_kv_checkpoint(itak_pool *pool, uint32_t slot, uint64_t max_roun
                          "round that long would overwrite a ring slot twice and no rewind could be "
                          "exact",
                          ULL(max_round_tokens), ULL(smallest_window));
-    // The device keeps no copies of evicted rows: the ring's headroom is what lets a round be
-    // undone, so a round may not be longer than it.
-    // (what the rings really hold beyond their windows: the configured headroom rounded up to
-    // whole 32-row blocks, the bound check_block_rows and check_ring_rewind use too)
-    uint64_t ring_room = ~0ull;
-    for (const LayerInfo &L : pool->layers)
-        if (L.windowed) ring_room = std::min<uint64_t>(ring_room, L.ring - L.window);
-    if (windowed && max_round_tokens > ring_room)
-        return set_error(pool->err, ITAK_CAPACITY_EXCEEDED, nullptr, 0, max_round_tokens,
-                         ring_room, 0,
-                         "a round of up to %llu tokens does not fit the %llu rows of ring headroom "
-                         "of the windowed layers; build the pool with a larger ring_headroom",
-                         ULL(max_round_tokens), ULL(ring_room));
+    // A round the ring's headroom covers needs no copies: the rows it overwrites are outside
+    // every window a rewind can bring back. A longer one (up to the smallest window, as the
+    // reference allows) sets the rows it may overwrite aside first, layer by layer where the
+    // headroom is too short, exactly the slots the reference saves (cache.rs:678-697).
+    std::vector<RingSave> saves;
+    uint64_t save_elems = 0;
+    for (uint64_t li = 0; li < pool->layers.size(); ++li) {
+        const LayerInfo &L = pool->layers[li];
+        if (!L.windowed || max_round_tokens <= L.ring - L.window) continue;
+        RingSave rs;
+        rs.layer = uint32_t(li);
+        rs.rows = uint32_t(max_round_tokens);
+        rs.saved_off = save_elems;
+        rs.high0 = s->high[li];
+        save_elems += 2 * max_round_tokens * pool->row;
+        saves.push_back(rs);
+    }
+    if (!saves.empty()) {
+        itak_status st = save_ring_rows(pool, slot, *s, saves, save_elems);
+        if (st != ITAK_OK) return st;
+    }
     s->next_serial += 1;
     s->cp.live = true;
     s->cp.serial = s->next_serial;
     s->cp.max_round_tokens = max_round_tokens;
     s->cp.bases = s->appended;
+    s->cp.ring_saves = std::move(saves);
     out->cache_id = s->cache_id;
     out->serial = s->cp.serial;
     out->max_round_tokens = max_round_tokens;
-    // What the reference's snapshot of the evictable ring slots would hold (cache.rs:678-697):
-    // reported for accounting; the device saves nothing, the rows stay in the ring's headroom.
+    // What the reference's snapshot of the evictable ring slots holds (cache.rs:678-697), as
+    // the reference counts it (f32 rows of every windowed layer); the device sets rows aside
+    // only on layers whose headroom the round outgrows, in the pool's element type.
     out->saved_bytes = windowed * max_round_tokens * 2 * pool->row * 4;
     ITAK_DIAG("checkpoint slot=%u serial=%llu max_round_tokens=%llu saved_bytes=%llu", slot,
               ULL(out->serial), ULL(max_round_tokens), ULL(out->saved_bytes));
@@ -1817,15 +1901,19 @@ itak_status itak_kv_checkpoint_bases(itak_pool *pool, uint32_t slot, const itak_
 // wrapped onto rows the target's view still needs: with H the highest position ever written
 // plus one, position x is overwritten once x + ring < H, and the view after the rewind starts
 // at target - window, so H - target may be at most ring - window.
-static itak_status check_ring_rewind(itak_pool *pool, const Slot &s, uint64_t target) {
+static itak_status check_ring_rewind(itak_pool *pool, const Slot &s, uint64_t target,
+                                     const std::vector<RingSave> *saves = nullptr) {
     for (uint64_t li = 0; li < s.appended.size(); ++li) {
         const LayerInfo &L = pool->layers[li];
         if (!L.windowed || target >= s.appended[li]) continue;
+        bool saved = false;  // a live checkpoint holds this layer's overwritten rows
+        if (saves)
+            for (const RingSave &rs : *saves) saved = saved || rs.layer == li;
         // A layer restored from a snapshot holds nothing older than the snapshot's first row:
         // the view of a target below first + window would reach under it.
         if (s.floor[li] > 0 && target < s.floor[li] + L.window)
             return rewind_range(pool->err, li, s.floor[li] + L.window, s.appended[li], target);
-        if (s.high[li] - target > L.ring - L.window)
+        if (!saved && s.high[li] - target > L.ring - L.window)
             return set_error(pool->err, ITAK_CAPACITY_EXCEEDED, nullptr, li, s.high[li] - target,
                              L.ring - L.window, 0,
                              "dropping windowed layer %llu back to position %llu discards rows up to "
@@ -1884,9 +1972,19 @@ itak_status itak_kv_rewind_to(itak_pool *pool, uint32_t slot, const itak_checkpo
         if (target < base || target > s->appended[li])
             return rewind_range(pool->err, li, base, s->appended[li], target);
     }
-    st = check_ring_rewind(pool, *s, target);
+    st = check_ring_rewind(pool, *s, target, &s->cp.ring_saves);
     if (st != ITAK_OK) return st;
     ITAK_DIAG("rewind slot=%u serial=%llu target=%llu", slot, ULL(cp->serial), ULL(target));
+    if (!s->cp.ring_saves.empty()) {
+        // The rows the dropped positions overwrote come back from the checkpoint's copy
+        // (cache.rs:792-812); what the ring then holds beyond `target` is what it held when
+        // the checkpoint was taken.
+        st = move_ring_rows(pool, slot, *s, s->cp.ring_saves, s->cp.bases.data(), target,
+                            s->high.data(), true);
+        if (st != ITAK_OK) return st;
+        for (const RingSave &rs : s->cp.ring_saves)
+            s->high[rs.layer] = std::max(target, std::min(rs.high0, s->high[rs.layer]));
+    }
     return truncate_slots(pool, &slot, &target, 1);
 }
 
@@ -1897,6 +1995,7 @@ itak_status itak_kv_release(itak_pool *pool, uint32_t slot, const itak_checkpoin
     itak_status st = live_data(pool, *s, cp);
     if (st != ITAK_OK) return st;
     s->cp.live = false;  // cache.rs:824-833
+    s->cp.ring_saves.clear();
     ITAK_DIAG("release slot=%u serial=%llu", slot, ULL(cp->serial));
     return ITAK_OK;
 }

@@ -278,11 +278,14 @@ def test_the_rings_headroom_bounds_blocks_rounds_and_truncates():
     for _ in range(4):
         pool.append_device(0, [(cache, 32)], rows.data_ptr(), rows.data_ptr())
     assert cache.next_position(0) == 128
-    # A round may be as long as the ring can undo: ring - window = 32 rows (the configured 16
-    # rounded up to whole blocks), the same bound blocks and truncates have; 33 is refused.
+    # A round longer than the ring can undo by itself (ring - window = 32 rows) is taken all
+    # the same, as the reference takes any round up to the window: the checkpoint sets the rows
+    # it may overwrite aside (the deep-round test below rewinds one).
+    cp = cache.checkpoint(33)
+    cache.release(cp)
     with pytest.raises(P().AttentionError) as e:
-        cache.checkpoint(33)
-    assert e.value.variant == "CapacityExceeded" and "ring headroom" in e.value.message
+        cache.checkpoint(65)
+    assert e.value == E("CheckpointTooDeep", max_round_tokens=65, window=64)
     pool.truncate([cache.slot], [100])   # 28 positions back: inside the 32 spare rows
     assert cache.next_position(0) == 100
     with pytest.raises(P().AttentionError) as e:
@@ -536,6 +539,102 @@ def test_speculative_rounds_on_a_windowed_layer_rewind_to_the_exact_continuation
         ref.release(rcp)
         assert view_snapshot(cache, 0) == view_snapshot(ref, 0)
         run_steps(pool, cache, ref, rng, q_heads, [1], elem)
+    pool.close()
+
+
+@pytest.mark.parametrize("elem", ["f32", "f16"])
+def test_rounds_deeper_than_the_ring_headroom_rewind_from_the_checkpoints_saved_rows(elem):
+    # KvCache::checkpoint takes any round up to the smallest window and saves the ring slots the
+    # round may overwrite (cache.rs:634-697); rewind_to puts back those the dropped positions
+    # took (cache.rs:792-812). The device ring undoes ring - window = 32 positions by itself; a
+    # deeper round (several blocks, each within the headroom) needs the saved rows: after every
+    # rewind the view and the next tokens' attention equal the oracle's, through second rewinds
+    # inside one checkpoint, rewinds below an earlier one, a round accepted whole, and a shallow
+    # round's leftovers under a deep one.
+    window, kvh, d, q_heads = 64, 4, 128, 32
+    pool, cache, ref, rng = pair(window, kvh, d, elem, seed=11, headroom=32)
+    run_steps(pool, cache, ref, rng, q_heads, [1] * 70 + [8] * 5, elem)   # wrapped once
+    for depth, blocks, cuts in (
+            (64, [32, 32], [40]),            # the whole window, rewound past the headroom
+            (60, [20, 20, 20], [48, 10]),    # second rewind below the first, more tokens between
+            (56, [28, 28], [5, 15, 2]),
+            (48, [16, 32], [48]),            # nothing dropped
+            (50, [25, 25], [1]),
+            (8, [8], [3]),                   # shallow: leaves dropped rows in the headroom ...
+            (64, [30, 30, 4], [0]),          # ... under a deep round that drops everything
+            (40, [8] * 5, [33])):
+        base = cache.next_position(0)
+        cp, rcp = cache.checkpoint(depth), ref.checkpoint(depth)
+        run_steps(pool, cache, ref, rng, q_heads, blocks, elem)
+        for i, cut in enumerate(cuts):
+            cache.rewind_to(cp, base + cut)
+            ref.rewind_to(rcp, base + cut)
+            assert cache.next_position(0) == ref.next_position(0) == base + cut
+            assert view_snapshot(cache, 0) == view_snapshot(ref, 0), (depth, cut)
+            if i + 1 < len(cuts):   # the round goes on before the next cut
+                run_steps(pool, cache, ref, rng, q_heads, [min(depth - cut, 12)], elem)
+        cache.release(cp)
+        ref.release(rcp)
+        run_steps(pool, cache, ref, rng, q_heads, [1, 1, 5], elem)
+        assert view_snapshot(cache, 0) == view_snapshot(ref, 0), depth
+    # The round bound still holds while the checkpoint is live, with the reference's fields.
+    base = cache.next_position(0)
+    cp, rcp = cache.checkpoint(40), ref.checkpoint(40)
+    run_steps(pool, cache, ref, rng, q_heads, [32], elem)
+    import torch
+    z = torch.zeros(9, kvh * d, device="cuda")
+    with pytest.raises(P().AttentionError) as e:
+        pool.append_device(0, [(cache, 9)], z.data_ptr(), z.data_ptr())
+    assert e.value.variant == "CheckpointRangeExceeded"
+    cache.rewind_to(cp, base)
+    ref.rewind_to(rcp, base)
+    cache.release(cp)
+    ref.release(rcp)
+    assert view_snapshot(cache, 0) == view_snapshot(ref, 0)
+    pool.close()
+
+
+def test_a_deep_round_on_a_hybrid_pattern_saves_only_the_layers_that_need_it():
+    # Windows 64 and 70 with 32 rows of headroom give rings of 96 and 128 rows: a round of 50
+    # outgrows the first ring's 32 spare rows and not the second's 58; the global layer
+    # truncates. All three must come back to the oracle's views.
+    import torch
+    kvh, d, q_heads = 2, 128, 8
+    pattern = [W(64), P().LayerKind.Global, W(70)]
+    rpattern = [oracle.LayerKind.windowed(64), oracle.LayerKind.Global, oracle.LayerKind.windowed(70)]
+    pool = P().KvPool(pattern, kvh, d, elem="f16", capacity_rows=512, ring_headroom=32)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    cache = pool.acquire()
+    ref = oracle.KvCache.new(rpattern, kvh, d, store_f16=True)
+    rng = np.random.default_rng(21)
+
+    def step(rows):
+        base = cache.next_position(0)
+        for layer in range(3):
+            q, k, v = normal(rng, rows, q_heads * d), normal(rng, rows, kvh * d), normal(rng, rows, kvh * d)
+            qd, kd, vd = (torch.from_numpy(x).cuda() for x in (q, k, v))
+            out = torch.empty_like(qd)
+            pool.attention_step_device(layer, [(cache, rows)], qd.data_ptr(), kd.data_ptr(),
+                                       vd.data_ptr(), out.data_ptr(), q_heads)
+            pool.synchronize()
+            want = oracle.attention_step(ref, layer, q, k, v, q_heads, base, threads=4)
+            assert max_abs(out.cpu().numpy().reshape(-1), want) <= 2e-3, (layer, base, rows)
+
+    for rows in [25] * 6:
+        step(rows)
+    for depth, blocks, cut in ((50, [25, 25], 7), (64, [32, 32], 33), (50, [20, 30], 50)):
+        base = cache.next_position(0)
+        cp, rcp = cache.checkpoint(depth), ref.checkpoint(depth)
+        for rows in blocks:
+            step(rows)
+        cache.rewind_to(cp, base + cut)
+        ref.rewind_to(rcp, base + cut)
+        cache.release(cp)
+        ref.release(rcp)
+        for layer in range(3):
+            assert view_snapshot(cache, layer) == view_snapshot(ref, layer), (depth, layer)
+        step(1)
+        step(4)
     pool.close()
 
 
