@@ -33,6 +33,12 @@
 //
 // The chunk's own K/V rows are appended before this kernel runs; row r of the chunk sits at
 // position pos0 + r and sees keys <= its position (attention.rs:77-85 with no window).
+// Blocks of up to kFuseRows rows in the one-tile form bring their rows along instead
+// (AttnParams::k_new / v_new): every workgroup whose run of key blocks reaches the new
+// positions converts them in its prologue, keeps them in registers (16 pieces of 4 channels a
+// thread) and writes them over what the ring's loads brought into LDS for those blocks, and
+// one workgroup per KV head stores them to the planes. That is one launch and its gap less per
+// layer for the blocks where a launch is a sixth of the layer.
 #include "internal.h"
 #include "mfma_common.h"
 #include "timeline.h"
@@ -52,6 +58,8 @@ constexpr int kWaves = 4;
 constexpr int kMaxTiles = 2;  // MFMA column tiles (16 query vectors) per wavefront: 1 or 2
 constexpr int kBlockElems = kBlockKeys * kD;        // 4096 halves = 8 KiB per plane block
 constexpr float kRefSlack = 8.0f;
+constexpr int kFuseRows = 64;  // new rows a launch that appends its own rows carries at most
+constexpr int kFusePieces = kFuseRows * 2 * (kD / 4) / (kWaves * 64);  // per thread
 
 __device__ __forceinline__ float column_max4(float v) {
     const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
@@ -163,7 +171,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     auto issue_block = [&](uint32_t kb) {
         // Past the end the last block is fetched again into a stage nobody reads: the
         // number of loads in flight stays the same in every iteration.
-        const uint64_t off = uint64_t(RING ? next_sb : min(kb, nblocks - 1)) * kBlockVec;
+        const uint64_t off = uint64_t(RING ? next_sb : min(kb, max(nblocks, 1u) - 1)) * kBlockVec;
         if (RING && kb + 1 < nblocks) next_sb = next_sb + 1 == ring_blocks ? 0 : next_sb + 1;
         const uint32_t dst = dma_base + (kb % STAGES) * kStageBytes;
         lds_dma16(kg + off, dst);
@@ -184,60 +192,132 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     // three to seven blocks of keys and values, which a short run of blocks could not hide.
     // The compiler cannot count the ring's loads (they are issued from assembly), so it would
     // wait for everything before the first use of Q: the Q loads are issued from assembly too
-    // and waited for by count. Rows past the block's end re-read its last row and are scaled
-    // to zero columns (no branch around a load).
+    // and waited for by count. Between such a load and the wait that names its registers the
+    // code is a straight line: across a branch the compiler may copy a register it believes
+    // loaded, and would copy what was there before. So the ring is always filled (a workgroup
+    // without blocks fetches block 0 into stages nobody reads), rows past the block's end
+    // re-read its last row and are scaled to zero columns, and the variant that also brings new
+    // rows is a second straight line, not a branch inside this one.
+    //
+    // New rows (one-tile form only): piece u of this thread is row (tid >> 6) + 4u, side
+    // (tid >> 5) & 1, channels (tid & 31) * 4 .. + 3, requested ahead of Q and waited for with it.
+    constexpr bool kCanFuse = kTiles == 1;
+    const bool fused = kCanFuse && p.k_new != nullptr;
+    const uint32_t nside = (tid >> 5) & 1u, nc4 = (tid & 31u) * 4;
+    // Does this workgroup's run of blocks reach the new positions? Is it the one that stores them?
+    const bool patches = fused && any_block && nblocks * kBlockKeys > item.pos0;
+    const bool stores_new = fused && unit < p.g.kv_heads && split == item.splits - 1;
+    const bool with_new = patches || stores_new;
+    [[maybe_unused]] uint2 npk[kCanFuse ? kFusePieces : 1];
     half8 qb[kTiles][4];
     uint32_t colpos[kTiles], collo[kTiles];
-    {
-        floatx4 qraw[kTiles][8];
+    const float *qp[kTiles];
+    float qsc[kTiles];
 #pragma unroll
-        for (int qt = 0; qt < kTiles; ++qt) {
-            const uint32_t j = qt * 16 + jl;
-            const uint32_t row = row_begin + j / group;
-            colpos[qt] = min(item.pos0 + row, item.kv_len - 1);
-            collo[qt] = lowest_visible(item.pos0 + row, window, kv_lo);
-            const uint32_t head = kv_head * group + j % group;
-            const float *qp =
-                p.q + (uint64_t(item.q_row0 + min(row, item.rows - 1)) * p.q_heads + head) * kD + g * 8;
-#pragma unroll
-            for (int s = 0; s < 8; ++s)
-                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qraw[qt][s]) : "v"(qp + (s >> 1) * 32 + (s & 1) * 4) : "memory");
-        }
-        if (any_block) {
-#pragma unroll
-            for (int ahead = 0; ahead < STAGES - 1; ++ahead) issue_block(kb_begin + ahead);
-        }
-        ITAK_MARK(2)
-        // Everything older than the ring's loads has landed: that is Q. A workgroup without
-        // blocks issued no ring loads, so there the count to wait for is zero: a Q load still in
-        // flight would land in a register the compiler has meanwhile given to something else
-        // (an address of the epilogue's stores, for one).
+    for (int qt = 0; qt < kTiles; ++qt) {
+        const uint32_t j = qt * 16 + jl;
+        const uint32_t row = row_begin + j / group;
+        colpos[qt] = min(item.pos0 + row, item.kv_len - 1);
+        collo[qt] = lowest_visible(item.pos0 + row, window, kv_lo);
+        const uint32_t head = kv_head * group + j % group;
+        qp[qt] = p.q + (uint64_t(item.q_row0 + min(row, item.rows - 1)) * p.q_heads + head) * kD + g * 8;
+        qsc[qt] = row < item.rows ? qscale : 0.0f;
+    }
+#define ITAK_Q_LOADS(qraw)                                                                      \
+    _Pragma("unroll") for (int qt = 0; qt < kTiles; ++qt)                                       \
+        _Pragma("unroll") for (int s = 0; s < 8; ++s)                                           \
+            asm volatile("global_load_dwordx4 %0, %1, off"                                      \
+                         : "=v"(qraw[qt][s])                                                    \
+                         : "v"(qp[qt] + (s >> 1) * 32 + (s & 1) * 4)                            \
+                         : "memory");
+#define ITAK_RING_FILL                                                                          \
+    _Pragma("unroll") for (int ahead = 0; ahead < STAGES - 1; ++ahead) issue_block(kb_begin + ahead);
 #define ITAK_Q_REGS(qt)                                                                         \
     "+v"(qraw[qt][0]), "+v"(qraw[qt][1]), "+v"(qraw[qt][2]), "+v"(qraw[qt][3]), "+v"(qraw[qt][4]), \
         "+v"(qraw[qt][5]), "+v"(qraw[qt][6]), "+v"(qraw[qt][7])
-        if (any_block) {
-            if constexpr (kTiles == 2)
-                asm volatile("s_waitcnt vmcnt(%16)" : ITAK_Q_REGS(0), ITAK_Q_REGS(1) : "n"(4 * (STAGES - 1)) : "memory");
-            else
-                asm volatile("s_waitcnt vmcnt(%8)" : ITAK_Q_REGS(0) : "n"(4 * (STAGES - 1)) : "memory");
-        } else {
-            if constexpr (kTiles == 2)
-                asm volatile("s_waitcnt vmcnt(0)" : ITAK_Q_REGS(0), ITAK_Q_REGS(1) : : "memory");
-            else
-                asm volatile("s_waitcnt vmcnt(0)" : ITAK_Q_REGS(0) : : "memory");
+#define ITAK_Q_CONVERT(qraw)                                                                    \
+    _Pragma("unroll") for (int qt = 0; qt < kTiles; ++qt)                                       \
+        _Pragma("unroll") for (int s = 0; s < 4; ++s) {                                         \
+            const floatx4 a = qraw[qt][2 * s], c = qraw[qt][2 * s + 1];                         \
+            const float sc = qsc[qt];                                                           \
+            qb[qt][s] = half8{static_cast<_Float16>(a[0] * sc), static_cast<_Float16>(a[1] * sc), \
+                              static_cast<_Float16>(a[2] * sc), static_cast<_Float16>(a[3] * sc), \
+                              static_cast<_Float16>(c[0] * sc), static_cast<_Float16>(c[1] * sc), \
+                              static_cast<_Float16>(c[2] * sc), static_cast<_Float16>(c[3] * sc)}; \
         }
+    bool took_new = false;
+    if constexpr (kCanFuse) {
+        if (with_new) {
+            took_new = true;
+            floatx4 nraw[kFusePieces], qraw[kTiles][8];
+            const uint32_t row_width = p.g.kv_heads * kD;
+            const float *src = (nside ? p.v_new : p.k_new) + uint64_t(item.q_row0) * row_width +
+                               kv_head * kD + nc4;
+#pragma unroll
+            for (int u = 0; u < kFusePieces; ++u) {
+                const uint32_t r = min((tid >> 6) + 4u * u, item.rows - 1);
+                asm volatile("global_load_dwordx4 %0, %1, off"
+                             : "=v"(nraw[u])
+                             : "v"(src + uint64_t(r) * row_width)
+                             : "memory");
+            }
+            ITAK_Q_LOADS(qraw)
+            ITAK_RING_FILL
+            ITAK_MARK(2)
+            static_assert(kFusePieces == 16, "the wait below names sixteen registers of new rows");
+            asm volatile("s_waitcnt vmcnt(%24)"
+                         : ITAK_Q_REGS(0), "+v"(nraw[0]), "+v"(nraw[1]), "+v"(nraw[2]), "+v"(nraw[3]),
+                           "+v"(nraw[4]), "+v"(nraw[5]), "+v"(nraw[6]), "+v"(nraw[7]), "+v"(nraw[8]),
+                           "+v"(nraw[9]), "+v"(nraw[10]), "+v"(nraw[11]), "+v"(nraw[12]),
+                           "+v"(nraw[13]), "+v"(nraw[14]), "+v"(nraw[15])
+                         : "n"(4 * (STAGES - 1))
+                         : "memory");
+            ITAK_Q_CONVERT(qraw)
+#pragma unroll
+            for (int u = 0; u < kFusePieces; ++u) {
+                const uint32_t h0 = f32_to_f16_bits(nraw[u][0]), h1 = f32_to_f16_bits(nraw[u][1]);
+                const uint32_t h2 = f32_to_f16_bits(nraw[u][2]), h3 = f32_to_f16_bits(nraw[u][3]);
+                npk[u] = uint2{h0 | (h1 << 16), h2 | (h3 << 16)};
+            }
+        }
+    }
+    if (!took_new) {
+        floatx4 qraw[kTiles][8];
+        ITAK_Q_LOADS(qraw)
+        ITAK_RING_FILL
+        ITAK_MARK(2)
+        // Everything older than the ring's loads has landed: that is Q.
+        if constexpr (kTiles == 2)
+            asm volatile("s_waitcnt vmcnt(%16)" : ITAK_Q_REGS(0), ITAK_Q_REGS(1) : "n"(4 * (STAGES - 1)) : "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(%8)" : ITAK_Q_REGS(0) : "n"(4 * (STAGES - 1)) : "memory");
+        ITAK_Q_CONVERT(qraw)
+    }
+#undef ITAK_Q_CONVERT
 #undef ITAK_Q_REGS
+#undef ITAK_RING_FILL
+#undef ITAK_Q_LOADS
+    if constexpr (kCanFuse) {
+        if (stores_new) {  // as the append kernel lays them out (k_offset / v_offset)
+            uint16_t *kp = const_cast<uint16_t *>(kplane), *vp = const_cast<uint16_t *>(vplane);
 #pragma unroll
-        for (int qt = 0; qt < kTiles; ++qt) {
-            const uint32_t row = row_begin + (qt * 16 + jl) / group;
-            const float sc = row < item.rows ? qscale : 0.0f;
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const floatx4 a = qraw[qt][2 * s], c = qraw[qt][2 * s + 1];
-                qb[qt][s] = half8{static_cast<_Float16>(a[0] * sc), static_cast<_Float16>(a[1] * sc),
-                                  static_cast<_Float16>(a[2] * sc), static_cast<_Float16>(a[3] * sc),
-                                  static_cast<_Float16>(c[0] * sc), static_cast<_Float16>(c[1] * sc),
-                                  static_cast<_Float16>(c[2] * sc), static_cast<_Float16>(c[3] * sc)};
+            for (int u = 0; u < kFusePieces; ++u) {
+                const uint32_t r = (tid >> 6) + 4u * u;
+                if (r >= item.rows) continue;
+                const uint32_t key = item.pos0 + r, kin = key % kBlockKeys;
+                const uint32_t sb = RING ? (key / kBlockKeys) % ring_blocks : key / kBlockKeys;
+                const uint64_t blk = uint64_t(sb) * kBlockElems;
+                if (nside == 0) {
+                    const uint32_t kt = (kin >> 2) & 1, ki = (kin >> 3) * 4 + (kin & 3);
+                    *reinterpret_cast<uint2 *>(kp + blk + ((kt * 16 + (nc4 >> 3)) * 16 + ki) * 8 +
+                                               (nc4 & 7)) = npk[u];
+                } else {
+                    uint16_t *vd = vp + blk + nc4 * kBlockKeys + kin;
+                    vd[0] = uint16_t(npk[u].x);
+                    vd[kBlockKeys] = uint16_t(npk[u].x >> 16);
+                    vd[2 * kBlockKeys] = uint16_t(npk[u].y);
+                    vd[3 * kBlockKeys] = uint16_t(npk[u].y >> 16);
+                }
             }
         }
     }
@@ -272,6 +352,35 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
         issue_block(kb + STAGES - 1);
         const uint16_t *lds_k = lds_ring + (kb % STAGES) * (kStageBytes / 2);
         const uint16_t *lds_v = lds_k + kBlockElems;
+        if constexpr (kCanFuse) {
+            if (patches && (kb + 1) * kBlockKeys > item.pos0) {
+                // The block holds new positions: what the loads brought for them is whatever
+                // the planes held (the storing workgroup may or may not have got there yet);
+                // the rows themselves go over it, in the stage's layouts.
+                uint16_t *sk = lds_ring + (kb % STAGES) * (kStageBytes / 2), *sv = sk + kBlockElems;
+#pragma unroll
+                for (int u = 0; u < kFusePieces; ++u) {
+                    const uint32_t r = (tid >> 6) + 4u * u;
+                    const uint32_t key = item.pos0 + r, kin = key % kBlockKeys;
+                    if (r >= item.rows || key / kBlockKeys != kb) continue;
+                    if (nside == 0) {
+                        const uint32_t kt = (kin >> 2) & 1, ki = (kin >> 3) * 4 + (kin & 3);
+                        *reinterpret_cast<uint2 *>(sk + ((kt * 16 + (nc4 >> 3)) * 16 + ki) * 8 +
+                                                   (nc4 & 7)) = npk[u];
+                    } else {
+                        // piece (channel c, keys g*8..g*8+7) sits at (c/16)*64 + g*16 + c%16
+                        uint16_t *vd = sv + (((nc4 >> 4) * 64 + (kin >> 3) * 16 + (nc4 & 15)) * 8) + (kin & 7);
+                        vd[0] = uint16_t(npk[u].x);
+                        vd[8] = uint16_t(npk[u].x >> 16);
+                        vd[16] = uint16_t(npk[u].y);
+                        vd[24] = uint16_t(npk[u].y >> 16);
+                    }
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+            }
+        }
 
         if (kb < wave_blocks && (!RING || kb >= wave_first)) {
             const uint32_t key_base = kb * kBlockKeys + g * 8;
@@ -398,7 +507,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
         if (kb == kb_begin) { ITAK_MARK(4) }
     }
     ITAK_MARK(5)
-    if (any_block) wait_vmcnt<0>();  // the surplus loads of the last iterations
+    wait_vmcnt<0>();  // the surplus loads of the last iterations (or of the prologue alone)
 
     // One split: the normalised output. Several: the partial (m, l, acc[128]) of this split
     // in the log2 domain, merged by the combine launch; a column that saw nothing writes
@@ -433,6 +542,14 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
 }
 
 }  // namespace
+
+// A launch may bring its items' new rows along (AttnParams::k_new / v_new) when it takes the
+// one-tile form and no item has more than kFuseRows rows.
+bool attn_prefill_f16_appends(const PoolGeom &g, uint32_t group, uint32_t most_rows,
+                              uint32_t most_blocks) {
+    return attn_prefill_f16_supports(g, group) && most_rows <= uint32_t(kFuseRows) &&
+           most_rows * group <= 512 && most_blocks <= 256;
+}
 
 bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group) {
     return g.v_block == kVBlock && g.head_dim == kD && group >= 1 && group <= 16 &&
@@ -474,7 +591,7 @@ static uint32_t unit_block_count(const AttnItem &it, uint32_t rows_per_group, ui
 }
 
 uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, uint32_t q_heads,
-                               uint32_t window) {
+                               uint32_t window, bool appends) {
     const uint32_t rows_per_group = uint32_t(tiles_for(b, group) * kWaves * 16) / group;
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess ||
@@ -502,7 +619,16 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
         const uint32_t nblocks = unit_block_count(it, rows_per_group, window);
         const uint32_t units = g.kv_heads * ((it.rows + rows_per_group - 1) / rows_per_group);
         uint32_t splits = std::max<uint32_t>(uint32_t((nblocks + T - 1) / T), 1);
-        const uint32_t bps = std::max<uint32_t>((nblocks + splits - 1) / splits, 1);
+        uint32_t bps = std::max<uint32_t>((nblocks + splits - 1) / splits, 1);
+        // A launch that appends its own rows: the workgroups of a unit's last split convert
+        // the new rows and write them over their last blocks, about a block's time for every
+        // eight rows, and the launch ends with them; their run is made that much shorter and
+        // the other splits share the difference.
+        if (appends && splits > 1) {
+            const uint32_t extra = std::min<uint32_t>(it.rows / 8 + 1, bps / 2);
+            const uint32_t longer = (nblocks + extra + splits - 1) / splits;
+            if (uint64_t(splits - 1) * longer < nblocks) bps = longer;
+        }
         splits = std::max<uint32_t>((nblocks + bps - 1) / bps, 1);
         it.splits = splits;
         it.keys_per_split = bps * kBlockKeys;
@@ -543,6 +669,7 @@ hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, uint
     if (b.total_blocks == 0) return hipSuccess;
     hipError_t e = hipSuccess;
     const bool one = tiles_for(b, p.group) == 1;
+    if (p.k_new && !one) return hipErrorInvalidValue;  // only the one-tile form appends
 #define ITAK_LAUNCH_TILES(SC, RING)                                                            \
     do {                                                                                       \
         if (one)                                                                               \

@@ -394,7 +394,11 @@ hipError_t launch_attn_splitk_f32(const AttnParams &p, const AttnBatch &b, uint3
 // otherwise not fill the device. Partials are in log2 domain (combine with base2 = 1).
 bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group);
 uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, uint32_t q_heads,
-                               uint32_t window);
+                               uint32_t window, bool appends = false);
+// True when a launch of the block kernel over items of at most `most_rows` rows and
+// `most_blocks` key blocks appends the items' rows itself (k_new / v_new in its parameters).
+bool attn_prefill_f16_appends(const PoolGeom &g, uint32_t group, uint32_t most_rows,
+                              uint32_t most_blocks);
 hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                    hipStream_t stream);
 // Merge of split partials; total_rows = query rows of the batch. With `gate` the merged rows

@@ -500,7 +500,7 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         if (mfma) {
             partials = attn_splitk_f16_plan(geom, b, uint32_t(q_heads));
         } else if (prefill) {
-            partials = attn_prefill_f16_plan(geom, b, group, uint32_t(q_heads), window);
+            partials = attn_prefill_f16_plan(geom, b, group, uint32_t(q_heads), window, k_new != nullptr);
         } else if (f32fast) {
             partials = attn_splitk_f32_plan(geom, b, uint32_t(q_heads));
         } else {
@@ -570,7 +570,7 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
                       ULL(layer), count, total_rows, ULL(q_heads), ULL(pool->g.kv_heads), ULL(view_len),
                       window, double(scale), double(softcap),
                       mfma ? "splitk_f16" : prefill ? "prefill_f16" : f32fast ? "splitk_f32" : "generic",
-                      b.total_blocks, splits, int(k_new != nullptr && (mfma || f32fast)),
+                      b.total_blocks, splits, int(k_new != nullptr && (mfma || f32fast || prefill)),
                       partials == 0 ? "none" : exchange_words ? "in_launch" : "launch");
         }
         AttnParams p{};
@@ -584,8 +584,8 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         p.ws = ws;
         p.exchange = exchange_words ? 1 : 0;
         p.spin_limit = pool->spin_limit;
-        p.k_new = (mfma || f32fast) ? k_new : nullptr;
-        p.v_new = (mfma || f32fast) ? v_new : nullptr;
+        p.k_new = (mfma || f32fast || prefill) ? k_new : nullptr;  // the caller passes them only to
+        p.v_new = (mfma || f32fast || prefill) ? v_new : nullptr;  // launches that append themselves
         p.q_heads = uint32_t(q_heads);
         p.group = group;
         p.group_magic = (65536u + group - 1) / group;
@@ -2101,8 +2101,16 @@ static itak_status step_on_device(itak_pool *pool, uint64_t layer, const itak_ba
         if (p.rows) active.push_back(p);
     uint32_t most_rows = 0;
     for (const PlanInput &p : active) most_rows = std::max(most_rows, p.rows);
+    // Mid-size blocks on f16 pools: the block kernel in its one-tile form appends too.
+    uint32_t most_blocks = 0;
+    for (const PlanInput &p : active)
+        most_blocks = std::max(most_blocks, (p.kv_len + 31) / 32 - p.kv_lo / 32);
+    const bool splitk = takes_splitk_f16(pool, active.data(), uint32_t(active.size()), num_q_heads, nullptr);
+    const bool block_fuses =
+        !splitk && pool->elem_f16 && !active.empty() &&
+        attn_prefill_f16_appends(pool->g, uint32_t(num_q_heads / pool->g.kv_heads), most_rows, most_blocks);
     const bool fuse =
-        takes_splitk_f16(pool, active.data(), uint32_t(active.size()), num_q_heads, nullptr) ||
+        splitk || block_fuses ||
         (!pool->elem_f16 && !active.empty() &&
          attn_splitk_f32_supports(pool->g, uint32_t(num_q_heads / pool->g.kv_heads), most_rows));
     // The allocation-free form plans first and refuses, before anything changes, a step whose

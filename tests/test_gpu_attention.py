@@ -306,7 +306,78 @@ def test_mid_size_blocks_split_over_the_context(rows, ctx, softcap):
     want = oracle.attention_step(ref, 0, q, k[ctx:], v[ctx:], q_heads, ctx,
                                  oracle.AttentionParams(softcap=softcap), threads=8)
     assert max_abs(out.cpu().numpy().reshape(-1), want) <= 2e-3
+    # Blocks of up to 64 rows bring their rows along (the block kernel appends them itself):
+    # what the cache then holds is what a separate append leaves, bit for bit.
+    _, rk, rv = ref.view(0).rows()
+    _, ck, cv = cache.view(0).rows()
+    as_f32 = lambda a: np.asarray(a).view(np.float16).astype(np.float32) if np.asarray(a).dtype == np.uint16 \
+        else np.asarray(a, dtype=np.float32)
+    assert as_f32(ck).tobytes() == as_f32(rk).tobytes()
+    assert as_f32(cv).tobytes() == as_f32(rv).tobytes()
     pool.close()
+
+
+@pytest.mark.parametrize("rows,ctx,window,group", [
+    (64, 4096, None, 8), (33, 1000, None, 8), (16, 4100, None, 8), (17, 31, None, 8),
+    (64, 200, None, 4), (40, 3000, None, 2), (64, 4096 + 13, None, 8),
+    (64, 5000, 1024, 8), (20, 2030, 1024, 8), (48, 1000, 256, 4)])
+def test_blocks_that_append_their_own_rows_leave_the_cache_as_a_separate_append_does(rows, ctx, window,
+                                                                                     group):
+    # The block kernel's one-tile form takes the new rows as parameters: converted in the
+    # prologue, written over the tail blocks in LDS by every workgroup that reads them, stored
+    # to the planes by one workgroup per KV head. Outputs against the oracle, stored rows bit for
+    # bit against a pool that appended first (through the append kernel), and the next steps on
+    # top of them; global and sliding-window layers (rings wrapped), several slots at once.
+    import torch
+    kv_heads, d = 4, 128
+    q_heads = kv_heads * group
+    rng = np.random.default_rng(rows * 7 + ctx)
+    kind = P().LayerKind.Global if window is None else P().LayerKind.windowed(window)
+    okind = oracle.LayerKind.Global if window is None else oracle.LayerKind.windowed(window)
+    slots = 2
+    pool = P().KvPool([kind], kv_heads, d, elem="f16", max_slots=slots, capacity_rows=ctx + 4 * rows + 8,
+                      ring_headroom=64)
+    plain = P().KvPool([kind], kv_heads, d, elem="f16", max_slots=slots, capacity_rows=ctx + 4 * rows + 8,
+                       ring_headroom=64)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    plain.set_stream(torch.cuda.current_stream().cuda_stream)
+    caches = [pool.acquire() for _ in range(slots)]
+    pcaches = [plain.acquire() for _ in range(slots)]
+    refs = [oracle.KvCache.new([okind], kv_heads, d, store_f16=True) for _ in range(slots)]
+    ctxs = [ctx, max(ctx - 37, 1)]
+    for s in range(slots):
+        k, v = normal(rng, ctxs[s], kv_heads * d), normal(rng, ctxs[s], kv_heads * d)
+        kd, vd = torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda()
+        for p0 in range(0, ctxs[s], 64):
+            n = min(64, ctxs[s] - p0)
+            pool.append_device(0, [(caches[s], n)], kd[p0:].data_ptr(), vd[p0:].data_ptr())
+            plain.append_device(0, [(pcaches[s], n)], kd[p0:].data_ptr(), vd[p0:].data_ptr())
+        for i in range(ctxs[s]):
+            refs[s].append(0, k[i], v[i], i)
+    for step_rows in (rows, rows, 1, max(rows // 2, 9)):
+        per = [step_rows, max(step_rows - 3, 9)]   # the second slot's block is a little shorter
+        total = sum(per)
+        q = normal(rng, total, q_heads * d)
+        k, v = normal(rng, total, kv_heads * d), normal(rng, total, kv_heads * d)
+        qd, kd, vd = (torch.from_numpy(a).cuda() for a in (q, k, v))
+        out = torch.empty_like(qd)
+        pool.attention_step_device(0, list(zip(caches, per)), qd.data_ptr(), kd.data_ptr(), vd.data_ptr(),
+                                   out.data_ptr(), q_heads)
+        plain.append_device(0, list(zip(pcaches, per)), kd.data_ptr(), vd.data_ptr())
+        pool.synchronize()
+        got = out.cpu().numpy()
+        row0 = 0
+        for s in range(slots):
+            base = refs[s].next_position(0)
+            want = oracle.attention_step(refs[s], 0, q[row0:row0 + per[s]], k[row0:row0 + per[s]],
+                                         v[row0:row0 + per[s]], q_heads, base, threads=8)
+            assert max_abs(got[row0:row0 + per[s]].reshape(-1), want) <= 2e-3, (s, step_rows)
+            row0 += per[s]
+            a, b = caches[s].read_raw(0), pcaches[s].read_raw(0)
+            assert a[0].tobytes() == b[0].tobytes() and a[1].tobytes() == b[1].tobytes(), (s, step_rows)
+            assert caches[s].next_position(0) == refs[s].next_position(0)
+    pool.close()
+    plain.close()
 
 
 @pytest.mark.gpu
