@@ -273,11 +273,31 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                          : "n"(4 * (STAGES - 1))
                          : "memory");
             ITAK_Q_CONVERT(qraw)
+            // The conversion rule (f32_to_f16_bits) is the hardware's rounding plus a fixed
+            // pattern for NaNs: a sum that is not a NaN proves its four terms are not, so the
+            // wavefront converts in pairs and takes the element-wise rule only when some lane
+            // met a NaN (or an infinity that cancelled). Pieces past the block's rows repeat
+            // its last row and are never written anywhere: skipped.
+            bool nan_seen = false;
 #pragma unroll
             for (int u = 0; u < kFusePieces; ++u) {
-                const uint32_t h0 = f32_to_f16_bits(nraw[u][0]), h1 = f32_to_f16_bits(nraw[u][1]);
-                const uint32_t h2 = f32_to_f16_bits(nraw[u][2]), h3 = f32_to_f16_bits(nraw[u][3]);
-                npk[u] = uint2{h0 | (h1 << 16), h2 | (h3 << 16)};
+                const float sum = (nraw[u][0] + nraw[u][1]) + (nraw[u][2] + nraw[u][3]);
+                nan_seen = nan_seen || sum != sum;
+            }
+            const bool by_element = __builtin_amdgcn_ballot_w64(nan_seen) != 0;
+#pragma unroll
+            for (int u = 0; u < kFusePieces; ++u) {
+                if (wave + 4u * u >= item.rows) continue;
+                if (by_element) {
+                    const uint32_t h0 = f32_to_f16_bits(nraw[u][0]), h1 = f32_to_f16_bits(nraw[u][1]);
+                    const uint32_t h2 = f32_to_f16_bits(nraw[u][2]), h3 = f32_to_f16_bits(nraw[u][3]);
+                    npk[u] = uint2{h0 | (h1 << 16), h2 | (h3 << 16)};
+                } else {
+                    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+                    const half2_t lo{static_cast<_Float16>(nraw[u][0]), static_cast<_Float16>(nraw[u][1])};
+                    const half2_t hi{static_cast<_Float16>(nraw[u][2]), static_cast<_Float16>(nraw[u][3])};
+                    npk[u] = uint2{__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi)};
+                }
             }
         }
     }

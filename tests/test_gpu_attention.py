@@ -317,6 +317,45 @@ def test_mid_size_blocks_split_over_the_context(rows, ctx, softcap):
     pool.close()
 
 
+@pytest.mark.parametrize("rows", [9, 40, 64])
+def test_blocks_that_append_their_own_rows_convert_every_class_of_value_as_append_does(rows):
+    # NaNs with payloads and either sign, infinities (a pair that cancels in a sum included),
+    # overflow, subnormals and ties among the new rows: the stored bits equal the append kernel's.
+    # (The outputs of such a step are NaN in any implementation and are not compared.)
+    import torch
+    kv_heads, d, ctx = 4, 128, 700
+    rng = np.random.default_rng(rows)
+    k, v = normal(rng, ctx + rows, kv_heads * d), normal(rng, ctx + rows, kv_heads * d)
+    specials = np.array([np.nan, -np.nan, np.inf, -np.inf, 65504.0, 65520.0, 1e9, -7e4, 6e-8, -3e-8,
+                         5.9604645e-8, 2.9802322e-8, 1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 0.0, -0.0],
+                        dtype=np.float32)
+    payload = np.array([0x7fc12345, 0xffa00001, 0x7f800001, 0xff812345], dtype=np.uint32).view(np.float32)
+    for arr in (k, v):
+        tail = arr[ctx:].reshape(-1)
+        idx = rng.choice(tail.size, size=400, replace=False)
+        tail[idx[:300]] = rng.choice(specials, size=300)
+        tail[idx[300:]] = rng.choice(payload, size=100)
+        tail[:4] = [np.inf, -np.inf, 1.0, 2.0]      # one piece whose sum is a NaN without a NaN in it
+    q = normal(rng, rows, 32 * d)
+    pools = [P().KvPool(1, kv_heads, d, elem="f16", capacity_rows=ctx + rows) for _ in range(2)]
+    caches = [p.acquire() for p in pools]
+    kd, vd, qd = (torch.from_numpy(a).cuda() for a in (k, v, q))
+    out = torch.empty_like(qd)
+    for p, c in zip(pools, caches):
+        p.set_stream(torch.cuda.current_stream().cuda_stream)
+        p.append_device(0, [(c, ctx)], kd.data_ptr(), vd.data_ptr())
+    pools[0].attention_step_device(0, [(caches[0], rows)], qd.data_ptr(), kd[ctx:].data_ptr(),
+                                   vd[ctx:].data_ptr(), out.data_ptr(), 32)
+    pools[1].append_device(0, [(caches[1], rows)], kd[ctx:].data_ptr(), vd[ctx:].data_ptr())
+    pools[0].synchronize()
+    a, b = caches[0].read_raw(0), caches[1].read_raw(0)
+    assert a[0].tobytes() == b[0].tobytes() and a[1].tobytes() == b[1].tobytes()
+    want = oracle.f32_to_f16_array(k[ctx:]).reshape(rows, kv_heads, d)
+    assert a[0][ctx:ctx + rows].view(np.uint16).tobytes() == np.asarray(want).view(np.uint16).tobytes()
+    for p in pools:
+        p.close()
+
+
 @pytest.mark.parametrize("rows,ctx,window,group", [
     (64, 4096, None, 8), (33, 1000, None, 8), (16, 4100, None, 8), (17, 31, None, 8),
     (64, 200, None, 4), (40, 3000, None, 2), (64, 4096 + 13, None, 8),
