@@ -59,6 +59,7 @@ constexpr int kMaxTiles = 2;  // MFMA column tiles (16 query vectors) per wavefr
 constexpr int kBlockElems = kBlockKeys * kD;        // 4096 halves = 8 KiB per plane block
 constexpr float kRefSlack = 8.0f;
 constexpr int kFuseRows = 64;  // new rows a launch that appends its own rows carries at most
+constexpr uint32_t kOneTileBlocks = 520;  // key blocks up to which blocks of <= 512 vectors take one tile
 constexpr int kFusePieces = kFuseRows * 2 * (kD / 4) / (kWaves * 64);  // per thread
 
 __device__ __forceinline__ float column_max4(float v) {
@@ -568,7 +569,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
 bool attn_prefill_f16_appends(const PoolGeom &g, uint32_t group, uint32_t most_rows,
                               uint32_t most_blocks) {
     return attn_prefill_f16_supports(g, group) && most_rows <= uint32_t(kFuseRows) &&
-           most_rows * group <= 512 && most_blocks <= 256;
+           most_rows * group <= 512 && most_blocks <= kOneTileBlocks;
 }
 
 bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group) {
@@ -578,12 +579,14 @@ bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group) {
 
 // Up to 64 query vectors per KV head (speculative blocks) take one 16-vector tile per
 // wavefront, so that all four wavefronts of the workgroup have columns; more take two.
-// So do blocks of up to 512 vectors over at most 256 key blocks (a draft tree of 16 to 32
-// tokens, or a 64-row chunk, at a context up to 8192): the launch has to split the context
-// anyway, and with twice the row tiles it needs half the splits, half the partials to write
-// and merge (measured at context 4096: 16 rows 20.6 -> 17.7 us, 32 rows 24.0 -> 21.2 us,
-// 64 rows 25.1 -> 23.7 us; at context 30720 the second pass over the keys costs more than
-// the partials saved).
+// So do blocks of up to 512 vectors over at most kOneTileBlocks key blocks (a draft tree of 16
+// to 32 tokens, or a 64-row chunk, at a context up to 16384): the launch has to split the
+// context anyway, with twice the row tiles it needs half the splits, half the partials to
+// write and merge, and the one-tile form appends the block's rows itself (measured per layer,
+// one tile and its own append against two tiles behind an append launch: context 8192, 9 / 16 /
+// 32 / 64 rows 19.7 / 22.6 / 25.9 / 30.3 -> 16.6 / 19.2 / 20.9 / 30.2 us; context 16384, 23.1 /
+// 25.6 / 30.2 / 37.6 -> 20.3 / 21.1 / 26.2 / 36.5; at context 30720 the second pass over the
+// keys costs more than it saves: 26.7 -> 29.0 and 38.4 -> 45.2 us for 9 and 32 rows).
 static int tiles_for(const AttnBatch &b, uint32_t group) {
     uint32_t nvec = 0, nblocks = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
@@ -591,7 +594,7 @@ static int tiles_for(const AttnBatch &b, uint32_t group) {
         nblocks = std::max(nblocks, item_block_count(b.item[i]));
     }
     if (nvec <= uint32_t(kWaves * 16)) return 1;
-    return nvec <= 512 && nblocks <= 256 ? 1 : kMaxTiles;
+    return nvec <= 512 && nblocks <= kOneTileBlocks ? 1 : kMaxTiles;
 }
 
 // Fills splits / keys_per_split / block0 / ws0 for a batch (slot, rows, pos0, q_row0, kv_len

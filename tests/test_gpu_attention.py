@@ -280,6 +280,8 @@ def test_speculative_round_trip_rewind_restores_the_exact_continuation():
     (9, 3000, 0.0), (40, 5000, 0.0),
     # 8 to 40 key blocks per compute unit in all: the block kernel's deep-ring instantiation.
     (130, 2100, 25.0), (64, 4096, 0.0), (48, 6000, 0.0),
+    # between 256 and 520 key blocks: still one tile per wavefront, rows appended by the kernel
+    (24, 9000, 0.0), (64, 16384, 30.0),
 ])
 def test_mid_size_blocks_split_over_the_context(rows, ctx, softcap):
     # Blocks too long for the decode kernel and too short to fill the device by rows alone:
@@ -359,7 +361,7 @@ def test_blocks_that_append_their_own_rows_convert_every_class_of_value_as_appen
 @pytest.mark.parametrize("rows,ctx,window,group", [
     (64, 4096, None, 8), (33, 1000, None, 8), (16, 4100, None, 8), (17, 31, None, 8),
     (64, 200, None, 4), (40, 3000, None, 2), (64, 4096 + 13, None, 8),
-    (64, 5000, 1024, 8), (20, 2030, 1024, 8), (48, 1000, 256, 4)])
+    (64, 5000, 1024, 8), (20, 2030, 1024, 8), (48, 1000, 256, 4), (31, 10000, None, 8)])
 def test_blocks_that_append_their_own_rows_leave_the_cache_as_a_separate_append_does(rows, ctx, window,
                                                                                      group):
     # The block kernel's one-tile form takes the new rows as parameters: converted in the
