@@ -398,7 +398,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", choices=["decode", "ragged", "verify", "prefill", "hybrid",
-                                           "prefill_windowed", "restore", "append"],
+                                           "prefill_windowed", "restore", "append", "chunk64"],
                     default="decode")
     ap.add_argument("--softcap", type=float, default=0.0)
     ap.add_argument("--kv", choices=["f16", "f32"], default="f16",
@@ -450,7 +450,7 @@ def main():
         # kernel's figure; `metric`, `value` and `config` stay those of the decode step.
         import copy
         workloads = {"decode": summary_of(result)}
-        for wl in ("ragged", "verify", "prefill", "restore"):
+        for wl in ("ragged", "verify", "prefill", "restore", "chunk64"):
             sub = copy.copy(args)
             sub.workload, sub.no_cpu_baseline, sub.prep = wl, True, False
             sub.steps, sub.warmup = max(10, args.steps // 4), max(3, args.warmup // 4)
@@ -494,6 +494,12 @@ def run_workload(args, pkg, torch, np, dev, stream, timed):
         layers, slots, rows, lengths = 16, 4, 7, [8192] * 4
         name = ("configs[3]: speculative verify block, 4 slots at context 8192, 7 query rows "
                 "appended and attended causally, 30B-class heads, f16 KV, 16 layers cycled")
+    elif wl == "chunk64":
+        layers, slots, rows, lengths = 16, 1, 64, [4096]
+        name = ("the reference's own prefill chunk (crates/wgpu-compute/src/session.rs:186-195): 64 rows "
+                "appended and attended causally at context 4096, 30B-class heads, f16 KV, 16 layers "
+                "cycled; the block kernel splits the context, appends the rows itself and a merge "
+                "launch follows")
     elif wl == "hybrid":
         layers, slots, rows, lengths = 8, 1, 1, [32768]
         name = ("hybrid decode step: sliding-window layers (window 2048) and global layers 3:1, "
@@ -539,7 +545,7 @@ def run_workload(args, pkg, torch, np, dev, stream, timed):
     q = torch.randn(layers, total_rows, Q_HEADS * D, device=dev)
     k_new = torch.randn(layers, total_rows, ROW, device=dev)
     v_new = torch.randn(layers, total_rows, ROW, device=dev)
-    if wl.startswith("prefill"):  # f16-valued Q/K/V
+    if wl.startswith("prefill") or wl == "chunk64":  # f16-valued Q/K/V
         q, k_new, v_new = q.half().float(), k_new.half().float(), v_new.half().float()
     out = torch.empty_like(q)
     for layer in range(layers):
@@ -677,7 +683,27 @@ def run_workload(args, pkg, torch, np, dev, stream, timed):
                      "append + attention; the gate in the merge kernel"),
         }
 
-    if wl.startswith("prefill"):
+    if wl == "chunk64":
+        # Neither roofline describes this shape (4.3 GFLOP and 8 MB of KV per layer, 5 us of
+        # either): the figure is the layer's time; TFLOP/s and the MFMA fraction go with it.
+        metric, unit = "prefill attention TFLOP/s (64-row chunk at context 4096)", "TFLOP/s"
+        value = flops_layer * layers / step_s / 1e12
+        roofline = {
+            "bound": "mfma",
+            "kernel": "attn_prefill_f16_kernel (one tile per wavefront, appends the chunk's rows) + "
+                      "attn_combine128_wave_kernel",
+            "achieved": round(value, 2),
+            "peak": MFMA_F16_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(value / MFMA_F16_PEAK_TFLOPS, 4),
+            "traffic": None,
+            "us_per_launch": round(step_s / layers * 1e6, 2),
+            "flops_per_launch": flops_layer,
+            "timed": "one layer of the timed step (HIP graph replay of all layers): append + "
+                     "attention in the block kernel's launch, then the merge launch",
+            "attention_only_us_per_launch": round(attn_s * 1e6, 2),
+        }
+    elif wl.startswith("prefill"):
         metric, unit = "prefill attention TFLOP/s (2048-row chunk over 30720 prefix)", "TFLOP/s"
         if wl == "prefill_windowed":
             metric = "prefill attention TFLOP/s (2048-row chunk, window 2048)"
