@@ -132,7 +132,9 @@ def test_long_positions_need_the_f64_angle_law():
 
 @pytest.mark.parametrize("rows,interleaved,rotary,norm,rope_base", [
     (7, True, 0, True, 1e6), (7, False, 0, True, 1e4), (5, False, 64, False, 1e4),
-    (5, True, 32, True, 5e5), (1, True, 0, True, 0.0), (200, True, 0, True, 1e6)])
+    (5, True, 32, True, 5e5), (1, True, 0, True, 0.0), (200, True, 0, True, 1e6),
+    # 9 to 64 rows: the preparation launch, then the block kernel that appends the prepared rows itself
+    (20, True, 0, True, 1e6), (40, False, 64, True, 1e4), (64, True, 0, True, 5e5)])
 def test_blocks_pairings_partial_rotary_and_nope(rows, interleaved, rotary, norm, rope_base):
     run_case("f16", 32, 4, 128, ctx=150, rows=rows, norm=norm, rope_base=rope_base,
              interleaved=interleaved, rotary=rotary, gate=(rows < 100), seed=rows)
