@@ -635,7 +635,21 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
     const bool deep = unit_blocks >= 8 * per_cu && unit_blocks <= 40 * per_cu;
     b.deep_ring = deep ? 1 : 0;
     const uint64_t target = deep ? per_cu : 2 * per_cu;
-    const uint64_t T = std::max<uint64_t>((unit_blocks + target - 1) / target, 8);
+    uint64_t T = std::max<uint64_t>((unit_blocks + target - 1) / target, 8);
+    // Rounding the splits up per unit can leave a few workgroups more than the device takes at
+    // once, and those few run alone in a second round (96 rows at context 4096: 264 workgroups
+    // on 256 compute units, 38.5 us where 128 rows take 34.4): lengthen the runs until the
+    // launch fits, when the first estimate says it nearly does (96 / 160 / 192 / 384 rows at
+    // context 4096: 38.5 / 48.1 / 51.9 / 63.0 -> 29.2 / 36.6 / 38.0 / 52.0 us).
+    for (; T < unit_blocks; ++T) {
+        uint64_t groups = 0;
+        for (uint32_t i = 0; i < b.n; ++i) {
+            const uint64_t nb = unit_block_count(b.item[i], rows_per_group, window);
+            const uint64_t units = uint64_t(g.kv_heads) * ((b.item[i].rows + rows_per_group - 1) / rows_per_group);
+            groups += units * std::max<uint64_t>((nb + T - 1) / T, 1);
+        }
+        if (groups <= target || groups > target + target / 4) break;
+    }
     uint32_t block0 = 0, ws0 = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         AttnItem &it = b.item[i];
