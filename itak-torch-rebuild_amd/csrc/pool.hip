@@ -1005,13 +1005,17 @@ itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out) {
     // in 69 us per layer with planes of 129 blocks of 8 KiB and in 51 us with 128 or 130 (127,
     // 254, 258, 387 and 516 blocks likewise 60 to 66 us against 52). Such a plane gets one more
     // block; the rows are never addressed (a ring's length is its own).
+    // The distance between two slots' planes of a head (2 * kv_heads planes) is held to the same
+    // rule: that is the spacing of a batch's streams.
     auto spread = [&](uint64_t rows) -> uint64_t {
         const uint64_t step = kVBlock;
-        for (int guard = 0; guard < 4; ++guard) {
+        auto bad = [](uint64_t bytes) {
+            return bytes != 0 && (bytes % ((1u << 20) + (1u << 13)) == 0 ||
+                                  bytes % ((1u << 20) - (1u << 13)) == 0);
+        };
+        for (int guard = 0; guard < 8; ++guard) {
             const uint64_t plane_bytes = rows * config->head_dim * elem_bytes;
-            if (plane_bytes == 0 || (plane_bytes % ((1u << 20) + (1u << 13)) != 0 &&
-                                     plane_bytes % ((1u << 20) - (1u << 13)) != 0))
-                break;
+            if (!bad(plane_bytes) && !bad(plane_bytes * 2 * config->num_kv_heads)) break;
             rows += step;
         }
         return rows;
