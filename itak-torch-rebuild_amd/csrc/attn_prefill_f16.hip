@@ -656,6 +656,12 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
         const uint32_t nblocks = unit_block_count(it, rows_per_group, window);
         const uint32_t units = g.kv_heads * ((it.rows + rows_per_group - 1) / rows_per_group);
         uint32_t splits = std::max<uint32_t>(uint32_t((nblocks + T - 1) / T), 1);
+        // A short context is not worth splitting once the row tiles alone keep a good part of
+        // the device busy: the partials and the merge launch cost more than the blocks saved
+        // (no prefix, 384 / 512 / 768 rows: 31.0 / 35.4 / 49.1 -> 20.7 / 25.4 / 31.6 us per
+        // layer; 192 / 256 / 512 rows over a 512-row prefix: 29.2 / 31.7 / 40.4 -> 25.4 / 26.6 /
+        // 35.0; with 32 units, a 64-row chunk, the splits are what fills the device and stay).
+        if (nblocks < 40 && units >= 48) splits = 1;
         uint32_t bps = std::max<uint32_t>((nblocks + splits - 1) / splits, 1);
         // A launch that appends its own rows: the workgroups of a unit's last split convert
         // the new rows and write them over their last blocks, about a block's time for every

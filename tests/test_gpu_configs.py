@@ -271,7 +271,9 @@ def test_reduced_prefill_matches_the_oracle_on_every_row():
     # The same path at a size the oracle covers completely, from an empty cache and over a
     # prefix, with and without softcap.
     rng = np.random.default_rng(7)
-    for prefix, chunk, softcap in ((0, 200, 0.0), (333, 150, 30.0)):
+    # (The last two: contexts short enough that the row tiles are left unsplit although the
+    # launch is far from filling the device; a prompt's first chunk.)
+    for prefix, chunk, softcap in ((0, 200, 0.0), (333, 150, 30.0), (0, 520, 0.0), (500, 390, 0.0)):
         k, v = normal(rng, prefix + chunk, ROW), normal(rng, prefix + chunk, ROW)
         q = normal(rng, chunk, Q_HEADS * D)
         pool = P().KvPool(1, KV_HEADS, D, elem="f16", capacity_rows=prefix + chunk)
