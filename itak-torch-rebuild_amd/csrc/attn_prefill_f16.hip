@@ -117,9 +117,19 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     const uint32_t rows_per_wave = kVecPerWave / group;
     // Workgroup -> (row tile, kv head, split of the context).
     const uint32_t local = blockIdx.x - item.block0;
-    const uint32_t unit = local / item.splits, split = local - unit * item.splits;
-    const uint32_t kv_head = unit % p.g.kv_heads;
+    uint32_t unit = local / item.splits;
+    const uint32_t split = local - unit * item.splits;
     const uint32_t tiles = (item.rows + rows_per_group - 1) / rows_per_group;
+    // Units are handed out longest row tile first. All of an unsplit causal launch's first two
+    // runs (one workgroup per compute unit each) are resident from the start, the second run
+    // beside the first: taken in the same order, the longest tiles would share their compute
+    // units with the longest of the second half. Every second run is taken in reverse.
+    if (p.fold_units) {
+        const uint32_t run = unit / p.fold_units, idx = unit - run * p.fold_units;
+        const uint32_t span = min(p.fold_units, tiles * p.g.kv_heads - run * p.fold_units);
+        if (run & 1) unit = run * p.fold_units + (span - 1 - idx);
+    }
+    const uint32_t kv_head = unit % p.g.kv_heads;
     const uint32_t tile = tiles - 1 - unit / p.g.kv_heads;  // longest first
     const uint32_t row_begin = tile * rows_per_group + wave * rows_per_wave;
     const uint32_t wg_row_end = min(item.rows, (tile + 1) * rows_per_group);
@@ -634,6 +644,7 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
     // context 30720 36.3 -> 31.6 us; above the range it loses, below it nothing changes).
     const bool deep = unit_blocks >= 8 * per_cu && unit_blocks <= 40 * per_cu;
     b.deep_ring = deep ? 1 : 0;
+    b.fold_units = 0;
     const uint64_t target = deep ? per_cu : 2 * per_cu;
     uint64_t T = std::max<uint64_t>((unit_blocks + target - 1) / target, 8);
     // Rounding the splits up per unit can leave a few workgroups more than the device takes at
@@ -662,6 +673,12 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
         // layer; 192 / 256 / 512 rows over a 512-row prefix: 29.2 / 31.7 / 40.4 -> 25.4 / 26.6 /
         // 35.0; with 32 units, a 64-row chunk, the splits are what fills the device and stay).
         if (nblocks < 40 && units >= 48) splits = 1;
+        // Nor is any context, once the units give most compute units their two workgroups
+        // (384 units, 1536 rows: no prefix 83.6 -> 49.3 us, over 2048 rows 138 -> 100, over
+        // 8192 290 -> 262, over 30720 829 -> 792), or each its one on a context under 128
+        // blocks (256 units over 2048 rows: 83.8 -> 77.4; from 160 blocks on the split form,
+        // two workgroups of half the run on every compute unit, is the faster one).
+        if (uint64_t(units) * 2 >= 3 * per_cu || (units >= per_cu && nblocks < 128)) splits = 1;
         uint32_t bps = std::max<uint32_t>((nblocks + splits - 1) / splits, 1);
         // A launch that appends its own rows: the workgroups of a unit's last split convert
         // the new rows and write them over their last blocks, about a block's time for every
@@ -683,6 +700,14 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
     }
     b.total_blocks = block0;
     b.rows_per_block = rows_per_group;
+    // One unsplit item whose row tiles see different numbers of blocks (no window) and whose
+    // workgroups are all resident from the start, two to a compute unit: fold the second run
+    // (see the kernel; 2048 rows without a prefix 64.9 -> 61.6 us per layer). With more runs
+    // the later workgroups go wherever one ends, which balances better unfolded (4096 and 8192
+    // rows measured 1 to 3 % slower folded).
+    if (b.n == 1 && b.item[0].splits == 1 && window == 0 && !deep && block0 > per_cu &&
+        block0 <= 2 * per_cu)
+        b.fold_units = uint32_t(per_cu);
     return ws0;
 }
 

@@ -233,6 +233,7 @@ struct AttnBatch {
     uint32_t total_blocks;
     uint32_t rows_per_block;
     uint32_t deep_ring;  // host side only: the block kernel's plan asks for its deeper LDS ring
+    uint32_t fold_units; // host side only: the block kernel's plan for AttnParams::fold_units
     AttnItem item[kMaxBatchItems];
 };
 // The kernel argument form of AttnBatch, sized to the batch: kernel arguments are
@@ -316,6 +317,10 @@ struct AttnParams {
     // gives up after spin_limit polls.
     uint32_t exchange;
     uint32_t spin_limit;
+    // Block kernel only, unsplit causal launches: workgroups reach the device in runs of this
+    // many (one per compute unit); every second run takes its units in reverse, so that the
+    // two workgroups that share a compute unit are a long row tile and a short one. 0 = off.
+    uint32_t fold_units;
 };
 // What the reference's model does around the step (muse-glimmer/src/model.rs:445-464),
 // folded into the step's own launches instead of running as launches of their own. `gate`

@@ -583,6 +583,7 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         p.q_pos = q_pos_dev;
         p.ws = ws;
         p.exchange = exchange_words ? 1 : 0;
+        p.fold_units = prefill ? b.fold_units : 0;
         p.spin_limit = pool->spin_limit;
         p.k_new = (mfma || f32fast || prefill) ? k_new : nullptr;  // the caller passes them only to
         p.v_new = (mfma || f32fast || prefill) ? v_new : nullptr;  // launches that append themselves
