@@ -58,6 +58,10 @@ constexpr int kWaves = 4;
 constexpr int kMaxTiles = 2;  // MFMA column tiles (16 query vectors) per wavefront: 1 or 2
 constexpr int kBlockElems = kBlockKeys * kD;        // 4096 halves = 8 KiB per plane block
 constexpr float kRefSlack = 8.0f;
+// The smallest divisor of 16 that holds a GQA group of up to 16 heads.
+__host__ __device__ inline uint32_t padded_group(uint32_t group) {
+    return group <= 1 ? 1 : group <= 2 ? 2 : group <= 4 ? 4 : group <= 8 ? 8 : 16;
+}
 constexpr int kFuseRows = 64;  // new rows a launch that appends its own rows carries at most
 constexpr uint32_t kOneTileBlocks = 520;  // key blocks up to which blocks of <= 512 vectors take one tile
 constexpr int kFusePieces = kFuseRows * 2 * (kD / 4) / (kWaves * 64);  // per thread
@@ -112,9 +116,12 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     ITAK_MARK(0)
 
     const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
-    const uint32_t group = p.group;
-    const uint32_t rows_per_group = kVecPerGroup / group;
-    const uint32_t rows_per_wave = kVecPerWave / group;
+    // A query row's heads of one KV group fill `gp` consecutive columns: the group size padded
+    // to the next divisor of 16 (a group of 5 takes 8 columns, three of them zero queries whose
+    // results are dropped), so that a row never straddles two MFMA tiles.
+    const uint32_t group = p.group, gp = padded_group(group);
+    const uint32_t rows_per_group = kVecPerGroup / gp;
+    const uint32_t rows_per_wave = kVecPerWave / gp;
     // Workgroup -> (row tile, kv head, split of the context).
     const uint32_t local = blockIdx.x - item.block0;
     uint32_t unit = local / item.splits;
@@ -227,12 +234,12 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
 #pragma unroll
     for (int qt = 0; qt < kTiles; ++qt) {
         const uint32_t j = qt * 16 + jl;
-        const uint32_t row = row_begin + j / group;
+        const uint32_t row = row_begin + j / gp, hq = j % gp;
         colpos[qt] = min(item.pos0 + row, item.kv_len - 1);
         collo[qt] = lowest_visible(item.pos0 + row, window, kv_lo);
-        const uint32_t head = kv_head * group + j % group;
+        const uint32_t head = kv_head * group + min(hq, group - 1);
         qp[qt] = p.q + (uint64_t(item.q_row0 + min(row, item.rows - 1)) * p.q_heads + head) * kD + g * 8;
-        qsc[qt] = row < item.rows ? qscale : 0.0f;
+        qsc[qt] = row < item.rows && hq < group ? qscale : 0.0f;
     }
 #define ITAK_Q_LOADS(qraw)                                                                      \
     _Pragma("unroll") for (int qt = 0; qt < kTiles; ++qt)                                       \
@@ -550,8 +557,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     for (int qt = 0; qt < kTiles; ++qt) {
         const float lt = l[qt][0];
         const uint32_t j = qt * 16 + jl;
-        const uint32_t row = row_begin + j / group, head = kv_head * group + j % group;
-        if (row >= item.rows) continue;
+        const uint32_t row = row_begin + j / gp, hq = j % gp, head = kv_head * group + hq;
+        if (row >= item.rows || hq >= group) continue;
         if (final_out) {
             const float inv = 1.0f / lt;
             float *dst = p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + g * 4;
@@ -579,12 +586,11 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
 bool attn_prefill_f16_appends(const PoolGeom &g, uint32_t group, uint32_t most_rows,
                               uint32_t most_blocks) {
     return attn_prefill_f16_supports(g, group) && most_rows <= uint32_t(kFuseRows) &&
-           most_rows * group <= 512 && most_blocks <= kOneTileBlocks;
+           most_rows * padded_group(group) <= 512 && most_blocks <= kOneTileBlocks;
 }
 
 bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group) {
-    return g.v_block == kVBlock && g.head_dim == kD && group >= 1 && group <= 16 &&
-           16 % group == 0;
+    return g.v_block == kVBlock && g.head_dim == kD && group >= 1 && group <= 16;
 }
 
 // Up to 64 query vectors per KV head (speculative blocks) take one 16-vector tile per
@@ -600,7 +606,7 @@ bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group) {
 static int tiles_for(const AttnBatch &b, uint32_t group) {
     uint32_t nvec = 0, nblocks = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
-        nvec = std::max(nvec, b.item[i].rows * group);
+        nvec = std::max(nvec, b.item[i].rows * padded_group(group));
         nblocks = std::max(nblocks, item_block_count(b.item[i]));
     }
     if (nvec <= uint32_t(kWaves * 16)) return 1;
@@ -625,7 +631,7 @@ static uint32_t unit_block_count(const AttnItem &it, uint32_t rows_per_group, ui
 
 uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, uint32_t q_heads,
                                uint32_t window, bool appends) {
-    const uint32_t rows_per_group = uint32_t(tiles_for(b, group) * kWaves * 16) / group;
+    const uint32_t rows_per_group = uint32_t(tiles_for(b, group) * kWaves * 16) / padded_group(group);
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)

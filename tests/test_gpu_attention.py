@@ -361,7 +361,9 @@ def test_blocks_that_append_their_own_rows_convert_every_class_of_value_as_appen
 @pytest.mark.parametrize("rows,ctx,window,group", [
     (64, 4096, None, 8), (33, 1000, None, 8), (16, 4100, None, 8), (17, 31, None, 8),
     (64, 200, None, 4), (40, 3000, None, 2), (64, 4096 + 13, None, 8),
-    (64, 5000, 1024, 8), (20, 2030, 1024, 8), (48, 1000, 256, 4), (31, 10000, None, 8)])
+    (64, 5000, 1024, 8), (20, 2030, 1024, 8), (48, 1000, 256, 4), (31, 10000, None, 8),
+    # groups that do not divide 16 take padded columns: 5 heads in 8, 3 in 4, 6 in 8, 12 in 16
+    (40, 1500, None, 5), (64, 900, None, 3), (30, 2000, 512, 6), (20, 1200, None, 12), (64, 700, None, 16)])
 def test_blocks_that_append_their_own_rows_leave_the_cache_as_a_separate_append_does(rows, ctx, window,
                                                                                      group):
     # The block kernel's one-tile form takes the new rows as parameters: converted in the

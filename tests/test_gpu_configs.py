@@ -296,6 +296,34 @@ def test_reduced_prefill_matches_the_oracle_on_every_row():
         pool.close()
 
 
+@pytest.mark.parametrize("q_heads,kv_heads", [(40, 8), (12, 4), (24, 4), (28, 4)])
+def test_prefill_chunks_with_groups_that_do_not_divide_sixteen(q_heads, kv_heads):
+    # Groups of 5, 3, 6 and 7 Q heads per KV head (40 / 8 is a common model shape): the block
+    # kernel pads a row's heads to 8 (or 4) MFMA columns instead of leaving such models to the
+    # generic kernel. A chunk over a prefix and a prompt's first chunk, every row checked.
+    rng = np.random.default_rng(q_heads)
+    row = kv_heads * D
+    for prefix, chunk in ((700, 300), (0, 260)):
+        k, v = normal(rng, prefix + chunk, row), normal(rng, prefix + chunk, row)
+        q = normal(rng, chunk, q_heads * D)
+        pool = P().KvPool(1, kv_heads, D, elem="f16", capacity_rows=prefix + chunk)
+        pool.set_stream(torch.cuda.current_stream().cuda_stream)
+        cache = pool.acquire()
+        kd, vd, qd = dev(k), dev(v), dev(q)
+        out = torch.empty_like(qd)
+        if prefix:
+            pool.append_device(0, [(cache, prefix)], kd.data_ptr(), vd.data_ptr())
+        pool.attention_step_device(0, [(cache, chunk)], qd.data_ptr(), kd[prefix:].data_ptr(),
+                                   vd[prefix:].data_ptr(), out.data_ptr(), q_heads)
+        torch.cuda.synchronize()
+        ref = oracle_cache(1, kv_heads, D, True)
+        if prefix:
+            ref.restore_bulk(0, 0, k[:prefix], v[:prefix])
+        want = oracle.attention_step(ref, 0, q, k[prefix:], v[prefix:], q_heads, prefix, threads=THREADS)
+        assert max_abs(out.cpu().numpy().reshape(-1), want) <= 2e-3
+        pool.close()
+
+
 def test_prefill_with_scores_that_climb_and_fall_along_the_context():
     # Key magnitudes ramp up and down along the context, so the softmax reference maximum
     # moves many times, by little and by a lot, and long runs of keys sit far below it; group sizes 8 and 2; with and without softcap.
