@@ -658,6 +658,10 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
     // on 256 compute units, 38.5 us where 128 rows take 34.4): lengthen the runs until the
     // launch fits, when the first estimate says it nearly does (96 / 160 / 192 / 384 rows at
     // context 4096: 38.5 / 48.1 / 51.9 / 63.0 -> 29.2 / 36.6 / 38.0 / 52.0 us).
+    // (Never by more than half: when the units alone outnumber the target, no run length fits,
+    // and a search to the end would leave every item unsplit, the decode rows of a mixed batch
+    // walking their whole context in one workgroup.)
+    const uint64_t T0 = T;
     for (; T < unit_blocks; ++T) {
         uint64_t groups = 0;
         for (uint32_t i = 0; i < b.n; ++i) {
@@ -666,6 +670,10 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
             groups += units * std::max<uint64_t>((nb + T - 1) / T, 1);
         }
         if (groups <= target || groups > target + target / 4) break;
+        if (T >= T0 + T0 / 2) {
+            T = T0;
+            break;
+        }
     }
     uint32_t block0 = 0, ws0 = 0;
     for (uint32_t i = 0; i < b.n; ++i) {

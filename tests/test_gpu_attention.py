@@ -319,6 +319,57 @@ def test_mid_size_blocks_split_over_the_context(rows, ctx, softcap):
     pool.close()
 
 
+@pytest.mark.parametrize("window", [None, 512])
+def test_a_step_that_mixes_decode_rows_a_verify_block_and_a_prefill_chunk(window):
+    # Continuous batching: one call carries slots that decode one row, a slot that verifies an
+    # 8-row block and a slot that prefills a 300-row chunk (a prompt's first chunk and a later
+    # one). Every slot's rows against the oracle, and the lengths afterwards.
+    import torch
+    q_heads, kv_heads, d = 32, 4, 128
+    rng = np.random.default_rng(77)
+    kind = P().LayerKind.Global if window is None else P().LayerKind.windowed(window)
+    okind = oracle.LayerKind.Global if window is None else oracle.LayerKind.windowed(window)
+    plan = [(3000, 1), (517, 1), (2100, 8), (0, 300), (1030, 300), (8000, 1)]   # (context, rows)
+    if window is not None:   # a ring takes a block no longer than its headroom
+        plan = [(3000, 1), (517, 1), (2100, 8), (0, 200), (1030, 200), (8000, 1)]
+    pool = P().KvPool([kind], kv_heads, d, elem="f16", max_slots=len(plan), capacity_rows=8400,
+                      ring_headroom=224)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    caches, refs = [], []
+    for ctx, _ in plan:
+        c = pool.acquire()
+        r = oracle.KvCache.new([okind], kv_heads, d, store_f16=True)
+        if ctx:
+            k, v = normal(rng, ctx, kv_heads * d), normal(rng, ctx, kv_heads * d)
+            kd, vd = torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda()
+            for p0 in range(0, ctx, 200):
+                n = min(200, ctx - p0)
+                pool.append_device(0, [(c, n)], kd[p0:].data_ptr(), vd[p0:].data_ptr())
+            first = 0 if window is None else max(0, ctx - window)
+            r.restore_bulk(0, first, k[first:], v[first:])
+        caches.append(c); refs.append(r)
+    for step in range(2):
+        rows = [n for _, n in plan]
+        total = sum(rows)
+        q = normal(rng, total, q_heads * d)
+        k, v = normal(rng, total, kv_heads * d), normal(rng, total, kv_heads * d)
+        qd, kd, vd = (torch.from_numpy(a).cuda() for a in (q, k, v))
+        out = torch.empty_like(qd)
+        pool.attention_step_device(0, list(zip(caches, rows)), qd.data_ptr(), kd.data_ptr(), vd.data_ptr(),
+                                   out.data_ptr(), q_heads)
+        pool.synchronize()
+        got = out.cpu().numpy()
+        row0 = 0
+        for s, n in enumerate(rows):
+            base = refs[s].next_position(0)
+            want = oracle.attention_step(refs[s], 0, q[row0:row0 + n], k[row0:row0 + n], v[row0:row0 + n],
+                                         q_heads, base, threads=8)
+            assert max_abs(got[row0:row0 + n].reshape(-1), want) <= 2e-3, (step, s)
+            assert caches[s].next_position(0) == refs[s].next_position(0) == base + n
+            row0 += n
+    pool.close()
+
+
 @pytest.mark.parametrize("rows", [9, 40, 64])
 def test_blocks_that_append_their_own_rows_convert_every_class_of_value_as_append_does(rows):
     # NaNs with payloads and either sign, infinities (a pair that cancels in a sum included),
