@@ -1,13 +1,15 @@
-// GQA flash-decode for gfx950 over f32 KV (the reference's own storage type), head_dim 128,
-// up to 16 query vectors per KV head (rows x group: decode steps and short blocks): split over
-// the context like the f16 kernel, products on v_mfma_f32_16x16x4_f32 (f32 in, f32 out: the
-// 1e-5 bar of f32 pools holds), K and V read straight from their row-major planes with 16-byte
-// loads, no LDS in the loop; a step's new rows are appended by the same launch. Everything
-// else (other head dims, more vectors, explicit query positions) stays on the generic kernel.
+// GQA attention for gfx950 over f32 KV (the reference's own storage type), head_dim 128:
+// decode steps, verify blocks and prefill chunks, split over the context like the f16 kernels,
+// products on v_mfma_f32_16x16x4_f32 (f32 in, f32 out: the 1e-5 bar of f32 pools holds), K and V
+// read straight from their row-major planes with 16-byte loads, no LDS in the loop; a short
+// step's new rows are appended by the same launch. Other head dims and explicit query
+// positions stay on the generic kernel.
 //
-// One workgroup of four wavefronts owns (item, kv head, split = a run of 32-key blocks); each
-// wavefront walks its own blocks with a private online softmax, the four merge once through
-// LDS. The MFMA takes one float per lane and operand: A[i][k] from lane i + 16k, B[k][j] from
+// One workgroup of four wavefronts owns (item, kv head, tile of 16 query vectors, split = a run
+// of 32-key blocks), a query vector being one row of one Q head of the group; a block of more
+// than 16 vectors is several tiles, each walking the keys its own rows see (tiles of later rows
+// first: they have the longest runs). Each wavefront walks its own blocks with a private online
+// softmax, the four merge once through LDS. The MFMA takes one float per lane and operand: A[i][k] from lane i + 16k, B[k][j] from
 // lane j + 16k, and returns rows 4g .. 4g+3 of column j to lane j + 16g. A dot product does
 // not care in which order its terms are taken, so the channels (for K.Q^T) and the keys (for
 // V^T.P^T) are assigned to the MFMA's k index in whatever order lets every lane fetch 16
@@ -63,19 +65,27 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
 
     const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
     const uint32_t local = blockIdx.x - item.block0;
-    const uint32_t kv_head = local / item.splits, split = local % item.splits;
+    const uint32_t unit = local / item.splits, split = local % item.splits;
     const uint32_t group = p.group, nvec = item.rows * group;
+    const uint32_t vtiles = (nvec + 15) / 16;
+    const uint32_t kv_head = unit % p.g.kv_heads, vtile = vtiles - 1 - unit / p.g.kv_heads;
+    // The rows this tile's vectors belong to bound the keys it walks.
+    const uint32_t row_first = (vtile * 16) / group;
+    const uint32_t row_last = min(item.rows - 1, (vtile * 16 + 15) / group);
 
     const float *kplane = static_cast<const float *>(p.layer_base) + item.slot * p.g.slot_stride +
                           kv_head * p.g.head_stride;
     const float *vplane = kplane + p.g.side_stride;
 
-    const uint32_t nblocks = (item.kv_len + kBlockKeys - 1) / kBlockKeys;
-    const uint32_t blocks_per_split = item.keys_per_split / kBlockKeys;
-    const uint32_t kb_begin = (RING ? item_first_block(item) : 0) + split * blocks_per_split;
-    const uint32_t kb_end = min(nblocks, kb_begin + blocks_per_split);
     const uint32_t ring = RING ? p.ring_blocks * kBlockKeys : 0;
     const uint32_t window = RING ? p.window : 0, kv_lo = RING ? item.kv_lo : 0;
+    const uint32_t nblocks =
+        (min(item.pos0 + row_last + 1, item.kv_len) + kBlockKeys - 1) / kBlockKeys;
+    const uint32_t blocks_per_split = item.keys_per_split / kBlockKeys;
+    const uint32_t kb_begin =
+        (RING ? lowest_visible(item.pos0 + row_first, window, kv_lo) / kBlockKeys : 0) +
+        split * blocks_per_split;
+    const uint32_t kb_end = min(nblocks, kb_begin + blocks_per_split);
 
     // Fused append (p.k_new set): the last `rows` positions are not in the planes yet. The
     // workgroups whose blocks reach them copy the new rows in (f32 to f32, all threads, 16 bytes
@@ -95,8 +105,9 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
         __syncthreads();
     }
 
-    // This lane's query vector (column jl) and what its mask and its output need.
-    const uint32_t j = min(jl, nvec - 1);
+    // This lane's query vector (column jl of the tile) and what its mask and its output need.
+    const uint32_t jv = vtile * 16 + jl;
+    const uint32_t j = min(jv, nvec - 1);
     const uint32_t row = j / group, head = kv_head * group + j % group;
     const uint32_t colpos = min(item.pos0 + row, item.kv_len - 1);
     const uint32_t collo = lowest_visible(item.pos0 + row, window, kv_lo);
@@ -112,7 +123,7 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             float4 a = *reinterpret_cast<const float4 *>(qp + 16 * s);
-            if (jl >= nvec) a = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (jv >= nvec) a = make_float4(0.f, 0.f, 0.f, 0.f);
             qreg[s] = make_float4(a.x * qscale, a.y * qscale, a.z * qscale, a.w * qscale);
         }
     }
@@ -238,7 +249,7 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
         wgt[w] = mw == -INFINITY ? 0.0f : fast_exp2(mw - M);
         L = fmaf(sm_l[w][jl], wgt[w], L);
     }
-    if (jl >= nvec) return;
+    if (jv >= nvec) return;
     const bool final_out = item.splits == 1;
     const uint64_t ps = item.ws0 + (uint64_t(row) * p.q_heads + head) * item.splits + split;
     float *dst = final_out ? p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD
@@ -268,8 +279,13 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
 }  // namespace
 
 bool attn_splitk_f32_supports(const PoolGeom &g, uint32_t group, uint32_t max_rows) {
-    return g.v_block == 0 && g.head_dim == kD && group >= 1 && max_rows >= 1 &&
-           max_rows * group <= 16;
+    return g.v_block == 0 && g.head_dim == kD && group >= 1 && max_rows >= 1;
+}
+// Steps of up to 16 query vectors per KV head bring their rows along: every workgroup that
+// reaches the new positions copies all of them in, which is nothing for a row or two and would
+// be the whole chunk for a prefill.
+bool attn_splitk_f32_appends(const PoolGeom &g, uint32_t group, uint32_t max_rows) {
+    return attn_splitk_f32_supports(g, group, max_rows) && max_rows * group <= 16;
 }
 
 // Fills splits / keys_per_split / block0 / ws0 (slot, rows, pos0, q_row0, kv_len, kv_lo are
@@ -282,16 +298,21 @@ uint32_t attn_splitk_f32_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads)
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
         (void)hipGetLastError();
     const uint64_t capacity = uint64_t(2) * uint64_t(cus > 0 ? cus : 256);
+    const uint32_t group = q_heads / g.kv_heads;
+    auto units_of = [&](const AttnItem &it) {
+        return uint64_t(g.kv_heads) * ((uint64_t(it.rows) * group + 15) / 16);
+    };
     uint64_t blocks = 0;
-    for (uint32_t i = 0; i < b.n; ++i) blocks += uint64_t(g.kv_heads) * item_block_count(b.item[i]);
+    for (uint32_t i = 0; i < b.n; ++i) blocks += units_of(b.item[i]) * item_block_count(b.item[i]);
     uint64_t T = std::max<uint64_t>((blocks + capacity - 1) / capacity, uint64_t(kWavesF32));
     for (;; ++T) {
         uint64_t groups = 0;
         for (uint32_t i = 0; i < b.n; ++i) {
             const uint64_t nb = item_block_count(b.item[i]);
-            groups += uint64_t(g.kv_heads) * std::max<uint64_t>((nb + T - 1) / T, 1);
+            groups += units_of(b.item[i]) * std::max<uint64_t>((nb + T - 1) / T, 1);
         }
-        if (groups <= capacity || T >= blocks) break;
+        // (Units that alone outnumber the device are left whole: nothing is gained by splitting.)
+        if (groups <= capacity || T >= blocks || T >= 4096) break;
     }
     uint32_t block0 = 0, ws0 = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
@@ -304,7 +325,7 @@ uint32_t attn_splitk_f32_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads)
         it.splits_magic = 0;
         it.block0 = block0;
         it.ws0 = ws0;
-        block0 += g.kv_heads * it.splits;
+        block0 += uint32_t(units_of(it)) * it.splits;
         if (it.splits > 1) ws0 += it.rows * q_heads * it.splits;
     }
     b.total_blocks = block0;

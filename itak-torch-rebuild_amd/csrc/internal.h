@@ -391,6 +391,8 @@ hipError_t launch_attn_decode_f16(const AttnParams &p, const AttnBatch &b, uint3
 // f32 MFMA split-K path: f32 pools (row-major planes), head_dim 128, rows*group <= 16, implied
 // query positions. Partials are in log2 domain (combine with base2 = 1).
 bool attn_splitk_f32_supports(const PoolGeom &g, uint32_t group, uint32_t max_rows);
+// True when such a launch also appends the step's rows (k_new / v_new in its parameters).
+bool attn_splitk_f32_appends(const PoolGeom &g, uint32_t group, uint32_t max_rows);
 uint32_t attn_splitk_f32_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads);
 hipError_t launch_attn_splitk_f32(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                   hipStream_t stream);

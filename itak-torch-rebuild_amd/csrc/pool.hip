@@ -2134,7 +2134,7 @@ static itak_status step_on_device(itak_pool *pool, uint64_t layer, const itak_ba
     const bool fuse =
         splitk || block_fuses ||
         (!pool->elem_f16 && !active.empty() &&
-         attn_splitk_f32_supports(pool->g, uint32_t(num_q_heads / pool->g.kv_heads), most_rows));
+         attn_splitk_f32_appends(pool->g, uint32_t(num_q_heads / pool->g.kv_heads), most_rows));
     // The allocation-free form plans first and refuses, before anything changes, a step whose
     // launches need more workspace than the static array has.
     struct NoAllocScope {

@@ -1,6 +1,7 @@
-"""Decode steps and short blocks on f32 pools of head_dim 128 (the reference's own storage type)
-run on the f32 MFMA split-K kernel; every other f32 shape stays on the generic kernel. Both are
-held to the oracle within 1e-5 relative to the largest output magnitude, the f32 bar."""
+"""Steps on f32 pools of head_dim 128 (the reference's own storage type) run on the f32 MFMA
+kernel: decode rows, verify blocks and prefill chunks as tiles of 16 query vectors; other head
+dims stay on the generic kernel. Both are held to the oracle within 1e-5 relative to the largest
+output magnitude, the f32 bar."""
 import numpy as np
 import pytest
 import torch
@@ -84,6 +85,19 @@ def test_softcap_and_a_block_of_rows_on_a_ring():
     run([400, 90], rows=2, q_heads=32, kv_heads=4, window=128, steps=40, seed=9)
 
 
-def test_other_shapes_keep_the_generic_kernel():
-    run([300], rows=3, q_heads=32, kv_heads=4, seed=10)       # 24 vectors: more than one tile
+@pytest.mark.parametrize("ctxs,rows,q_heads,kv_heads,window,softcap", [
+    ([300], 3, 32, 4, None, 0.0),            # 24 vectors: two tiles, the second half empty
+    ([2100, 700, 0, 45], 8, 32, 4, None, 0.0),   # verify blocks, four slots
+    ([1000], 64, 32, 4, None, 30.0),         # the reference's prefill chunk
+    ([0], 300, 32, 4, None, 0.0),            # a prompt's first chunk: tiles see different runs of keys
+    ([500], 200, 40, 8, None, 0.0),          # a group of five: tiles straddle rows
+    ([900], 40, 16, 2, 256, 0.0),            # a block on a ring, the window inside the block's span
+    ([3000, 100], 20, 12, 4, 1024, 0.0),
+])
+def test_blocks_of_any_length_run_as_tiles_of_sixteen_vectors(ctxs, rows, q_heads, kv_heads, window, softcap):
+    run(ctxs, rows=rows, q_heads=q_heads, kv_heads=kv_heads, window=window, softcap=softcap, steps=2,
+        seed=rows + len(ctxs))
+
+
+def test_other_head_dims_keep_the_generic_kernel():
     run([300], rows=1, q_heads=8, kv_heads=2, d=64, seed=11)  # head_dim 64
