@@ -52,12 +52,16 @@ __device__ __forceinline__ float lanes4_sum(float v) {
     return __uint_as_float(c[0]) + __uint_as_float(c[1]);
 }
 
-template <int N, bool RING>
+// D = head_dim: 64 or 128 (a multiple of 64: a value row is read as D / 64 float4 per lane).
+template <int N, bool RING, int D>
 __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnParams p,
                                                                          AttnBatchT<N> b,
                                                                          uint32_t total_partials) {
+    constexpr int kD = D;          // shadows the f16 kernels' constant inside this kernel
+    constexpr int kSteps = D / 16;  // float4 steps of a key row per lane group
+    constexpr int kH = D / 64;      // float4 pieces of a value row per lane
     __shared__ float sm_m[kWavesF32][16], sm_l[kWavesF32][16];
-    __shared__ float sm_o[kWavesF32][8][64][4];  // [wave][tile (h, e)][lane][row of the lane]
+    __shared__ float sm_o[kWavesF32][kH * 4][64][4];  // [wave][tile (h, e)][lane][row of the lane]
 
     const uint32_t tid = threadIdx.x;
     const uint32_t wave = tid >> 6, lane = tid & 63;
@@ -93,8 +97,9 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
     // them both write the same bytes. No other workgroup reads these positions.
     if (p.k_new != nullptr && kb_end * kBlockKeys > item.pos0) {
         const uint32_t row_width = p.g.kv_heads * kD;
-        for (uint32_t f = tid; f < item.rows * 64; f += kWavesF32 * 64) {
-            const uint32_t r = f >> 6, side = (f >> 5) & 1, c4 = (f & 31) * 4;
+        constexpr uint32_t kChunks = kD / 4;  // float4 pieces of one side of a row
+        for (uint32_t f = tid; f < item.rows * 2 * kChunks; f += kWavesF32 * 64) {
+            const uint32_t r = f / (2 * kChunks), side = (f / kChunks) & 1, c4 = (f % kChunks) * 4;
             const float *src = (side ? p.v_new : p.k_new) + uint64_t(item.q_row0 + r) * row_width +
                                kv_head * kD + c4;
             const uint32_t pos = item.pos0 + r;
@@ -117,11 +122,11 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
     const float qscale = softcap > 0.0f ? p.scale : p.scale * kLog2e;
 
     // Q^T as B operands: step (s, e) takes channel 16s + 4g + e of vector jl.
-    float4 qreg[8];
+    float4 qreg[kSteps];
     {
         const float *qp = p.q + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + 4 * g;
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
+        for (int s = 0; s < kSteps; ++s) {
             float4 a = *reinterpret_cast<const float4 *>(qp + 16 * s);
             if (jv >= nvec) a = make_float4(0.f, 0.f, 0.f, 0.f);
             qreg[s] = make_float4(a.x * qscale, a.y * qscale, a.z * qscale, a.w * qscale);
@@ -129,9 +134,9 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
     }
 
     float m_run = -INFINITY, l_run = 0.0f;
-    floatx4 o[2][4];
+    floatx4 o[kH][4];
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int h = 0; h < kH; ++h)
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[h][e] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 
@@ -143,12 +148,12 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
             const uint32_t q = min(pos, item.kv_len - 1);
             return RING ? q % ring : q;
         };
-        float4 kreg[2][8], vreg[2][4][2];
+        float4 kreg[2][kSteps], vreg[2][4][kH];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const float *kr = kplane + uint64_t(storage_row(key0 + 16 * t + jl)) * kD + 4 * g;
 #pragma unroll
-            for (int s = 0; s < 8; ++s) kreg[t][s] = *reinterpret_cast<const float4 *>(kr + 16 * s);
+            for (int s = 0; s < kSteps; ++s) kreg[t][s] = *reinterpret_cast<const float4 *>(kr + 16 * s);
         }
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -156,7 +161,7 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
             for (int r = 0; r < 4; ++r) {
                 const float *vr = vplane + uint64_t(storage_row(key0 + 16 * t + 4 * g + r)) * kD + 4 * jl;
 #pragma unroll
-                for (int h = 0; h < 2; ++h)
+                for (int h = 0; h < kH; ++h)
                     vreg[t][r][h] = *reinterpret_cast<const float4 *>(vr + 64 * h);
             }
 
@@ -166,7 +171,7 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
         for (int t = 0; t < 2; ++t) {
             floatx4 acc = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int s = 0; s < 8; ++s) {
+            for (int s = 0; s < kSteps; ++s) {
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[t][s].x, qreg[s].x, acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[t][s].y, qreg[s].y, acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[t][s].z, qreg[s].z, acc, 0, 0, 0);
@@ -190,7 +195,7 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
                 // oldest window on a ring) may hold anything: keep it out of P.V even as 0*x.
                 if (kp >= item.kv_len || (RING && kp < lo_min)) {
 #pragma unroll
-                    for (int h = 0; h < 2; ++h) vreg[t][r][h] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    for (int h = 0; h < kH; ++h) vreg[t][r][h] = make_float4(0.f, 0.f, 0.f, 0.f);
                 }
             }
         mx = lanes4_max(mx);
@@ -209,7 +214,7 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
         l_run = l_run * alpha + sum;
         m_run = m_new;
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+        for (int h = 0; h < kH; ++h)
 #pragma unroll
             for (int e = 0; e < 4; ++e) o[h][e] *= alpha;
 #pragma unroll
@@ -217,7 +222,7 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
 #pragma unroll
             for (int r = 0; r < 4; ++r)
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
+                for (int h = 0; h < kH; ++h) {
                     const float4 a = vreg[t][r][h];
                     o[h][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, sc[t][r], o[h][0], 0, 0, 0);
                     o[h][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, sc[t][r], o[h][1], 0, 0, 0);
@@ -233,7 +238,7 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
         sm_l[wave][jl] = l_col;
     }
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int h = 0; h < kH; ++h)
 #pragma unroll
         for (int e = 0; e < 4; ++e)
             *reinterpret_cast<floatx4 *>(&sm_o[wave][h * 4 + e][lane][0]) = o[h][e];
@@ -255,23 +260,33 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
     float *dst = final_out ? p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD
                            : p.ws + ps * kD;
     const float post = final_out ? 1.0f / L : 1.0f;
-    // Tile (h, e), lane (jl, g), register rr holds channel 64h + 16g + 4rr + e: the four e of
-    // one (h, rr) are 16 contiguous bytes, and this wavefront owns e = 2 (wave % 2) .. +1 of
-    // h = wave / 2.
-    const uint32_t h = wave >> 1, e0 = (wave & 1) * 2;
-    floatx4 fin[2];
+    // Tile (h, e), lane (jl, g), register rr holds channel 64h + 16g + 4rr + e. The kH * 4 tiles
+    // are shared out among the four wavefronts: two consecutive e of one h each at head_dim 128
+    // (8 contiguous bytes per register), one tile each at head_dim 64.
+    constexpr int kTilesPerWave = kH * 4 / kWavesF32;
+    floatx4 fin[kTilesPerWave];
 #pragma unroll
-    for (int x = 0; x < 2; ++x) {
+    for (int x = 0; x < kTilesPerWave; ++x) {
         fin[x] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int w = 0; w < kWavesF32; ++w)
-            fin[x] += *reinterpret_cast<const floatx4 *>(&sm_o[w][h * 4 + e0 + x][lane][0]) * wgt[w];
+            fin[x] += *reinterpret_cast<const floatx4 *>(&sm_o[w][wave * kTilesPerWave + x][lane][0]) * wgt[w];
         fin[x] *= post;
     }
+    if constexpr (kTilesPerWave == 2) {
+        const uint32_t h = wave >> 1, e0 = (wave & 1) * 2;
 #pragma unroll
-    for (int rr = 0; rr < 4; ++rr)
-        *reinterpret_cast<float2 *>(dst + 64 * h + 16 * g + 4 * rr + e0) =
-            make_float2(fin[0][rr], fin[1][rr]);
+        for (int rr = 0; rr < 4; ++rr)
+            *reinterpret_cast<float2 *>(dst + 64 * h + 16 * g + 4 * rr + e0) =
+                make_float2(fin[0][rr], fin[1][rr]);
+    } else {
+#pragma unroll
+        for (int x = 0; x < kTilesPerWave; ++x) {
+            const uint32_t tile = wave * kTilesPerWave + x, h = tile >> 2, e = tile & 3;
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) dst[64 * h + 16 * g + 4 * rr + e] = fin[x][rr];
+        }
+    }
     if (!final_out && wave == 0 && g == 0)
         *reinterpret_cast<float2 *>(p.ws + uint64_t(total_partials) * kD + ps * 2) = make_float2(M, L);
 }
@@ -279,7 +294,7 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
 }  // namespace
 
 bool attn_splitk_f32_supports(const PoolGeom &g, uint32_t group, uint32_t max_rows) {
-    return g.v_block == 0 && g.head_dim == kD && group >= 1 && max_rows >= 1;
+    return g.v_block == 0 && (g.head_dim == 128 || g.head_dim == 64) && group >= 1 && max_rows >= 1;
 }
 // Steps of up to 16 query vectors per KV head bring their rows along: every workgroup that
 // reaches the new positions copies all of them in, which is nothing for a row or two and would
@@ -336,12 +351,15 @@ uint32_t attn_splitk_f32_plan(const PoolGeom &g, AttnBatch &b, uint32_t q_heads)
 hipError_t launch_attn_splitk_f32(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                   hipStream_t stream) {
     if (b.total_blocks == 0) return hipSuccess;
-    if (p.ring_blocks)
-        ITAK_DISPATCH_BATCH(b.n, (attn_splitk_f32_kernel<N, true><<<b.total_blocks, kWavesF32 * 64, 0, stream>>>(
-                                     p, AttnBatchT<N>(b), total_partials)));
-    else
-        ITAK_DISPATCH_BATCH(b.n, (attn_splitk_f32_kernel<N, false><<<b.total_blocks, kWavesF32 * 64, 0, stream>>>(
-                                     p, AttnBatchT<N>(b), total_partials)));
+#define ITAK_LAUNCH_F32(RING, D)                                                                  \
+    ITAK_DISPATCH_BATCH(b.n, (attn_splitk_f32_kernel<N, RING, D>                                    \
+                              <<<b.total_blocks, kWavesF32 * 64, 0, stream>>>(p, AttnBatchT<N>(b), total_partials)))
+    if (p.g.head_dim == 64) {
+        if (p.ring_blocks) ITAK_LAUNCH_F32(true, 64); else ITAK_LAUNCH_F32(false, 64);
+    } else {
+        if (p.ring_blocks) ITAK_LAUNCH_F32(true, 128); else ITAK_LAUNCH_F32(false, 128);
+    }
+#undef ITAK_LAUNCH_F32
     return hipGetLastError();
 }
 

@@ -99,5 +99,14 @@ def test_blocks_of_any_length_run_as_tiles_of_sixteen_vectors(ctxs, rows, q_head
         seed=rows + len(ctxs))
 
 
+@pytest.mark.parametrize("ctxs,rows,q_heads,kv_heads,window", [
+    ([512], 1, 32, 4, None),                 # configs[0]: the reference's CPU-runnable case
+    ([0, 31, 1000], 1, 8, 2, None), ([700], 2, 32, 4, None), ([300, 64], 8, 32, 4, None),
+    ([0], 200, 16, 4, None), ([900], 1, 32, 4, 256), ([600], 30, 8, 8, 128)])
+def test_head_dim_64_runs_on_the_same_kernel(ctxs, rows, q_heads, kv_heads, window):
+    run(ctxs, rows=rows, q_heads=q_heads, kv_heads=kv_heads, window=window, steps=3, seed=rows + 64, d=64)
+
+
 def test_other_head_dims_keep_the_generic_kernel():
-    run([300], rows=1, q_heads=8, kv_heads=2, d=64, seed=11)  # head_dim 64
+    run([300], rows=1, q_heads=8, kv_heads=2, d=96, seed=11)
+    run([300], rows=3, q_heads=4, kv_heads=2, d=256, seed=12)
