@@ -1,4 +1,5 @@
-// Chunked causal prefill attention for gfx950, f16 KV, head_dim 128: QK^T and PV on
+// Chunked causal prefill attention for gfx950, f16 KV, head_dim 64, 128 or 256 (a template
+// argument; the figures in these comments are those of head_dim 128): QK^T and PV on
 // v_mfma_f32_16x16x32_f16, everything else (scale, softcap, mask, online softmax) in f32.
 //
 // One workgroup of four wavefronts owns (item, kv head, tile of 128 query vectors), where a
@@ -56,15 +57,18 @@ namespace {
 
 constexpr int kWaves = 4;
 constexpr int kMaxTiles = 2;  // MFMA column tiles (16 query vectors) per wavefront: 1 or 2
-constexpr int kBlockElems = kBlockKeys * kD;        // 4096 halves = 8 KiB per plane block
+// Halves in one plane block (8 KiB at head_dim 128) and bytes in one stage of the LDS ring (one
+// key block + one value block).
+constexpr int block_elems(int d) { return kBlockKeys * d; }
+constexpr int stage_bytes(int d) { return 2 * block_elems(d) * 2; }
 constexpr float kRefSlack = 8.0f;
 // The smallest divisor of 16 that holds a GQA group of up to 16 heads.
 __host__ __device__ inline uint32_t padded_group(uint32_t group) {
     return group <= 1 ? 1 : group <= 2 ? 2 : group <= 4 ? 4 : group <= 8 ? 8 : 16;
 }
-constexpr int kFuseRows = 64;  // new rows a launch that appends its own rows carries at most
+// New rows a launch that appends its own rows carries at most: sixteen 16-byte pieces a thread.
+constexpr int fuse_rows(int d) { return d <= 128 ? 64 : 16; }
 constexpr uint32_t kOneTileBlocks = 520;  // key blocks up to which blocks of <= 512 vectors take one tile
-constexpr int kFusePieces = kFuseRows * 2 * (kD / 4) / (kWaves * 64);  // per thread
 
 __device__ __forceinline__ float column_max4(float v) {
     const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
@@ -85,7 +89,6 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
 // is ordered by the explicit s_waitcnt vmcnt + s_barrier at the top of each iteration.
 constexpr int kStages = 4;      // blocks of the LDS ring: three in flight while one is read
 constexpr int kDeepStages = 8;  // for short runs of blocks, one workgroup per compute unit
-constexpr int kStageBytes = 2 * kBlockElems * 2;  // one key block + one value block
 
 __device__ __forceinline__ void lds_dma16(const void *src, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
@@ -101,10 +104,22 @@ __device__ __forceinline__ void wait_vmcnt() {
 
 // RING = the layer is windowed (blocks start at the window, live in a ring, the mask has a
 // lower edge); global layers run the instantiation without any of it.
-template <int N, bool SOFTCAP, int kTiles, bool RING, int STAGES>
-__global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnParams p,
-                                                                           AttnBatchT<N> b,
-                                                                           uint32_t total_partials) {
+// D = head_dim. At 256 a stage of the ring is 32 KiB and a wavefront's accumulators alone are 64
+// to 128 registers: one workgroup per compute unit, up to 512 registers a lane.
+template <int N, bool SOFTCAP, int kTiles, bool RING, int STAGES, int D>
+__global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f16_kernel(
+    AttnParams p, AttnBatchT<N> b, uint32_t total_partials) {
+    constexpr int kD = D;
+    constexpr int kSteps = D / 32;  // MFMAs of one score tile (32 channels each)
+    constexpr int kOut = D / 16;    // output tiles of 16 channels
+    constexpr int kBlockElems = block_elems(D);
+    constexpr int kStageBytes = stage_bytes(D);
+    constexpr int kPieces = D / 64;      // KiB pieces of a key (or value) block each wavefront moves
+    constexpr int kLoads = 2 * kPieces;  // ring loads a thread issues per block
+    constexpr int kChunks = D / 4;       // 16-byte pieces of one side of a new f32 row
+    constexpr int kRowsPerPass = kWaves * 64 / (2 * kChunks);  // new rows the workgroup loads at once
+    constexpr int kFuseRows = fuse_rows(D);
+    constexpr int kFusePieces = kFuseRows / kRowsPerPass;  // per thread
     constexpr int kVecPerWave = kTiles * 16;
     constexpr int kVecPerGroup = kWaves * kVecPerWave;  // query vectors per workgroup
     extern __shared__ __attribute__((aligned(16))) uint16_t lds_ring[];  // [kStages][K block | V block]
@@ -170,7 +185,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     const uint32_t low_masked_end =
         (lowest_visible(item.pos0 + wave_row_end - 1, window, kv_lo) + kBlockKeys - 1) / kBlockKeys;
 
-    // Each wavefront moves two 1 KiB pieces of the key block and two of the value block.
+    // Each wavefront moves kPieces 1 KiB pieces of the key block and as many of the value block
+    // (piece w + 4i for wavefront w).
     const uint4 *kg = reinterpret_cast<const uint4 *>(kplane) + tid;
     // Value pieces are permuted on the way in: LDS position dt*64 + g*16 + jl holds the
     // 16 bytes (channel dt*16 + jl, keys g*8 .. g*8+7), so that the operand read of a
@@ -192,10 +208,11 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
         const uint64_t off = uint64_t(RING ? next_sb : min(kb, max(nblocks, 1u) - 1)) * kBlockVec;
         if (RING && kb + 1 < nblocks) next_sb = next_sb + 1 == ring_blocks ? 0 : next_sb + 1;
         const uint32_t dst = dma_base + (kb % STAGES) * kStageBytes;
-        lds_dma16(kg + off, dst);
-        lds_dma16(kg + off + 256, dst + 4096);
-        lds_dma16(vg + off, dst + 8192);
-        lds_dma16(vg + off + 256, dst + 12288);
+#pragma unroll
+        for (int i = 0; i < kPieces; ++i) lds_dma16(kg + off + 256 * i, dst + 4096 * i);
+#pragma unroll
+        for (int i = 0; i < kPieces; ++i)
+            lds_dma16(vg + off + 256 * i, dst + 2 * kBlockElems + 4096 * i);
     };
     const bool any_block = kb_begin < nblocks;  // a split past the rows' horizon has none
     ITAK_MARK(1)
@@ -217,17 +234,19 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     // re-read its last row and are scaled to zero columns, and the variant that also brings new
     // rows is a second straight line, not a branch inside this one.
     //
-    // New rows (one-tile form only): piece u of this thread is row (tid >> 6) + 4u, side
-    // (tid >> 5) & 1, channels (tid & 31) * 4 .. + 3, requested ahead of Q and waited for with it.
+    // New rows (one-tile form only): piece u of this thread is row nrow + kRowsPerPass * u, side
+    // nside, channels nc4 .. nc4 + 3 (at head_dim 128: row (tid >> 6) + 4u, side (tid >> 5) & 1,
+    // channels (tid & 31) * 4), requested ahead of Q and waited for with it.
     constexpr bool kCanFuse = kTiles == 1;
     const bool fused = kCanFuse && p.k_new != nullptr;
-    const uint32_t nside = (tid >> 5) & 1u, nc4 = (tid & 31u) * 4;
+    const uint32_t nrow = tid / (2 * kChunks);
+    const uint32_t nside = (tid / kChunks) & 1u, nc4 = (tid % kChunks) * 4;
     // Does this workgroup's run of blocks reach the new positions? Is it the one that stores them?
     const bool patches = fused && any_block && nblocks * kBlockKeys > item.pos0;
     const bool stores_new = fused && unit < p.g.kv_heads && split == item.splits - 1;
     const bool with_new = patches || stores_new;
     [[maybe_unused]] uint2 npk[kCanFuse ? kFusePieces : 1];
-    half8 qb[kTiles][4];
+    half8 qb[kTiles][kSteps];
     uint32_t colpos[kTiles], collo[kTiles];
     const float *qp[kTiles];
     float qsc[kTiles];
@@ -243,19 +262,22 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     }
 #define ITAK_Q_LOADS(qraw)                                                                      \
     _Pragma("unroll") for (int qt = 0; qt < kTiles; ++qt)                                       \
-        _Pragma("unroll") for (int s = 0; s < 8; ++s)                                           \
+        _Pragma("unroll") for (int s = 0; s < 2 * kSteps; ++s)                                  \
             asm volatile("global_load_dwordx4 %0, %1, off"                                      \
                          : "=v"(qraw[qt][s])                                                    \
                          : "v"(qp[qt] + (s >> 1) * 32 + (s & 1) * 4)                            \
                          : "memory");
 #define ITAK_RING_FILL                                                                          \
     _Pragma("unroll") for (int ahead = 0; ahead < STAGES - 1; ++ahead) issue_block(kb_begin + ahead);
-#define ITAK_Q_REGS(qt)                                                                         \
-    "+v"(qraw[qt][0]), "+v"(qraw[qt][1]), "+v"(qraw[qt][2]), "+v"(qraw[qt][3]), "+v"(qraw[qt][4]), \
-        "+v"(qraw[qt][5]), "+v"(qraw[qt][6]), "+v"(qraw[qt][7])
+// Everything older than the ring's loads has landed. The registers named after the wait pass
+// through an (empty) statement behind it, so that nothing that reads them is scheduled ahead.
+#define ITAK_WAIT_BEHIND_RING asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kLoads * (STAGES - 1)) : "memory");
+#define ITAK_Q_ARRIVED(qraw)                                                                    \
+    _Pragma("unroll") for (int qt = 0; qt < kTiles; ++qt)                                       \
+        _Pragma("unroll") for (int s = 0; s < 2 * kSteps; ++s) asm volatile("" : "+v"(qraw[qt][s]));
 #define ITAK_Q_CONVERT(qraw)                                                                    \
     _Pragma("unroll") for (int qt = 0; qt < kTiles; ++qt)                                       \
-        _Pragma("unroll") for (int s = 0; s < 4; ++s) {                                         \
+        _Pragma("unroll") for (int s = 0; s < kSteps; ++s) {                                    \
             const floatx4 a = qraw[qt][2 * s], c = qraw[qt][2 * s + 1];                         \
             const float sc = qsc[qt];                                                           \
             qb[qt][s] = half8{static_cast<_Float16>(a[0] * sc), static_cast<_Float16>(a[1] * sc), \
@@ -267,13 +289,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     if constexpr (kCanFuse) {
         if (with_new) {
             took_new = true;
-            floatx4 nraw[kFusePieces], qraw[kTiles][8];
+            floatx4 nraw[kFusePieces], qraw[kTiles][2 * kSteps];
             const uint32_t row_width = p.g.kv_heads * kD;
             const float *src = (nside ? p.v_new : p.k_new) + uint64_t(item.q_row0) * row_width +
                                kv_head * kD + nc4;
 #pragma unroll
             for (int u = 0; u < kFusePieces; ++u) {
-                const uint32_t r = min((tid >> 6) + 4u * u, item.rows - 1);
+                const uint32_t r = min(nrow + uint32_t(kRowsPerPass) * u, item.rows - 1);
                 asm volatile("global_load_dwordx4 %0, %1, off"
                              : "=v"(nraw[u])
                              : "v"(src + uint64_t(r) * row_width)
@@ -282,14 +304,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
             ITAK_Q_LOADS(qraw)
             ITAK_RING_FILL
             ITAK_MARK(2)
-            static_assert(kFusePieces == 16, "the wait below names sixteen registers of new rows");
-            asm volatile("s_waitcnt vmcnt(%24)"
-                         : ITAK_Q_REGS(0), "+v"(nraw[0]), "+v"(nraw[1]), "+v"(nraw[2]), "+v"(nraw[3]),
-                           "+v"(nraw[4]), "+v"(nraw[5]), "+v"(nraw[6]), "+v"(nraw[7]), "+v"(nraw[8]),
-                           "+v"(nraw[9]), "+v"(nraw[10]), "+v"(nraw[11]), "+v"(nraw[12]),
-                           "+v"(nraw[13]), "+v"(nraw[14]), "+v"(nraw[15])
-                         : "n"(4 * (STAGES - 1))
-                         : "memory");
+            ITAK_WAIT_BEHIND_RING
+            ITAK_Q_ARRIVED(qraw)
+#pragma unroll
+            for (int u = 0; u < kFusePieces; ++u) asm volatile("" : "+v"(nraw[u]));
             ITAK_Q_CONVERT(qraw)
             // The conversion rule (f32_to_f16_bits) is the hardware's rounding plus a fixed
             // pattern for NaNs: a sum that is not a NaN proves its four terms are not, so the
@@ -305,7 +323,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
             const bool by_element = __builtin_amdgcn_ballot_w64(nan_seen) != 0;
 #pragma unroll
             for (int u = 0; u < kFusePieces; ++u) {
-                if (wave + 4u * u >= item.rows) continue;
+                // (Uniform over the wavefront when a row is 64 lanes.)
+                if ((2 * kChunks == 64 ? wave : nrow) + uint32_t(kRowsPerPass) * u >= item.rows) continue;
                 if (by_element) {
                     const uint32_t h0 = f32_to_f16_bits(nraw[u][0]), h1 = f32_to_f16_bits(nraw[u][1]);
                     const uint32_t h2 = f32_to_f16_bits(nraw[u][2]), h3 = f32_to_f16_bits(nraw[u][3]);
@@ -320,19 +339,17 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
         }
     }
     if (!took_new) {
-        floatx4 qraw[kTiles][8];
+        floatx4 qraw[kTiles][2 * kSteps];
         ITAK_Q_LOADS(qraw)
         ITAK_RING_FILL
         ITAK_MARK(2)
-        // Everything older than the ring's loads has landed: that is Q.
-        if constexpr (kTiles == 2)
-            asm volatile("s_waitcnt vmcnt(%16)" : ITAK_Q_REGS(0), ITAK_Q_REGS(1) : "n"(4 * (STAGES - 1)) : "memory");
-        else
-            asm volatile("s_waitcnt vmcnt(%8)" : ITAK_Q_REGS(0) : "n"(4 * (STAGES - 1)) : "memory");
+        ITAK_WAIT_BEHIND_RING  // that is Q
+        ITAK_Q_ARRIVED(qraw)
         ITAK_Q_CONVERT(qraw)
     }
 #undef ITAK_Q_CONVERT
-#undef ITAK_Q_REGS
+#undef ITAK_Q_ARRIVED
+#undef ITAK_WAIT_BEHIND_RING
 #undef ITAK_RING_FILL
 #undef ITAK_Q_LOADS
     if constexpr (kCanFuse) {
@@ -340,14 +357,14 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
             uint16_t *kp = const_cast<uint16_t *>(kplane), *vp = const_cast<uint16_t *>(vplane);
 #pragma unroll
             for (int u = 0; u < kFusePieces; ++u) {
-                const uint32_t r = (tid >> 6) + 4u * u;
+                const uint32_t r = nrow + uint32_t(kRowsPerPass) * u;
                 if (r >= item.rows) continue;
                 const uint32_t key = item.pos0 + r, kin = key % kBlockKeys;
                 const uint32_t sb = RING ? (key / kBlockKeys) % ring_blocks : key / kBlockKeys;
                 const uint64_t blk = uint64_t(sb) * kBlockElems;
                 if (nside == 0) {
                     const uint32_t kt = (kin >> 2) & 1, ki = (kin >> 3) * 4 + (kin & 3);
-                    *reinterpret_cast<uint2 *>(kp + blk + ((kt * 16 + (nc4 >> 3)) * 16 + ki) * 8 +
+                    *reinterpret_cast<uint2 *>(kp + blk + ((kt * (kD / 8) + (nc4 >> 3)) * 16 + ki) * 8 +
                                                (nc4 & 7)) = npk[u];
                 } else {
                     uint16_t *vd = vp + blk + nc4 * kBlockKeys + kin;
@@ -370,7 +387,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
     floatx4 negref[kTiles];
     const half8 ones = {_Float16(1.0f), _Float16(1.0f), _Float16(1.0f), _Float16(1.0f),
                         _Float16(1.0f), _Float16(1.0f), _Float16(1.0f), _Float16(1.0f)};
-    floatx4 o[kTiles][8];
+    floatx4 o[kTiles][kOut];
 #pragma unroll
     for (int qt = 0; qt < kTiles; ++qt) {
         ref[qt] = 0.0f;
@@ -378,14 +395,14 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
         l[qt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
         negref[qt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int dt = 0; dt < 8; ++dt) o[qt][dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int dt = 0; dt < kOut; ++dt) o[qt][dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
     for (uint32_t kb = kb_begin; kb < nblocks; ++kb) {
-        // This thread's pieces of block kb have landed (the 8 loads of the next two blocks
+        // This thread's pieces of block kb have landed (the loads of the next STAGES - 2 blocks
         // may still fly); after the barrier everybody's have, and everybody is done with
         // block kb - 1, whose stage the loads for block kb + 3 may now overwrite.
-        wait_vmcnt<4 * (STAGES - 2)>();
+        wait_vmcnt<kLoads * (STAGES - 2)>();
         __builtin_amdgcn_s_barrier();
         issue_block(kb + STAGES - 1);
         const uint16_t *lds_k = lds_ring + (kb % STAGES) * (kStageBytes / 2);
@@ -398,12 +415,12 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                 uint16_t *sk = lds_ring + (kb % STAGES) * (kStageBytes / 2), *sv = sk + kBlockElems;
 #pragma unroll
                 for (int u = 0; u < kFusePieces; ++u) {
-                    const uint32_t r = (tid >> 6) + 4u * u;
+                    const uint32_t r = nrow + uint32_t(kRowsPerPass) * u;
                     const uint32_t key = item.pos0 + r, kin = key % kBlockKeys;
                     if (r >= item.rows || key / kBlockKeys != kb) continue;
                     if (nside == 0) {
                         const uint32_t kt = (kin >> 2) & 1, ki = (kin >> 3) * 4 + (kin & 3);
-                        *reinterpret_cast<uint2 *>(sk + ((kt * 16 + (nc4 >> 3)) * 16 + ki) * 8 +
+                        *reinterpret_cast<uint2 *>(sk + ((kt * (kD / 8) + (nc4 >> 3)) * 16 + ki) * 8 +
                                                    (nc4 & 7)) = npk[u];
                     } else {
                         // piece (channel c, keys g*8..g*8+7) sits at (c/16)*64 + g*16 + c%16
@@ -425,29 +442,29 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
             floatx4 x[kTiles][2];
             __builtin_amdgcn_s_setprio(0);  // raised again below, for the block's second half
             {
-                half8 ka[2][4];
+                half8 ka[2][kSteps];
                 const uint16_t *kl = lds_k + (g * 16 + jl) * 8;
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
-                    for (int s = 0; s < 4; ++s)
+                    for (int s = 0; s < kSteps; ++s)
                         ka[t][s] =
-                            *reinterpret_cast<const half8 *>(kl + ((t * 16 + s * 4) * 16) * 8);
+                            *reinterpret_cast<const half8 *>(kl + ((t * (kD / 8) + s * 4) * 16) * 8);
 #pragma unroll
                 for (int qt = 0; qt < kTiles; ++qt)
 #pragma unroll
                     for (int t = 0; t < 2; ++t) {
                         floatx4 s = negref[qt];
 #pragma unroll
-                        for (int k = 0; k < 4; ++k)
+                        for (int k = 0; k < kSteps; ++k)
                             s = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[t][k], qb[qt][k], s, 0, 0, 0);
                         x[qt][t] = s;
                     }
             }
-            half8 va[8];
+            half8 va[kOut];
             const uint16_t *vl = lds_v + lane * 8;
 #pragma unroll
-            for (int dt = 0; dt < 8; ++dt)
+            for (int dt = 0; dt < kOut; ++dt)
                 va[dt] = *reinterpret_cast<const half8 *>(vl + dt * 64 * 8);
 
             if constexpr (SOFTCAP) {  // negref stays zero: x is the raw scaled score here
@@ -466,7 +483,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                 if (kb * kBlockKeys < item_lo) {
                     // Ring rows older than anything the item's queries see may be stale.
 #pragma unroll
-                    for (int dt = 0; dt < 8; ++dt)
+                    for (int dt = 0; dt < kOut; ++dt)
 #pragma unroll
                         for (int e = 0; e < 8; ++e)
                             if (key_base + e < item_lo) va[dt][e] = _Float16(0.0f);
@@ -481,7 +498,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                 if ((kb + 1) * kBlockKeys > item.kv_len) {
                     // Rows past the stored length may hold stale data: keep them out of P.V.
 #pragma unroll
-                    for (int dt = 0; dt < 8; ++dt)
+                    for (int dt = 0; dt < kOut; ++dt)
 #pragma unroll
                         for (int e = 0; e < 8; ++e)
                             if (key_base + e >= item.kv_len) va[dt][e] = _Float16(0.0f);
@@ -510,7 +527,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                     if (cm != -INFINITY) thr[qt] = kRefSlack;
                     l[qt] *= alpha;
 #pragma unroll
-                    for (int dt = 0; dt < 8; ++dt) o[qt][dt] *= alpha;
+                    for (int dt = 0; dt < kOut; ++dt) o[qt][dt] *= alpha;
 #pragma unroll
                     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -538,7 +555,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
                 for (int e = 0; e < 8; ++e) pb[e] = static_cast<_Float16>(pe[e]);
                 l[qt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pb, l[qt], 0, 0, 0);
 #pragma unroll
-                for (int dt = 0; dt < 8; ++dt)
+                for (int dt = 0; dt < kOut; ++dt)
                     o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[dt], pb, o[qt][dt], 0, 0, 0);
             }
         }
@@ -563,13 +580,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
             const float inv = 1.0f / lt;
             float *dst = p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * kD + g * 4;
 #pragma unroll
-            for (int dt = 0; dt < 8; ++dt)
+            for (int dt = 0; dt < kOut; ++dt)
                 *reinterpret_cast<floatx4 *>(dst + dt * 16) = o[qt][dt] * inv;
         } else {
             const uint64_t ps = item.ws0 + (uint64_t(row) * p.q_heads + head) * item.splits + split;
             float *dst = ws_acc + ps * kD + g * 4;
 #pragma unroll
-            for (int dt = 0; dt < 8; ++dt) *reinterpret_cast<floatx4 *>(dst + dt * 16) = o[qt][dt];
+            for (int dt = 0; dt < kOut; ++dt) *reinterpret_cast<floatx4 *>(dst + dt * 16) = o[qt][dt];
             if (g == 0)
                 *reinterpret_cast<float2 *>(ws_ml + ps * 2) =
                     make_float2(thr[qt] == -INFINITY ? -INFINITY : ref[qt], lt);
@@ -585,12 +602,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void attn_prefill_f16_kernel(AttnPa
 // one-tile form and no item has more than kFuseRows rows.
 bool attn_prefill_f16_appends(const PoolGeom &g, uint32_t group, uint32_t most_rows,
                               uint32_t most_blocks) {
-    return attn_prefill_f16_supports(g, group) && most_rows <= uint32_t(kFuseRows) &&
+    return attn_prefill_f16_supports(g, group) && most_rows <= uint32_t(fuse_rows(int(g.head_dim))) &&
            most_rows * padded_group(group) <= 512 && most_blocks <= kOneTileBlocks;
 }
 
 bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group) {
-    return g.v_block == kVBlock && g.head_dim == kD && group >= 1 && group <= 16;
+    return g.v_block == kVBlock && (g.head_dim == 64 || g.head_dim == 128 || g.head_dim == 256) &&
+           group >= 1 && group <= 16;
 }
 
 // Up to 64 query vectors per KV head (speculative blocks) take one 16-vector tile per
@@ -648,7 +666,8 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
     // that its handful of blocks arrive behind one another after a single memory latency
     // (measured: 64 rows at context 4096 30.8 -> 27.1 us, 256 rows 52.6 -> 48.4 us, 16 rows at
     // context 30720 36.3 -> 31.6 us; above the range it loses, below it nothing changes).
-    const bool deep = unit_blocks >= 8 * per_cu && unit_blocks <= 40 * per_cu;
+    // (Eight stages of head_dim 256 do not fit the LDS.)
+    const bool deep = unit_blocks >= 8 * per_cu && unit_blocks <= 40 * per_cu && g.head_dim <= 128;
     b.deep_ring = deep ? 1 : 0;
     b.fold_units = 0;
     const uint64_t target = deep ? per_cu : 2 * per_cu;
@@ -725,25 +744,44 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
     return ws0;
 }
 
-template <int N, bool SOFTCAP, int TILES, bool RING, int STAGES>
+template <int N, bool SOFTCAP, int TILES, bool RING, int STAGES, int D>
 static hipError_t launch_prefill_ring(const AttnParams &p, const AttnBatch &b,
                                       uint32_t total_partials, hipStream_t stream) {
-    constexpr size_t lds = size_t(STAGES) * kStageBytes;
+    constexpr size_t lds = size_t(STAGES) * stage_bytes(D);
     static const hipError_t granted = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(&attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING, STAGES>),
+        reinterpret_cast<const void *>(&attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING, STAGES, D>),
         hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
     if (granted != hipSuccess) return granted;
-    attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING, STAGES>
+    attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING, STAGES, D>
         <<<b.total_blocks, kWaves * 64, lds, stream>>>(p, AttnBatchT<N>(b), total_partials);
     return hipGetLastError();
 }
 
-template <int N, bool SOFTCAP, int TILES, bool RING>
+template <int N, bool SOFTCAP, int TILES, bool RING, int D>
 static hipError_t launch_prefill(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                  hipStream_t stream) {
-    return b.deep_ring
-               ? launch_prefill_ring<N, SOFTCAP, TILES, RING, kDeepStages>(p, b, total_partials, stream)
-               : launch_prefill_ring<N, SOFTCAP, TILES, RING, kStages>(p, b, total_partials, stream);
+    if constexpr (D <= 128) {
+        if (b.deep_ring)
+            return launch_prefill_ring<N, SOFTCAP, TILES, RING, kDeepStages, D>(p, b, total_partials, stream);
+    } else if (b.deep_ring) {
+        return hipErrorInvalidValue;
+    }
+    return launch_prefill_ring<N, SOFTCAP, TILES, RING, kStages, D>(p, b, total_partials, stream);
+}
+
+// head_dim 128 has an instantiation per batch size class (the batch table is a kernel argument:
+// a decode-sized launch should not carry 64 entries); the other head dims take the largest.
+template <bool SOFTCAP, int TILES, bool RING>
+static hipError_t launch_prefill_dim(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                                     hipStream_t stream) {
+    hipError_t e = hipErrorInvalidValue;
+    if (p.g.head_dim == 128)
+        ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, SOFTCAP, TILES, RING, 128>(p, b, total_partials, stream)));
+    else if (p.g.head_dim == 64)
+        e = launch_prefill<64, SOFTCAP, TILES, RING, 64>(p, b, total_partials, stream);
+    else if (p.g.head_dim == 256)
+        e = launch_prefill<64, SOFTCAP, TILES, RING, 256>(p, b, total_partials, stream);
+    return e;
 }
 
 hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
@@ -752,12 +790,12 @@ hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, uint
     hipError_t e = hipSuccess;
     const bool one = tiles_for(b, p.group) == 1;
     if (p.k_new && !one) return hipErrorInvalidValue;  // only the one-tile form appends
-#define ITAK_LAUNCH_TILES(SC, RING)                                                            \
-    do {                                                                                       \
-        if (one)                                                                               \
-            ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, SC, 1, RING>(p, b, total_partials, stream))); \
-        else                                                                                   \
-            ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, SC, 2, RING>(p, b, total_partials, stream))); \
+#define ITAK_LAUNCH_TILES(SC, RING)                                             \
+    do {                                                                        \
+        if (one)                                                                \
+            e = launch_prefill_dim<SC, 1, RING>(p, b, total_partials, stream);  \
+        else                                                                    \
+            e = launch_prefill_dim<SC, 2, RING>(p, b, total_partials, stream);  \
     } while (0)
 #define ITAK_LAUNCH_RING(SC)              \
     do {                                  \
