@@ -143,3 +143,26 @@ def test_head_dim_64_rewinds_a_speculative_round():
             r.release(cp)
         step(pool, caches, refs, rng, [1, 1], q_heads)
     pool.close()
+
+
+@pytest.mark.parametrize("elem,d,q_heads,kv_heads,rows,ctx,window", [
+    ("f16", 64, 32, 4, 1, 3000, None),     # splits merged by the general merge kernel, which applies the gate
+    ("f16", 64, 32, 4, 1, 20, None),       # one split: the gate is a launch of its own
+    ("f16", 64, 8, 2, 7, 500, 128),        # a block on a ring
+    ("f16", 64, 32, 4, 150, 200, None),    # a chunk behind the append launch
+    ("f16", 256, 16, 4, 1, 2500, None),
+    ("f16", 256, 8, 2, 12, 300, None),
+    ("f32", 64, 32, 4, 1, 2500, None),     # the f32 matrix-pipe kernel at head_dim 64
+    ("f32", 64, 32, 4, 40, 600, None),
+])
+def test_norms_rotation_and_gate_around_the_step(elem, d, q_heads, kv_heads, rows, ctx, window):
+    # The fused preparation (RMS norms, rotation, append) and the output gate at the head dims
+    # whose steps run on the block kernel or the f32 kernel: the preparation is a launch of its
+    # own there, the gate is applied by whichever kernel writes the output.
+    from test_gpu_prep import run_case
+    run_case(elem, q_heads, kv_heads, d, ctx=ctx, rows=rows, norm=True, rope_base=1e6, interleaved=True,
+             rotary=0, gate=True, seed=ctx + rows, window=window)
+    # (Normed in both: the case's raw Q and K are drawn at three and two times unit scale, past
+    # what f16 operands hold to 2e-3 without the norm.)
+    run_case(elem, q_heads, kv_heads, d, ctx=ctx, rows=rows, norm=True, rope_base=1e4, interleaved=False,
+             rotary=d // 2, gate=True, seed=ctx + rows + 1, window=window)
