@@ -90,7 +90,7 @@ enum {
    over the same rounded rows as long as the scaled scores q.k*scale have a standard deviation
    of at most about 3 (3e-5 at unit scale, 1.5e-3 at 3, above the bar from about 4.5 on). Q and K
    normed per head, as the reference's model norms them, stay at unit scale.
-   Matrix-pipe kernels exist for f16 pools at head_dim 64, 128 and 256 with up to 16 Q heads per
+   Matrix-pipe kernels exist for f16 pools at head_dim 64, 96, 128 and 256 with up to 16 Q heads per
    KV head and for f32 pools at head_dim 64 and 128; every other shape (any head_dim up to 256)
    runs on a general kernel that is correct and one to two orders of magnitude slower. */
 enum { ITAK_ELEM_F32 = 0, ITAK_ELEM_F16 = 1 };

@@ -1,4 +1,4 @@
-// Chunked causal prefill attention for gfx950, f16 KV, head_dim 64, 128 or 256 (a template
+// Chunked causal prefill attention for gfx950, f16 KV, head_dim 64, 96, 128 or 256 (a template
 // argument; the figures in these comments are those of head_dim 128): QK^T and PV on
 // v_mfma_f32_16x16x32_f16, everything else (scale, softcap, mask, online softmax) in f32.
 //
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     constexpr int kOut = D / 16;    // output tiles of 16 channels
     constexpr int kBlockElems = block_elems(D);
     constexpr int kStageBytes = stage_bytes(D);
-    constexpr int kPieces = D / 64;      // KiB pieces of a key (or value) block each wavefront moves
+    constexpr int kPieces = (D + 63) / 64;  // KiB pieces of a key (or value) block each wavefront moves
     constexpr int kLoads = 2 * kPieces;  // ring loads a thread issues per block
     constexpr int kChunks = D / 4;       // 16-byte pieces of one side of a new f32 row
     constexpr int kRowsPerPass = kWaves * 64 / (2 * kChunks);  // new rows the workgroup loads at once
@@ -146,10 +146,17 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     // runs (one workgroup per compute unit each) are resident from the start, the second run
     // beside the first: taken in the same order, the longest tiles would share their compute
     // units with the longest of the second half. Every second run is taken in reverse.
+    // The row tiles are reversed, not the KV heads: workgroup i of a launch runs on compute die
+    // i mod 8, so with unit mod kv_heads as the head every die keeps reading the K/V of one head
+    // (two dies per head with 4 KV heads) and the head's blocks are fetched into two L2s, not four.
     if (p.fold_units) {
         const uint32_t run = unit / p.fold_units, idx = unit - run * p.fold_units;
         const uint32_t span = min(p.fold_units, tiles * p.g.kv_heads - run * p.fold_units);
-        if (run & 1) unit = run * p.fold_units + (span - 1 - idx);
+        if (run & 1) {
+            const uint32_t t = idx / p.g.kv_heads, h = idx - t * p.g.kv_heads;
+            unit = run * p.fold_units + (span / p.g.kv_heads - 1 - t) * p.g.kv_heads + h;
+        }
+        unit = __builtin_amdgcn_readfirstlane(unit);  // (the divisions run on the vector unit)
     }
     const uint32_t kv_head = unit % p.g.kv_heads;
     const uint32_t tile = tiles - 1 - unit / p.g.kv_heads;  // longest first
@@ -186,7 +193,11 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
         (lowest_visible(item.pos0 + wave_row_end - 1, window, kv_lo) + kBlockKeys - 1) / kBlockKeys;
 
     // Each wavefront moves kPieces 1 KiB pieces of the key block and as many of the value block
-    // (piece w + 4i for wavefront w).
+    // (piece w + 4i for wavefront w). When the block is not a multiple of 4 KiB (head_dim 96: six
+    // pieces), the wavefronts whose last piece would lie past it fetch their previous piece twice:
+    // every wavefront then has the same number of loads in flight, which is what the waits count.
+    static_assert(D % 32 == 0 && (D % 64 == 0 || kPieces >= 2), "piece plan");
+    const uint32_t last_piece = wave + 4u * (kPieces - 1) < uint32_t(D / 16) ? kPieces - 1 : kPieces - 2;
     const uint4 *kg = reinterpret_cast<const uint4 *>(kplane) + tid;
     // Value pieces are permuted on the way in: LDS position dt*64 + g*16 + jl holds the
     // 16 bytes (channel dt*16 + jl, keys g*8 .. g*8+7), so that the operand read of a
@@ -209,10 +220,15 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
         if (RING && kb + 1 < nblocks) next_sb = next_sb + 1 == ring_blocks ? 0 : next_sb + 1;
         const uint32_t dst = dma_base + (kb % STAGES) * kStageBytes;
 #pragma unroll
-        for (int i = 0; i < kPieces; ++i) lds_dma16(kg + off + 256 * i, dst + 4096 * i);
+        for (int i = 0; i < kPieces; ++i) {
+            const uint32_t ii = i == kPieces - 1 ? last_piece : uint32_t(i);
+            lds_dma16(kg + off + 256 * ii, dst + 4096 * ii);
+        }
 #pragma unroll
-        for (int i = 0; i < kPieces; ++i)
-            lds_dma16(vg + off + 256 * i, dst + 2 * kBlockElems + 4096 * i);
+        for (int i = 0; i < kPieces; ++i) {
+            const uint32_t ii = i == kPieces - 1 ? last_piece : uint32_t(i);
+            lds_dma16(vg + off + 256 * ii, dst + 2 * kBlockElems + 4096 * ii);
+        }
     };
     const bool any_block = kb_begin < nblocks;  // a split past the rows' horizon has none
     ITAK_MARK(1)
@@ -237,7 +253,8 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     // New rows (one-tile form only): piece u of this thread is row nrow + kRowsPerPass * u, side
     // nside, channels nc4 .. nc4 + 3 (at head_dim 128: row (tid >> 6) + 4u, side (tid >> 5) & 1,
     // channels (tid & 31) * 4), requested ahead of Q and waited for with it.
-    constexpr bool kCanFuse = kTiles == 1;
+    // (and only where the pieces of a row pair off with the threads: not at head_dim 96)
+    constexpr bool kCanFuse = kTiles == 1 && (kWaves * 64) % (2 * kChunks) == 0;
     const bool fused = kCanFuse && p.k_new != nullptr;
     const uint32_t nrow = tid / (2 * kChunks);
     const uint32_t nside = (tid / kChunks) & 1u, nc4 = (tid % kChunks) * 4;
@@ -602,12 +619,14 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
 // one-tile form and no item has more than kFuseRows rows.
 bool attn_prefill_f16_appends(const PoolGeom &g, uint32_t group, uint32_t most_rows,
                               uint32_t most_blocks) {
-    return attn_prefill_f16_supports(g, group) && most_rows <= uint32_t(fuse_rows(int(g.head_dim))) &&
+    return attn_prefill_f16_supports(g, group) && (kWaves * 64) % (g.head_dim / 2) == 0 &&
+           most_rows <= uint32_t(fuse_rows(int(g.head_dim))) &&
            most_rows * padded_group(group) <= 512 && most_blocks <= kOneTileBlocks;
 }
 
 bool attn_prefill_f16_supports(const PoolGeom &g, uint32_t group) {
-    return g.v_block == kVBlock && (g.head_dim == 64 || g.head_dim == 128 || g.head_dim == 256) &&
+    return g.v_block == kVBlock &&
+           (g.head_dim == 64 || g.head_dim == 96 || g.head_dim == 128 || g.head_dim == 256) &&
            group >= 1 && group <= 16;
 }
 
@@ -739,7 +758,7 @@ uint32_t attn_prefill_f16_plan(const PoolGeom &g, AttnBatch &b, uint32_t group, 
     // the later workgroups go wherever one ends, which balances better unfolded (4096 and 8192
     // rows measured 1 to 3 % slower folded).
     if (b.n == 1 && b.item[0].splits == 1 && window == 0 && !deep && block0 > per_cu &&
-        block0 <= 2 * per_cu)
+        block0 <= 2 * per_cu && per_cu % g.kv_heads == 0)
         b.fold_units = uint32_t(per_cu);
     return ws0;
 }
@@ -779,6 +798,8 @@ static hipError_t launch_prefill_dim(const AttnParams &p, const AttnBatch &b, ui
         ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, SOFTCAP, TILES, RING, 128>(p, b, total_partials, stream)));
     else if (p.g.head_dim == 64)
         e = launch_prefill<64, SOFTCAP, TILES, RING, 64>(p, b, total_partials, stream);
+    else if (p.g.head_dim == 96)
+        e = launch_prefill<64, SOFTCAP, TILES, RING, 96>(p, b, total_partials, stream);
     else if (p.g.head_dim == 256)
         e = launch_prefill<64, SOFTCAP, TILES, RING, 256>(p, b, total_partials, stream);
     return e;

@@ -68,4 +68,4 @@ def test_registers_of_hand_issued_loads_are_untouched_until_their_wait():
         operands = line.split(None, 1)[1] if " " in line else ""
         assert not (registers(operands) & pending), \
             f"line {n}: a register with a load in flight is used before the wait: {line}"
-    assert kernels >= 72 and runs >= kernels, (kernels, runs)
+    assert kernels >= 88 and runs >= kernels, (kernels, runs)

@@ -1,4 +1,4 @@
-"""f16 pools at head_dim 64 and 256 run on the block kernel (head_dim is a template argument of
+"""f16 pools at head_dim 64, 96 and 256 run on the block kernel (head_dim is a template argument of
 it): decode steps, speculative blocks that append their own rows, prefill chunks, windowed rings
 and ragged batches, against the CPU oracle evaluated over the same f16-rounded cache.
 
@@ -55,7 +55,8 @@ def step(pool, caches, refs, rng, rows, q_heads, softcap=0.0, layer=0):
         at += r
 
 
-@pytest.mark.parametrize("d,q_heads,kv_heads", [(64, 32, 4), (64, 8, 8), (64, 24, 8), (256, 16, 4), (256, 8, 1)])
+@pytest.mark.parametrize("d,q_heads,kv_heads", [(64, 32, 4), (64, 8, 8), (64, 24, 8), (256, 16, 4), (256, 8, 1),
+                                                  (96, 32, 32), (96, 32, 8), (96, 12, 4)])
 @pytest.mark.parametrize("softcap", [0.0, 30.0])
 def test_decode_steps_blocks_and_chunks(d, q_heads, kv_heads, softcap):
     G = P().LayerKind.Global
@@ -64,7 +65,8 @@ def test_decode_steps_blocks_and_chunks(d, q_heads, kv_heads, softcap):
     cache, ref = caches[0], refs[0]
     row = kv_heads * d
     # A prompt's first chunk (no prefix), then decode rows, blocks that append their own rows
-    # (up to 64 at head_dim 64, up to 16 at 256), blocks behind the append launch, a second chunk.
+    # (up to 64 at head_dim 64, up to 16 at 256, never at 96), blocks behind the append launch, a
+    # second chunk.
     kept = []
     for rows in (300, 1, 1, 7, 16, 1, 17, 40, 64, 65, 1, 330, 1, 3):
         base = ref.next_position(0)
@@ -89,7 +91,7 @@ def test_decode_steps_blocks_and_chunks(d, q_heads, kv_heads, softcap):
     pool.close()
 
 
-@pytest.mark.parametrize("d,q_heads,kv_heads", [(64, 32, 4), (256, 8, 2)])
+@pytest.mark.parametrize("d,q_heads,kv_heads", [(64, 32, 4), (256, 8, 2), (96, 16, 4)])
 def test_ragged_batches_split_their_contexts(d, q_heads, kv_heads):
     # Slots of very different lengths in one launch, long enough that the planner splits the
     # context (the merge of head dims other than 128 is the general merge kernel), a slot that
@@ -110,7 +112,8 @@ def test_ragged_batches_split_their_contexts(d, q_heads, kv_heads):
     pool.close()
 
 
-@pytest.mark.parametrize("d,q_heads,kv_heads,window", [(64, 32, 4, 256), (64, 8, 2, 100), (256, 8, 2, 128)])
+@pytest.mark.parametrize("d,q_heads,kv_heads,window", [(64, 32, 4, 256), (64, 8, 2, 100), (256, 8, 2, 128),
+                                                         (96, 8, 2, 100)])
 @pytest.mark.parametrize("softcap", [0.0, 30.0])
 def test_windowed_layers_beside_global_ones(d, q_heads, kv_heads, window, softcap):
     # A windowed ring and a global layer in one pool; the ring wraps several times, by single
@@ -152,6 +155,8 @@ def test_head_dim_64_rewinds_a_speculative_round():
     ("f16", 64, 32, 4, 150, 200, None),    # a chunk behind the append launch
     ("f16", 256, 16, 4, 1, 2500, None),
     ("f16", 256, 8, 2, 12, 300, None),
+    ("f16", 96, 32, 8, 1, 3000, None),
+    ("f16", 96, 8, 8, 9, 300, 128),
     ("f32", 64, 32, 4, 1, 2500, None),     # the f32 matrix-pipe kernel at head_dim 64
     ("f32", 64, 32, 4, 40, 600, None),
 ])
