@@ -48,7 +48,8 @@
 
 // Timeline marks of attn_prefill_f16_kernel: 0 first instruction, 1 addresses known, 2 first
 // blocks and Q requested, 3 Q converted (it has arrived), 4 first block multiplied, 5 last block
-// multiplied, 6 output or partials issued, 11 all done.
+// multiplied, 6 output or partials issued, 11 all done; of the first block: 7 its loads have
+// landed, 8 past the barrier, 9 new rows written over it.
 ITAK_TIMELINE_READER(itak_timeline_read_prefill)
 
 namespace itak {
@@ -82,6 +83,17 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
     float r;
     asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
     return r;
+}
+
+// A mask over the eight halves of an operand register group that keeps the first n (a lane's
+// eight keys of a value piece; element-wise conditional stores into such a vector compile to
+// hundreds of permutes on a path every last block takes).
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x4 first_halves(uint32_t n) {
+    u32x4 m;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) m[j] = n > 2u * j + 1 ? 0xffffffffu : n > 2u * j ? 0x0000ffffu : 0u;
+    return m;
 }
 
 // The direct-to-LDS load is issued from inline assembly: the compiler then neither tracks it
@@ -119,7 +131,7 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     constexpr int kChunks = D / 4;       // 16-byte pieces of one side of a new f32 row
     constexpr int kRowsPerPass = kWaves * 64 / (2 * kChunks);  // new rows the workgroup loads at once
     constexpr int kFuseRows = fuse_rows(D);
-    constexpr int kFusePieces = kFuseRows / kRowsPerPass;  // per thread
+    constexpr int kFusePieces = (kFuseRows + kRowsPerPass - 1) / kRowsPerPass;  // per thread
     constexpr int kVecPerWave = kTiles * 16;
     constexpr int kVecPerGroup = kWaves * kVecPerWave;  // query vectors per workgroup
     extern __shared__ __attribute__((aligned(16))) uint16_t lds_ring[];  // [kStages][K block | V block]
@@ -253,10 +265,11 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     // New rows (one-tile form only): piece u of this thread is row nrow + kRowsPerPass * u, side
     // nside, channels nc4 .. nc4 + 3 (at head_dim 128: row (tid >> 6) + 4u, side (tid >> 5) & 1,
     // channels (tid & 31) * 4), requested ahead of Q and waited for with it.
-    // (and only where the pieces of a row pair off with the threads: not at head_dim 96)
-    constexpr bool kCanFuse = kTiles == 1 && (kWaves * 64) % (2 * kChunks) == 0;
+    // At head_dim 96 a row is 48 pieces: five rows a pass, the last sixteen threads idle.
+    constexpr bool kCanFuse = kTiles == 1;
     const bool fused = kCanFuse && p.k_new != nullptr;
     const uint32_t nrow = tid / (2 * kChunks);
+    const bool nlane = nrow < uint32_t(kRowsPerPass);  // false only where a row is not a divisor of 256 lanes
     const uint32_t nside = (tid / kChunks) & 1u, nc4 = (tid % kChunks) * 4;
     // Does this workgroup's run of blocks reach the new positions? Is it the one that stores them?
     const bool patches = fused && any_block && nblocks * kBlockKeys > item.pos0;
@@ -341,7 +354,7 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
 #pragma unroll
             for (int u = 0; u < kFusePieces; ++u) {
                 // (Uniform over the wavefront when a row is 64 lanes.)
-                if ((2 * kChunks == 64 ? wave : nrow) + uint32_t(kRowsPerPass) * u >= item.rows) continue;
+                if (!nlane || (2 * kChunks == 64 ? wave : nrow) + uint32_t(kRowsPerPass) * u >= item.rows) continue;
                 if (by_element) {
                     const uint32_t h0 = f32_to_f16_bits(nraw[u][0]), h1 = f32_to_f16_bits(nraw[u][1]);
                     const uint32_t h2 = f32_to_f16_bits(nraw[u][2]), h3 = f32_to_f16_bits(nraw[u][3]);
@@ -375,7 +388,7 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
 #pragma unroll
             for (int u = 0; u < kFusePieces; ++u) {
                 const uint32_t r = nrow + uint32_t(kRowsPerPass) * u;
-                if (r >= item.rows) continue;
+                if (!nlane || r >= item.rows) continue;
                 const uint32_t key = item.pos0 + r, kin = key % kBlockKeys;
                 const uint32_t sb = RING ? (key / kBlockKeys) % ring_blocks : key / kBlockKeys;
                 const uint64_t blk = uint64_t(sb) * kBlockElems;
@@ -420,7 +433,9 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
         // may still fly); after the barrier everybody's have, and everybody is done with
         // block kb - 1, whose stage the loads for block kb + 3 may now overwrite.
         wait_vmcnt<kLoads * (STAGES - 2)>();
+        if (kb == kb_begin) { ITAK_MARK(7) }
         __builtin_amdgcn_s_barrier();
+        if (kb == kb_begin) { ITAK_MARK(8) }
         issue_block(kb + STAGES - 1);
         const uint16_t *lds_k = lds_ring + (kb % STAGES) * (kStageBytes / 2);
         const uint16_t *lds_v = lds_k + kBlockElems;
@@ -434,7 +449,7 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
                 for (int u = 0; u < kFusePieces; ++u) {
                     const uint32_t r = nrow + uint32_t(kRowsPerPass) * u;
                     const uint32_t key = item.pos0 + r, kin = key % kBlockKeys;
-                    if (r >= item.rows || key / kBlockKeys != kb) continue;
+                    if (!nlane || r >= item.rows || key / kBlockKeys != kb) continue;
                     if (nside == 0) {
                         const uint32_t kt = (kin >> 2) & 1, ki = (kin >> 3) * 4 + (kin & 3);
                         *reinterpret_cast<uint2 *>(sk + ((kt * (kD / 8) + (nc4 >> 3)) * 16 + ki) * 8 +
@@ -451,6 +466,7 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
                 __builtin_amdgcn_s_barrier();
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+                if (kb == kb_begin) { ITAK_MARK(9) }
             }
         }
 
@@ -499,11 +515,11 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
                         if (key_base + e < collo[qt]) x[qt][e >> 2][e & 3] = -INFINITY;
                 if (kb * kBlockKeys < item_lo) {
                     // Ring rows older than anything the item's queries see may be stale.
+                    const uint32_t stale = min(item_lo - min(item_lo, key_base), 8u);
+                    const u32x4 keep = ~first_halves(stale);
 #pragma unroll
                     for (int dt = 0; dt < kOut; ++dt)
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (key_base + e < item_lo) va[dt][e] = _Float16(0.0f);
+                        va[dt] = __builtin_bit_cast(half8, __builtin_bit_cast(u32x4, va[dt]) & keep);
                 }
             }
             if (kb >= first_masked) {
@@ -514,11 +530,11 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
                         if (key_base + e > colpos[qt]) x[qt][e >> 2][e & 3] = -INFINITY;
                 if ((kb + 1) * kBlockKeys > item.kv_len) {
                     // Rows past the stored length may hold stale data: keep them out of P.V.
+                    const uint32_t stored = min(item.kv_len - min(item.kv_len, key_base), 8u);
+                    const u32x4 keep = first_halves(stored);
 #pragma unroll
                     for (int dt = 0; dt < kOut; ++dt)
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (key_base + e >= item.kv_len) va[dt][e] = _Float16(0.0f);
+                        va[dt] = __builtin_bit_cast(half8, __builtin_bit_cast(u32x4, va[dt]) & keep);
                 }
             }
             float lmax[kTiles];
@@ -619,8 +635,7 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
 // one-tile form and no item has more than kFuseRows rows.
 bool attn_prefill_f16_appends(const PoolGeom &g, uint32_t group, uint32_t most_rows,
                               uint32_t most_blocks) {
-    return attn_prefill_f16_supports(g, group) && (kWaves * 64) % (g.head_dim / 2) == 0 &&
-           most_rows <= uint32_t(fuse_rows(int(g.head_dim))) &&
+    return attn_prefill_f16_supports(g, group) && most_rows <= uint32_t(fuse_rows(int(g.head_dim))) &&
            most_rows * padded_group(group) <= 512 && most_blocks <= kOneTileBlocks;
 }
 
@@ -788,8 +803,16 @@ static hipError_t launch_prefill(const AttnParams &p, const AttnBatch &b, uint32
     return launch_prefill_ring<N, SOFTCAP, TILES, RING, kStages, D>(p, b, total_partials, stream);
 }
 
-// head_dim 128 has an instantiation per batch size class (the batch table is a kernel argument:
-// a decode-sized launch should not carry 64 entries); the other head dims take the largest.
+// head_dim 128 has an instantiation per batch size class (the batch table is a kernel argument,
+// and a large argument block costs a launch about a microsecond); the other head dims have two,
+// one item and any number.
+template <bool SOFTCAP, int TILES, bool RING, int D>
+static hipError_t launch_prefill_other(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                                       hipStream_t stream) {
+    if (b.n <= 1) return launch_prefill<1, SOFTCAP, TILES, RING, D>(p, b, total_partials, stream);
+    return launch_prefill<kMaxBatchItems, SOFTCAP, TILES, RING, D>(p, b, total_partials, stream);
+}
+
 template <bool SOFTCAP, int TILES, bool RING>
 static hipError_t launch_prefill_dim(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                      hipStream_t stream) {
@@ -797,11 +820,11 @@ static hipError_t launch_prefill_dim(const AttnParams &p, const AttnBatch &b, ui
     if (p.g.head_dim == 128)
         ITAK_DISPATCH_BATCH(b.n, (e = launch_prefill<N, SOFTCAP, TILES, RING, 128>(p, b, total_partials, stream)));
     else if (p.g.head_dim == 64)
-        e = launch_prefill<64, SOFTCAP, TILES, RING, 64>(p, b, total_partials, stream);
+        e = launch_prefill_other<SOFTCAP, TILES, RING, 64>(p, b, total_partials, stream);
     else if (p.g.head_dim == 96)
-        e = launch_prefill<64, SOFTCAP, TILES, RING, 96>(p, b, total_partials, stream);
+        e = launch_prefill_other<SOFTCAP, TILES, RING, 96>(p, b, total_partials, stream);
     else if (p.g.head_dim == 256)
-        e = launch_prefill<64, SOFTCAP, TILES, RING, 256>(p, b, total_partials, stream);
+        e = launch_prefill_other<SOFTCAP, TILES, RING, 256>(p, b, total_partials, stream);
     return e;
 }
 

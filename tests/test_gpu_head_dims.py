@@ -65,8 +65,8 @@ def test_decode_steps_blocks_and_chunks(d, q_heads, kv_heads, softcap):
     cache, ref = caches[0], refs[0]
     row = kv_heads * d
     # A prompt's first chunk (no prefix), then decode rows, blocks that append their own rows
-    # (up to 64 at head_dim 64, up to 16 at 256, never at 96), blocks behind the append launch, a
-    # second chunk.
+    # (up to 64 at head_dim 64 and 96, up to 16 at 256), blocks behind the append launch, a second
+    # chunk.
     kept = []
     for rows in (300, 1, 1, 7, 16, 1, 17, 40, 64, 65, 1, 330, 1, 3):
         base = ref.next_position(0)
