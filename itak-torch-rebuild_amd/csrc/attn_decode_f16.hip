@@ -168,25 +168,13 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
         if (j >= group) h = half4{0, 0, 0, 0};
         *reinterpret_cast<half4 *>(sm_q + j * kQStride + c4) = h;
     }
+    uint2 packed{0u, 0u};
     if (owns_new && wave == 0) {
         const uint32_t c4 = (lane & 31) * 4;
-        const uint16_t h0 = f32_to_f16_bits(nraw.x), h1 = f32_to_f16_bits(nraw.y);
-        const uint16_t h2 = f32_to_f16_bits(nraw.z), h3 = f32_to_f16_bits(nraw.w);
-        const uint2 packed{uint32_t(h0) | (uint32_t(h1) << 16), uint32_t(h2) | (uint32_t(h3) << 16)};
+        const uint32_t h0 = f32_to_f16_bits(nraw.x), h1 = f32_to_f16_bits(nraw.y);
+        const uint32_t h2 = f32_to_f16_bits(nraw.z), h3 = f32_to_f16_bits(nraw.w);
+        packed = uint2{h0 | (h1 << 16), h2 | (h3 << 16)};
         *reinterpret_cast<uint2 *>(sm_new + (lane >> 5) * kD + c4) = packed;
-        uint32_t nsb = new_kb;
-        if (RING) nsb %= ring_blocks;
-        const uint64_t blk = uint64_t(nsb) * (kBlockKeys * kD);
-        if (lane < 32) {
-            const uint32_t kt = (kk >> 2) & 1, ki = (kk >> 3) * 4 + (kk & 3);
-            *reinterpret_cast<uint2 *>(kplane + blk + ((kt * 16 + (c4 >> 3)) * 16 + ki) * 8 + (c4 & 7)) = packed;
-        } else {
-            uint16_t *vd = vplane + blk + c4 * kBlockKeys + kk;
-            vd[0] = h0;
-            vd[kBlockKeys] = h1;
-            vd[2 * kBlockKeys] = h2;
-            vd[3 * kBlockKeys] = h3;
-        }
     }
     lds_barrier();
     half8 qb[4];
@@ -202,18 +190,6 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
             for (int s = 0; s < 4; ++s) {
                 const half8 h = *reinterpret_cast<const half8 *>(sm_new + s * 32 + g * 8);
                 if (t_new == 0) bk[0][s] = h; else bk[1][s] = h;
-            }
-        }
-        // Values: lane (g, jl) holds keys g*8 .. g*8+7 of channel dt*16 + jl.
-        if (g == (kk >> 3)) {
-            _Float16 vn[8];
-#pragma unroll
-            for (int dt = 0; dt < 8; ++dt) vn[dt] = sm_new[kD + dt * 16 + jl];
-            switch (kk & 7u) {  // uniform: the element index becomes a constant
-#define ITAK_PUT(E) case E: _Pragma("unroll") for (int dt = 0; dt < 8; ++dt) bv[dt][E] = vn[dt]; break;
-                ITAK_PUT(0) ITAK_PUT(1) ITAK_PUT(2) ITAK_PUT(3) ITAK_PUT(4) ITAK_PUT(5) ITAK_PUT(6)
-                default: _Pragma("unroll") for (int dt = 0; dt < 8; ++dt) bv[dt][7] = vn[dt]; break;
-#undef ITAK_PUT
             }
         }
     }
@@ -248,11 +224,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
     if ((kb + 1) * kBlockKeys > pos + 1 || (RING && kb * kBlockKeys < lo)) {
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-            if (key_base + e > pos || (RING && key_base + e < lo)) {
-                sc[e] = -INFINITY;
-#pragma unroll
-                for (int dt = 0; dt < 8; ++dt) bv[dt][e] = _Float16(0.0f);
-            }
+            if (key_base + e > pos || (RING && key_base + e < lo)) sc[e] = -INFINITY;
     }
     float mx = sc[0];
 #pragma unroll
@@ -268,6 +240,31 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
         pb[e] = static_cast<_Float16>(pe);
     }
     // ---- O^T = V^T . P^T, then the wavefronts meet in LDS.
+    // What touches the value registers comes here, after the scores: the keys arrive first and
+    // the softmax runs while the values are still on their way.
+    if (owns_new && kb == new_kb) {
+        // Values: lane (g, jl) holds keys g*8 .. g*8+7 of channel dt*16 + jl.
+        if (g == (kk >> 3)) {
+            // Half kk % 8 of each register group is replaced through a mask: no jump into one
+            // of eight copies of the insertion, on a path one workgroup per KV head runs, cold.
+            const u32x4 at = first_halves((kk & 7u) + 1) & ~first_halves(kk & 7u);
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) {
+                const uint32_t h = reinterpret_cast<const uint16_t *>(sm_new)[kD + dt * 16 + jl];
+                const uint32_t both = h | (h << 16);
+                const u32x4 old = __builtin_bit_cast(u32x4, bv[dt]);
+                bv[dt] = __builtin_bit_cast(half8, (old & ~at) | (u32x4{both, both, both, both} & at));
+            }
+        }
+    }
+    if ((kb + 1) * kBlockKeys > pos + 1 || (RING && kb * kBlockKeys < lo)) {
+        // This lane's keys [first, end) stay.
+        const uint32_t end = min(pos + 1 - min(pos + 1, key_base), 8u);
+        const uint32_t first = RING ? min(lo - min(lo, key_base), 8u) : 0u;
+        const u32x4 keep = first_halves(end) & ~first_halves(first);
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) bv[dt] = keep_halves(bv[dt], keep);
+    }
     const float l_wave = column_sum4(sum);
     if (g == 0) {
         sm_m[wave * 16 + jl] = dead ? -INFINITY : mx;
@@ -280,6 +277,24 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
         *reinterpret_cast<floatx4 *>(sm_o + ((wave * 8 + dt) * 64 + lane) * 4) = o;
     }
     ITAK_MARK(4)
+    if (owns_new && wave == 0) {
+        // The new row goes to the planes as append lays it out (k_offset / v_offset); nothing in
+        // this launch reads it from there, so the stores wait until the products are under way.
+        const uint32_t c4 = (lane & 31) * 4;
+        uint32_t nsb = new_kb;
+        if (RING) nsb %= ring_blocks;
+        const uint64_t blk = uint64_t(nsb) * (kBlockKeys * kD);
+        if (lane < 32) {
+            const uint32_t kt = (kk >> 2) & 1, ki = (kk >> 3) * 4 + (kk & 3);
+            *reinterpret_cast<uint2 *>(kplane + blk + ((kt * 16 + (c4 >> 3)) * 16 + ki) * 8 + (c4 & 7)) = packed;
+        } else {
+            uint16_t *vd = vplane + blk + c4 * kBlockKeys + kk;
+            vd[0] = uint16_t(packed.x);
+            vd[kBlockKeys] = uint16_t(packed.x >> 16);
+            vd[2 * kBlockKeys] = uint16_t(packed.y);
+            vd[3 * kBlockKeys] = uint16_t(packed.y >> 16);
+        }
+    }
     lds_barrier();
     ITAK_MARK(5)
     // Wavefront w finishes channel tiles 2w and 2w+1 of every column.

@@ -85,17 +85,6 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
     return r;
 }
 
-// A mask over the eight halves of an operand register group that keeps the first n (a lane's
-// eight keys of a value piece; element-wise conditional stores into such a vector compile to
-// hundreds of permutes on a path every last block takes).
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ u32x4 first_halves(uint32_t n) {
-    u32x4 m;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) m[j] = n > 2u * j + 1 ? 0xffffffffu : n > 2u * j ? 0x0000ffffu : 0u;
-    return m;
-}
-
 // The direct-to-LDS load is issued from inline assembly: the compiler then neither tracks it
 // (it would make every LDS read wait for all of them) nor needs to, because the only consumer
 // is ordered by the explicit s_waitcnt vmcnt + s_barrier at the top of each iteration.
@@ -519,7 +508,7 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
                     const u32x4 keep = ~first_halves(stale);
 #pragma unroll
                     for (int dt = 0; dt < kOut; ++dt)
-                        va[dt] = __builtin_bit_cast(half8, __builtin_bit_cast(u32x4, va[dt]) & keep);
+                        va[dt] = keep_halves(va[dt], keep);
                 }
             }
             if (kb >= first_masked) {
@@ -534,7 +523,7 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
                     const u32x4 keep = first_halves(stored);
 #pragma unroll
                     for (int dt = 0; dt < kOut; ++dt)
-                        va[dt] = __builtin_bit_cast(half8, __builtin_bit_cast(u32x4, va[dt]) & keep);
+                        va[dt] = keep_halves(va[dt], keep);
                 }
             }
             float lmax[kTiles];

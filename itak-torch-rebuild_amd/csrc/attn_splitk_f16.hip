@@ -149,12 +149,11 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
     auto zero_tail = [&] {
         // Rows past the stored length, and ring rows older than anything the block's queries
         // see, may hold stale data: keep them out of P.V even as 0*x.
+        const uint32_t end = min(kv_len - min(kv_len, key_base), 8u);
+        const uint32_t first = RING ? min(lo_min - min(lo_min, key_base), 8u) : 0u;
+        const u32x4 keep = first_halves(end) & ~first_halves(first);
 #pragma unroll
-        for (int dt = 0; dt < 8; ++dt)
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                if (key_base + e >= kv_len || (RING && key_base + e < lo_min))
-                    b.v[dt][e] = _Float16(0.0f);
+        for (int dt = 0; dt < 8; ++dt) b.v[dt] = keep_halves(b.v[dt], keep);
     };
     if (NQ <= 2 && tail) zero_tail();
     [[maybe_unused]] half8 pbs[NQ > 2 ? NQ : 1];

@@ -19,6 +19,22 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// A mask over the eight halves of an operand register group (a lane's eight keys of a value
+// piece) that keeps the first n. Element-wise conditional stores into such a vector compile to
+// a permute and a shift per half under execution masks, hundreds of instructions on a path that
+// every workgroup holding a last or oldest block takes once, cold: rows are dropped with an AND.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x4 first_halves(uint32_t n) {
+    u32x4 m;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) m[j] = n > 2u * j + 1 ? 0xffffffffu : n > 2u * j ? 0x0000ffffu : 0u;
+    return m;
+}
+// Zeroes the halves of v whose mask bits are clear.
+__device__ __forceinline__ half8 keep_halves(half8 v, u32x4 keep) {
+    return __builtin_bit_cast(half8, __builtin_bit_cast(u32x4, v) & keep);
+}
+
 // The value of another lane of the same 16-lane row, chosen by a DPP control word.
 template <int CTRL>
 __device__ __forceinline__ float dpp_lane(float v) {
