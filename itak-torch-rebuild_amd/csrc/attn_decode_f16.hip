@@ -277,24 +277,6 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
         *reinterpret_cast<floatx4 *>(sm_o + ((wave * 8 + dt) * 64 + lane) * 4) = o;
     }
     ITAK_MARK(4)
-    if (owns_new && wave == 0) {
-        // The new row goes to the planes as append lays it out (k_offset / v_offset); nothing in
-        // this launch reads it from there, so the stores wait until the products are under way.
-        const uint32_t c4 = (lane & 31) * 4;
-        uint32_t nsb = new_kb;
-        if (RING) nsb %= ring_blocks;
-        const uint64_t blk = uint64_t(nsb) * (kBlockKeys * kD);
-        if (lane < 32) {
-            const uint32_t kt = (kk >> 2) & 1, ki = (kk >> 3) * 4 + (kk & 3);
-            *reinterpret_cast<uint2 *>(kplane + blk + ((kt * 16 + (c4 >> 3)) * 16 + ki) * 8 + (c4 & 7)) = packed;
-        } else {
-            uint16_t *vd = vplane + blk + c4 * kBlockKeys + kk;
-            vd[0] = uint16_t(packed.x);
-            vd[kBlockKeys] = uint16_t(packed.x >> 16);
-            vd[2 * kBlockKeys] = uint16_t(packed.y);
-            vd[3 * kBlockKeys] = uint16_t(packed.y >> 16);
-        }
-    }
     lds_barrier();
     ITAK_MARK(5)
     // Wavefront w finishes channel tiles 2w and 2w+1 of every column.
@@ -322,6 +304,27 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
         acc[0] += ow[0][w] * wgt;
         acc[1] += ow[1][w] * wgt;
     }
+    // The new row goes to the planes as append lays it out (k_offset / v_offset). Nothing in this
+    // launch reads it from there, so the stores are the last thing their wavefront issues: the
+    // others of its workgroup never wait behind them.
+    auto store_new_row = [&] {
+    if (owns_new && wave == 0) {
+            const uint32_t c4 = (lane & 31) * 4;
+            uint32_t nsb = new_kb;
+            if (RING) nsb %= ring_blocks;
+            const uint64_t blk = uint64_t(nsb) * (kBlockKeys * kD);
+            if (lane < 32) {
+                const uint32_t kt = (kk >> 2) & 1, ki = (kk >> 3) * 4 + (kk & 3);
+                *reinterpret_cast<uint2 *>(kplane + blk + ((kt * 16 + (c4 >> 3)) * 16 + ki) * 8 + (c4 & 7)) = packed;
+            } else {
+                uint16_t *vd = vplane + blk + c4 * kBlockKeys + kk;
+                vd[0] = uint16_t(packed.x);
+                vd[kBlockKeys] = uint16_t(packed.x >> 16);
+                vd[2 * kBlockKeys] = uint16_t(packed.y);
+                vd[3 * kBlockKeys] = uint16_t(packed.y >> 16);
+            }
+        }
+    };
     if (item.splits == 1) {
         if (jl < group) {
             float *dst = p.out + (uint64_t(item.q_row0) * p.q_heads + kv_head * group + jl) * kD;
@@ -330,6 +333,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
             for (int x = 0; x < 2; ++x)
                 *reinterpret_cast<floatx4 *>(dst + (wave * 2 + x) * 16 + g * 4) = acc[x] * inv;
         }
+        store_new_row();
         ITAK_MARK_END
         return;
     }
@@ -346,6 +350,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
                     make_float2(M, L);
         }
         ITAK_MARK(6)
+        store_new_row();
         ITAK_MARK_END
         return;
     }
@@ -356,6 +361,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
         xg.publish(jl, wave * 2 + 1, g, acc[1], M, L);
     }
     ITAK_MARK(6)
+    store_new_row();
     unsigned long long gathered_at = 0;
     xg.template finish<kWaves * 64, kDecodeWords, kDecodeLooks>(reinterpret_cast<unsigned long long *>(sm_o), p, item, kv_head, group,
                                     p.group_magic, nullptr, &gathered_at);
