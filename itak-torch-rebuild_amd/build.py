@@ -38,7 +38,11 @@ def _compile(src: str, timeline: bool = False) -> str:
            os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
-    lines = [l for l in res.stderr.splitlines() if noise not in l]
+    raw = res.stderr.splitlines()
+    # (Notes and remarks about code in a header arrive under an "In file included from" line.)
+    lines = [l for i, l in enumerate(raw) if noise not in l and not (
+        l.startswith("In file included from") and i + 1 < len(raw) and
+        (noise in raw[i + 1] or "remark:" in raw[i + 1]))]
     remarks = [l for l in lines if "-Rpass-analysis=kernel-resource-usage" in l]
     err = "\n".join(l for l in lines if l not in remarks and "remark" not in l)
     if res.returncode != 0:

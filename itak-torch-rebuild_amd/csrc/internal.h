@@ -408,6 +408,10 @@ bool attn_prefill_f16_appends(const PoolGeom &g, uint32_t group, uint32_t most_r
                               uint32_t most_blocks);
 hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                    hipStream_t stream);
+// The same at head dims 64, 96 and 256 (instantiated in a file of their own); `one` = the
+// one-tile form, as launch_attn_prefill_f16 decides it.
+hipError_t launch_attn_prefill_f16_dims(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                                        bool one, hipStream_t stream);
 // Merge of split partials; total_rows = query rows of the batch. With `gate` the merged rows
 // are multiplied by sigmoid(gate) as they are written (items with one split are not touched:
 // their writer was the attention kernel).
