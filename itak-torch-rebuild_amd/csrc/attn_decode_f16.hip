@@ -98,8 +98,22 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
                      "s"(b.item[0].kv_lo), "s"(p.window), "s"(p.ring_blocks));
     const AttnItem item = b.item[b.find_by_block(blockIdx.x)];
     const uint32_t local = blockIdx.x - item.block0;
-    const uint32_t kv_head = item.splits > 1 ? __umulhi(local, item.splits_magic) : local;
-    const uint32_t split = local - kv_head * item.splits;
+    // Workgroups reach the device in the order of their index and the launch ends with its
+    // slowest: the last split of every KV head, which holds the new position and has the most to
+    // do, takes the first indices (split-major order, last split first).
+    const uint32_t heads = p.g.kv_heads;
+    uint32_t kv_head = local, split = 0;
+    if (item.splits > 1) {
+        uint32_t behind;  // splits after this one
+        if ((heads & (heads - 1)) == 0) {
+            behind = local >> __builtin_ctz(heads);
+            kv_head = local & (heads - 1);
+        } else {
+            behind = local / heads;
+            kv_head = local - behind * heads;
+        }
+        split = item.splits - 1 - behind;
+    }
     const uint32_t group = p.group;
 
     uint16_t *kplane = static_cast<uint16_t *>(const_cast<void *>(p.layer_base)) +
