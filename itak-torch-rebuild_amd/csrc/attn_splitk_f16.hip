@@ -1057,17 +1057,31 @@ __global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(AttnParam
     }
 }
 
-// The same merge for head_dim 128, shaped for latency (it runs for about two microseconds
-// per decode layer): grid = (Q head, query row), thread = (4 channels c, split lane sl of 8).
-// A thread issues every load of its first 8 splits, accumulators and (m, l) pairs alike,
-// before it waits for anything, folds them with its own running maximum, and the eight
-// split lanes meet once in LDS. One memory round trip and one barrier.
+// The same merge for head_dim 128, shaped for latency (it runs for under two microseconds per
+// decode layer): grid = (Q head, query row); wavefront w owns channels 32w .. 32w+31, lane =
+// (4 channels c of its 8 chunks, split lane sl of 8). A lane issues every load of its first 8
+// splits, accumulators and (m, l) pairs alike, before it waits for anything, folds them with its
+// own running maximum, and the eight split lanes meet through lane permutes: one memory round
+// trip, no LDS and no barrier, and no stretch that a single wavefront runs while three wait (the
+// form with a barrier and 32 threads finishing cost 0.4 us more per launch).
+__device__ __forceinline__ float split_lanes_max(float v) {  // over lane bits 3, 4, 5
+    v = fmaxf(v, dpp_lane<0x128>(v));  // row_ror:8
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(c[0]), __uint_as_float(c[1]));
+}
+__device__ __forceinline__ float split_lanes_sum(float v) {
+    v += dpp_lane<0x128>(v);
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(c[0]) + __uint_as_float(c[1]);
+}
 template <int N, bool BASE2, bool GATE>
 __device__ __forceinline__ void attn_combine128_body(const AttnParams &p, const AttnBatchT<N> &b,
                                                      uint32_t total_partials,
                                                      [[maybe_unused]] const float *gate) {
-    __shared__ float4 part[256];
-    __shared__ float part_m[8], part_l[8];
     const uint32_t tid = threadIdx.x;
     ITAK_MARK_BEGIN
     ITAK_MARK(0)
@@ -1082,14 +1096,14 @@ __device__ __forceinline__ void attn_combine128_body(const AttnParams &p, const 
     if (S == 1) return;
     const uint32_t row = grow - (item.q_row0 - b.base_row);
     const uint64_t ps0 = item.ws0 + (uint64_t(row) * p.q_heads + head) * S;
-    const uint32_t c = tid & 31, sl = tid >> 5;
+    const uint32_t wave = tid >> 6, lane = tid & 63;
+    const uint32_t c = wave * 8 + (lane & 7), sl = lane >> 3;  // chunk of 4 channels, split lane
     const float *ws_acc = p.ws + ps0 * 128 + c * 4;
     const float2 *ws_ml = reinterpret_cast<const float2 *>(p.ws + uint64_t(total_partials) * 128) + ps0;
-    // The gate of the 32 threads that write the output, fetched with the partials.
+    const uint64_t at = (uint64_t(item.q_row0 + row) * p.q_heads + head) * 128 + c * 4;
+    // The gate of the lanes that write the output, fetched with the partials.
     [[maybe_unused]] float4 gt = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (GATE && tid < 32)
-        gt = *reinterpret_cast<const float4 *>(
-            gate + (uint64_t(item.q_row0 + row) * p.q_heads + head) * 128 + tid * 4);
+    if (GATE && sl == 0) gt = *reinterpret_cast<const float4 *>(gate + at);
     ITAK_MARK(1)
 
     float m_run = -INFINITY, l_run = 0.0f;
@@ -1125,38 +1139,21 @@ __device__ __forceinline__ void attn_combine128_body(const AttnParams &p, const 
             acc.w = fmaf(x[u].w, w, acc.w);
         }
     }
-    part[tid] = acc;
-    if (c == 0) {
-        part_m[sl] = m_run;
-        part_l[sl] = l_run;
-    }
     ITAK_MARK(7)
-    __syncthreads();
+    // The eight split lanes of a chunk: a common maximum, then the weighted sums.
+    const float M = split_lanes_max(m_run);
+    const float w = m_run == -INFINITY ? 0.0f : (BASE2 ? fast_exp2(m_run - M) : __expf(m_run - M));
+    const float L = split_lanes_sum(l_run * w);
+    float4 sum = make_float4(split_lanes_sum(acc.x * w), split_lanes_sum(acc.y * w),
+                             split_lanes_sum(acc.z * w), split_lanes_sum(acc.w * w));
     ITAK_MARK(8)
-    if (tid < 32) {
-        float M = part_m[0];
-#pragma unroll
-        for (int l = 1; l < 8; ++l) M = fmaxf(M, part_m[l]);
-        float L = 0.0f;
-        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-        for (int l = 0; l < 8; ++l) {
-            const float ml = part_m[l];
-            const float w = ml == -INFINITY ? 0.0f : (BASE2 ? fast_exp2(ml - M) : __expf(ml - M));
-            const float4 y = part[l * 32 + tid];
-            L = fmaf(part_l[l], w, L);
-            sum.x = fmaf(y.x, w, sum.x);
-            sum.y = fmaf(y.y, w, sum.y);
-            sum.z = fmaf(y.z, w, sum.z);
-            sum.w = fmaf(y.w, w, sum.w);
-        }
+    if (sl == 0) {
         const float inv = 1.0f / L;
-        float *dst = p.out + (uint64_t(item.q_row0 + row) * p.q_heads + head) * 128;
         float4 o = make_float4(sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv);
         if (GATE)
             o = make_float4(o.x * sigmoid_fast(gt.x), o.y * sigmoid_fast(gt.y),
                             o.z * sigmoid_fast(gt.z), o.w * sigmoid_fast(gt.w));
-        *reinterpret_cast<float4 *>(dst + tid * 4) = o;
+        *reinterpret_cast<float4 *>(p.out + at) = o;
     }
     ITAK_MARK(9)
     ITAK_MARK_END_AT(ITAK_TIMELINE_WAVES / 2)
