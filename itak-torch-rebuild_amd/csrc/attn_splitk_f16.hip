@@ -1117,6 +1117,9 @@ __device__ __forceinline__ void attn_combine128_body(const AttnParams &p, const 
             x[u] = *reinterpret_cast<const float4 *>(ws_acc + uint64_t(s) * 128);
             ml[u] = ws_ml[s];
         }
+        // Nothing below may move above this line and no load below it: left to itself the
+        // scheduler issues half of the accumulator loads after the first weights are computed.
+        __builtin_amdgcn_sched_barrier(0);
         if (s0 == 0) { ITAK_MARK(2) }
         float mx = m_run;
 #pragma unroll
@@ -1124,14 +1127,18 @@ __device__ __forceinline__ void attn_combine128_body(const AttnParams &p, const 
             if (s0 + sl + u * 8 >= S) ml[u].x = -INFINITY;
             mx = fmaxf(mx, ml[u].x);
         }
-        if (mx == -INFINITY) continue;  // nothing visible in these splits (nor before)
-        const float alpha = BASE2 ? fast_exp2(m_run - mx) : __expf(m_run - mx);  // 0 at first
+        // Nothing visible in these splits (nor before): every weight below is exp(-inf) = 0
+        // against a finite stand-in. No branch around the arithmetic: behind one the compiler
+        // fetches the maxima first and the accumulators after it has looked at them, two memory
+        // round trips instead of one.
+        const float ref = mx == -INFINITY ? 0.0f : mx;
+        const float alpha = BASE2 ? fast_exp2(m_run - ref) : __expf(m_run - ref);  // 0 at first
         acc.x *= alpha, acc.y *= alpha, acc.z *= alpha, acc.w *= alpha;
         l_run *= alpha;
         m_run = mx;
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-            const float w = BASE2 ? fast_exp2(ml[u].x - mx) : __expf(ml[u].x - mx);  // exp(-inf) = 0
+            const float w = BASE2 ? fast_exp2(ml[u].x - ref) : __expf(ml[u].x - ref);  // exp(-inf) = 0
             l_run = fmaf(ml[u].y, w, l_run);
             acc.x = fmaf(x[u].x, w, acc.x);
             acc.y = fmaf(x[u].y, w, acc.y);
@@ -1148,7 +1155,7 @@ __device__ __forceinline__ void attn_combine128_body(const AttnParams &p, const 
                              split_lanes_sum(acc.z * w), split_lanes_sum(acc.w * w));
     ITAK_MARK(8)
     if (sl == 0) {
-        const float inv = 1.0f / L;
+        const float inv = __builtin_amdgcn_rcpf(L);  // within an ulp: far inside either pool's bar
         float4 o = make_float4(sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv);
         if (GATE)
             o = make_float4(o.x * sigmoid_fast(gt.x), o.y * sigmoid_fast(gt.y),
