@@ -340,7 +340,7 @@ def timeline(args, pkg, torch, np):
         table(f"attn_combine128_kernel ({merge_rows[0].shape[0]} wavefronts per launch)", merge_rows, [
             (0, "first instruction"), (1, "kernel arguments in, addresses known"),
             (2, "every load issued"), (7, "sums done (partials arrived)"),
-            (8, "past the workgroup barrier"), (9, "output issued"),
+            (8, "split lanes joined"), (9, "output issued"),
             (11, "everything in flight done (stores acknowledged)")])
     pool.close()
 
