@@ -321,6 +321,10 @@ struct AttnParams {
     // many (one per compute unit); every second run takes its units in reverse, so that the
     // two workgroups that share a compute unit are a long row tile and a short one. 0 = off.
     uint32_t fold_units;
+    // The step's keys and values, over all layers of the pool, are more than the last-level cache
+    // holds (so the next step will not find them there): kernels that read each row once may ask
+    // for them with the streaming hint.
+    uint32_t kv_streams;
 };
 // What the reference's model does around the step (muse-glimmer/src/model.rs:445-464),
 // folded into the step's own launches instead of running as launches of their own. `gate`

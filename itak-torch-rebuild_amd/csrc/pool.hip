@@ -584,6 +584,13 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         p.ws = ws;
         p.exchange = exchange_words ? 1 : 0;
         p.fold_units = prefill ? b.fold_units : 0;
+        {
+            uint64_t rows_read = 0;
+            for (uint32_t i = 0; i < count; ++i) rows_read += b.item[i].kv_len - b.item[i].kv_lo;
+            const uint64_t layer_bytes = rows_read * 2 * pool->g.kv_heads * pool->g.head_dim *
+                                         (pool->elem_f16 ? 2 : 4);
+            p.kv_streams = layer_bytes * pool->layers.size() > (uint64_t(512) << 20) ? 1 : 0;  // twice the cache: well clear of it
+        }
         p.spin_limit = pool->spin_limit;
         p.k_new = (mfma || f32fast || prefill) ? k_new : nullptr;  // the caller passes them only to
         p.v_new = (mfma || f32fast || prefill) ? v_new : nullptr;  // launches that append themselves
