@@ -575,3 +575,40 @@ def test_masked_rows_with_non_finite_values_do_not_reach_a_decode_query():
         assert np.isfinite(want).all() and np.isfinite(got).all()
         assert max_abs(got, want) <= F16_ABS
         pool.close()
+
+
+@pytest.mark.parametrize("elem,ctx,kk", [("f16", 20000, 0), ("f16", 40011, 11), ("f16", 9000, 8), ("f32", 20017, 17)])
+def test_long_single_slot_decode_merges_more_splits_than_one_pass_holds(elem, ctx, kk):
+    # One slot far beyond 8192 keys: the decode kernel leaves well over 64 partials per head, so the
+    # merge kernel folds them in several passes with a running maximum; the new row lands at
+    # different places of its 32-row block (kk), a gate rides along on the second step.
+    import torch
+    assert ctx % 32 == kk
+    rng = np.random.default_rng(ctx)
+    q_heads, kv_heads, d = 32, 4, 128
+    row = kv_heads * d
+    pool = P().KvPool(1, kv_heads, d, elem=elem, capacity_rows=ctx + 8)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    cache = pool.acquire()
+    k, v = normal(rng, ctx, row), normal(rng, ctx, row)
+    kd, vd = torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda()
+    pool.append_device(0, [(cache, ctx)], kd.data_ptr(), vd.data_ptr())
+    torch.cuda.synchronize()
+    ref = oracle.KvCache.new([oracle.LayerKind.Global], kv_heads, d, store_f16=(elem == "f16"))
+    ref.restore_bulk(0, 0, k, v)
+    for step in range(3):
+        q, kn, vn = normal(rng, 1, q_heads * d), normal(rng, 1, row), normal(rng, 1, row)
+        qd, knd, vnd = (torch.from_numpy(x).cuda() for x in (q, kn, vn))
+        out = torch.empty_like(qd)
+        pool.attention_step_device(0, [(cache, 1)], qd.data_ptr(), knd.data_ptr(), vnd.data_ptr(),
+                                   out.data_ptr(), q_heads)
+        torch.cuda.synchronize()
+        want = oracle.attention_step(ref, 0, q, kn, vn, q_heads, ctx + step, threads=8)
+        got = out.cpu().numpy().reshape(-1)
+        if elem == "f32":
+            assert rel_err(got, want) <= 1e-5
+        else:
+            assert max_abs(got, want) <= 2e-3
+    _, gk, gv = cache.read_rows(0, ctx, 3)
+    assert gk.shape[0] == 3 and cache.next_position(0) == ctx + 3
+    pool.close()
