@@ -1064,24 +1064,34 @@ __global__ __launch_bounds__(kCombineThreads) void attn_combine_kernel(AttnParam
 // own running maximum, and the eight split lanes meet through lane permutes: one memory round
 // trip, no LDS and no barrier, and no stretch that a single wavefront runs while three wait (the
 // form with a barrier and 32 threads finishing cost 0.4 us more per launch).
-__device__ __forceinline__ float split_lanes_max(float v) {  // over lane bits 3, 4, 5
-    v = fmaxf(v, dpp_lane<0x128>(v));  // row_ror:8
+// SL = split lanes of a chunk: lanes that differ in the bits above log2(64 / SL).
+template <int SL>
+__device__ __forceinline__ float split_lanes_max(float v) {
+    if constexpr (SL >= 16) v = fmaxf(v, dpp_lane<0x124>(v));  // row_ror:4
+    if constexpr (SL >= 8) v = fmaxf(v, dpp_lane<0x128>(v));   // row_ror:8
     const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
     v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
     const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
     return fmaxf(__uint_as_float(c[0]), __uint_as_float(c[1]));
 }
+template <int SL>
 __device__ __forceinline__ float split_lanes_sum(float v) {
-    v += dpp_lane<0x128>(v);
+    if constexpr (SL >= 16) v += dpp_lane<0x124>(v);
+    if constexpr (SL >= 8) v += dpp_lane<0x128>(v);
     const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
     v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
     const auto c = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
     return __uint_as_float(c[0]) + __uint_as_float(c[1]);
 }
-template <int N, bool BASE2, bool GATE>
+// D = head_dim (64, 96, 128 or 256): a wavefront owns D/4 channels, i.e. D/16 chunks, in the next
+// power of two of lanes (at 96 two of eight sit idle), and the other lane bits are split lanes.
+template <int N, bool BASE2, bool GATE, int D = 128>
 __device__ __forceinline__ void attn_combine128_body(const AttnParams &p, const AttnBatchT<N> &b,
                                                      uint32_t total_partials,
                                                      [[maybe_unused]] const float *gate) {
+    constexpr uint32_t kChunks = D / 16;                                   // per wavefront
+    constexpr uint32_t kChunkLanes = kChunks <= 4 ? 4 : kChunks <= 8 ? 8 : 16;
+    constexpr int SL = 64 / kChunkLanes;                                   // split lanes
     const uint32_t tid = threadIdx.x;
     ITAK_MARK_BEGIN
     ITAK_MARK(0)
@@ -1097,24 +1107,26 @@ __device__ __forceinline__ void attn_combine128_body(const AttnParams &p, const 
     const uint32_t row = grow - (item.q_row0 - b.base_row);
     const uint64_t ps0 = item.ws0 + (uint64_t(row) * p.q_heads + head) * S;
     const uint32_t wave = tid >> 6, lane = tid & 63;
-    const uint32_t c = wave * 8 + (lane & 7), sl = lane >> 3;  // chunk of 4 channels, split lane
-    const float *ws_acc = p.ws + ps0 * 128 + c * 4;
-    const float2 *ws_ml = reinterpret_cast<const float2 *>(p.ws + uint64_t(total_partials) * 128) + ps0;
-    const uint64_t at = (uint64_t(item.q_row0 + row) * p.q_heads + head) * 128 + c * 4;
+    const uint32_t cl = lane % kChunkLanes, sl = lane / kChunkLanes;  // chunk of the wavefront, split lane
+    const bool holds = cl < kChunks;                                   // (false only at head_dim 96)
+    const uint32_t c = wave * kChunks + min(cl, kChunks - 1);          // chunk of 4 channels
+    const float *ws_acc = p.ws + ps0 * D + c * 4;
+    const float2 *ws_ml = reinterpret_cast<const float2 *>(p.ws + uint64_t(total_partials) * D) + ps0;
+    const uint64_t at = (uint64_t(item.q_row0 + row) * p.q_heads + head) * D + c * 4;
     // The gate of the lanes that write the output, fetched with the partials.
     [[maybe_unused]] float4 gt = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (GATE && sl == 0) gt = *reinterpret_cast<const float4 *>(gate + at);
+    if (GATE && sl == 0 && holds) gt = *reinterpret_cast<const float4 *>(gate + at);
     ITAK_MARK(1)
 
     float m_run = -INFINITY, l_run = 0.0f;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (uint32_t s0 = 0; s0 < S; s0 += 64) {
+    for (uint32_t s0 = 0; s0 < S; s0 += 8 * SL) {
         float4 x[8];
         float2 ml[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {  // clamped, so the loads need no branch
-            const uint32_t s = min(s0 + sl + u * 8, S - 1);
-            x[u] = *reinterpret_cast<const float4 *>(ws_acc + uint64_t(s) * 128);
+            const uint32_t s = min(s0 + sl + u * SL, S - 1);
+            x[u] = *reinterpret_cast<const float4 *>(ws_acc + uint64_t(s) * D);
             ml[u] = ws_ml[s];
         }
         // Nothing below may move above this line and no load below it: left to itself the
@@ -1124,7 +1136,7 @@ __device__ __forceinline__ void attn_combine128_body(const AttnParams &p, const 
         float mx = m_run;
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-            if (s0 + sl + u * 8 >= S) ml[u].x = -INFINITY;
+            if (s0 + sl + u * SL >= S) ml[u].x = -INFINITY;
             mx = fmaxf(mx, ml[u].x);
         }
         // Nothing visible in these splits (nor before): every weight below is exp(-inf) = 0
@@ -1148,13 +1160,13 @@ __device__ __forceinline__ void attn_combine128_body(const AttnParams &p, const 
     }
     ITAK_MARK(7)
     // The eight split lanes of a chunk: a common maximum, then the weighted sums.
-    const float M = split_lanes_max(m_run);
+    const float M = split_lanes_max<SL>(m_run);
     const float w = m_run == -INFINITY ? 0.0f : (BASE2 ? fast_exp2(m_run - M) : __expf(m_run - M));
-    const float L = split_lanes_sum(l_run * w);
-    float4 sum = make_float4(split_lanes_sum(acc.x * w), split_lanes_sum(acc.y * w),
-                             split_lanes_sum(acc.z * w), split_lanes_sum(acc.w * w));
+    const float L = split_lanes_sum<SL>(l_run * w);
+    float4 sum = make_float4(split_lanes_sum<SL>(acc.x * w), split_lanes_sum<SL>(acc.y * w),
+                             split_lanes_sum<SL>(acc.z * w), split_lanes_sum<SL>(acc.w * w));
     ITAK_MARK(8)
-    if (sl == 0) {
+    if (sl == 0 && holds) {
         const float inv = __builtin_amdgcn_rcpf(L);  // within an ulp: far inside either pool's bar
         float4 o = make_float4(sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv);
         if (GATE)
@@ -1176,6 +1188,15 @@ __global__ __launch_bounds__(256) void attn_combine128_gate_kernel(AttnParams p,
                                                                    uint32_t total_partials,
                                                                    const float *gate) {
     attn_combine128_body<N, BASE2, true>(p, b, total_partials, gate);
+}
+
+// The same merge at head dims 64, 96 and 256 (the partials of the block kernel and, at 64, of the
+// f32 kernel).
+template <int N, bool BASE2, bool GATE, int D>
+__global__ __launch_bounds__(256) void attn_combine_lanes_kernel(AttnParams p, AttnBatchT<N> b,
+                                                                 uint32_t total_partials,
+                                                                 const float *gate) {
+    attn_combine128_body<N, BASE2, GATE, D>(p, b, total_partials, gate);
 }
 
 // The same merge for items of at most 16 splits, one wavefront per (row, Q head): lane =
@@ -1284,6 +1305,25 @@ hipError_t launch_attn_combine(const AttnParams &p, const AttnBatch &b, uint32_t
         else
             ITAK_DISPATCH_BATCH(b.n, (attn_combine128_kernel<N, false><<<grid, 256, 0, stream>>>(
                                          p, AttnBatchT<N>(b), total_partials)));
+        return hipGetLastError();
+    }
+    if (p.g.head_dim == 64 || p.g.head_dim == 96 || p.g.head_dim == 256) {
+        const dim3 grid(p.q_heads, total_rows);
+#define ITAK_LANES(B2, G, D)                                                                  \
+    ITAK_DISPATCH_BATCH(b.n, (attn_combine_lanes_kernel<N, B2, G, D><<<grid, 256, 0, stream>>>( \
+                                 p, AttnBatchT<N>(b), total_partials, gate)))
+#define ITAK_LANES_D(D)                                \
+    do {                                               \
+        if (gate && base2) ITAK_LANES(true, true, D);  \
+        else if (gate) ITAK_LANES(false, true, D);     \
+        else if (base2) ITAK_LANES(true, false, D);    \
+        else ITAK_LANES(false, false, D);              \
+    } while (0)
+        if (p.g.head_dim == 64) ITAK_LANES_D(64);
+        else if (p.g.head_dim == 96) ITAK_LANES_D(96);
+        else ITAK_LANES_D(256);
+#undef ITAK_LANES_D
+#undef ITAK_LANES
         return hipGetLastError();
     }
     ITAK_DISPATCH_BATCH(b.n, (attn_combine_kernel<N><<<total_rows * p.q_heads, kCombineThreads, 0,
