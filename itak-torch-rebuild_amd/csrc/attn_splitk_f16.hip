@@ -1307,7 +1307,10 @@ hipError_t launch_attn_combine(const AttnParams &p, const AttnBatch &b, uint32_t
                                          p, AttnBatchT<N>(b), total_partials)));
         return hipGetLastError();
     }
-    if (p.g.head_dim == 64 || p.g.head_dim == 96 || p.g.head_dim == 256) {
+    // (A workgroup per output pays where the merge is a matter of latency; with thousands of
+    // outputs, a 512-row chunk, the general kernel below is the faster one by a tenth of the step.)
+    if ((p.g.head_dim == 64 || p.g.head_dim == 96 || p.g.head_dim == 256) &&
+        uint64_t(total_rows) * p.q_heads <= 4096) {
         const dim3 grid(p.q_heads, total_rows);
 #define ITAK_LANES(B2, G, D)                                                                  \
     ITAK_DISPATCH_BATCH(b.n, (attn_combine_lanes_kernel<N, B2, G, D><<<grid, 256, 0, stream>>>( \
