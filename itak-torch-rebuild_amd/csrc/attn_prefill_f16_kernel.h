@@ -264,6 +264,7 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     const bool patches = fused && any_block && nblocks * kBlockKeys > item.pos0;
     const bool stores_new = fused && unit < p.g.kv_heads && split == item.splits - 1;
     const bool with_new = patches || stores_new;
+    const bool by_stage = stores_new && patches && item.rows >= 8;  // see the stores below
     [[maybe_unused]] uint2 npk[kCanFuse ? kFusePieces : 1];
     half8 qb[kTiles][kSteps];
     uint32_t colpos[kTiles], collo[kTiles];
@@ -372,13 +373,21 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
 #undef ITAK_RING_FILL
 #undef ITAK_Q_LOADS
     if constexpr (kCanFuse) {
-        if (stores_new) {  // as the append kernel lays them out (k_offset / v_offset)
+        // As the append kernel lays them out (k_offset / v_offset). From registers, a value row
+        // leaves as one two-byte store per channel (sixty-four such stores a thread for a 64-row
+        // block, each touching as many cache lines as it has lanes: 6 us in the one workgroup per
+        // KV head that stores, the last to finish). Blocks of eight rows or more are therefore
+        // stored block by block from the LDS stage once the rows have been written over it (below),
+        // sixteen bytes a thread and store; what remains here are short blocks and rows of key
+        // blocks that lie before this workgroup's run.
+        if (stores_new) {
             uint16_t *kp = const_cast<uint16_t *>(kplane), *vp = const_cast<uint16_t *>(vplane);
 #pragma unroll
             for (int u = 0; u < kFusePieces; ++u) {
                 const uint32_t r = nrow + uint32_t(kRowsPerPass) * u;
                 if (!nlane || r >= item.rows) continue;
                 const uint32_t key = item.pos0 + r, kin = key % kBlockKeys;
+                if (by_stage && key / kBlockKeys >= kb_begin) continue;
                 const uint32_t sb = RING ? (key / kBlockKeys) % ring_blocks : key / kBlockKeys;
                 const uint64_t blk = uint64_t(sb) * kBlockElems;
                 if (nside == 0) {
@@ -455,6 +464,21 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
                 __builtin_amdgcn_s_barrier();
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+                if (by_stage) {
+                    // The stage now is what the planes' block should hold (rows past the new ones
+                    // are what the loads brought from there): back it goes, the key block as it
+                    // lies, the value pieces to where their load took them from.
+                    const uint32_t sb = RING ? kb % ring_blocks : kb;
+                    uint4 *kdst = reinterpret_cast<uint4 *>(const_cast<uint16_t *>(kplane)) + uint64_t(sb) * kBlockVec;
+                    uint4 *vdst = reinterpret_cast<uint4 *>(const_cast<uint16_t *>(vplane)) + uint64_t(sb) * kBlockVec;
+                    const uint4 *ks = reinterpret_cast<const uint4 *>(sk), *vs = reinterpret_cast<const uint4 *>(sv);
+#pragma unroll
+                    for (uint32_t i = tid; i < kBlockVec; i += kWaves * 64) {
+                        kdst[i] = ks[i];
+                        const uint32_t dt = i >> 6, gg = (i >> 4) & 3, jj = i & 15;
+                        vdst[(dt * 16 + jj) * 4 + gg] = vs[i];
+                    }
+                }
                 if (kb == kb_begin) { ITAK_MARK(9) }
             }
         }
