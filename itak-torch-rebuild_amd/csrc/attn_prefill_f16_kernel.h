@@ -264,7 +264,10 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     const bool patches = fused && any_block && nblocks * kBlockKeys > item.pos0;
     const bool stores_new = fused && unit < p.g.kv_heads && split == item.splits - 1;
     const bool with_new = patches || stores_new;
-    const bool by_stage = stores_new && patches && item.rows >= 8;  // see the stores below
+    // (See the stores below. The new rows touch up to three consecutive position blocks; on a ring
+    // of fewer storage blocks two of them are the same storage block, and the stage of the later
+    // one, fetched before the earlier one was stored, would put the old rows back over the new.)
+    const bool by_stage = stores_new && patches && item.rows >= 8 && (!RING || ring_blocks >= 3);
     [[maybe_unused]] uint2 npk[kCanFuse ? kFusePieces : 1];
     half8 qb[kTiles][kSteps];
     uint32_t colpos[kTiles], collo[kTiles];

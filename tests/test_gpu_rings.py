@@ -483,6 +483,22 @@ def test_steps_on_a_windowed_layer_match_the_oracle(elem, window, q_heads, kvh, 
     pool.close()
 
 
+@pytest.mark.parametrize("window,headroom,d,q_heads", [(7, 16, 128, 32), (20, 40, 128, 32), (7, 16, 64, 16),
+                                                        (40, 50, 128, 8), (70, 20, 128, 32)])
+def test_blocks_on_rings_of_one_to_three_storage_blocks_leave_exactly_their_rows(window, headroom, d, q_heads):
+    # Blocks of eight rows or more are stored by writing whole 32-row storage blocks back. On a
+    # ring of one or two storage blocks, consecutive position blocks are the same storage block:
+    # a block that crosses a 32-row boundary must still leave its first rows in place. The
+    # cache is compared after every step.
+    pool, cache, ref, rng = pair(window, 4, d, "f16", seed=window + headroom, headroom=headroom)
+    most = min(headroom, 64)
+    for rows in [5, 16, 9, 16, 16, 8, 13, 16, 12, 16, 16, 10, most, 1, most, 11, most]:
+        rows = min(rows, most)
+        run_steps(pool, cache, ref, rng, q_heads, [rows], "f16")
+        assert view_snapshot(cache, 0) == view_snapshot(ref, 0), (rows, cache.next_position(0))
+    pool.close()
+
+
 def test_steps_with_softcap_and_several_slots_on_a_mixed_pattern():
     import torch
     rng = np.random.default_rng(9)
