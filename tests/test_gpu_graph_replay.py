@@ -163,3 +163,57 @@ def test_replays_of_a_captured_step_equal_the_eager_step(elem, windows, contexts
         assert err <= (2e-3 if elem == "f16" else 1e-5), (s, err)
     other.close()
     pool.close()
+
+
+@pytest.mark.parametrize("rows", [1, 20])
+def test_replays_of_a_captured_prepared_step_equal_the_eager_step(rows):
+    # The step with its norms, rotation and output gate (a preparation launch of its own from nine
+    # rows on): captured, replayed with new inputs, compared with the eager call bit for bit. The
+    # eager call itself is held to the oracle by the preparation's own tests.
+    ctx, layers = 700, 2
+    rng = np.random.default_rng(rows)
+    stream = torch.cuda.current_stream()
+    pool = P().KvPool(layers, KV_HEADS, D, elem="f16", capacity_rows=ctx + rows + 8)
+    pool.set_stream(stream.cuda_stream)
+    cache = pool.acquire()
+    for layer in range(layers):
+        kd = torch.from_numpy(normal(rng, ctx, ROW)).cuda()
+        pool.append_device(layer, [(cache, ctx)], kd.data_ptr(), kd.data_ptr())
+        pool.synchronize()
+    qw, kw = (torch.from_numpy(1.0 + 0.1 * normal(rng, D)).cuda() for _ in range(2))
+    inputs = [tuple(normal(rng, layers * rows, w).reshape(layers, rows, w)
+                    for w in (Q_HEADS * D, ROW, ROW, Q_HEADS * D)) for _ in range(2)]
+    q, kn, vn, gate = (torch.from_numpy(x).cuda() for x in inputs[0])
+    out = torch.empty_like(q)
+
+    def step():
+        for layer in range(layers):
+            pool.attention_prep_step_device(
+                layer, [(cache, rows)], q[layer].data_ptr(), kn[layer].data_ptr(), vn[layer].data_ptr(),
+                out[layer].data_ptr(), Q_HEADS, q_norm_ptr=qw.data_ptr(), k_norm_ptr=kw.data_ptr(), eps=1e-6,
+                rope_base=1e6, interleaved=True, rotary_dim=0, gate_ptr=gate[layer].data_ptr())
+        pool.truncate([cache], [ctx])
+
+    def eager():
+        out.fill_(float("nan"))
+        step()
+        torch.cuda.synchronize()
+        return out.cpu().numpy().copy()
+
+    want = [eager(), None]
+    graph = capture(pool, stream, step)
+    for replay in range(4):
+        which = replay % 2
+        for t, x in zip((q, kn, vn, gate), inputs[which]):
+            t.copy_(torch.from_numpy(x))
+        if want[which] is None:
+            want[which] = eager()
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        assert np.isfinite(got).all(), replay
+        assert np.array_equal(got, want[which]), (replay, float(np.abs(got - want[which]).max()))
+    assert cache.next_position(0) == ctx
+    pool.close()
