@@ -489,7 +489,9 @@ itak_status itak_gqa_attention(itak_pool *pool, uint32_t slot, uint64_t layer, c
    [rows][q_heads*head_dim], k and v [rows][kv_heads*head_dim]; out has q_len
    elements. The slot is never advanced past what was appended: a failed call
    leaves it ahead of the caller's position and the next call refuses until
-   itak_slot_reset, as the reference does. */
+   itak_slot_reset, as the reference does. The rotation uses f64 angles, sines and
+   cosines like rope_interleaved.rs:103-114, on every shape: the K rows the call stores
+   are the reference's rotated rows, rounded once where the pool is f16. */
 itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t layer, const float *q,
                                    uint64_t q_len, const float *k, uint64_t k_len, const float *v,
                                    uint64_t v_len, uint64_t num_q_heads, uint64_t cache_position,

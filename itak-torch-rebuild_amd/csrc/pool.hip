@@ -2486,14 +2486,12 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
     // several blocks.
     const LayerInfo &L = pool->layers[layer];
     const uint64_t block_cap = L.windowed ? L.ring - L.window : std::max<uint64_t>(rows, 1);
-    // The rotation of a sliding-window layer (row i at position appended + i): inside the
-    // attention launch where the split-K kernel takes the block, else in place on the staged
-    // rows beforehand.
-    FoldedParams folded{};
-    folded.prep_on = 1;
-    folded.prep_interleaved = 1;
-    folded.prep_rot = pool->g.head_dim;
-    folded.prep_freq_step = rotate ? -2.0 * std::log2(double(rope_freq_base_swa)) / double(pool->g.head_dim) : 0.0;
+    // The rotation of a sliding-window layer (row i at position appended + i): in place on the
+    // staged rows, by the preparation launch, whose f64 angles, sines and cosines are the
+    // reference's (rope_interleaved.rs:103-114), so that the K rows this call stores are the
+    // reference's rounded once. (The split-K kernel can rotate inside its own launch, with the
+    // hardware's sine and cosine, within one f16 step of that; the device-resident step uses it,
+    // where a launch counts. Here the call already copies its rows in and its output out.)
     auto rotate_block = [&](uint64_t done, uint64_t n, bool with_q) -> itak_status {
         PrepArgs a{};
         a.q_in = a.q_out = qd + done * q_width;
@@ -2532,12 +2530,11 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
         const uint64_t lo = (L.window && base + 1 > L.window) ? base + 1 - L.window : 0;
         std::vector<PlanInput> plan{
             PlanInput{slot, uint32_t(n), uint32_t(base), uint32_t(base + n), uint32_t(lo)}};
-        const bool folds = rotate && takes_splitk_f16(pool, plan.data(), 1, num_q_heads, nullptr);
-        if (rotate && !folds && (st = rotate_block(done, n, true)) != ITAK_OK) return st;
+        if (rotate && (st = rotate_block(done, n, true)) != ITAK_OK) return st;
         st = step_on_device(pool, layer, &item, 1, plan, qd + done * q_width, kd + done * pool->row,
                             vd + done * pool->row, out_dev + done * q_width, num_q_heads,
                             default_scale(pool->g.head_dim),  // AttentionParams::new(), cpu.rs:584
-                            softcap, folds ? &folded : nullptr);
+                            softcap, nullptr);
         if (st != ITAK_OK) return st;
     }
     if (!out_pinned) {
