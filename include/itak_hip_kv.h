@@ -572,7 +572,10 @@ itak_status itak_attention_prep_step_device(itak_pool *pool, uint64_t layer,
                                             float softcap, const itak_prep_params *prep);
 /* The attention half alone: query row r of item i attends at position
    len_i - rows_i + r, i.e. over rows the slot already holds (gqa_attention over the
-   slot's view, attention.rs:104-215, with the last rows_i positions as queries). */
+   slot's view, attention.rs:104-215, with the last rows_i positions as queries). On a
+   windowed layer the view starts at the window of the newest row: an earlier query row sees
+   what of its own window is still in the view, and more rows than the window are refused with
+   the reference's NoVisibleKeys for the first of them (attention.rs:160-173). */
 itak_status itak_attention_device(itak_pool *pool, uint64_t layer, const itak_batch_item *items,
                                   uint32_t item_count, const float *q_dev, float *out_dev,
                                   uint64_t num_q_heads, float scale, float softcap);

@@ -2368,9 +2368,13 @@ itak_status itak_attention_device(itak_pool *pool, uint64_t layer, const itak_ba
         if (items[i].rows > len)
             return shape_mismatch(pool->err, "query rows", len, items[i].rows);
         // The newest `rows` positions query the view as it stands: nothing older than the
-        // view's first row is promised to be in the ring.
+        // view's first row is promised to be in the ring. A query that stands before that row
+        // (more rows than a windowed layer's window) sees none of the view: the reference's
+        // refusal for its position (attention.rs:160-173), the lowest such query first.
+        const uint64_t first = first_visible(pool, *s, layer);
+        if (len - items[i].rows < first) return no_visible_keys(pool->err, len - items[i].rows);
         plan.push_back(PlanInput{items[i].slot, items[i].rows, uint32_t(len - items[i].rows),
-                                 uint32_t(len), uint32_t(first_visible(pool, *s, layer))});
+                                 uint32_t(len), uint32_t(first)});
     }
     if (std::isnan(scale)) scale = default_scale(pool->g.head_dim);
     return run_attention(pool, layer, plan.data(), uint32_t(plan.size()), q_dev, out_dev, nullptr,
