@@ -146,3 +146,55 @@ def test_a_step_beyond_the_static_workspace_is_refused_before_anything_changes()
     assert cache2.next_position(0) == ctx + rows2
     pool.close()
     pool2.close()
+
+
+@pytest.mark.parametrize("in_launch", [False, True])
+def test_the_call_is_captured_into_a_graph_on_its_first_use_and_replays(in_launch):
+    # The callers the entry point is for: its very first call on a pool is made under stream
+    # capture (nothing before it has sized a workspace), the graph is replayed with new inputs
+    # in the captured buffers, and every replay equals the eager call of the allocating entry
+    # point on a twin pool, bit for bit.
+    pools = twin_pools(2, 2200, in_launch)
+    contexts, rows = [2048, 700], 3
+    rng = np.random.default_rng(8)
+    stream = torch.cuda.current_stream()
+    for pool, caches in pools:
+        for s, n in enumerate(contexts):
+            kd = dev(normal(np.random.default_rng(100 + s), n, ROW))
+            pool.append_device(0, [(caches[s], n)], kd.data_ptr(), kd.data_ptr())
+            pool.synchronize()
+    inputs = [tuple(normal(rng, 2 * rows, w) for w in (Q_HEADS * D, ROW, ROW)) for _ in range(2)]
+    q, k, v = (dev(x) for x in inputs[0])
+    out = torch.full((2 * rows, Q_HEADS * D), float("nan"), device="cuda")
+    (eager_pool, eager_caches), (pool, caches) = pools
+    items = [(c, rows) for c in caches]
+
+    def step():
+        assert call(pool, "itak_attention_step_device_noalloc", 0, items, q, k, v, out) == 0, \
+            P()._native.load().itak_last_error(pool._h)
+        pool.truncate(caches, contexts)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(stream)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        pool.set_stream(side.cuda_stream)
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.synchronize()
+    pool.set_stream(stream.cuda_stream)
+    for replay in range(4):
+        for t, x in zip((q, k, v), inputs[replay % 2]):
+            t.copy_(torch.from_numpy(x))
+        want = torch.full_like(out, float("nan"))
+        assert call(eager_pool, "itak_attention_step_device", 0, [(c, rows) for c in eager_caches],
+                    q, k, v, want) == 0
+        eager_pool.truncate(eager_caches, contexts)
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.isfinite(out).all(), replay
+        assert torch.equal(out, want), replay
+    for p, _ in pools:
+        p.close()
