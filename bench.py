@@ -408,6 +408,10 @@ def main():
     ap.add_argument("--merge-in-launch", action="store_true",
                     help="merge split partials inside the attention launch (workgroups exchange "
                          "them through a buffer) instead of with a launch of its own")
+    ap.add_argument("--die-merge", action="store_true",
+                    help="merge each unit's splits on its compute die inside the split-K launch "
+                         "(ITAK_POOL_DIE_MERGE) where the batch suits it, instead of with a launch "
+                         "of its own")
     ap.add_argument("--prep", action="store_true",
                     help="also time the step with the fused Q/K preparation (per-head RMSNorm + "
                          "RoPE) before it and the sigmoid gate after it, reported as 'with_prep'")
@@ -461,6 +465,29 @@ def main():
                 workloads[wl] = {"error": f"{type(e).__name__}: {e}"}
         result["workloads"] = workloads
     print(json.dumps(result))
+
+
+def merge_form_of(pkg, pool, step):
+    """How the step's split partials are merged ("launch", "on_die", "in_launch", "none"), read
+    from the library's diagnostic line for the step's first attention launch."""
+    import re
+    import tempfile
+
+    with tempfile.TemporaryFile(mode="w+b") as tmp:
+        sys.stderr.flush()
+        saved = os.dup(2)
+        os.dup2(tmp.fileno(), 2)
+        try:
+            pkg.set_debug_enabled(True)
+            step()
+            pool.synchronize()
+        finally:
+            pkg.set_debug_enabled(False)
+            os.dup2(saved, 2)
+            os.close(saved)
+        tmp.seek(0)
+        forms = re.findall(r"merge=(\w+)", tmp.read().decode(errors="replace"))
+    return forms[0] if forms else None
 
 
 def summary_of(result):
@@ -536,7 +563,8 @@ def run_workload(args, pkg, torch, np, dev, stream, timed):
     pool = pkg.KvPool(pattern, KV_HEADS, D, elem=args.kv, max_slots=slots,
                       capacity_rows=max_len + rows + 8, scrub_on_truncate=False,
                       ring_headroom=rows if wl == "prefill_windowed" else 0,
-                      merge_in_launch=args.merge_in_launch)
+                      merge_in_launch=args.merge_in_launch,
+                      die_merge=getattr(args, "die_merge", False))
     pool.set_stream(stream.cuda_stream)
     caches = [pool.acquire() for _ in range(slots)]
 
@@ -579,6 +607,7 @@ def run_workload(args, pkg, torch, np, dev, stream, timed):
     for _ in range(max(args.warmup, 1)):
         step()
     torch.cuda.synchronize()
+    merge_form = merge_form_of(pkg, pool, step)
     probe = probes(torch, pool, timed, dev)
 
     eager_s, eager_wall_s = timed(step, args.steps)
@@ -740,6 +769,8 @@ def run_workload(args, pkg, torch, np, dev, stream, timed):
             "bound": "hbm",
             "kernel": (("attn_decode_f16_kernel" if lean else f"attn_splitk_{args.kv}_kernel") +
                        (" (splits merged inside the launch)" if args.merge_in_launch else
+                        " (each unit's splits merged on its compute die by the unit's last "
+                        "workgroup: one launch per layer)" if merge_form == "on_die" else
                         " + attn_combine128_kernel (the two launches of one layer's attention)")),
             "achieved": round(kv_bytes_layer / layer_s / 1e9, 2),
             "peak": HBM_PEAK_GBS,
@@ -786,6 +817,8 @@ def run_workload(args, pkg, torch, np, dev, stream, timed):
         "device_probes": probe,
         "roofline": roofline,
     }
+    if merge_form is not None:
+        result["config"]["split_merge"] = merge_form
     if with_prep is not None:
         result["with_prep"] = with_prep
     if host_call is not None:

@@ -110,7 +110,21 @@ enum {
        instead of two; results agree with the default form to rounding. On an MI355X the
        exchange costs what the second launch costs (a round trip through memory between
        compute dies, then the stores that hand the buffer back), so it is not the default. */
-    ITAK_POOL_MERGE_IN_LAUNCH = 2u
+    ITAK_POOL_MERGE_IN_LAUNCH = 2u,
+    /* Merge split partials on the compute die that produced them, inside the attention launch.
+       Split steps of f16 pools at head_dim 128 with at most 32 query vectors per KV head whose
+       (sequence, KV head) units deal out evenly over the device's eight compute dies (1, 2, 4 or
+       8 KV heads; at least 8 / kv_heads sequences of similar total length) place each unit's
+       splits on one die, and the unit's last workgroup to finish merges the unit's partials out
+       of that die's L2: no merge launch and no wait inside the launch. Other steps keep the
+       merge launch. Pool creation probes that the device deals workgroup i to die i % 8 and
+       ignores the flag if it does not; every such launch checks again, and
+       itak_pool_synchronize reports ITAK_STEP_FAILED if a workgroup ran elsewhere. Results
+       agree with the merge launch's to the rounding of another split plan. On an MI355X it is
+       2 to 4 % faster than the merge launch on batches of a hundred MB of KV per layer and more,
+       level or slower below (the launch's own tail and a slower start cost what the second
+       launch costs), so it is not the default. */
+    ITAK_POOL_DIE_MERGE = 4u
 };
 
 typedef struct itak_pool itak_pool;

@@ -30,6 +30,7 @@ ELEM_F32, ELEM_F16 = 0, 1
 LAYER_GLOBAL, LAYER_WINDOWED = 0, 1
 POOL_SCRUB_ON_TRUNCATE = 1
 POOL_MERGE_IN_LAUNCH = 2
+POOL_DIE_MERGE = 4
 
 
 class PoolConfig(C.Structure):

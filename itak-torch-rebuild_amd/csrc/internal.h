@@ -386,6 +386,37 @@ constexpr unsigned long long kExchangeEmptyWord = 0xffffffffffffffffull;
 hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                   uint32_t max_rows, hipStream_t stream,
                                   const FoldedParams *folded = nullptr);
+// ---- the split merge on a unit's compute die (attn_splitk_f16_die.hip) ---------------------
+// The device's workgroups are dealt round-robin over its eight compute dies, each with an L2 of
+// its own. A launch planned for it puts every split of a unit = (item, KV head, part of the
+// query vectors) on one die; the unit's last workgroup to finish merges the partials out of
+// that die's L2, so there is neither a merge launch nor a wait.
+constexpr uint32_t kDieCount = 8;
+constexpr uint32_t kDieTicketStride = 32;  // words from one unit's ticket to the next: a cache line each
+constexpr uint32_t kDieMaxUnits = 1024;
+constexpr uint64_t kDieTicketBytes = uint64_t(kDieMaxUnits) * kDieTicketStride * 4;
+struct DieMap {
+    uint32_t *tickets;  // kDieMaxUnits words kDieTicketStride apart, zero whenever no launch runs
+    uint32_t *faults;   // workgroups that found themselves on another die than their index names
+    const float *gate;  // merged rows are multiplied by sigmoid(gate) as they are written, or null
+    uint32_t shift;     // log2(heads a bin's dies share out): die = bin << shift | KV head
+    uint32_t pad;
+    uint32_t bin_first[kDieCount + 1];  // items of bin i: [bin_first[i], bin_first[i + 1])
+    uint32_t bin_count[kDieCount];      // workgroups of a die of bin i
+};
+// True when the current device deals workgroup i to compute die i % 8 (probed once per device:
+// a small launch whose workgroups report the hardware's die number).
+bool die_layout_ok(int device);
+// Plans `b` (slot, rows, pos0, q_row0, kv_len, kv_lo set) for the die-local merge: `out` gets
+// the items in bin order with splits, keys_per_split, block0 (first index on the die), ws0 and
+// the unit's first ticket (in splits_magic); `map` the bins. Returns the partials the launch
+// writes, 0 when the batch is better served by the ordinary plan (too few or too uneven units,
+// a KV head count that does not deal out over eight dies, nothing to split).
+uint32_t attn_splitk_f16_plan_die(const PoolGeom &g, const AttnBatch &b, uint32_t q_heads,
+                                  AttnBatch &out, DieMap &map);
+hipError_t launch_attn_splitk_f16_die(const AttnParams &p, const AttnBatch &b, const DieMap &map,
+                                      uint32_t total_partials, hipStream_t stream,
+                                      const FoldedParams *folded = nullptr);
 // The latency-shaped form of the same path for decode steps (attn_decode_f16.hip): every item
 // one new row, at most one block per wavefront, splits merged inside the launch. `takes` is
 // asked after the batch has been planned and AttnParams::exchange set.

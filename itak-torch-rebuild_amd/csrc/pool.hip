@@ -134,6 +134,11 @@ struct itak_pool {
     bool no_alloc_call = false;
     bool scratch_exchange_used = false;  // its give-up counter is then looked at too
     bool merge_in_launch = false;
+    // ITAK_POOL_DIE_MERGE: split-K launches whose units deal out evenly over the compute dies
+    // merge each unit's splits on its die (attn_splitk_f16_die.hip): one ticket word per unit, then the count of
+    // workgroups that found themselves on another die than planned.
+    bool die_merge = false;
+    uint32_t *die_words = nullptr;
     // Per slot: the side buffer of a deep checkpoint's ring rows, kept for the next one
     // (cache.rs:620-625: allocated once per cache, not once per round).
     std::vector<void *> ring_saved;
@@ -538,6 +543,21 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         uint64_t exchange_words = 0;
         if (mfma && pool->merge_in_launch && (!gate || prepares))
             exchange_words = attn_splitk_f16_plan_exchange(geom, b, uint32_t(q_heads));
+        // Or on the units' compute dies, when the batch deals out evenly over them and is not
+        // one the single-row decode kernel takes.
+        AttnBatch bd{};
+        DieMap dm{};
+        uint32_t die_partials = 0;
+        if (mfma && pool->die_merge && !exchange_words) {
+            AttnParams probe{};
+            probe.g = geom;
+            probe.group = group;
+            if (prepares || !attn_decode_f16_takes(probe, b))
+                die_partials = attn_splitk_f16_plan_die(geom, b, uint32_t(q_heads), bd, dm);
+        }
+        const bool on_die = die_partials != 0;
+        if (on_die) partials = die_partials;
+        const AttnBatch &bl = on_die ? bd : b;  // the batch the attention launch takes
         const uint64_t partial_floats = uint64_t(partials) * (pool->g.head_dim + 2);
         if (need_only) {  // planning only: nothing is allocated, launched or changed
             need_only->exchange_words = std::max(need_only->exchange_words, exchange_words);
@@ -561,7 +581,7 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
             uint32_t splits = 0;
             uint64_t view_len = 0;
             for (uint32_t i = 0; i < count; ++i) {
-                splits = std::max(splits, b.item[i].splits);
+                splits = std::max(splits, bl.item[i].splits);
                 view_len = std::max<uint64_t>(view_len, b.item[i].kv_len - b.item[i].kv_lo);
             }
             diag_emit("gqa_attention layer=%llu items=%u queries=%u q_heads=%llu kv_heads=%llu "
@@ -570,8 +590,8 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
                       ULL(layer), count, total_rows, ULL(q_heads), ULL(pool->g.kv_heads), ULL(view_len),
                       window, double(scale), double(softcap),
                       mfma ? "splitk_f16" : prefill ? "prefill_f16" : f32fast ? "splitk_f32" : "generic",
-                      b.total_blocks, splits, int(k_new != nullptr && (mfma || f32fast || prefill)),
-                      partials == 0 ? "none" : exchange_words ? "in_launch" : "launch");
+                      bl.total_blocks, splits, int(k_new != nullptr && (mfma || f32fast || prefill)),
+                      partials == 0 ? "none" : on_die ? "on_die" : exchange_words ? "in_launch" : "launch");
         }
         AttnParams p{};
         p.layer_base = layer_base(pool, layer);
@@ -603,9 +623,17 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         // splits; for items of one split the split-K kernel, which only its preparing
         // variants can; otherwise a launch of its own over the chunk's rows.
         bool merged_only = mfma || prefill;
-        for (uint32_t i = 0; i < count; ++i) merged_only = merged_only && b.item[i].splits > 1;
+        for (uint32_t i = 0; i < count; ++i) merged_only = merged_only && bl.item[i].splits > 1;
         const bool gate_folded = gate && (prepares || (mfma && merged_only));
-        if (mfma) {
+        if (on_die) {
+            dm.tickets = pool->die_words;
+            dm.faults = pool->die_words + kDieTicketBytes / sizeof(uint32_t);
+            dm.gate = gate_folded ? gate : nullptr;
+            HIP_TRY(pool,
+                    launch_attn_splitk_f16_die(p, bd, dm, partials, pool->stream,
+                                               prepares ? folded : nullptr),
+                    "launch split-K attention");
+        } else if (mfma) {
             HIP_TRY(pool,
                     launch_attn_splitk_f16(p, b, partials, max_rows, pool->stream,
                                            prepares ? folded : nullptr),
@@ -620,7 +648,7 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
             HIP_TRY(pool, launch_attn_generic(pool->elem_f16, p, b, partials, pool->stream),
                     "launch attention");
         }
-        if (!exchange_words)
+        if (!exchange_words && !on_die)
             HIP_TRY(pool, launch_attn_combine(p, b, partials, total_rows, (mfma || prefill || f32fast) ? 1 : 0,
                                               pool->stream, gate_folded ? gate : nullptr),
                     "launch split merge");
@@ -1075,6 +1103,18 @@ itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out) {
     pool->ring_saved.assign(config->max_slots, nullptr);
     pool->ring_saved_bytes.assign(config->max_slots, 0);
     pool->merge_in_launch = (config->flags & ITAK_POOL_MERGE_IN_LAUNCH) != 0;
+    if (pool->elem_f16 && !pool->merge_in_launch && (config->flags & ITAK_POOL_DIE_MERGE) &&
+        die_layout_ok(config->device)) {
+        he = hipMalloc(reinterpret_cast<void **>(&pool->die_words), kDieTicketBytes + 256);
+        if (he == hipSuccess) he = hipMemset(pool->die_words, 0, kDieTicketBytes + 256);
+        if (he != hipSuccess) {
+            if (pool->die_words) (void)hipFree(pool->die_words);
+            (void)hipFree(pool->base);
+            delete pool;
+            return hip_error(e, he, "allocate the split tickets");
+        }
+        pool->die_merge = true;
+    }
     he = bind_scratch(config->device, &pool->scratch_dev);
     if (he != hipSuccess) {
         (void)hipFree(pool->base);
@@ -1098,6 +1138,7 @@ void itak_pool_destroy(itak_pool *pool) {
     if (pool->ws) (void)hipFree(pool->ws);
     if (pool->prep) (void)hipFree(pool->prep);
     if (pool->xws) (void)hipFree(pool->xws);
+    if (pool->die_words) (void)hipFree(pool->die_words);
     for (void *buf : pool->ring_saved)
         if (buf) (void)hipFree(buf);
     if (pool->hstage) (void)hipHostFree(pool->hstage);
@@ -1139,6 +1180,23 @@ itak_status itak_pool_synchronize(itak_pool *pool) {
                          "attention: %u workgroups of a split merge gave up waiting for their "
                          "group; the outputs of that step are NaN",
                          total);
+    if (pool->die_words) {
+        // A launch that merges on the units' compute dies relies on where the device runs each
+        // workgroup; every workgroup checks, and one that ran elsewhere has counted itself.
+        uint32_t strays = 0;
+        uint32_t *faults = pool->die_words + kDieTicketBytes / sizeof(uint32_t);
+        HIP_TRY(pool, hipMemcpy(&strays, faults, sizeof(strays), hipMemcpyDeviceToHost),
+                "read the die check's counter");
+        if (strays) {
+            pool->die_merge = false;  // the ordinary merge launch from here on
+            HIP_TRY(pool, hipMemset(pool->die_words, 0, kDieTicketBytes + 256), "clear the split tickets");
+            return set_error(pool->err, ITAK_STEP_FAILED, "attention", strays, 0, 0, 0,
+                             "attention: %u workgroups of a split merge ran on another compute die "
+                             "than their index names; outputs of the steps since the last "
+                             "synchronize may be wrong (later steps use the merge launch)",
+                             strays);
+        }
+    }
     return ITAK_OK;
 }
 

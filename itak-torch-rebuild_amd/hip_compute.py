@@ -13,6 +13,7 @@ that one launch can serve all of them.
 from __future__ import annotations
 
 import ctypes as C
+import os
 import math
 from dataclasses import dataclass, field
 from typing import List, Optional, Sequence, Tuple, Union
@@ -193,7 +194,7 @@ class KvPool:
     def __init__(self, pattern: Union[int, Sequence[LayerKind]], num_kv_heads: int, head_dim: int,
                  *, elem: str = "f16", max_slots: int = 1, capacity_rows: int = 4096,
                  device: int = 0, scrub_on_truncate: bool = True, ring_headroom: int = 0,
-                 merge_in_launch: bool = False):
+                 merge_in_launch: bool = False, die_merge: Optional[bool] = None):
         if isinstance(pattern, int):
             pattern = [LayerKind.Global] * pattern
         self.pattern = list(pattern)
@@ -215,6 +216,13 @@ class KvPool:
         cfg.device = device
         cfg.flags = (N.POOL_SCRUB_ON_TRUNCATE if scrub_on_truncate else 0) | \
                     (N.POOL_MERGE_IN_LAUNCH if merge_in_launch else 0)
+        # Split merges on the units' compute dies are opt-in; ITAK_HIP_KV_DIE_MERGE=1 in the
+        # environment turns them on for pools that do not say otherwise (how the test suite is
+        # run over that form).
+        if die_merge is None:
+            die_merge = os.environ.get("ITAK_HIP_KV_DIE_MERGE", "0") == "1"
+        if die_merge:
+            cfg.flags |= N.POOL_DIE_MERGE
         cfg.ring_headroom = ring_headroom
         handle = C.c_void_p()
         self._h = None
