@@ -398,7 +398,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", choices=["decode", "ragged", "verify", "prefill", "hybrid",
-                                           "prefill_windowed", "restore", "append", "chunk64"],
+                                           "prefill_windowed", "restore", "append", "chunk64", "sweep"],
                     default="decode")
     ap.add_argument("--softcap", type=float, default=0.0)
     ap.add_argument("--kv", choices=["f16", "f32"], default="f16",
@@ -446,6 +446,9 @@ def main():
     stream = torch.cuda.current_stream()
     timed = Timer(torch, stream)
 
+    if args.workload == "sweep":
+        print(json.dumps(decode_sweep(args, pkg, torch, stream, full=True)))
+        return
     result = run_workload(args, pkg, torch, np, dev, stream, timed)
     primary = (args.workload == "decode" and args.kv == "f16" and args.softcap == 0.0
                and not args.only and not args.merge_in_launch)
@@ -464,7 +467,83 @@ def main():
             except Exception as e:  # a secondary figure must not take the contract line down
                 workloads[wl] = {"error": f"{type(e).__name__}: {e}"}
         result["workloads"] = workloads
+        # The same decode step over context and batch, a coarse grid: where the 70 % of the HBM
+        # peak that the headline asks for is met (`--workload sweep` prints the whole table).
+        try:
+            torch.cuda.empty_cache()
+            sweep = decode_sweep(args, pkg, torch, stream, full=False)
+            result["decode_sweep"] = {k: sweep[k] for k in ("summary", "seventy_pct_met_from_mb_per_launch",
+                                                            "points")}
+        except Exception as e:
+            result["decode_sweep"] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(result))
+
+
+def decode_sweep(args, pkg, torch, stream, full):
+    """One decode row per slot (fused append + attention, 32 Q / 4 KV heads, f16) over a grid of
+    context lengths and slot counts: us per layer and KV bytes / time as a fraction of the HBM
+    peak, 4 layers cycled in a HIP graph. Also the smallest launch (MB of KV) from which every
+    larger launch of the grid meets 70 % of the peak."""
+    layers = 4
+    if full:
+        contexts = [512, 1024, 2048, 4096, 8192, 16384, 32768, 65536, 131072]
+        batches = [1, 2, 4, 8, 16, 32, 64]
+    else:
+        contexts, batches = [1024, 4096, 16384, 65536], [1, 4, 16, 64]
+    points = []
+    for ctx in contexts:
+        for batch in batches:
+            if batch * ctx * 2 * ROW * 2 * layers > 24e9:
+                continue
+            pool = pkg.KvPool(layers, KV_HEADS, D, elem="f16", max_slots=batch, capacity_rows=ctx + 9,
+                              scrub_on_truncate=False, die_merge=getattr(args, "die_merge", False))
+            pool.set_stream(stream.cuda_stream)
+            caches = [pool.acquire() for _ in range(batch)]
+            k = torch.randn(ctx, ROW, device="cuda")
+            v = torch.randn(ctx, ROW, device="cuda")
+            for layer in range(layers):
+                for c in caches:
+                    pool.append_device(layer, [(c, ctx)], k.data_ptr(), v.data_ptr())
+            torch.cuda.synchronize()
+            q = torch.randn(layers, batch, Q_HEADS * D, device="cuda")
+            kn = torch.randn(layers, batch, ROW, device="cuda")
+            vn = torch.randn(layers, batch, ROW, device="cuda")
+            out = torch.empty_like(q)
+            items = [(c, 1) for c in caches]
+
+            def step():
+                for layer in range(layers):
+                    pool.attention_step_device(layer, items, q[layer].data_ptr(), kn[layer].data_ptr(),
+                                               vn[layer].data_ptr(), out[layer].data_ptr(), Q_HEADS)
+                pool.truncate(caches, [ctx] * batch)
+
+            for _ in range(3):
+                step()
+            torch.cuda.synchronize()
+            graph = capture(torch, pool, stream, step)
+            for _ in range(3):
+                graph.replay()
+            reps = 20 if full else 10
+            us = Timer(torch, stream)(graph.replay, reps)[0] / reps / layers * 1e6
+            kv_bytes = 2 * batch * (ctx + 1) * ROW * 2
+            points.append({"context": ctx, "slots": batch, "us_per_layer": round(us, 2),
+                           "kv_mb_per_launch": round(kv_bytes / 1e6, 1),
+                           "frac": round(kv_bytes / us / 1e3 / HBM_PEAK_GBS, 3)})
+            pool.close()
+            del pool, caches, graph
+            torch.cuda.empty_cache()
+    # The smallest size from which every launch of the grid at least as large meets 70 %.
+    by_size = sorted(points, key=lambda p: p["kv_mb_per_launch"])
+    met_from = None
+    for i, p in enumerate(by_size):
+        if all(r["frac"] >= 0.70 for r in by_size[i:]):
+            met_from = p["kv_mb_per_launch"]
+            break
+    summary = ("70 % of the HBM peak is not met on this grid" if met_from is None else
+               f"70 % of the HBM peak is met from {met_from:.0f} MB of KV per launch")
+    return {"metric": "decode-attn KV GB/s over context and batch", "unit": "fraction of 8 TB/s",
+            "layers_cycled": layers, "summary": summary,
+            "seventy_pct_met_from_mb_per_launch": met_from, "points": points}
 
 
 def merge_form_of(pkg, pool, step):

@@ -254,9 +254,17 @@ itak_status itak_pool_set_stream(itak_pool *pool, void *hip_stream);
 itak_status itak_pool_synchronize(itak_pool *pool);
 /* No counterpart in the reference. Workgroups of a launch that merges its own splits
    (ITAK_POOL_MERGE_IN_LAUNCH) wait for each other's partials by polling; `polls` bounds that
-   wait (default 131072, about a microsecond each). A workgroup that runs out writes NaN outputs and is reported by the next
-   itak_pool_synchronize as ITAK_STEP_FAILED. 0 makes every wait a single look: for tests of
-   that report. */
+   wait. The unit is one look at the exchange buffer (default 131072 looks). A kernel keeps
+   several looks in flight, four in the single-row decode kernel and one elsewhere, each a round
+   trip to memory of 1 to 1.5 microseconds, so the default bounds the wait at about 40 ms in
+   the decode kernel and 170 ms in the others. A workgroup that runs out writes NaN into the
+   outputs it owns, counts itself, and still hands back to the buffer, as empty, the words it had
+   already gathered; the words it was still waiting for stay as they are, and producers that
+   arrive late write theirs. itak_pool_synchronize then returns ITAK_STEP_FAILED and refills the
+   buffer. Everything launched on the pool between the give-up and that synchronize must be
+   taken as invalid, not only the step that gave up: later launches of the same stream read the
+   same buffer and may have taken leftover words for published ones. 0 makes every wait a
+   single look: for tests of that report. */
 itak_status itak_pool_set_merge_spin_limit(itak_pool *pool, uint32_t polls);
 /* Bytes of device memory the pool holds for KV rows. */
 uint64_t itak_pool_device_bytes(const itak_pool *pool);
@@ -544,8 +552,13 @@ itak_status itak_attention_step_device(itak_pool *pool, uint64_t layer,
    hipMalloc, hipFree or other allocating routine. A step whose launches would need more
    (8 MiB of partials = rows x q_heads x splits x 520 bytes summed over the slots) is
    refused with ITAK_CAPACITY_EXCEEDED before anything is changed. Every call on a device
-   shares that device's array, whichever pool makes it: calls that overlap on one device (two
-   pools on two streams) race on it, and so must be ordered by the caller. */
+   shares that device's array, whichever pool makes it. Eager calls are kept apart by the
+   library: each records an event behind its launches, and a call whose stream is not the
+   stream of the device's previous such call makes its stream wait for that event first (a wait
+   on the device, nothing the host blocks on). Calls made while their stream is being captured
+   are outside that: graphs captured from this entry point on different streams of one device
+   must not be replayed at the same time, nor beside eager calls of it; that ordering is the
+   caller's. */
 itak_status itak_attention_step_device_noalloc(itak_pool *pool, uint64_t layer,
                                                const itak_batch_item *items, uint32_t item_count,
                                                const float *q_dev, const float *k_dev,

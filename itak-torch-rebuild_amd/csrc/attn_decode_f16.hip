@@ -30,6 +30,8 @@
 
 #include <math.h>
 
+#include <algorithm>
+
 
 // Timeline marks of attn_decode_f16_kernel: 0 first instruction, 1 addresses known (the kernel
 // arguments have arrived), 2 every load issued, 3 scores done (keys and queries have arrived),
@@ -402,6 +404,34 @@ bool attn_decode_f16_takes(const AttnParams &p, const AttnBatch &b) {
         }
     }
     return true;
+}
+
+uint32_t attn_decode_f16_resident_groups() {
+    static uint32_t cached = 0;
+    if (cached) return cached;
+    int cus = 0, dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    const void *kernels[] = {reinterpret_cast<const void *>(&attn_decode_f16_kernel<1, false>),
+                             reinterpret_cast<const void *>(&attn_decode_f16_kernel<8, false>),
+                             reinterpret_cast<const void *>(&attn_decode_f16_kernel<64, false>),
+                             reinterpret_cast<const void *>(&attn_decode_f16_kernel<1, true>),
+                             reinterpret_cast<const void *>(&attn_decode_f16_kernel<8, true>),
+                             reinterpret_cast<const void *>(&attn_decode_f16_kernel<64, true>)};
+    int least = 1 << 30;
+    for (const void *k : kernels) {
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k, kWaves * 64, 0) != hipSuccess || per_cu < 1) {
+            (void)hipGetLastError();
+            return 256;
+        }
+        least = std::min(least, per_cu);
+    }
+    cached = uint32_t(least) * uint32_t(cus);
+    return cached;
 }
 
 hipError_t launch_attn_decode_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,

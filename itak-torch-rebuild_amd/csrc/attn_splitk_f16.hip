@@ -91,24 +91,46 @@ static hipError_t grant_lds(size_t lds) {
     return e;
 }
 // Workgroups of a variant the device holds at once (registers and LDS decide), asked of the
-// runtime once per variant. A launch of at most this many workgroups runs in one wave of
-// dispatch, so its duration is that of its largest workgroup.
+// runtime once per variant: the smallest figure over every instantiation a launch of the
+// variant may be (batch sizes, ring and preparing forms differ in registers). A launch of at
+// most this many workgroups runs in one wave of dispatch, so its duration is that of its
+// largest workgroup, and every one of its workgroups is running or done when another waits
+// for it (the in-launch exchange relies on that).
 template <int NQ, int W>
 static uint32_t resident_groups() {
     static uint32_t cached = 0;
     if (cached) return cached;
     const size_t lds = variant_lds(NQ, W);
-    int per_cu = 0, cus = 0, dev = 0;
-    if (grant_lds<NQ, W>(lds) != hipSuccess || hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-        hipOccupancyMaxActiveBlocksPerMultiprocessor(
-            &per_cu, reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 1, false>), W * 64,
-            lds) != hipSuccess ||
-        per_cu < 1 || cus < 1) {
+    int cus = 0, dev = 0;
+    if (grant_lds<NQ, W>(lds) != hipSuccess || grant_lds<NQ, W, true>(lds) != hipSuccess ||
+        hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
         (void)hipGetLastError();
         return 256;
     }
-    cached = uint32_t(per_cu) * uint32_t(cus);
+    const void *kernels[] = {
+        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 1, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 8, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 64, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 1, true>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 8, true>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_kernel<NQ, W, 64, true>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<NQ, W, 1, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<NQ, W, 8, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<NQ, W, 64, false>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<NQ, W, 1, true>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<NQ, W, 8, true>),
+        reinterpret_cast<const void *>(&attn_splitk_f16_prep_kernel<NQ, W, 64, true>)};
+    int least = 1 << 30;
+    for (const void *k : kernels) {
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k, W * 64, lds) != hipSuccess || per_cu < 1) {
+            (void)hipGetLastError();
+            return 256;
+        }
+        least = std::min(least, per_cu);
+    }
+    cached = uint32_t(least) * uint32_t(cus);
     return cached;
 }
 static uint32_t variant_capacity(const Variant &v) {
@@ -179,6 +201,12 @@ uint64_t attn_splitk_f16_plan_exchange(const PoolGeom &g, AttnBatch &b, uint32_t
         if (slices + it.splits >= 65536) return 0;  // the kernel divides by multiplication
     }
     if (!any) return 0;
+    // A workgroup of the exchange polls for its group's others: all of the launch must be on the
+    // device together. The launch may be the single-row decode kernel (its own registers and
+    // LDS), so that kernel's figure bounds 16-vector launches too.
+    uint64_t held = variant_capacity(v);
+    if (v.index == 0) held = std::min<uint64_t>(held, attn_decode_f16_resident_groups());
+    if (b.total_blocks > held) return 0;
     uint64_t records = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         AttnItem &it = b.item[i];

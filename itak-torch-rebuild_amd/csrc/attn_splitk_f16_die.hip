@@ -186,34 +186,33 @@ uint32_t attn_splitk_f16_plan_die(const PoolGeom &g, const AttnBatch &b, uint32_
     }
     if (!splits_any) return 0;
     // The shortest run of blocks per split, T, with which every die takes its workgroups at
-    // once. For each T the items go over the bins by their workgroup counts at that T, most
-    // first into the bin with the fewest (ties: the lighter bin by blocks); the first T whose
-    // fullest bin fits a die's compute units is taken, if the bins' blocks are then even enough.
+    // once. For each T the items go over the bins longest first, each into the lightest bin (by
+    // blocks) that still has room for its workgroups at that T; the first T at which every item
+    // finds room is taken, if the bins' blocks are then even enough.
     const uint64_t cap = uint64_t(variant_groups_per_cu(v)) * cus_per_die;
+    for (uint32_t i = 0; i < b.n; ++i) order[i] = i;
+    std::stable_sort(order, order + b.n, [&](uint32_t x, uint32_t y) { return nb[x] > nb[y]; });
     uint64_t T = std::max<uint64_t>((total + cap * bins - 1) / (cap * bins), uint64_t(v.waves));
     uint64_t heaviest = 0;
     for (;; ++T) {
-        uint32_t count_of[kMaxBatchItems];
-        for (uint32_t i = 0; i < b.n; ++i) {
-            count_of[i] = uint32_t((nb[i] + T - 1) / T);
-            order[i] = i;
-        }
-        std::stable_sort(order, order + b.n, [&](uint32_t x, uint32_t y) {
-            return count_of[x] != count_of[y] ? count_of[x] > count_of[y] : nb[x] > nb[y];
-        });
         uint64_t count[kDieCount] = {0}, load[kDieCount] = {0};
+        bool fits = true;
         for (uint32_t k = 0; k < b.n; ++k) {
             const uint32_t i = order[k];
-            uint32_t best = 0;
-            for (uint32_t bin = 1; bin < bins; ++bin)
-                if (count[bin] < count[best] || (count[bin] == count[best] && load[bin] < load[best]))
-                    best = bin;
+            const uint64_t mine = (nb[i] + T - 1) / T;
+            uint32_t best = bins;
+            for (uint32_t bin = 0; bin < bins; ++bin)
+                if (count[bin] + mine <= cap && (best == bins || load[bin] < load[best])) best = bin;
+            if (best == bins) {  // no room anywhere: the lightest bin, and a longer T next
+                fits = false;
+                best = uint32_t(std::min_element(load, load + bins) - load);
+            }
             bin_of[i] = best;
-            count[best] += count_of[i];
+            count[best] += mine;
             load[best] += nb[i];
         }
         heaviest = *std::max_element(load, load + bins);
-        if (*std::max_element(count, count + bins) <= cap || T >= longest) break;
+        if (fits || T >= longest) break;
     }
     // A die that carries a tenth more than its share would cost more than the merge launch.
     if (heaviest * bins * 10 > total * 11) return 0;

@@ -421,6 +421,9 @@ hipError_t launch_attn_splitk_f16_die(const AttnParams &p, const AttnBatch &b, c
 // one new row, at most one block per wavefront, splits merged inside the launch. `takes` is
 // asked after the batch has been planned and AttnParams::exchange set.
 bool attn_decode_f16_takes(const AttnParams &p, const AttnBatch &b);
+// Workgroups of that kernel the device holds at once (the smallest figure over its
+// instantiations, asked of the runtime once).
+uint32_t attn_decode_f16_resident_groups();
 hipError_t launch_attn_decode_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                   hipStream_t stream);
 // f32 MFMA split-K path: f32 pools (row-major planes), head_dim 128, rows*group <= 16, implied

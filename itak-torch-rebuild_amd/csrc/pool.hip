@@ -87,6 +87,17 @@ constexpr uint64_t kScratchExchangeBytes = 8ull << 20;
 constexpr int kMaxDevices = 64;
 unsigned char *g_scratch_of_device[kMaxDevices];
 std::mutex g_scratch_mutex;
+// Every pool and stream of a device shares the device's copy of the array. Eager calls are kept
+// apart by an event (made with the address, at set-up): recorded behind every allocation-free
+// step on the stream it ran on, and waited for, on the device, by the next such step when that
+// one runs on another stream. Calls made while their stream is being captured into a graph are
+// outside this guard: nothing runs at the call, and when the replays run is the caller's matter.
+struct ScratchGuard {
+    hipEvent_t done = nullptr;     // behind the last eager allocation-free step of the device
+    hipStream_t stream = nullptr;  // the stream that step ran on
+    bool recorded = false;
+};
+ScratchGuard g_scratch_guard[kMaxDevices];
 std::atomic<uint64_t> g_next_cache_id{1};  // cache.rs:32
 
 }  // namespace
@@ -127,7 +138,7 @@ struct itak_pool {
     // the consumers that gave up waiting (checked by itak_pool_synchronize).
     unsigned long long *xws = nullptr;
     uint64_t xws_words = 0;
-    uint32_t spin_limit = 1u << 17;  // polls a consumer makes (about a microsecond each)
+    uint32_t spin_limit = 1u << 17;  // looks at the buffer a consumer makes before it gives up
     // This device's copy of the static split workspace, and whether the call in progress must
     // use it instead of the pool's own buffers (itak_attention_step_device_noalloc).
     unsigned char *scratch_dev = nullptr;
@@ -416,10 +427,38 @@ hipError_t bind_scratch(int device, unsigned char **out) {
         if (e == hipSuccess) e = launch_fill_words(reinterpret_cast<unsigned long long *>(ptr), 1, 0, nullptr);
         if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
         if (e != hipSuccess) return e;
+        e = hipEventCreateWithFlags(&g_scratch_guard[device].done, hipEventDisableTiming);
+        if (e != hipSuccess) return e;
         g_scratch_of_device[device] = ptr;
     }
     *out = g_scratch_of_device[device];
     return hipSuccess;
+}
+
+// Before an allocation-free step is enqueued on `stream`: if the device's last such step ran on
+// another stream, this one waits for it on the device. Returns whether the stream is being
+// captured (the guard then stands aside).
+hipError_t scratch_guard_enter(int device, hipStream_t stream, bool *capturing) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    hipError_t e = hipStreamIsCapturing(stream, &status);
+    if (e != hipSuccess) return e;
+    *capturing = status != hipStreamCaptureStatusNone;
+    if (*capturing) return hipSuccess;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    ScratchGuard &g = g_scratch_guard[device];
+    if (g.recorded && g.stream != stream) return hipStreamWaitEvent(stream, g.done, 0);
+    return hipSuccess;
+}
+// After it: the event now stands behind this step.
+hipError_t scratch_guard_leave(int device, hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    ScratchGuard &g = g_scratch_guard[device];
+    const hipError_t e = hipEventRecord(g.done, stream);
+    if (e == hipSuccess) {
+        g.stream = stream;
+        g.recorded = true;
+    }
+    return e;
 }
 
 // What the launches of one attention call need beyond their inputs and outputs.
@@ -1178,7 +1217,8 @@ itak_status itak_pool_synchronize(itak_pool *pool) {
     if (total)
         return set_error(pool->err, ITAK_STEP_FAILED, "attention", total, 0, 0, 0,
                          "attention: %u workgroups of a split merge gave up waiting for their "
-                         "group; the outputs of that step are NaN",
+                         "group; their outputs are NaN and every step launched on this pool since "
+                         "the last successful synchronize is invalid",
                          total);
     if (pool->die_words) {
         // A launch that merges on the units' compute dies relies on where the device runs each
@@ -2304,8 +2344,15 @@ itak_status itak_attention_step_device_noalloc(itak_pool *pool, uint64_t layer,
     itak_status st = plan_step(pool, layer, items, item_count, num_q_heads, plan);
     if (st != ITAK_OK) return st;
     if (std::isnan(scale)) scale = default_scale(pool->g.head_dim);
-    return step_on_device(pool, layer, items, item_count, plan, q_dev, k_dev, v_dev, out_dev,
-                          num_q_heads, scale, softcap, nullptr, true);
+    bool capturing = false;
+    HIP_TRY(pool, scratch_guard_enter(pool->cfg.device, pool->stream, &capturing),
+            "order the step behind the static workspace's last user");
+    st = step_on_device(pool, layer, items, item_count, plan, q_dev, k_dev, v_dev, out_dev,
+                        num_q_heads, scale, softcap, nullptr, true);
+    if (!capturing)
+        HIP_TRY(pool, scratch_guard_leave(pool->cfg.device, pool->stream),
+                "mark the static workspace's last user");
+    return st;
 }
 
 itak_status itak_attention_prep_step_device(itak_pool *pool, uint64_t layer,

@@ -198,3 +198,51 @@ def test_the_call_is_captured_into_a_graph_on_its_first_use_and_replays(in_launc
         assert torch.equal(out, want), replay
     for p, _ in pools:
         p.close()
+
+
+def test_two_pools_on_two_streams_take_the_static_workspace_in_turn():
+    # Every pool and stream of a device shares the one static array. Eager calls on different
+    # streams are ordered by the library (each waits, on the device, for the array's last user);
+    # without that the launches of the two streams overlap and one step's merge reads the
+    # other's partials. Two pools with different batch shapes, each on a stream of its own,
+    # call in turn with no host synchronisation in between; every output equals the allocating
+    # entry point's on a twin pool, bit for bit.
+    shapes = [([4096, 3000, 2500, 3900], 1), ([2048, 1800], 3)]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    rounds = 12
+    rng = np.random.default_rng(31)
+    sides = []
+    for (contexts, rows), stream in zip(shapes, streams):
+        slots = len(contexts)
+        pools = []
+        for _ in range(2):  # the allocating twin, then the allocation-free pool
+            pool = P().KvPool(1, KV_HEADS, D, elem="f16", max_slots=slots, capacity_rows=max(contexts) + 16)
+            pool.set_stream(stream.cuda_stream)
+            pools.append((pool, [pool.acquire() for _ in range(slots)]))
+        fill = [dev(normal(rng, n, ROW)) for n in contexts]
+        inputs = [tuple(dev(normal(rng, slots * rows, w)) for w in (Q_HEADS * D, ROW, ROW))
+                  for _ in range(rounds)]
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            for pool, caches in pools:
+                for c, kd, n in zip(caches, fill, contexts):
+                    pool.append_device(0, [(c, n)], kd.data_ptr(), kd.data_ptr())
+        outs = [[torch.full((slots * rows, Q_HEADS * D), float("nan"), device="cuda")
+                 for _ in range(rounds)] for _ in range(2)]
+        sides.append((pools, contexts, rows, inputs, outs))
+    torch.cuda.synchronize()
+    for r in range(rounds):
+        for pools, contexts, rows, inputs, outs in sides:
+            q, k, v = inputs[r]
+            for which, name in enumerate(("itak_attention_step_device", "itak_attention_step_device_noalloc")):
+                pool, caches = pools[which]
+                st = call(pool, name, 0, [(c, rows) for c in caches], q, k, v, outs[which][r])
+                assert st == 0, P()._native.load().itak_last_error(pool._h)
+                pool.truncate(caches, contexts)
+    torch.cuda.synchronize()
+    for pools, contexts, rows, inputs, outs in sides:
+        for r in range(rounds):
+            assert torch.isfinite(outs[1][r]).all(), r
+            assert torch.equal(outs[0][r], outs[1][r]), r
+        for pool, _ in pools:
+            pool.close()
