@@ -22,7 +22,7 @@
 use std::cell::RefCell;
 
 use cpu_compute::CpuCompute;
-use itak_hip_sys::safe::{Checkpoint, Elem, HipKvError, Layer, Pool, PoolConfig, Slot};
+use itak_hip_sys::safe::{Checkpoint, Elem, HipKvError, Layer, Pool, PoolConfig, Slot, Store};
 use muse_glimmer::{
     AttentionRequest, Cache, Compute, GlimmerConfig, GlimmerError, LayerKind, LayerWeights,
     Result, TensorView,
@@ -142,6 +142,41 @@ impl HipCompute {
             )
         })?;
         state.slot.cache_release(checkpoint).map_err(|e| from_hip(step, &e))
+    }
+
+    /// Drops the positions from `new_len` on, on every layer (the device session's rewind,
+    /// `crates/wgpu-compute/src/session.rs:5397-5428`: no checkpoint involved).
+    pub fn truncate(&self, new_len: usize) -> Result<()> {
+        let step = "session";
+        let guard = self.kv.borrow();
+        let state = guard.as_ref().ok_or_else(|| step_failed(step, "no KV state yet"))?;
+        state.slot.truncate(new_len as u64).map_err(|e| from_hip(step, &e))
+    }
+
+    /// The read half of a session start (`ResidentSession::restore_prefix_from_store`,
+    /// `crates/wgpu-compute/src/session.rs:5000-5053`): with no row stored yet, installs the
+    /// longest stored prefix of `tokens` into this backend's slot (built here if the first
+    /// attention call has not built it) and returns its length, `None` when the cold prefill
+    /// serves. The caller advances its position cache by the same count.
+    pub fn restore_prefix_from_store(&self, cfg: &GlimmerConfig, store: &Store, tokens: &[u32],
+                                     fingerprint: &str) -> Result<Option<usize>> {
+        let step = "prefix_restore";
+        let mut guard = self.kv.borrow_mut();
+        if guard.is_none() {
+            *guard = Some(self.build(cfg)?);
+        }
+        let state = guard.as_ref().ok_or_else(|| step_failed(step, "no KV state"))?;
+        let matched = store.restore_prefix(&state.slot, tokens, fingerprint).map_err(|e| from_hip(step, &e))?;
+        Ok(if matched == 0 { None } else { Some(matched as usize) })
+    }
+
+    /// The write half (`ResidentSession::capture_and_store_prefix`, `session.rs:5056-5094`):
+    /// files the slot's rows under `tokens`, which must be exactly the forwarded prefix.
+    pub fn capture_and_store_prefix(&self, store: &Store, tokens: &[u32], fingerprint: &str) -> Result<()> {
+        let step = "prefix_store";
+        let guard = self.kv.borrow();
+        let state = guard.as_ref().ok_or_else(|| step_failed(step, "no KV state yet: nothing was forwarded"))?;
+        store.capture_and_put(&state.slot, tokens, fingerprint, self.elem).map_err(|e| from_hip(step, &e))
     }
 
     /// `KvState::build` (`cpu.rs:207-231`): one pool of one slot in the config's layer pattern.

@@ -10,7 +10,9 @@ use crate::{
     itak_attention_step_device, itak_attention_step_device_noalloc, itak_batch_item,
     itak_checkpoint, itak_compute_attention, itak_compute_cache_checkpoint,
     itak_compute_cache_release, itak_compute_cache_rewind, itak_error_info, itak_kv_next_position,
-    itak_kv_truncate, itak_last_error, itak_last_error_info, itak_pool, itak_pool_config,
+    itak_kv_now_unix, itak_kv_truncate, itak_last_error, itak_last_error_info, itak_pool,
+    itak_pool_config, itak_store, itak_store_capture_and_put, itak_store_close,
+    itak_store_last_error, itak_store_open, itak_store_restore_prefix,
     itak_pool_create, itak_pool_destroy, itak_pool_set_stream, itak_pool_synchronize,
     itak_slot_acquire, itak_slot_release, itak_slot_reset, itak_status, ITAK_ELEM_F16,
     ITAK_ELEM_F32, ITAK_LAYER_GLOBAL, ITAK_LAYER_WINDOWED, ITAK_OK,
@@ -375,4 +377,76 @@ pub unsafe fn attention_step_device(
         call(pool.raw(), layer, raw.as_ptr(), count, tensors.q, tensors.k, tensors.v, tensors.out,
              num_q_heads, scale, softcap)
     })
+}
+
+/// `itak_kv::PrefixStore` (`crates/itak-kv/src/store.rs:128-543`) as the library keeps it: the
+/// same directory, the same entry files, and the two store halves of a session start against a
+/// pool slot.
+pub struct Store(*mut itak_store);
+
+impl Drop for Store {
+    fn drop(&mut self) {
+        // SAFETY: the handle came from itak_store_open and is closed exactly once.
+        unsafe { itak_store_close(self.0) }
+    }
+}
+
+fn store_error(store: *const itak_store, code: itak_status) -> HipKvError {
+    // SAFETY: `store` is null (the last failed open on this thread) or a live handle; the
+    // message pointer is read before any further call on the store.
+    let message = unsafe {
+        let text = itak_store_last_error(store);
+        if text.is_null() { String::new() } else { CStr::from_ptr(text).to_string_lossy().into_owned() }
+    };
+    HipKvError { code, message, what: String::new(), fields: [0; 4] }
+}
+
+impl Store {
+    /// `PrefixStore::open` (`store.rs:147-168`).
+    pub fn open(root: &str, max_bytes: u64) -> Result<Store, HipKvError> {
+        let root = std::ffi::CString::new(root).map_err(|_| HipKvError {
+            code: crate::ITAK_INVALID_ARGUMENT as itak_status,
+            message: "store root holds a NUL byte".to_string(),
+            what: String::new(),
+            fields: [0; 4],
+        })?;
+        let mut raw: *mut itak_store = ptr::null_mut();
+        // SAFETY: `root` is a live C string; `raw` is a valid out-pointer.
+        let status = unsafe { itak_store_open(root.as_ptr(), max_bytes, &mut raw) };
+        if status == ITAK_OK as itak_status { Ok(Store(raw)) } else { Err(store_error(ptr::null(), status)) }
+    }
+
+    /// `itak_kv::now_unix` (`store.rs:120-126`).
+    #[must_use]
+    pub fn now_unix() -> u64 {
+        // SAFETY: reads the clock.
+        unsafe { itak_kv_now_unix() }
+    }
+
+    /// `ResidentSession::restore_prefix_from_store` (`crates/wgpu-compute/src/session.rs:
+    /// 5000-5053`) into a slot that stands at position zero: the tokens restored, 0 when the
+    /// cold prefill serves. Only a device failure is an error.
+    pub fn restore_prefix(&self, slot: &Slot, tokens: &[u32], fingerprint: &str) -> Result<u64, HipKvError> {
+        let mut matched = 0u64;
+        // SAFETY: slices and the string outlive the call; lengths are theirs.
+        let status = unsafe {
+            itak_store_restore_prefix(self.0, slot.pool.raw(), slot.slot, tokens.as_ptr(),
+                                      tokens.len() as u64, fingerprint.as_ptr().cast(),
+                                      fingerprint.len() as u64, Store::now_unix(), &mut matched)
+        };
+        if status == ITAK_OK as itak_status { Ok(matched) } else { Err(store_error(self.0, status)) }
+    }
+
+    /// `ResidentSession::capture_and_store_prefix` (`session.rs:5056-5094`): the slot must stand
+    /// at exactly `tokens.len()` positions.
+    pub fn capture_and_put(&self, slot: &Slot, tokens: &[u32], fingerprint: &str, elem: Elem) -> Result<(), HipKvError> {
+        let elem = match elem { Elem::F32 => ITAK_ELEM_F32, Elem::F16 => ITAK_ELEM_F16 };
+        // SAFETY: as above.
+        let status = unsafe {
+            itak_store_capture_and_put(self.0, slot.pool.raw(), slot.slot, tokens.as_ptr(),
+                                       tokens.len() as u64, fingerprint.as_ptr().cast(),
+                                       fingerprint.len() as u64, elem as u32, Store::now_unix())
+        };
+        if status == ITAK_OK as itak_status { Ok(()) } else { Err(store_error(self.0, status)) }
+    }
 }

@@ -2036,10 +2036,15 @@ static itak_status check_ring_rewind(itak_pool *pool, const Slot &s, uint64_t ta
         bool saved = false;  // a live checkpoint holds this layer's overwritten rows
         if (saves)
             for (const RingSave &rs : *saves) saved = saved || rs.layer == li;
-        // A layer restored from a snapshot holds nothing older than the snapshot's first row:
-        // the view of a target below first + window would reach under it.
-        if (s.floor[li] > 0 && target < s.floor[li] + L.window)
-            return rewind_range(pool->err, li, s.floor[li] + L.window, s.appended[li], target);
+        // A layer restored from a snapshot holds nothing older than the snapshot's first row.
+        // The query appended next stands at `target` and sees down to target + 1 - window:
+        // that must not reach under the first row. The lowest target that passes, first +
+        // window - 1, is the resident session's rewind by one after a stored prefix covered
+        // the whole prompt (crates/wgpu-compute/src/session.rs:5138-5143); the view at that
+        // length has one row in it, the oldest, that was never written and reads as a fresh
+        // ring's zeros, as after the reference's restore of fewer rows than the window.
+        if (s.floor[li] > 0 && target + 1 < s.floor[li] + L.window)
+            return rewind_range(pool->err, li, s.floor[li] + L.window - 1, s.appended[li], target);
         if (!saved && s.high[li] - target > L.ring - L.window)
             return set_error(pool->err, ITAK_CAPACITY_EXCEEDED, nullptr, li, s.high[li] - target,
                              L.ring - L.window, 0,

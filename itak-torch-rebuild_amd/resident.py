@@ -30,8 +30,14 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import List, Optional, Sequence, Tuple
 
+import sys
+
 from . import itak_kv as _kv
-from .hip_compute import GlimmerConfig, KvCache, KvPool, StepFailed
+from . import prefix_store as _store
+from .hip_compute import GlimmerConfig, KvCache, KvPool, StepFailed, debug_enabled
+
+
+PREFILL_CHUNK = 64  # rows of a prompt forwarded per block (session.rs:186-195)
 
 
 @dataclass
@@ -80,8 +86,16 @@ class ResidentTarget:
         return self._position
 
     def forward(self, tokens: Sequence[int]):
-        """Forward `tokens`, returning the last token's logits."""
-        logits, _ = self.forward_block_capturing(tokens, [])
+        """Forward `tokens`, returning the last token's logits. A prompt goes through in chunks,
+        as the reference's session sends it (64 rows a chunk, crates/wgpu-compute/src/session.rs:
+        186-195), and no longer than the rings' headroom lets one block be."""
+        tokens = list(tokens)
+        if not tokens:
+            raise StepFailed("forward", "no tokens to forward")
+        chunk = PREFILL_CHUNK if self._rewind_room is None else max(1, min(PREFILL_CHUNK, self._rewind_room))
+        logits = None
+        for at in range(0, len(tokens), chunk):
+            logits, _ = self.forward_block_capturing(tokens[at:at + chunk], [])
         return logits[-1]
 
     def forward_capturing(self, tokens: Sequence[int], capture_layers: Sequence[int]):
@@ -145,6 +159,62 @@ class ResidentTarget:
             self._records.append(SpecRoundRecord(_kv.prefix_hash(list(proposed)), len(proposed),
                                                  accepted))
 
+    # ---- the prefix store in the loop -------------------------------------------------
+    def restore_prefix_from_store(self, store, tokens: Sequence[int], fingerprint: str) -> Optional[int]:
+        """ResidentSession::restore_prefix_from_store (session.rs:5000-5053): at position zero
+        with the switch on, installs the longest stored prefix of `tokens` and returns its
+        length; None when nothing was installed (switch off, a live sequence, no usable hit:
+        the cold prefill serves)."""
+        if not _store.prefix_store_enabled():
+            return None
+        if self._position != 0:
+            _diag(f"prefix restore skipped: session position is {self._position}, not 0; a restore "
+                  "is a session-start act and the live sequence is left alone")
+            return None
+        matched = store.restore_prefix(self._cache, tokens, fingerprint)
+        if matched == 0:
+            return None
+        self._position = matched
+        return matched
+
+    def capture_and_store_prefix(self, store, tokens: Sequence[int], fingerprint: str,
+                                 elem: str = "f32") -> None:
+        """ResidentSession::capture_and_store_prefix (session.rs:5056-5094): files the slot's rows
+        under `tokens`, which must be exactly the forwarded prefix."""
+        if not _store.prefix_store_enabled():
+            raise StepFailed("prefix_store", f"the prefix store switch {_store.ENABLE_ENV} is off")
+        if self._position != len(tokens):
+            raise StepFailed("prefix_store",
+                             f"session position {self._position} does not equal the {len(tokens)} "
+                             "tokens to store under; a snapshot covers exactly the forwarded "
+                             "prefix, so any other token list would file one sequence's KV under "
+                             "another's key")
+        store.capture_and_put(self._cache, tokens, fingerprint, elem=elem)
+
+    def forward_with_prefix_store(self, store, tokens: Sequence[int], fingerprint: str,
+                                  elem: str = "f32"):
+        """ResidentSession::forward_with_prefix_store (session.rs:5122-5151), the session-level
+        flow in one call. With the switch off, or mid-sequence, exactly `forward`. Otherwise the
+        longest stored prefix of `tokens` is installed and only the rest is forwarded; a hit that
+        covers the whole prompt is rewound by one position and its last token forwarded again,
+        because the returned logits are that token's forward product and no snapshot carries
+        logits. Afterwards the whole prefix is captured and stored, hit or miss; a failure
+        there is named on the diagnostic channel and the forward's result stands."""
+        tokens = list(tokens)
+        if not _store.prefix_store_enabled() or self._position != 0:
+            return self.forward(tokens)
+        matched = self.restore_prefix_from_store(store, tokens, fingerprint) or 0
+        if matched > 0 and matched == len(tokens):
+            self.rewind(self.checkpoint(1), matched - 1)
+            logits = self.forward(tokens[matched - 1:])
+        else:
+            logits = self.forward(tokens[matched:])
+        try:
+            self.capture_and_store_prefix(store, tokens, fingerprint, elem=elem)
+        except Exception as e:  # store and capture refusals alike: the logits are computed
+            _diag(f"prefix store: post-forward capture/store failed: {e}; the forward's result stands")
+        return logits
+
     # ---- beyond the trait --------------------------------------------------------------
     def spec_round_records(self) -> List[SpecRoundRecord]:
         return list(self._records or [])
@@ -153,6 +223,12 @@ class ResidentTarget:
         """ResidentSession::reset: drop the sequence, positions restart at 0."""
         self._cache.reset()
         self._position = 0
+
+
+def _diag(line: str) -> None:
+    """One line on the library's diagnostic channel (stderr, its prefix), when it is on."""
+    if debug_enabled():
+        print(f"[itak_hip_kv::diag] {line}", file=sys.stderr, flush=True)
 
 
 def pool_ring_rows(cache: KvCache, layer: int) -> int:

@@ -9,6 +9,8 @@ the device step. The oracle replays what the device was given: for every block a
 q, k, v rows the model produced are appended to an oracle KvCache (with the reference's
 checkpoint / rewind_to / release around the round) and attended on the CPU. Bars: attention
 outputs within 2e-3, every layer's visible cache rows bit-exact at the end of every round."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -174,4 +176,100 @@ def test_resident_rewind_refusals_follow_the_session():
     assert driver.position() == 0
     driver.forward([2, 3])
     assert driver.position() == 2
+    pool.close()
+
+
+def _hybrid_target(seed, slots=1, softcap=0.0):
+    W, G = P().LayerKind.windowed, P().LayerKind.Global
+    pattern = [W(48), W(48), G, W(48)]
+    pool = P().KvPool(pattern, KV_HEADS, D, elem="f16", max_slots=slots, capacity_rows=512,
+                      ring_headroom=32)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    config = P().GlimmerConfig(layers=pattern, q_heads=Q_HEADS, kv_heads=KV_HEADS, key_length=D,
+                               value_length=D, sliding_window=48)
+    return pool, config, pattern
+
+
+def _view_bytes(cache, layers):
+    out = []
+    for layer in range(layers):
+        n = cache.stored_len(layer)
+        positions, k, v = cache.read_rows(layer, 0, n)
+        out.append((list(positions), k.tobytes(), v.tobytes()))
+    return out
+
+
+@pytest.mark.parametrize("elem", ["f32", "f16"])
+def test_forward_with_prefix_store_cold_partial_and_full_hits(tmp_path, monkeypatch, capfd, elem):
+    # ResidentSession::forward_with_prefix_store (crates/wgpu-compute/src/session.rs:5122-5151)
+    # on a hybrid pool. Chunks are 48 rows here (what the rings hold beyond their window), and the prompts are cut so
+    # that a run that restores a prefix makes the same launches over the same rows as the cold
+    # run it is compared with: logits and stored rows are then equal bit for bit, which is the
+    # reference's claim for its own chunking ("reproduces exactly the cold run's last step").
+    monkeypatch.setenv("ITAK_KV_PREFIX_STORE", "1")
+    rng = np.random.default_rng(77)
+    tokens = rng.integers(0, VOCAB, size=146).tolist()
+    fp = "toy-model"
+    pool, config, pattern = _hybrid_target(5, slots=6)
+    layers = len(pattern)
+
+    def target():
+        return P().ResidentTarget(pool, pool.acquire(), config, ToyLayers(layers, 5))
+
+    # A prompt of 97 tokens = chunks of 48, 48 and 1: cold (a miss that files the prefix), then
+    # the same prompt again: a hit over the whole prompt, rewound by one, the last token
+    # forwarded again.
+    store = P().PrefixStore.open(str(tmp_path / "one"), 1 << 30)
+    cold = target()
+    cold_logits = cold.forward_with_prefix_store(store, tokens[:97], fp, elem=elem)
+    assert cold.position() == 97 and store.stats().entries == 1
+    assert store.entries()[0].token_count == 97
+    full = target()
+    full_logits = full.forward_with_prefix_store(store, tokens[:97], fp, elem=elem)
+    assert full.position() == 97
+    assert len(full._layers.seen) == layers  # one block of one row per layer, nothing else
+    assert all(rows.shape[0] == 1 and pos == 96 for _, pos, rows, _, _ in full._layers.seen)
+    assert torch.equal(full_logits, cold_logits)
+    assert _view_bytes(full._cache, layers) == _view_bytes(cold._cache, layers)
+
+    # A stored prefix of 96 tokens under a prompt of 144: the rest is one chunk of 48, as the
+    # cold run's third chunk is.
+    store2 = P().PrefixStore.open(str(tmp_path / "two"), 1 << 30)
+    first = target()
+    first.forward_with_prefix_store(store2, tokens[:96], fp, elem=elem)
+    assert store2.entries()[0].token_count == 96
+    partial = target()
+    partial_logits = partial.forward_with_prefix_store(store2, tokens[:144], fp, elem=elem)
+    assert partial.position() == 144
+    assert [pos for _, pos, _, _, _ in partial._layers.seen] == [96] * layers
+    assert sorted(e.token_count for e in store2.entries()) == [96, 144]  # hit or miss, the whole prefix is filed
+    monkeypatch.setenv("ITAK_KV_PREFIX_STORE", "0")   # the switch off: exactly forward
+    plain = target()
+    plain_logits = plain.forward_with_prefix_store(store2, tokens[:144], fp, elem=elem)
+    assert len(store2.entries()) == 2
+    assert torch.equal(partial_logits, plain_logits)
+    assert _view_bytes(partial._cache, layers) == _view_bytes(plain._cache, layers)
+    monkeypatch.setenv("ITAK_KV_PREFIX_STORE", "1")
+
+    # Mid-sequence the store is not consulted and nothing is filed.
+    entries = len(store2.entries())
+    more = partial.forward_with_prefix_store(store2, tokens[144:145], fp, elem=elem)
+    assert partial.position() == 145 and len(store2.entries()) == entries and more.shape == (VOCAB,)
+
+    # A store whose directory has gone (a file stands in its place): the lookup is refused, the
+    # cold prefill serves, the capture fails, and the forward's result stands; the failure is
+    # named on the diagnostic channel.
+    root = tmp_path / "three"
+    store3 = P().PrefixStore.open(str(root), 1 << 30)
+    os.rmdir(root)
+    root.write_text("not a directory")
+    P().set_debug_enabled(True)
+    capfd.readouterr()
+    try:
+        broken = target()
+        broken_logits = broken.forward_with_prefix_store(store3, tokens[:97], fp, elem=elem)
+    finally:
+        P().set_debug_enabled(False)
+    assert torch.equal(broken_logits, cold_logits)
+    assert "post-forward capture/store failed" in capfd.readouterr().err
     pool.close()

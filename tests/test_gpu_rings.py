@@ -362,8 +362,10 @@ def test_a_ring_rewound_to_empty_restores_like_a_fresh_one():
 
 
 def test_a_restored_ring_cannot_be_cut_back_under_its_snapshot():
-    # A snapshot of a windowed layer carries its last `window` rows only: a length below
-    # first + window would put rows in view that the slot never held.
+    # A snapshot of a windowed layer carries its last `window` rows only. The query appended
+    # after a cut stands at the new length and sees `window` positions down from there: the cut
+    # may go to first + window - 1 (the resident session's rewind by one after a stored prefix
+    # covered the whole prompt) and no further.
     pool = P().KvPool([W(8)], 1, 2, elem="f32", ring_headroom=16)
     cache = pool.acquire()
     rows = np.arange(16, dtype=np.float32).reshape(8, 2)
@@ -373,10 +375,16 @@ def test_a_restored_ring_cannot_be_cut_back_under_its_snapshot():
     pool.truncate([cache.slot], [49])
     assert cache.view(0).rows()[0].tolist() == list(range(41, 49))
     with pytest.raises(P().AttentionError) as e:
-        pool.truncate([cache.slot], [47])
-    assert e.value == E("RewindOutOfRange", layer=0, base=48, appended=49, target=47)
+        pool.truncate([cache.slot], [46])
+    assert e.value == E("RewindOutOfRange", layer=0, base=47, appended=49, target=46)
     pool.truncate([cache.slot], [48])
     assert cache.view(0).rows()[0].tolist() == list(range(40, 48))
+    # One further: position 47 goes, and the next row appended sees 40..47 again.
+    pool.truncate([cache.slot], [47])
+    cache.append(0, [47.5] * 2, [47.5] * 2, 47)
+    positions, keys, _ = cache.view(0).rows()
+    assert positions.tolist() == list(range(40, 48))
+    assert keys.reshape(8, 2)[:, 0].tolist() == [0.0, 2.0, 4.0, 6.0, 8.0, 10.0, 12.0, 47.5]
     pool.close()
 
 
