@@ -53,15 +53,18 @@ struct Variant {
     int nq, waves, index;
 };
 static Variant pick_variant(const PoolGeom &g, const AttnBatch &b, uint32_t group) {
-    uint32_t nvec = 0;
+    uint32_t nvec = 0, rows = 0;
     uint64_t blocks = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         nvec = std::max(nvec, b.item[i].rows * group);
+        rows = std::max(rows, b.item[i].rows);
         blocks += uint64_t(g.kv_heads) * item_block_count(b.item[i]);
     }
     if (nvec > 32) return {4, 4, 3};
     if (nvec > 16) return {2, 4, 2};
-    return blocks >= 4096 ? Variant{1, 8, 1} : Variant{1, 4, 0};
+    // (Eight wavefronts for one-row steps only: that variant leaves out the exact treatment of
+    // non-finite values that a step of several rows may need.)
+    return blocks >= 4096 && rows == 1 ? Variant{1, 8, 1} : Variant{1, 4, 0};
 }
 template <int NQ, int W, bool PREP = false>
 static hipError_t grant_lds(size_t lds) {
@@ -478,7 +481,13 @@ __device__ __forceinline__ void attn_combine128_body(const AttnParams &p, const 
         float mx = m_run;
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-            if (s0 + sl + u * SL >= S) ml[u].x = -INFINITY;
+            // A lane past the last split holds a second copy of that split's partial: its
+            // weight is zero, and so must the copy be, or a value in it that is not finite
+            // (which the rows that see the key are due) would make the product NaN.
+            if (s0 + sl + u * SL >= S) {
+                ml[u].x = -INFINITY;
+                x[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
             mx = fmaxf(mx, ml[u].x);
         }
         // Nothing visible in these splits (nor before): every weight below is exp(-inf) = 0
@@ -593,7 +602,10 @@ __global__ __launch_bounds__(256) void attn_combine128_wave_kernel(AttnParams p,
     float mx = -INFINITY;
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-        if (sl + u * 2 >= S) ml[u].x = -INFINITY;
+        if (sl + u * 2 >= S) {  // a second copy of the last split: weight zero, and cleared
+            ml[u].x = -INFINITY;
+            x[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
         mx = fmaxf(mx, ml[u].x);
     }
     const float M = half_max(mx);

@@ -37,14 +37,15 @@ struct DieVariant {
 };
 // 16-vector steps with four or eight wavefronts, as the ordinary plan picks them, or 32 vectors.
 DieVariant pick_die_variant(const PoolGeom &g, const AttnBatch &b, uint32_t group) {
-    uint32_t nvec = 0;
+    uint32_t nvec = 0, rows = 0;
     uint64_t blocks = 0;
     for (uint32_t i = 0; i < b.n; ++i) {
         nvec = std::max(nvec, b.item[i].rows * group);
+        rows = std::max(rows, b.item[i].rows);
         blocks += uint64_t(g.kv_heads) * item_block_count(b.item[i]);
     }
     if (nvec > 16) return {2, 4, 2};
-    return blocks >= 4096 ? DieVariant{1, 8, 1} : DieVariant{1, 4, 0};
+    return blocks >= 4096 && rows == 1 ? DieVariant{1, 8, 1} : DieVariant{1, 4, 0};
 }
 
 template <int NQ, int W>

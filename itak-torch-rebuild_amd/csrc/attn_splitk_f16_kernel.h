@@ -106,17 +106,66 @@ __device__ __forceinline__ float column_sum(float v) {
     return __uint_as_float(c[0]) + __uint_as_float(c[1]);
 }
 
+// What the exact treatment of non-finite value rows needs to know of the item's query rows.
+struct RowSpan {
+    uint32_t pos0;    // position of the item's first query row (not clamped)
+    uint32_t rows;
+    uint32_t window;  // 0 on a global layer
+    uint32_t kv_lo;
+    uint32_t magic;   // j / group == (j * magic) >> 16
+    // The step appends its own rows (they are then the only keys at the causal edge that some
+    // rows see and others do not), and whether one of their values is not finite.
+    bool appends, new_not_finite;
+};
+
+// O^T += V^T . P^T of one tile of query vectors, row of the step by row, for a block in which
+// the rows do not all see the same keys and some value is not finite. The rows of a step share
+// the block's value operand, a key that only some of them see is one column of it, and a
+// masked key's zero weight times a value that is not finite is NaN in every row of the
+// product, where gqa_attention never reads the value row of a key a query does not see
+// (crates/attention/src/attention.rs:160-173). So the product is taken once per query row,
+// with the value columns of the keys that row does not see cleared, and each lane keeps the
+// result of the row its own column belongs to.
+template <bool RING>
+__device__ __forceinline__ void accumulate_by_row(floatx4 (&o)[8], const BlockOperands &b, half8 pb,
+                                                  uint32_t qt, uint32_t key_base, uint32_t jl,
+                                                  uint32_t kv_len, const RowSpan &span) {
+    const uint32_t my_row = ((qt * 16 + jl) * span.magic) >> 16;
+#pragma unroll 1
+    for (uint32_t r = 0; r < span.rows; ++r) {
+        const uint32_t pos = min(span.pos0 + r, kv_len - 1);
+        const uint32_t lo = RING ? lowest_visible(span.pos0 + r, span.window, span.kv_lo) : 0u;
+        const uint32_t end = min(pos + 1 - min(pos + 1, key_base), 8u);   // this lane's keys up to pos
+        const uint32_t first = min(lo - min(lo, key_base), 8u);             // and from lo on
+        const u32x4 keep = first_halves(end) & ~first_halves(first);
+        const bool mine = my_row == r;
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) {
+            const floatx4 part = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                keep_halves(b.v[dt], keep), pb, floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+            if (mine) o[dt] += part;
+            // One channel tile at a time: left to itself the scheduler starts all eight products
+            // before it adds the first, and their 32 registers do not fit beside the loop's.
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
 // One 32-key block against all NQ tiles of query vectors. FIRST = the wavefront's first
 // block: the running state is written, not rescaled (most decode wavefronts see one block).
 // Up to 32 vectors the Q^T operand lives in registers (qreg), beyond that it is re-read
 // from LDS per block: lane (g, jl) holds channels k*32 + g*8 .. +8 of vector jl.
-template <int NQ, bool FIRST, bool RING>
+// BYROW = false compiles the exact treatment of non-finite values out: for the eight-wavefront
+// variant, which the planners give to steps of one row per item only (its registers are all
+// taken, and one row alone never needs it).
+template <int NQ, bool FIRST, bool RING, bool BYROW>
 __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &b,
                                               const half8 *qreg, const _Float16 *sm_q,
                                               uint32_t kb, uint32_t g, uint32_t jl,
                                               const uint32_t *colpos, const uint32_t *collo,
                                               uint32_t pos0, uint32_t kv_len, uint32_t lo_min,
-                                              uint32_t lo_max, float softcap, float inv_cap) {
+                                              uint32_t lo_max, float softcap, float inv_cap,
+                                              const RowSpan &span) {
     const uint32_t key_base = kb * kBlockKeys + g * 8;  // first of this lane's 8 keys
     const bool tail = (kb + 1) * kBlockKeys > kv_len || (RING && kb * kBlockKeys < lo_min);
     auto zero_tail = [&] {
@@ -133,6 +182,17 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
     [[maybe_unused]] float alphas[NQ > 2 ? NQ : 1];
     const bool need_mask =
         (kb + 1) * kBlockKeys > pos0 + 1 || (RING && kb * kBlockKeys < lo_max);
+    // A block of several rows that do not all see the same keys: values that are not finite go
+    // the exact way (accumulate_by_row). One row alone sees what zero_tail left.
+    // (Where the step appends its own rows the answer for the causal edge was settled when they
+    // were converted; looking through the operand registers is a hundred instructions that the
+    // workgroup at the end of every item would otherwise run, cold.)
+    auto suspect = [&]() -> bool {
+        const bool low_edge = RING && kb * kBlockKeys < lo_max;
+        if (!low_edge && span.appends) return span.new_not_finite;
+        return any_not_finite(b.v);
+    };
+    const bool by_row = BYROW && span.rows > 1 && need_mask && (NQ <= 2 || !tail) && suspect();
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
         half8 qb[4];
@@ -199,6 +259,11 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
             // four tiles of score MFMAs and softmax have run.
             pbs[qt] = pb;
             alphas[qt] = alpha;
+        } else if (__builtin_expect(by_row, false)) {
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt)
+                st.o[qt][dt] = FIRST ? floatx4{0.0f, 0.0f, 0.0f, 0.0f} : st.o[qt][dt] * alpha;
+            accumulate_by_row<RING>(st.o[qt], b, pb, qt, key_base, jl, kv_len, span);
         } else if constexpr (FIRST) {
 #pragma unroll
             for (int dt = 0; dt < 8; ++dt)
@@ -215,6 +280,9 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
     }
     if constexpr (NQ > 2) {
         if (tail) zero_tail();
+        // (The values are looked at after the tail is cleared: what lies past the stored rows
+        // is nobody's to see.)
+        const bool by_row_late = by_row || (BYROW && span.rows > 1 && need_mask && tail && suspect());
         if constexpr (!FIRST) {
 #pragma unroll
             for (int qt = 0; qt < NQ; ++qt)
@@ -222,6 +290,17 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
 #pragma unroll
                     for (int dt = 0; dt < 8; ++dt) st.o[qt][dt] *= alphas[qt];
                 }
+        }
+        if (__builtin_expect(by_row_late, false)) {
+#pragma unroll
+            for (int qt = 0; qt < NQ; ++qt) {
+                if constexpr (FIRST) {
+#pragma unroll
+                    for (int dt = 0; dt < 8; ++dt) st.o[qt][dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+                }
+                accumulate_by_row<RING>(st.o[qt], b, pbs[qt], qt, key_base, jl, kv_len, span);
+            }
+            return;
         }
 #pragma unroll
         for (int qt = 0; qt < NQ; ++qt)
@@ -384,7 +463,10 @@ __device__ __forceinline__ void die_merge(const AttnParams &p, const AttnItem &i
             float mx = m_run;
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
-                if (s0 + u >= S) ml[u].x = -INFINITY;
+                if (s0 + u >= S) {  // a second copy of the last split: weight zero, and cleared
+                    ml[u].x = -INFINITY;
+                    x[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
                 mx = fmaxf(mx, ml[u].x);
             }
             const float ref = mx == -INFINITY ? 0.0f : mx;  // exp2(-inf - finite) = 0
@@ -618,7 +700,9 @@ __device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const 
         if (j >= nvec) h = half4{0, 0, 0, 0};
         *reinterpret_cast<half4 *>(sm_q + j * kQStride + c4) = h;
     }
+    __shared__ uint32_t sm_new_not_finite[WAVES];
     if (owns_new) {
+        uint32_t not_finite = 0;  // exponent field all ones in some half of a new value row
 #pragma unroll
         for (int u = 0; u < NL; ++u) {
             const uint32_t f = tid + u * WAVES * 64;
@@ -635,6 +719,8 @@ __device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const 
             const uint16_t h0 = f32_to_f16_bits(a.x), h1 = f32_to_f16_bits(a.y);
             const uint16_t h2 = f32_to_f16_bits(a.z), h3 = f32_to_f16_bits(a.w);
             uint2 packed{uint32_t(h0) | (uint32_t(h1) << 16), uint32_t(h2) | (uint32_t(h3) << 16)};
+            if (side)
+                not_finite |= ((packed.x & 0x7c007c00u) + 0x04000400u) | ((packed.y & 0x7c007c00u) + 0x04000400u);
             *reinterpret_cast<uint2 *>((side ? sm_newv : sm_newk) + r * kNewStride + c4) = packed;
             const uint32_t key = item.pos0 + r, kin = key % kBlockKeys;
             const uint64_t blk =
@@ -651,9 +737,16 @@ __device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const 
                 vd[3 * kBlockKeys] = h3;
             }
         }
+        const bool wave_saw = __builtin_amdgcn_ballot_w64((not_finite & 0x80008000u) != 0) != 0;
+        if (lane == 0) sm_new_not_finite[wave] = wave_saw ? 1u : 0u;
     }
     ITAK_MARK(4)
     __syncthreads();
+    bool new_not_finite = false;
+    if (owns_new) {
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) new_not_finite = new_not_finite || sm_new_not_finite[w] != 0;
+    }
     half8 qreg[NQ <= 2 ? NQ * 4 : 1];
     if constexpr (NQ <= 2) {
 #pragma unroll
@@ -669,13 +762,29 @@ __device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const 
     // operand sets, so the next block's loads fly while the current one is multiplied; with
     // 64 vectors the accumulators take that room and the other wavefronts hide the latency.
     WaveState<NQ> st;
+    const RowSpan span{item.pos0, item.rows, window, kv_lo, magic, fused, new_not_finite};
 #define ITAK_BLOCK(FIRST, BUF, KB)                                                               \
     do {                                                                                         \
         if (fused && ((KB) + 1) * kBlockKeys > item.pos0)                                        \
             patch_new_rows(BUF, sm_newk, sm_newv, KB, g, jl, item.pos0, item.kv_len);            \
-        process_block<NQ, FIRST, RING>(st, BUF, qreg, sm_q, KB, g, jl, colpos, collo,                  \
+        /* Two copies of the block's arithmetic: the one with the exact treatment of values   \
+           that are not finite only for blocks in which the step's rows do not all see the    \
+           same keys, so that every other block runs code that knows nothing of it. */        \
+        if constexpr (NQ > 2) { /* (no room for two copies beside 128 accumulators; the one copy  \
+           costs the 7-row verify block 3 %: 23.7 -> 24.5 us per layer, same box) */             \
+            process_block<NQ, FIRST, RING, true>(st, BUF, qreg, sm_q, KB, g, jl, colpos,         \
+                                 collo, min(item.pos0, item.kv_len - 1), item.kv_len, lo_min,    \
+                                 lo_max, softcap, inv_cap, span);                                \
+        } else if (WAVES != 8 && item.rows > 1 &&                                                \
+            (((KB) + 1) * kBlockKeys > min(item.pos0, item.kv_len - 1) + 1 ||                    \
+             (RING && (KB) * kBlockKeys < lo_max)))                                              \
+            process_block<NQ, FIRST, RING, WAVES != 8>(st, BUF, qreg, sm_q, KB, g, jl, colpos,   \
+                                 collo, min(item.pos0, item.kv_len - 1), item.kv_len, lo_min,    \
+                                 lo_max, softcap, inv_cap, span);                                \
+        else                                                                                     \
+            process_block<NQ, FIRST, RING, false>(st, BUF, qreg, sm_q, KB, g, jl, colpos, collo, \
                                  min(item.pos0, item.kv_len - 1), item.kv_len, lo_min, lo_max,   \
-                                 softcap, inv_cap);                                              \
+                                 softcap, inv_cap, span);                                        \
     } while (0)
     if (has_block) {
         if constexpr (NQ <= 2) {

@@ -69,7 +69,9 @@ __device__ __forceinline__ float4 kv_load(const float *p) {
     }
 }
 
-template <int N, bool RING, int D, bool STREAM>
+// BYROW: the launch holds an item of several rows (the exact treatment of values that are not
+// finite is compiled in; launches of one row per item run the kernel without it).
+template <int N, bool RING, int D, bool STREAM, bool BYROW>
 __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnParams p,
                                                                          AttnBatchT<N> b,
                                                                          uint32_t total_partials) {
@@ -233,6 +235,62 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
         for (int h = 0; h < kH; ++h)
 #pragma unroll
             for (int e = 0; e < 4; ++e) o[h][e] *= alpha;
+        // A block in which the tile's rows do not all see the same keys, holding a value that is
+        // not finite: gqa_attention never reads the value row of a key a query does not see
+        // (crates/attention/src/attention.rs:160-173), but the rows share the value operand here
+        // and a masked key's zero weight times such a value is NaN. The product is then taken
+        // once per query row of the tile, the values of the keys that row does not see
+        // cleared, and each lane keeps the result of the row its own column belongs to.
+        if (BYROW && row_last > row_first &&
+            (key0 + kBlockKeys > min(item.pos0 + row_first, item.kv_len - 1) + 1 ||
+             (RING && key0 < lowest_visible(item.pos0 + row_last, window, kv_lo)))) {
+            uint32_t seen = 0;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+#pragma unroll
+                    for (int h = 0; h < kH; ++h) {
+                        const float4 a = vreg[t][r][h];  // exponent all ones: 0x7f800000 + 0x00800000 = 0x80000000
+                        seen |= ((__float_as_uint(a.x) & 0x7f800000u) + 0x00800000u) |
+                                ((__float_as_uint(a.y) & 0x7f800000u) + 0x00800000u) |
+                                ((__float_as_uint(a.z) & 0x7f800000u) + 0x00800000u) |
+                                ((__float_as_uint(a.w) & 0x7f800000u) + 0x00800000u);
+                    }
+            if (__builtin_amdgcn_ballot_w64((seen & 0x80000000u) != 0) != 0) {
+#pragma unroll 1
+                for (uint32_t rr = row_first; rr <= row_last; ++rr) {
+                    const uint32_t pos = min(item.pos0 + rr, item.kv_len - 1);
+                    const uint32_t lo = RING ? lowest_visible(item.pos0 + rr, window, kv_lo) : 0u;
+                    const bool mine = row == rr;
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const uint32_t kp = key0 + 16 * t + 4 * g + r;
+                            const bool seen_by_row = kp <= pos && kp >= lo;
+#pragma unroll
+                            for (int h = 0; h < kH; ++h) {
+                                const float4 v = vreg[t][r][h];
+                                const float4 a = seen_by_row ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+                                const floatx4 zero = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+                                const floatx4 p0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, sc[t][r], zero, 0, 0, 0);
+                                const floatx4 p1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, sc[t][r], zero, 0, 0, 0);
+                                const floatx4 p2 = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, sc[t][r], zero, 0, 0, 0);
+                                const floatx4 p3 = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, sc[t][r], zero, 0, 0, 0);
+                                if (mine) {
+                                    o[h][0] += p0;
+                                    o[h][1] += p1;
+                                    o[h][2] += p2;
+                                    o[h][3] += p3;
+                                }
+                                __builtin_amdgcn_sched_barrier(0);
+                            }
+                        }
+                }
+                continue;
+            }
+        }
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -373,9 +431,18 @@ hipError_t launch_attn_splitk_f32(const AttnParams &p, const AttnBatch &b, uint3
     // of 8192 rows on two layers.)
     bool single = p.kv_streams != 0;
     for (uint32_t i = 0; i < b.n; ++i) single = single && b.item[i].rows * p.group <= 16;
-#define ITAK_LAUNCH_F32_S(RING, D, STREAM)                                                        \
-    ITAK_DISPATCH_BATCH(b.n, (attn_splitk_f32_kernel<N, RING, D, STREAM>                            \
+    bool several = false;
+    for (uint32_t i = 0; i < b.n; ++i) several = several || b.item[i].rows > 1;
+#define ITAK_LAUNCH_F32_B(RING, D, STREAM, BYROW)                                                 \
+    ITAK_DISPATCH_BATCH(b.n, (attn_splitk_f32_kernel<N, RING, D, STREAM, BYROW>                     \
                               <<<b.total_blocks, kWavesF32 * 64, 0, stream>>>(p, AttnBatchT<N>(b), total_partials)))
+#define ITAK_LAUNCH_F32_S(RING, D, STREAM)              \
+    do {                                                \
+        if (several)                                    \
+            ITAK_LAUNCH_F32_B(RING, D, STREAM, true);   \
+        else                                            \
+            ITAK_LAUNCH_F32_B(RING, D, STREAM, false);  \
+    } while (0)
 #define ITAK_LAUNCH_F32(RING, D)                 \
     do {                                         \
         if (single)                              \
@@ -389,6 +456,7 @@ hipError_t launch_attn_splitk_f32(const AttnParams &p, const AttnBatch &b, uint3
         if (p.ring_blocks) ITAK_LAUNCH_F32(true, 128); else ITAK_LAUNCH_F32(false, 128);
     }
 #undef ITAK_LAUNCH_F32_S
+#undef ITAK_LAUNCH_F32_B
 #undef ITAK_LAUNCH_F32
     return hipGetLastError();
 }

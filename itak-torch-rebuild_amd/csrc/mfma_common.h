@@ -35,6 +35,20 @@ __device__ __forceinline__ half8 keep_halves(half8 v, u32x4 keep) {
     return __builtin_bit_cast(half8, __builtin_bit_cast(u32x4, v) & keep);
 }
 
+// True when some half of the N operand register groups is an infinity or a NaN (exponent field
+// all ones), in any lane of the wavefront.
+template <int N>
+__device__ __forceinline__ bool any_not_finite(const half8 (&v)[N]) {
+    uint32_t seen = 0;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const u32x4 x = __builtin_bit_cast(u32x4, v[i]);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) seen |= (x[c] & 0x7c007c00u) + 0x04000400u;  // 0x7c00 + 0x0400 = 0x8000
+    }
+    return __builtin_amdgcn_ballot_w64((seen & 0x80008000u) != 0) != 0;
+}
+
 // The value of another lane of the same 16-lane row, chosen by a DPP control word.
 template <int CTRL>
 __device__ __forceinline__ float dpp_lane(float v) {
