@@ -412,6 +412,9 @@ def main():
                     help="merge each unit's splits on its compute die inside the split-K launch "
                          "(ITAK_POOL_DIE_MERGE) where the batch suits it, instead of with a launch "
                          "of its own")
+    ap.add_argument("--q-two-halves", action="store_true",
+                    help="queries as two f16 halves in the split-K kernels' score products "
+                         "(ITAK_POOL_Q_TWO_HALVES): the 2e-3 bar then holds off unit scale")
     ap.add_argument("--prep", action="store_true",
                     help="also time the step with the fused Q/K preparation (per-head RMSNorm + "
                          "RoPE) before it and the sigmoid gate after it, reported as 'with_prep'")
@@ -451,7 +454,8 @@ def main():
         return
     result = run_workload(args, pkg, torch, np, dev, stream, timed)
     primary = (args.workload == "decode" and args.kv == "f16" and args.softcap == 0.0
-               and not args.only and not args.merge_in_launch)
+               and not args.only and not args.merge_in_launch and not args.die_merge
+               and not args.q_two_halves)
     if primary:
         # The other configurations in short runs of their own, so that one line carries every
         # kernel's figure; `metric`, `value` and `config` stay those of the decode step.
@@ -643,7 +647,8 @@ def run_workload(args, pkg, torch, np, dev, stream, timed):
                       capacity_rows=max_len + rows + 8, scrub_on_truncate=False,
                       ring_headroom=rows if wl == "prefill_windowed" else 0,
                       merge_in_launch=args.merge_in_launch,
-                      die_merge=getattr(args, "die_merge", False))
+                      die_merge=getattr(args, "die_merge", False),
+                      q_two_halves=getattr(args, "q_two_halves", False))
     pool.set_stream(stream.cuda_stream)
     caches = [pool.acquire() for _ in range(slots)]
 

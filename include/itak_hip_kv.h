@@ -83,13 +83,27 @@ enum {
     ITAK_KV_IO = 35                       /* what = context, a = errno; message as std::io::Error prints it */
 };
 
-/* Storage / source element types. An f32 pool computes in f32 throughout. An f16 pool rounds
-   the rows it stores to f16 (round to nearest even, as the reference's f16 session does) and its
-   attention kernels feed Q and the softmax weights to the matrix pipe as f16 too (scores,
-   softmax state and accumulators stay f32): outputs are within 2e-3 (max abs) of f32 arithmetic
-   over the same rounded rows as long as the scaled scores q.k*scale have a standard deviation
-   of at most about 3 (3e-5 at unit scale, 1.5e-3 at 3, above the bar from about 4.5 on). Q and K
-   normed per head, as the reference's model norms them, stay at unit scale.
+/* Storage / source element types.
+   An f32 pool computes in f32 throughout. Its outputs are within 1e-5 of the reference's f32
+   arithmetic, as the largest deviation over the largest output magnitude, on unit-scale inputs
+   (3e-6 to 5e-6 observed). That figure is a distance between two f32 evaluations that sum in
+   different orders: with Q at three and K at two times unit scale (scaled scores of standard
+   deviation 6) each of the two is 2e-6 to 8e-6 from a float64 evaluation and they have been
+   seen 1.08e-5 apart; off unit scale the bar that holds is 1e-5 against float64, not against
+   the reference's own rounding.
+   An f16 pool rounds the rows it stores to f16 (round to nearest even, as the reference's f16
+   session does) and its attention kernels feed Q and the softmax weights to the matrix pipe as
+   f16 too (scores, softmax state and accumulators stay f32): outputs are within 2e-3 (max abs)
+   of f32 arithmetic over the same rounded rows as long as the scaled scores q.k*scale have a
+   standard deviation of at most about 3 (3e-5 at unit scale, 1.5e-3 at 3, above the bar from
+   about 4.5 on). Q and K normed per head, as the reference's model norms them, stay at unit
+   scale. ITAK_POOL_Q_TWO_HALVES lifts the limit for decode steps and blocks of up to 8 rows at
+   head_dim 128 (4e-5 to 2.6e-4 observed at standard deviation 6).
+   A value row that is not finite reaches the outputs of exactly the query rows that see its key
+   (the reference never reads the value row of a masked key) on f32 pools and, on f16 pools, in
+   decode steps and blocks of up to 8 rows at head_dim 128; in longer blocks and at the other
+   head dims of f16 pools the rows of a step share one product, and the rows of the step that
+   do not see the key come out NaN in the channels where the value is not finite.
    Matrix-pipe kernels exist for f16 pools at head_dim 64, 96, 128 and 256 with up to 16 Q heads per
    KV head and for f32 pools at head_dim 64 and 128; every other shape (any head_dim up to 256)
    runs on a general kernel that is correct and one to two orders of magnitude slower. */
@@ -124,7 +138,16 @@ enum {
        2 to 4 % faster than the merge launch on batches of a hundred MB of KV per layer and more,
        level or slower below (the launch's own tail and a slower start cost what the second
        launch costs), so it is not the default. */
-    ITAK_POOL_DIE_MERGE = 4u
+    ITAK_POOL_DIE_MERGE = 4u,
+    /* f16 pools at head_dim 128, decode steps and blocks of up to 8 rows (the split-K kernels):
+       the queries enter the score products as two f16 halves, q = hi + lo, and every score is
+       K.hi + K.lo. Without the flag Q is rounded to f16 once, an error relative to each channel
+       that grows with the scores: outputs meet the 2e-3 bar up to scaled scores of standard
+       deviation 3 (see ITAK_ELEM_F16). With it the queries are good to 2^-22 and what is left is
+       the rounding of the softmax weights to f16. These kernels wait for memory, not for the
+       matrix pipe, so the second product costs nothing measurable. Longer blocks and prefill
+       chunks (the block kernel) are not affected by the flag. */
+    ITAK_POOL_Q_TWO_HALVES = 8u
 };
 
 typedef struct itak_pool itak_pool;

@@ -31,6 +31,7 @@ LAYER_GLOBAL, LAYER_WINDOWED = 0, 1
 POOL_SCRUB_ON_TRUNCATE = 1
 POOL_MERGE_IN_LAUNCH = 2
 POOL_DIE_MERGE = 4
+POOL_Q_TWO_HALVES = 8
 
 
 class PoolConfig(C.Structure):

@@ -73,13 +73,16 @@ __device__ __forceinline__ half8 to_half8_rne(float4 a, float4 b) {
     return h;
 }
 
-template <int N, bool RING>
+// QLO: the queries as two f16 halves, q = hi + lo, scores K.hi + K.lo (attn_splitk_f16_qlo.hip
+// says why).
+template <int N, bool RING, bool QLO = false>
 __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams p, AttnBatchT<N> b,
                                                                        uint32_t total_partials) {
     __shared__ float sm_m[kWaves * 16];
     __shared__ float sm_l[kWaves * 16];
     __shared__ __attribute__((aligned(16))) float sm_o[kWaves * 8 * 64 * 4];
     __shared__ __attribute__((aligned(16))) _Float16 sm_q[16 * kQStride];
+    [[maybe_unused]] __shared__ __attribute__((aligned(16))) _Float16 sm_q_lo[QLO ? 16 * kQStride : 8];
     __shared__ __attribute__((aligned(16))) _Float16 sm_new[2 * kD];  // the new K row, then the new V row
 
     const uint32_t tid = threadIdx.x;
@@ -183,6 +186,12 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
                 static_cast<_Float16>(qraw[u].z), static_cast<_Float16>(qraw[u].w)};
         if (j >= group) h = half4{0, 0, 0, 0};
         *reinterpret_cast<half4 *>(sm_q + j * kQStride + c4) = h;
+        if constexpr (QLO) {
+            half4 l{static_cast<_Float16>(qraw[u].x - float(h[0])), static_cast<_Float16>(qraw[u].y - float(h[1])),
+                    static_cast<_Float16>(qraw[u].z - float(h[2])), static_cast<_Float16>(qraw[u].w - float(h[3]))};
+            if (j >= group) l = half4{0, 0, 0, 0};
+            *reinterpret_cast<half4 *>(sm_q_lo + j * kQStride + c4) = l;
+        }
     }
     uint2 packed{0u, 0u};
     if (owns_new && wave == 0) {
@@ -220,6 +229,15 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
 #pragma unroll
         for (int k = 0; k < 4; ++k)
             s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bk[t][k], qb[k], s[t], 0, 0, 0);
+    }
+    if constexpr (QLO) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const half8 ql = *reinterpret_cast<const half8 *>(sm_q_lo + jl * kQStride + k * 32 + g * 8);
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bk[t][k], ql, s[t], 0, 0, 0);
+        }
     }
     ITAK_MARK(3)
     float sc[8];
@@ -435,8 +453,20 @@ uint32_t attn_decode_f16_resident_groups() {
 }
 
 hipError_t launch_attn_decode_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
-                                  hipStream_t stream) {
+                                  hipStream_t stream, bool q_two_halves) {
     if (b.total_blocks == 0) return hipSuccess;
+    if (q_two_halves) {
+#define ITAK_LAUNCH_DECODE_QLO()                                                                   \
+    do {                                                                                           \
+        if (p.ring_blocks)                                                                         \
+            attn_decode_f16_kernel<N, true, true><<<b.total_blocks, kWaves * 64, 0, stream>>>(p, AttnBatchT<N>(b), total_partials); \
+        else                                                                                       \
+            attn_decode_f16_kernel<N, false, true><<<b.total_blocks, kWaves * 64, 0, stream>>>(p, AttnBatchT<N>(b), total_partials); \
+    } while (0)
+        ITAK_DISPATCH_BATCH(b.n, ITAK_LAUNCH_DECODE_QLO());
+#undef ITAK_LAUNCH_DECODE_QLO
+        return hipGetLastError();
+    }
 #define ITAK_LAUNCH_DECODE()                                                                       \
     do {                                                                                           \
         if (p.ring_blocks)                                                                         \

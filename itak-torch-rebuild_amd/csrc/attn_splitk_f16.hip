@@ -66,6 +66,11 @@ static Variant pick_variant(const PoolGeom &g, const AttnBatch &b, uint32_t grou
     // non-finite values that a step of several rows may need.)
     return blocks >= 4096 && rows == 1 ? Variant{1, 8, 1} : Variant{1, 4, 0};
 }
+// The variant a planned batch takes: 0 = 16 vectors on four wavefronts, 1 = on eight, 2 = 32
+// vectors, 3 = 64 vectors.
+int attn_splitk_f16_variant(const PoolGeom &g, const AttnBatch &b, uint32_t group) {
+    return pick_variant(g, b, group).index;
+}
 template <int NQ, int W, bool PREP = false>
 static hipError_t grant_lds(size_t lds) {
     static size_t granted = 64 * 1024;
@@ -225,12 +230,14 @@ uint64_t attn_splitk_f16_plan_exchange(const PoolGeom &g, AttnBatch &b, uint32_t
 
 hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                   uint32_t max_rows, hipStream_t stream,
-                                  const FoldedParams *folded) {
+                                  const FoldedParams *folded, bool q_two_halves) {
     (void)max_rows;
     if (b.total_blocks == 0) return hipSuccess;
     const Variant v = pick_variant(p.g, b, p.group);
     const bool prep = folded && folded->prep_on;
-    if (!prep && v.index == 0 && attn_decode_f16_takes(p, b)) return launch_attn_decode_f16(p, b, total_partials, stream);
+    if (!prep && v.index == 0 && attn_decode_f16_takes(p, b))
+        return launch_attn_decode_f16(p, b, total_partials, stream, q_two_halves);
+    if (q_two_halves) return launch_attn_splitk_f16_qlo(p, b, total_partials, stream, folded);
 #define ITAK_LAUNCH(NQ, W)                                                                \
     do {                                                                                  \
         const size_t lds = variant_lds(NQ, W);                                            \

@@ -158,9 +158,14 @@ __device__ __forceinline__ void accumulate_by_row(floatx4 (&o)[8], const BlockOp
 // BYROW = false compiles the exact treatment of non-finite values out: for the eight-wavefront
 // variant, which the planners give to steps of one row per item only (its registers are all
 // taken, and one row alone never needs it).
-template <int NQ, bool FIRST, bool RING, bool BYROW>
+// QLO: the scaled queries are held as two halves, q = hi + lo with hi = f16(q) and lo = f16(q -
+// hi), and every score is K.hi + K.lo: the queries' rounding to f16, which is relative to each
+// channel and so grows with the scores, leaves the scores (the keys are exact, they are stored
+// as f16). The low halves are read from LDS (sm_q_lo) block by block.
+template <int NQ, bool FIRST, bool RING, bool BYROW, bool QLO>
 __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &b,
                                               const half8 *qreg, const _Float16 *sm_q,
+                                              [[maybe_unused]] const _Float16 *sm_q_lo,
                                               uint32_t kb, uint32_t g, uint32_t jl,
                                               const uint32_t *colpos, const uint32_t *collo,
                                               uint32_t pos0, uint32_t kv_len, uint32_t lo_min,
@@ -211,6 +216,16 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
 #pragma unroll
             for (int k = 0; k < 4; ++k)
                 s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b.k[t][k], qb[k], s[t], 0, 0, 0);
+        }
+        if constexpr (QLO) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const half8 ql = *reinterpret_cast<const half8 *>(sm_q_lo + (qt * 16 + jl) * kQStride +
+                                                                  k * 32 + g * 8);
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b.k[t][k], ql, s[t], 0, 0, 0);
+            }
         }
         float sc[8];
 #pragma unroll
@@ -406,9 +421,10 @@ __device__ __forceinline__ float4 prep_chunk(float4 x, bool norm, float4 w, floa
 
 
 // Dynamic LDS of a variant: the wavefronts' (m, l) and O^T for their merge, Q^T, the new rows.
-inline size_t variant_lds(int nq, int waves) {
+inline size_t variant_lds(int nq, int waves, bool q_two_halves = false) {
     return (size_t(2) * waves * nq * 16 + size_t(waves) * nq * 8 * 64 * 4) * 4 +
-           size_t(nq) * 16 * kQStride * 2 + size_t(2) * kMaxNewRows * kNewStride * 2;
+           size_t(nq) * 16 * kQStride * 2 * (q_two_halves && nq <= 2 ? 2 : 1) +
+           size_t(2) * kMaxNewRows * kNewStride * 2;
 }
 
 // ---- the merge of a unit's splits on the unit's own compute die (DIE instantiations) -------
@@ -499,7 +515,7 @@ __device__ __forceinline__ void die_merge(const AttnParams &p, const AttnItem &i
     }
 }
 
-template <int NQ, int WAVES, int N, bool RING, bool PREP, bool DIE>
+template <int NQ, int WAVES, int N, bool RING, bool PREP, bool DIE, bool QLO = false>
 __device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const AttnBatchT<N> &b,
                                                      uint32_t total_partials,
                                                      [[maybe_unused]] const FoldedParams &fold,
@@ -511,6 +527,11 @@ __device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const 
     _Float16 *sm_q = reinterpret_cast<_Float16 *>(sm_o + WAVES * NQ * 8 * 64 * 4);  // [NQ*16][kQStride]
     _Float16 *sm_newk = sm_q + NQ * 16 * kQStride;  // [kMaxNewRows][kNewStride]
     _Float16 *sm_newv = sm_newk + kMaxNewRows * kNewStride;
+    // QLO: the queries' low halves, [NQ*16][kQStride]. With 64 vectors there is no LDS left for
+    // them: they lie in the area the wavefronts' merge takes over when the blocks are done
+    // (a barrier stands between the last read and the merge's first write).
+    [[maybe_unused]] _Float16 *sm_q_lo =
+        NQ > 2 ? reinterpret_cast<_Float16 *>(sm_o) : sm_newv + kMaxNewRows * kNewStride;
 
     const uint32_t tid = threadIdx.x;
     const uint32_t wave = tid >> 6, lane = tid & 63;
@@ -695,10 +716,17 @@ __device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const 
             if (prot && row != 0) prep_trig(t, double(item.pos0 + row), freq, trig_pairs);
             a = prep_chunk(a, fold.prep_q_weight != nullptr, wq, fold.prep_eps, c4, lane, prot, pinter, t);
         }
-        half4 h{static_cast<_Float16>(a.x * qscale), static_cast<_Float16>(a.y * qscale),
-                static_cast<_Float16>(a.z * qscale), static_cast<_Float16>(a.w * qscale)};
+        const float4 as = make_float4(a.x * qscale, a.y * qscale, a.z * qscale, a.w * qscale);
+        half4 h{static_cast<_Float16>(as.x), static_cast<_Float16>(as.y),
+                static_cast<_Float16>(as.z), static_cast<_Float16>(as.w)};
         if (j >= nvec) h = half4{0, 0, 0, 0};
         *reinterpret_cast<half4 *>(sm_q + j * kQStride + c4) = h;
+        if constexpr (QLO) {  // what the rounding to f16 dropped, as a second f16
+            half4 l{static_cast<_Float16>(as.x - float(h[0])), static_cast<_Float16>(as.y - float(h[1])),
+                    static_cast<_Float16>(as.z - float(h[2])), static_cast<_Float16>(as.w - float(h[3]))};
+            if (j >= nvec) l = half4{0, 0, 0, 0};
+            *reinterpret_cast<half4 *>(sm_q_lo + j * kQStride + c4) = l;
+        }
     }
     __shared__ uint32_t sm_new_not_finite[WAVES];
     if (owns_new) {
@@ -772,17 +800,17 @@ __device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const 
            same keys, so that every other block runs code that knows nothing of it. */        \
         if constexpr (NQ > 2) { /* (no room for two copies beside 128 accumulators; the one copy  \
            costs the 7-row verify block 3 %: 23.7 -> 24.5 us per layer, same box) */             \
-            process_block<NQ, FIRST, RING, true>(st, BUF, qreg, sm_q, KB, g, jl, colpos,         \
+            process_block<NQ, FIRST, RING, true, QLO>(st, BUF, qreg, sm_q, sm_q_lo, KB, g, jl, colpos, \
                                  collo, min(item.pos0, item.kv_len - 1), item.kv_len, lo_min,    \
                                  lo_max, softcap, inv_cap, span);                                \
         } else if (WAVES != 8 && item.rows > 1 &&                                                \
             (((KB) + 1) * kBlockKeys > min(item.pos0, item.kv_len - 1) + 1 ||                    \
              (RING && (KB) * kBlockKeys < lo_max)))                                              \
-            process_block<NQ, FIRST, RING, WAVES != 8>(st, BUF, qreg, sm_q, KB, g, jl, colpos,   \
+            process_block<NQ, FIRST, RING, WAVES != 8, QLO>(st, BUF, qreg, sm_q, sm_q_lo, KB, g, jl, colpos, \
                                  collo, min(item.pos0, item.kv_len - 1), item.kv_len, lo_min,    \
                                  lo_max, softcap, inv_cap, span);                                \
         else                                                                                     \
-            process_block<NQ, FIRST, RING, false>(st, BUF, qreg, sm_q, KB, g, jl, colpos, collo, \
+            process_block<NQ, FIRST, RING, false, QLO>(st, BUF, qreg, sm_q, sm_q_lo, KB, g, jl, colpos, collo, \
                                  min(item.pos0, item.kv_len - 1), item.kv_len, lo_min, lo_max,   \
                                  softcap, inv_cap, span);                                        \
     } while (0)
@@ -823,6 +851,7 @@ __device__ __forceinline__ void attn_splitk_f16_body(const AttnParams &p, const 
 
     // ---- merge the wavefronts through LDS ------------------------------------------------
     ITAK_MARK(6)
+    if constexpr (QLO && NQ > 2) __syncthreads();  // everybody is done with the low halves in sm_o
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
         const float l = column_sum(st.l[qt]);
@@ -949,6 +978,19 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_prep_kernel(AttnPa
                                                                           uint32_t total_partials,
                                                                           FoldedParams f) {
     attn_splitk_f16_body<NQ, WAVES, N, RING, true, false>(p, b, total_partials, f, DieMap{});
+}
+// The same with the queries as two halves (ITAK_POOL_Q_TWO_HALVES).
+template <int NQ, int WAVES, int N, bool RING>
+__global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_qlo_kernel(AttnParams p, AttnBatchT<N> b,
+                                                                         uint32_t total_partials) {
+    attn_splitk_f16_body<NQ, WAVES, N, RING, false, false, true>(p, b, total_partials, FoldedParams{}, DieMap{});
+}
+template <int NQ, int WAVES, int N, bool RING>
+__global__ __launch_bounds__(WAVES * 64) void attn_splitk_f16_qlo_prep_kernel(AttnParams p,
+                                                                              AttnBatchT<N> b,
+                                                                              uint32_t total_partials,
+                                                                              FoldedParams f) {
+    attn_splitk_f16_body<NQ, WAVES, N, RING, true, false, true>(p, b, total_partials, f, DieMap{});
 }
 // The variants that merge each unit's splits on the unit's compute die.
 template <int NQ, int WAVES, int N, bool RING>

@@ -383,9 +383,15 @@ hipError_t launch_fill_words(unsigned long long *dst, uint64_t count, unsigned l
 constexpr unsigned long long kExchangeEmptyWord = 0xffffffffffffffffull;
 // `folded` with prep_on set selects the variants that prepare Q and the new K rows themselves
 // and gate what they write (every item must then be a 16-vector step); otherwise it is ignored.
+// `q_two_halves`: the queries enter the score products as f16 hi + f16 lo (two products per
+// score tile), so that their rounding to f16 leaves the scores (ITAK_POOL_Q_TWO_HALVES).
 hipError_t launch_attn_splitk_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                   uint32_t max_rows, hipStream_t stream,
-                                  const FoldedParams *folded = nullptr);
+                                  const FoldedParams *folded = nullptr, bool q_two_halves = false);
+// The two-halves instantiations (attn_splitk_f16_qlo.hip) and the variant a batch takes.
+hipError_t launch_attn_splitk_f16_qlo(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                                      hipStream_t stream, const FoldedParams *folded);
+int attn_splitk_f16_variant(const PoolGeom &g, const AttnBatch &b, uint32_t group);
 // ---- the split merge on a unit's compute die (attn_splitk_f16_die.hip) ---------------------
 // The device's workgroups are dealt round-robin over its eight compute dies, each with an L2 of
 // its own. A launch planned for it puts every split of a unit = (item, KV head, part of the
@@ -425,7 +431,7 @@ bool attn_decode_f16_takes(const AttnParams &p, const AttnBatch &b);
 // instantiations, asked of the runtime once).
 uint32_t attn_decode_f16_resident_groups();
 hipError_t launch_attn_decode_f16(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
-                                  hipStream_t stream);
+                                  hipStream_t stream, bool q_two_halves = false);
 // f32 MFMA split-K path: f32 pools (row-major planes), head_dim 128, rows*group <= 16, implied
 // query positions. Partials are in log2 domain (combine with base2 = 1).
 bool attn_splitk_f32_supports(const PoolGeom &g, uint32_t group, uint32_t max_rows);

@@ -150,6 +150,7 @@ struct itak_pool {
     // workgroups that found themselves on another die than planned.
     bool die_merge = false;
     uint32_t *die_words = nullptr;
+    bool q_two_halves = false;  // ITAK_POOL_Q_TWO_HALVES
     // Per slot: the side buffer of a deep checkpoint's ring rows, kept for the next one
     // (cache.rs:620-625: allocated once per cache, not once per round).
     std::vector<void *> ring_saved;
@@ -587,7 +588,7 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         AttnBatch bd{};
         DieMap dm{};
         uint32_t die_partials = 0;
-        if (mfma && pool->die_merge && !exchange_words) {
+        if (mfma && pool->die_merge && !exchange_words && !pool->q_two_halves) {
             AttnParams probe{};
             probe.g = geom;
             probe.group = group;
@@ -675,7 +676,7 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         } else if (mfma) {
             HIP_TRY(pool,
                     launch_attn_splitk_f16(p, b, partials, max_rows, pool->stream,
-                                           prepares ? folded : nullptr),
+                                           prepares ? folded : nullptr, pool->q_two_halves),
                     "launch split-K attention");
         } else if (prefill) {
             HIP_TRY(pool, launch_attn_prefill_f16(p, b, partials, pool->stream),
@@ -1142,6 +1143,7 @@ itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out) {
     pool->ring_saved.assign(config->max_slots, nullptr);
     pool->ring_saved_bytes.assign(config->max_slots, 0);
     pool->merge_in_launch = (config->flags & ITAK_POOL_MERGE_IN_LAUNCH) != 0;
+    pool->q_two_halves = pool->elem_f16 && (config->flags & ITAK_POOL_Q_TWO_HALVES) != 0;
     if (pool->elem_f16 && !pool->merge_in_launch && (config->flags & ITAK_POOL_DIE_MERGE) &&
         die_layout_ok(config->device)) {
         he = hipMalloc(reinterpret_cast<void **>(&pool->die_words), kDieTicketBytes + 256);

@@ -194,7 +194,8 @@ class KvPool:
     def __init__(self, pattern: Union[int, Sequence[LayerKind]], num_kv_heads: int, head_dim: int,
                  *, elem: str = "f16", max_slots: int = 1, capacity_rows: int = 4096,
                  device: int = 0, scrub_on_truncate: bool = True, ring_headroom: int = 0,
-                 merge_in_launch: bool = False, die_merge: Optional[bool] = None):
+                 merge_in_launch: bool = False, die_merge: Optional[bool] = None,
+                 q_two_halves: bool = False):
         if isinstance(pattern, int):
             pattern = [LayerKind.Global] * pattern
         self.pattern = list(pattern)
@@ -223,6 +224,8 @@ class KvPool:
             die_merge = os.environ.get("ITAK_HIP_KV_DIE_MERGE", "0") == "1"
         if die_merge:
             cfg.flags |= N.POOL_DIE_MERGE
+        if q_two_halves:
+            cfg.flags |= N.POOL_Q_TWO_HALVES
         cfg.ring_headroom = ring_headroom
         handle = C.c_void_p()
         self._h = None
