@@ -144,8 +144,9 @@ enum {
        K.hi + K.lo. Without the flag Q is rounded to f16 once, an error relative to each channel
        that grows with the scores: outputs meet the 2e-3 bar up to scaled scores of standard
        deviation 3 (see ITAK_ELEM_F16). With it the queries are good to 2^-22 and what is left is
-       the rounding of the softmax weights to f16. These kernels wait for memory, not for the
-       matrix pipe, so the second product costs nothing measurable. Longer blocks and prefill
+       the rounding of the softmax weights to f16. These kernels wait for memory more than for
+       the matrix pipe: the second product costs 1 % on a decode step or a ragged batch and 7 %
+       on a speculative block of 64 query vectors per KV head. Longer blocks and prefill
        chunks (the block kernel) are not affected by the flag. */
     ITAK_POOL_Q_TWO_HALVES = 8u
 };

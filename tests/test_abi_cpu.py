@@ -185,3 +185,44 @@ def test_rust_binding_declares_the_header_symbol_for_symbol():
     header_text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
     for name in re.findall(r"typedef\s+struct\s+(\w+)", header_text):
         assert f"pub struct {name} " in text, name
+
+
+def _rust_calls(path):
+    """(name, argument count, line) of every call of an `itak_*` function in a Rust source:
+    arguments are counted by the commas at the call's own nesting depth."""
+    import re
+    text = re.sub(r"//[^\n]*", "", open(path).read())
+    calls = []
+    for m in re.finditer(r"\b(itak_[a-z0-9_]+)\s*\(", text):
+        if re.search(r"\bfn\s+$", text[:m.start()]):
+            continue  # a declaration, not a call
+        depth, commas, i, seen = 1, 0, m.end(), False
+        while depth:
+            c = text[i]
+            depth += c in "([{"
+            depth -= c in ")]}"
+            commas += c == "," and depth == 1
+            seen = seen or (depth >= 1 and not c.isspace())
+            trailing = c == "," and depth == 1 and text[i + 1:].lstrip().startswith(")")
+            commas -= trailing
+            i += 1
+        calls.append((m.group(1), commas + 1 if seen else 0, text.count("\n", 0, m.start()) + 1))
+    return calls
+
+
+def test_the_safe_rust_layer_calls_the_header_with_the_headers_arity():
+    # The crates are source only here (no Rust toolchain): what a compiler would check of the
+    # safe layer's calls into the extern block is checked as text, so that a function renamed or
+    # given another argument in the header does not leave the wrappers behind.
+    header = _header_functions()
+    seen = set()
+    for rel in (("itak-hip-sys", "src", "safe.rs"), ("hip-compute", "src", "lib.rs"),
+                ("hip-compute", "src", "target.rs")):
+        path = os.path.join(ROOT, "crates", *rel)
+        for name, count, line in _rust_calls(path):
+            assert name in header, f"{'/'.join(rel)}:{line} calls {name}, which the header does not declare"
+            assert count == header[name], \
+                f"{'/'.join(rel)}:{line} calls {name} with {count} arguments, the header declares {header[name]}"
+            seen.add(name)
+    assert {"itak_pool_create", "itak_compute_attention", "itak_kv_truncate",
+            "itak_store_restore_prefix", "itak_store_capture_and_put"} <= seen

@@ -38,10 +38,10 @@ def call(pool, name, layer, items, q, k, v, out):
                               out.data_ptr(), Q_HEADS, C.c_float(math.nan), C.c_float(0.0))
 
 
-def twin_pools(slots, capacity, in_launch):
+def twin_pools(slots, capacity, in_launch, elem="f16"):
     pools = []
     for _ in range(2):
-        pool = P().KvPool(1, KV_HEADS, D, elem="f16", max_slots=slots, capacity_rows=capacity,
+        pool = P().KvPool(1, KV_HEADS, D, elem=elem, max_slots=slots, capacity_rows=capacity,
                           merge_in_launch=in_launch)
         pool.set_stream(torch.cuda.current_stream().cuda_stream)
         pools.append((pool, [pool.acquire() for _ in range(slots)]))
@@ -148,14 +148,11 @@ def test_a_step_beyond_the_static_workspace_is_refused_before_anything_changes()
     pool2.close()
 
 
-@pytest.mark.parametrize("in_launch", [False, True])
-def test_the_call_is_captured_into_a_graph_on_its_first_use_and_replays(in_launch):
-    # The callers the entry point is for: its very first call on a pool is made under stream
-    # capture (nothing before it has sized a workspace), the graph is replayed with new inputs
-    # in the captured buffers, and every replay equals the eager call of the allocating entry
-    # point on a twin pool, bit for bit.
-    pools = twin_pools(2, 2200, in_launch)
-    contexts, rows = [2048, 700], 3
+def captured_on_first_use(pools, contexts, rows):
+    """The callers the entry point is for: its very first call on a pool is made under stream
+    capture (nothing before it has sized a workspace), the graph is replayed with new inputs
+    in the captured buffers, and every replay equals the eager call of the allocating entry
+    point on a twin pool, bit for bit."""
     rng = np.random.default_rng(8)
     stream = torch.cuda.current_stream()
     for pool, caches in pools:
@@ -163,9 +160,9 @@ def test_the_call_is_captured_into_a_graph_on_its_first_use_and_replays(in_launc
             kd = dev(normal(np.random.default_rng(100 + s), n, ROW))
             pool.append_device(0, [(caches[s], n)], kd.data_ptr(), kd.data_ptr())
             pool.synchronize()
-    inputs = [tuple(normal(rng, 2 * rows, w) for w in (Q_HEADS * D, ROW, ROW)) for _ in range(2)]
+    inputs = [tuple(normal(rng, len(contexts) * rows, w) for w in (Q_HEADS * D, ROW, ROW)) for _ in range(2)]
     q, k, v = (dev(x) for x in inputs[0])
-    out = torch.full((2 * rows, Q_HEADS * D), float("nan"), device="cuda")
+    out = torch.full((len(contexts) * rows, Q_HEADS * D), float("nan"), device="cuda")
     (eager_pool, eager_caches), (pool, caches) = pools
     items = [(c, rows) for c in caches]
 
@@ -198,6 +195,19 @@ def test_the_call_is_captured_into_a_graph_on_its_first_use_and_replays(in_launc
         assert torch.equal(out, want), replay
     for p, _ in pools:
         p.close()
+
+
+@pytest.mark.parametrize("in_launch", [False, True])
+def test_the_call_is_captured_into_a_graph_on_its_first_use_and_replays(in_launch):
+    captured_on_first_use(twin_pools(2, 2200, in_launch), [2048, 700], 3)
+
+
+@pytest.mark.parametrize("elem,rows", [("f16", 16), ("f32", 1), ("f32", 3)])
+def test_the_other_kernels_workspaces_are_captured_on_first_use_too(elem, rows):
+    # A 16-row block goes to the block kernel with its context split (partials and a merge of
+    # their own), an f32 pool to the f32 kernel: each sizes its workspace by its own plan, and
+    # each must find the static array bound when the first call is the captured one.
+    captured_on_first_use(twin_pools(2, 2200, False, elem), [2048, 700], rows)
 
 
 def test_two_pools_on_two_streams_take_the_static_workspace_in_turn():
