@@ -46,11 +46,11 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # known size: (bytes, the summary under profiles/ that holds the run and the scaling factors).
 # They are not measured by this run: `traffic_source` says where each came from.
 PROFILE_TRAFFIC = {
-    ("decode", "f16"): (9_800_561, "profiles/attn_decode_f16_ctx4096_traffic.md"),
-    ("ragged", "f16"): (216_790_832, "profiles/attn_splitk_f16_ragged16_traffic.md"),
-    ("prefill", "f16"): (201_442_358, "profiles/attn_prefill_f16_chunk2048_prefix30720_traffic.md"),
-    ("verify", "f16"): (87_356_285, "profiles/attn_splitk_f16_verify_traffic.md"),
-    ("decode", "f32"): (18_238_750, "profiles/attn_splitk_f32_decode_ctx4096_traffic.md"),
+    ("decode", "f16"): (9_805_775, "profiles/attn_decode_f16_ctx4096_traffic.md"),
+    ("ragged", "f16"): (216_797_776, "profiles/attn_splitk_f16_ragged16_traffic.md"),
+    ("prefill", "f16"): (201_442_441, "profiles/attn_prefill_f16_chunk2048_prefix30720_traffic.md"),
+    ("verify", "f16"): (87_437_369, "profiles/attn_splitk_f16_verify_traffic.md"),
+    ("decode", "f32"): (18_240_825, "profiles/attn_splitk_f32_decode_ctx4096_traffic.md"),
 }
 
 
