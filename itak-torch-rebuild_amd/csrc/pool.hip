@@ -885,12 +885,39 @@ PtrKind classify(const void *p, const void **usable) {
     return PtrKind::PlainHost;
 }
 
+// The same for the many sources of one restore: a snapshot's layers usually lie in one or two
+// device allocations, and the runtime's lookup costs microseconds a pointer (two lookups a
+// layer and side were more host time than the gather of a 48-layer prefix takes the device).
+// The extent of the last device allocation seen answers for every pointer inside it.
+struct PtrClassifier {
+    uintptr_t lo = 0, hi = 0;  // a device allocation already looked up
+    PtrKind operator()(const void *p, const void **usable) {
+        const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+        if (a >= lo && a < hi) {
+            *usable = p;
+            return PtrKind::Device;
+        }
+        const PtrKind kind = classify(p, usable);
+        if (kind == PtrKind::Device) {
+            hipDeviceptr_t base = nullptr;
+            size_t size = 0;
+            if (hipMemGetAddressRange(&base, &size, const_cast<void *>(p)) == hipSuccess && size) {
+                lo = reinterpret_cast<uintptr_t>(base);
+                hi = lo + size;
+            } else {
+                (void)hipGetLastError();
+            }
+        }
+        return kind;
+    }
+};
+
 // Rows the gather kernel cannot read where they lie: ordinary host memory, or a source that
 // is not aligned to its element size (the payload of an encoded snapshot starts wherever
 // its fingerprint ends).
-bool must_stage(const void *p, uint64_t elem_bytes) {
+bool must_stage(PtrClassifier &kind_of, const void *p, uint64_t elem_bytes) {
     const void *usable;
-    return classify(p, &usable) == PtrKind::PlainHost ||
+    return kind_of(p, &usable) == PtrKind::PlainHost ||
            reinterpret_cast<uintptr_t>(p) % elem_bytes != 0;
 }
 
@@ -1418,11 +1445,12 @@ static itak_status restore_layers(itak_pool *pool, uint32_t slot, Slot &s,
     const uint64_t src_bytes_per_elem = src_elem == ITAK_ELEM_F16 ? 2 : 4;
     // Sources the device cannot read in place are staged through one temporary buffer.
     uint64_t stage_need = 0;
+    PtrClassifier kind_of;
     for (uint64_t i = 0; i < count; ++i) {
         if (layers[i].rows == 0) continue;
         const uint64_t bytes = layers[i].rows * pool->row * src_bytes_per_elem;
-        if (must_stage(layers[i].keys, src_bytes_per_elem)) stage_need += align_up(bytes, 256);
-        if (must_stage(layers[i].values, src_bytes_per_elem)) stage_need += align_up(bytes, 256);
+        if (must_stage(kind_of, layers[i].keys, src_bytes_per_elem)) stage_need += align_up(bytes, 256);
+        if (must_stage(kind_of, layers[i].values, src_bytes_per_elem)) stage_need += align_up(bytes, 256);
     }
     unsigned char *temp = nullptr;
     if (stage_need) HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&temp), stage_need), "allocate restore staging");
@@ -1468,8 +1496,8 @@ static itak_status restore_layers(itak_pool *pool, uint32_t slot, Slot &s,
         const void *src[2] = {L.keys, L.values};
         for (int side = 0; side < 2; ++side) {
             const void *usable;
-            if (!must_stage(src[side], src_bytes_per_elem)) {
-                classify(src[side], &usable);
+            if (!must_stage(kind_of, src[side], src_bytes_per_elem)) {
+                kind_of(src[side], &usable);
                 src[side] = usable;
                 continue;
             }

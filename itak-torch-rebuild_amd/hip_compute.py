@@ -431,12 +431,19 @@ class KvCache:
             self._h, self.slot, layer, first_position, keys_ptr, elems, values_ptr, elems,
             N.ELEM_F16 if src_f16 else N.ELEM_F32))
 
-    def restore_snapshot_ptrs(self, token_count: int, layers: Sequence[Tuple[int, int, int, int]],
-                              src_f16: bool) -> None:
-        """layers: (first_position, rows, keys_ptr, values_ptr) per layer."""
+    @staticmethod
+    def snapshot_layer_table(layers: Sequence[Tuple[int, int, int, int]]):
+        """The itak_snapshot_layer array for (first_position, rows, keys_ptr, values_ptr) per
+        layer: a caller that restores the same sources again builds it once."""
         raw = (N.SnapshotLayer * len(layers))()
         for i, (first, rows, kp, vp) in enumerate(layers):
             raw[i].first_position, raw[i].rows, raw[i].keys, raw[i].values = first, rows, kp, vp
+        return raw
+
+    def restore_snapshot_ptrs(self, token_count: int, layers, src_f16: bool) -> None:
+        """layers: (first_position, rows, keys_ptr, values_ptr) per layer, or the array
+        `snapshot_layer_table` made of them."""
+        raw = layers if isinstance(layers, C.Array) else self.snapshot_layer_table(layers)
         _check(self._h, self._lib.itak_kv_restore_snapshot(
             self._h, self.slot, token_count, raw, len(layers),
             N.ELEM_F16 if src_f16 else N.ELEM_F32), "restore_snapshot")
