@@ -68,6 +68,11 @@ void for_each_index(uint64_t count, F f) {
 // sums itself.
 uint64_t fnv1a64_blocks(const uint8_t *bytes, uint64_t count);
 uint64_t fnv1a64_of_sums(const uint64_t *sums, uint64_t blocks);
+// Block sums of blocks [first, first + n) of `count` bytes, n <= kItkvSumGroup, into sums[first..].
+// A sum is a chain of one multiply per byte, each waiting for the last: one thread walks up to
+// four blocks side by side, four chains in the multiplier at once (0.7 -> 2.7 GB/s a thread).
+constexpr uint64_t kItkvSumGroup = 4;
+void fnv1a64_block_group(const uint8_t *bytes, uint64_t count, uint64_t first, uint64_t n, uint64_t *sums);
 // The trailer a snapshot of `version` carries for the `count` bytes before it.
 inline uint64_t itkv_trailer(uint32_t version, const uint8_t *bytes, uint64_t count) {
     return version == kItkvVersionTyped ? fnv1a64_blocks(bytes, count) : fnv1a64(bytes, count, kFnvOffset);

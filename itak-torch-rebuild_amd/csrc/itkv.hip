@@ -57,12 +57,42 @@ uint64_t fnv1a64_of_sums(const uint64_t *sums, uint64_t blocks) {
     return hash;
 }
 
+void fnv1a64_block_group(const uint8_t *bytes, uint64_t count, uint64_t first, uint64_t n, uint64_t *sums) {
+    const uint8_t *p[kItkvSumGroup];
+    uint64_t len[kItkvSumGroup], h[kItkvSumGroup];
+    uint64_t common = kItkvSumBlock;
+    for (uint64_t j = 0; j < kItkvSumGroup; ++j) {
+        const uint64_t k = first + std::min(j, n - 1);  // short groups walk their last block again
+        const uint64_t at = k * kItkvSumBlock;
+        p[j] = bytes + at;
+        len[j] = std::min(kItkvSumBlock, count - at);
+        h[j] = kFnvOffset;
+        common = std::min(common, len[j]);
+    }
+    uint64_t a = h[0], b = h[1], c = h[2], d = h[3];
+    const uint8_t *pa = p[0], *pb = p[1], *pc = p[2], *pd = p[3];
+    for (uint64_t i = 0; i < common; ++i) {
+        a ^= pa[i];
+        b ^= pb[i];
+        c ^= pc[i];
+        d ^= pd[i];
+        a *= kFnvPrime;
+        b *= kFnvPrime;
+        c *= kFnvPrime;
+        d *= kFnvPrime;
+    }
+    h[0] = a, h[1] = b, h[2] = c, h[3] = d;
+    for (uint64_t j = 0; j < n; ++j)  // only the snapshot's last block can be longer than the others are short
+        sums[first + j] = len[j] > common ? fnv1a64(p[j] + common, len[j] - common, h[j]) : h[j];
+}
+
 uint64_t fnv1a64_blocks(const uint8_t *bytes, uint64_t count) {
     const uint64_t blocks = count / kItkvSumBlock + (count % kItkvSumBlock ? 1 : 0);
     std::vector<uint64_t> sums(blocks);
-    for_each_index(blocks, [&](uint64_t k) {
-        const uint64_t at = k * kItkvSumBlock;
-        sums[k] = fnv1a64(bytes + at, std::min(kItkvSumBlock, count - at), kFnvOffset);
+    const uint64_t groups = (blocks + kItkvSumGroup - 1) / kItkvSumGroup;
+    for_each_index(groups, [&](uint64_t g) {
+        const uint64_t first = g * kItkvSumGroup;
+        fnv1a64_block_group(bytes, count, first, std::min(kItkvSumGroup, blocks - first), sums.data());
     });
     return fnv1a64_of_sums(sums.data(), blocks);
 }

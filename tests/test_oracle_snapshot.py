@@ -313,7 +313,8 @@ def test_block_checksum_is_the_sum_of_block_sums_at_every_boundary():
     rng = np.random.default_rng(2)
     B = okv.SUM_BLOCK
     assert P.checksum_blocks(b"") == okv.FNV_OFFSET == okv.block_checksum(b"")
-    for size in (1, 77, B - 1, B, B + 1, 2 * B, 3 * B + 5):
+    # (The library walks blocks in groups of four: sizes on both sides of a group's edge too.)
+    for size in (1, 77, B - 1, B, B + 1, 2 * B, 3 * B + 5, 4 * B, 4 * B + 1, 5 * B + 17, 8 * B - 3, 9 * B):
         data = rng.integers(0, 256, size=size, dtype=np.uint8).tobytes()
         want = okv.block_checksum(data, _fast_sum)
         assert P.checksum_blocks(data) == want, size
