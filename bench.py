@@ -274,6 +274,8 @@ def timeline(args, pkg, torch, np):
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     stream = torch.cuda.current_stream()
+    if args.workload in ("verify", "ragged"):
+        return timeline_splitk(args, pkg, torch, np, raw, dev, stream)
     layers, ctx = 48, 4096
     pool = pkg.KvPool(layers, KV_HEADS, D, elem="f16", max_slots=1, capacity_rows=ctx + 8,
                       scrub_on_truncate=False, merge_in_launch=args.merge_in_launch)
@@ -349,6 +351,87 @@ def timeline(args, pkg, torch, np):
             (2, "every load issued"), (7, "sums done (partials arrived)"),
             (8, "split lanes joined"), (9, "output issued"),
             (11, "everything in flight done (stores acknowledged)")])
+    pool.close()
+
+
+def timeline_splitk(args, pkg, torch, np, raw, dev, stream):
+    """The same for the split-K kernel on the verify block or the ragged batch (--workload),
+    merge launch or die form (--die-merge): stage times of every wavefront over ten replays,
+    and the last replay's stages by compute die (workgroup index mod 8)."""
+    import ctypes as C
+
+    die = bool(getattr(args, "die_merge", False))
+    if args.workload == "ragged":
+        layers, slots, rows = 4, 16, 1
+        lengths = np.random.default_rng(3).integers(256, 16384, size=slots, endpoint=True).tolist()
+    else:
+        layers, slots, rows, lengths = 4, 4, 7, [8192] * 4
+    pool = pkg.KvPool(layers, KV_HEADS, D, elem="f16", max_slots=slots, capacity_rows=max(lengths) + 16,
+                      scrub_on_truncate=False, die_merge=die)
+    pool.set_stream(stream.cuda_stream)
+    caches = [pool.acquire() for _ in range(slots)]
+    torch.manual_seed(0)
+    for layer in range(layers):
+        for s_, n in enumerate(lengths):
+            k, v = torch.randn(n, ROW, device=dev), torch.randn(n, ROW, device=dev)
+            pool.append_device(layer, [(caches[s_], n)], k.data_ptr(), v.data_ptr())
+            torch.cuda.synchronize()
+    total = slots * rows
+    q = torch.randn(layers, total, Q_HEADS * D, device=dev)
+    kn, vn = torch.randn(layers, total, ROW, device=dev), torch.randn(layers, total, ROW, device=dev)
+    out = torch.empty_like(q)
+    items = [(c, rows) for c in caches]
+
+    def step():
+        for layer in range(layers):
+            pool.attention_step_device(layer, items, q[layer].data_ptr(), kn[layer].data_ptr(),
+                                       vn[layer].data_ptr(), out[layer].data_ptr(), Q_HEADS)
+        pool.truncate(caches, lengths)
+
+    for _ in range(3):
+        step()
+    form = merge_form_of(pkg, pool, step)
+    pool.truncate(caches, lengths)
+    graph = capture(torch, pool, stream, step)
+    marks, waves = 12, 8192
+    buf = np.zeros(waves * marks, dtype=np.uint64)
+    reader = "itak_timeline_read_splitk_die" if form == "on_die" else "itak_timeline_read_splitk"
+    replays, groups = [], None
+    for _ in range(10):
+        graph.replay()
+        torch.cuda.synchronize()
+        rc = getattr(raw, reader)(buf.ctypes.data_as(C.c_void_p), C.c_ulonglong(buf.size))
+        assert rc == 0, f"{reader} failed with HIP error {rc}"
+        t = buf.reshape(waves, marks).astype(np.int64)
+        if form != "on_die":
+            t = t[:waves // 2]  # the second half holds the merge launch's records
+        keep = t[:, 0] > 0
+        groups = (np.arange(t.shape[0]) // 8)[keep]
+        t = t[keep]
+        replays.append((t - t[:, 0].min()) * 10)
+    step_s = Timer(torch, stream)(graph.replay, 50)[0] / 50
+    print(f"split-K timeline, {args.workload} (the last of {layers} layers in a HIP graph), split partials "
+          f"merged by: {form}; {step_s / layers * 1e6:.2f} us per layer with the timestamps compiled in; "
+          f"{replays[0].shape[0]} wavefronts per launch; ns from the launch's first instruction")
+    allr = np.concatenate(replays)
+    names = ["first instruction", "kernel arguments in, addresses known", "first block's loads issued",
+             "mask and epilogue bookkeeping done", "Q^T (and new rows) staged in LDS", "query operands in registers (past the barrier)",
+             "the wavefront's blocks done", "O^T written to LDS", "past the workgroup barrier",
+             "partials issued", "arrival ticket drawn (die form)", "everything in flight done"]
+    for i, name in enumerate(names):
+        col = allr[:, i]
+        col = col[col > 0] if i else col
+        if len(col):
+            print(f"  {name:42s} min {col.min():6d}  p50 {int(np.median(col)):6d}  "
+                  f"p90 {int(np.percentile(col, 90)):6d}  max {col.max():6d}")
+    last, die_of = replays[-1], groups % 8
+    print("  by compute die (workgroup index mod 8), last replay: loads issued p50 / blocks done p50 / "
+          "blocks done max / all done max")
+    for d in range(8):
+        r = last[die_of == d]
+        if len(r):
+            print(f"    die {d}: {int(np.median(r[:, 2])):6d} {int(np.median(r[:, 6])):6d} "
+                  f"{r[:, 6].max():6d} {r[:, 11].max():6d}")
     pool.close()
 
 
@@ -428,7 +511,8 @@ def main():
     ap.add_argument("--timeline", action="store_true",
                     help="print where a decode layer's time goes: stage timestamps from the "
                          "measurement build of the library (python itak-torch-rebuild_amd/build.py "
-                         "--timeline), a table instead of the JSON line")
+                         "--timeline), a table instead of the JSON line; with --workload verify or "
+                         "ragged the split-K kernel's stages, by compute die too")
     ap.add_argument("--only", action="store_true",
                     help="measure the named workload alone (the default decode run otherwise "
                          "adds short runs of the other configurations under 'workloads')")
