@@ -357,6 +357,43 @@ def test_f16_snapshot_restores_raw_and_pinned_host_sources_are_read_in_place():
     assert e.value.variant == "Unsupported"
 
 
+def test_a_snapshot_whose_layers_lie_in_different_allocations_of_different_kinds():
+    # The library asks the runtime what kind of memory a source is once per device allocation
+    # and answers the rest from that allocation's extent: sources in two device allocations
+    # (one of them large enough to hold several layers), in pinned host memory and in ordinary
+    # host memory, mixed within one snapshot and given as a prebuilt layer table, each land
+    # where a snapshot from one place lands.
+    import torch
+
+    rng = np.random.default_rng(21)
+    kv_heads, head_dim, tokens, layers = 2, 128, 70, 6
+    width = kv_heads * head_dim
+    k32, v32 = normal(rng, layers, tokens, width), normal(rng, layers, tokens, width)
+    want_k, want_v = oracle.f32_to_f16_array(k32), oracle.f32_to_f16_array(v32)
+    big = torch.from_numpy(np.concatenate([k32[:3], v32[:3]])).cuda()          # layers 0-2, K then V
+    other = torch.from_numpy(k32[3:5]).cuda()                                    # K of layers 3, 4
+    pinned = torch.from_numpy(v32[3:5]).pin_memory()                             # V of layers 3, 4
+    plain_k, plain_v = np.ascontiguousarray(k32[5]), np.ascontiguousarray(v32[5])  # layer 5: staged
+    table = []
+    for l in range(layers):
+        if l < 3:
+            table.append((0, tokens, big[l].data_ptr(), big[3 + l].data_ptr()))
+        elif l < 5:
+            table.append((0, tokens, other[l - 3].data_ptr(), pinned[l - 3].data_ptr()))
+        else:
+            table.append((0, tokens, plain_k.ctypes.data, plain_v.ctypes.data))
+    pool = P().KvPool(layers, kv_heads, head_dim, elem="f16", max_slots=2, capacity_rows=96)
+    a, b = pool.acquire(), pool.acquire()
+    a.restore_snapshot_ptrs(tokens, P().KvCache.snapshot_layer_table(table), src_f16=False)
+    b.restore_snapshot_ptrs(tokens, table, src_f16=False)
+    for cache in (a, b):
+        for l in range(layers):
+            assert cache.next_position(l) == tokens
+            _, gk, gv = cache.view(l).rows()
+            assert np.array_equal(gk.reshape(tokens, -1), want_k[l]), l
+            assert np.array_equal(gv.reshape(tokens, -1), want_v[l]), l
+
+
 def test_batched_truncate_then_reappend_is_bitwise_never_appended():
     import torch
 
