@@ -133,7 +133,8 @@ enum {
        of that die's L2: no merge launch and no wait inside the launch. Other steps keep the
        merge launch. Pool creation probes that the device deals workgroup i to die i % 8 and
        ignores the flag if it does not; every such launch checks again, and
-       itak_pool_synchronize reports ITAK_STEP_FAILED if a workgroup ran elsewhere. Results
+       itak_pool_synchronize reports ITAK_STEP_FAILED if a workgroup ran elsewhere (seen
+       rarely, on small launches between other work; the pool then keeps the merge launch). Results
        agree with the merge launch's to the rounding of another split plan. On an MI355X it is
        2 to 4 % faster than the merge launch on batches of a hundred MB of KV per layer and more,
        level or slower below (the launch's own tail and a slower start cost what the second
