@@ -195,7 +195,7 @@ class KvPool:
                  *, elem: str = "f16", max_slots: int = 1, capacity_rows: int = 4096,
                  device: int = 0, scrub_on_truncate: bool = True, ring_headroom: int = 0,
                  merge_in_launch: bool = False, die_merge: Optional[bool] = None,
-                 q_two_halves: bool = False):
+                 q_two_halves: Optional[bool] = None):
         if isinstance(pattern, int):
             pattern = [LayerKind.Global] * pattern
         self.pattern = list(pattern)
@@ -224,6 +224,9 @@ class KvPool:
             die_merge = os.environ.get("ITAK_HIP_KV_DIE_MERGE", "0") == "1"
         if die_merge:
             cfg.flags |= N.POOL_DIE_MERGE
+        # The same for the queries as two halves: ITAK_HIP_KV_Q_TWO_HALVES=1.
+        if q_two_halves is None:
+            q_two_halves = os.environ.get("ITAK_HIP_KV_Q_TWO_HALVES", "0") == "1"
         if q_two_halves:
             cfg.flags |= N.POOL_Q_TWO_HALVES
         cfg.ring_headroom = ring_headroom

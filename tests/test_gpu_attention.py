@@ -549,6 +549,7 @@ def _worst_error_at_scale(rows, q_scale, k_scale, ctx, slots=1, **pool_args):
     worst = 0.0
     for seed in range(2):
         rng = np.random.default_rng(1000 + seed)
+        pool_args.setdefault("q_two_halves", False)  # whatever the environment's default says
         pool = P().KvPool(1, 4, 128, elem="f16", max_slots=slots, capacity_rows=ctx + rows, **pool_args)
         pool.set_stream(torch.cuda.current_stream().cuda_stream)
         caches = [pool.acquire() for _ in range(slots)]

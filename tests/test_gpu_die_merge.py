@@ -58,7 +58,8 @@ class Twin:
     def __init__(self, kinds, kv_heads, slots, capacity, lengths, rng, ring_headroom=0):
         self.kv_heads, self.width = kv_heads, kv_heads * D
         self.pools = [P().KvPool(kinds, kv_heads, D, elem="f16", max_slots=slots,
-                                 capacity_rows=capacity, die_merge=form, ring_headroom=ring_headroom)
+                                 capacity_rows=capacity, die_merge=form, ring_headroom=ring_headroom,
+                                 q_two_halves=False)  # (the two forms exclude each other)
                       for form in (True, False)]
         self.caches = []
         self.k0 = [normal(rng, int(n), self.width) for n in lengths]
