@@ -122,6 +122,13 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     constexpr int kFuseRows = fuse_rows(D);
     constexpr int kFusePieces = (kFuseRows + kRowsPerPass - 1) / kRowsPerPass;  // per thread
     constexpr int kVecPerWave = kTiles * 16;
+    // The row-by-row product for values that are not finite is compiled into every form but two.
+    // The one-tile form at head_dim 128, which also converts and stages a step's own rows, holds
+    // all 256 registers, and with the product in it the compiler keeps three to seven values of
+    // the product's own loop in scratch memory (the two-tile form stands at 190 to 210
+    // registers without it). At head_dim 96 the product's presence made a 512-row chunk 10 %
+    // slower (65 -> 71 us per layer), the other head dims 1 %.
+    constexpr bool kByRow = D == 128 ? kTiles == 2 : D != 96;
     constexpr int kVecPerGroup = kWaves * kVecPerWave;  // query vectors per workgroup
     extern __shared__ __attribute__((aligned(16))) uint16_t lds_ring[];  // [kStages][K block | V block]
 
@@ -180,6 +187,7 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
         min((min(item.pos0 + wg_row_end, item.kv_len) + kBlockKeys - 1) / kBlockKeys,
             kb_begin + blocks_per_split);
     const uint32_t wave_row_end = min(item.rows, row_begin + rows_per_wave);
+    [[maybe_unused]] const uint32_t wave_rows = wave_row_end - min(wave_row_end, row_begin);
     const uint32_t wave_blocks =
         row_begin < item.rows
             ? (min(item.pos0 + wave_row_end, item.kv_len) + kBlockKeys - 1) / kBlockKeys
@@ -523,6 +531,11 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
                     for (int e = 0; e < 8; ++e)
                         x[qt][e >> 2][e & 3] = softcap_of_exp2_arg(x[qt][e >> 2][e & 3], cap2, ref[qt]);
             }
+            // A block at an edge of the mask whose values are not all finite: the wavefront's rows
+            // share the value operand, and a masked key's zero weight times such a value is NaN,
+            // where gqa_attention never reads the value row of a key a query does not see
+            // (crates/attention/src/attention.rs:160-173). P.V is then taken row by row (below).
+            [[maybe_unused]] bool by_row = false;
             if (RING && kb < low_masked_end) {
 #pragma unroll
                 for (int qt = 0; qt < kTiles; ++qt)
@@ -537,6 +550,7 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
                     for (int dt = 0; dt < kOut; ++dt)
                         va[dt] = keep_halves(va[dt], keep);
                 }
+                if constexpr (kByRow) by_row = true;
             }
             if (kb >= first_masked) {
 #pragma unroll
@@ -551,6 +565,24 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
 #pragma unroll
                     for (int dt = 0; dt < kOut; ++dt)
                         va[dt] = keep_halves(va[dt], keep);
+                }
+                if constexpr (kByRow) by_row = true;
+            }
+            if constexpr (kByRow) {
+                if (by_row && wave_rows > 1) {
+                    // Is any value of the block not finite? Asked of the matrix pipe: the values
+                    // times a zero operand sum to zero unless one of them is an infinity or a NaN
+                    // (eight MFMAs and a comparison, where looking at the 32 registers' exponent
+                    // fields takes a hundred vector instructions).
+                    floatx4 t = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+                    const half8 zero = half8{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                    for (int dt = 0; dt < kOut; ++dt)
+                        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[dt], zero, t, 0, 0, 0);
+                    const float any = (t[0] + t[1]) + (t[2] + t[3]);
+                    by_row = __builtin_amdgcn_ballot_w64(any != any) != 0;
+                } else {
+                    by_row = false;
                 }
             }
             float lmax[kTiles];
@@ -594,18 +626,54 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
             // drifting into step (measured on the 2048-row chunk: +4.5 %; the other placements
             // of the raised stretch tried, scores only or masks and maxima only, gave +3 %).
             __builtin_amdgcn_s_setprio(1);
+            half8 pb[kTiles];
 #pragma unroll
             for (int qt = 0; qt < kTiles; ++qt) {
                 float pe[8];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) pe[e] = fast_exp2(x[qt][e >> 2][e & 3]);
-                half8 pb;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) pb[e] = static_cast<_Float16>(pe[e]);
-                l[qt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pb, l[qt], 0, 0, 0);
+                for (int e = 0; e < 8; ++e) pb[qt][e] = static_cast<_Float16>(pe[e]);
+            }
+            if constexpr (kByRow) {
+                if (__builtin_expect(by_row, false)) {
+                    // Once per row of the wavefront's tile, with the columns of the keys that row
+                    // does not see cleared; a lane keeps the sum of its own column's row. The
+                    // accumulators are written in place, and the value operand is cleared
+                    // afterwards, so that the products below, which every block runs, add zeros:
+                    // one definition of the accumulators reaches the loop's end, not two that the
+                    // compiler would have to copy into one another every block.
+#pragma unroll
+                    for (int qt = 0; qt < kTiles; ++qt) {
+                        __builtin_amdgcn_sched_barrier(0);  // one tile after the other: registers
+                        const uint32_t my_row = row_begin + (uint32_t(qt) * 16 + jl) / gp;
+#pragma unroll 1
+                        for (uint32_t r = row_begin; r < wave_row_end; ++r) {
+                            const uint32_t pos = min(item.pos0 + r, item.kv_len - 1);
+                            const uint32_t lo = RING ? lowest_visible(item.pos0 + r, window, kv_lo) : 0u;
+                            const uint32_t end = min(pos + 1 - min(pos + 1, key_base), 8u);
+                            u32x4 keep = first_halves(end);
+                            if constexpr (RING) keep &= ~first_halves(min(lo - min(lo, key_base), 8u));
+                            const bool mine = my_row == r;
+#pragma unroll
+                            for (int dt = 0; dt < kOut; ++dt) {
+                                const floatx4 sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                    keep_halves(va[dt], keep), pb[qt], o[qt][dt], 0, 0, 0);
+                                if (mine) o[qt][dt] = sum;
+                                __builtin_amdgcn_sched_barrier(0);
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int dt = 0; dt < kOut; ++dt) va[dt] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+                }
+            }
+#pragma unroll
+            for (int qt = 0; qt < kTiles; ++qt) {
+                l[qt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pb[qt], l[qt], 0, 0, 0);
 #pragma unroll
                 for (int dt = 0; dt < kOut; ++dt)
-                    o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[dt], pb, o[qt][dt], 0, 0, 0);
+                    o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[dt], pb[qt], o[qt][dt], 0, 0, 0);
             }
         }
         if (kb == kb_begin) { ITAK_MARK(4) }
@@ -619,10 +687,14 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     const bool final_out = item.splits == 1;
     float *const ws_acc = p.ws;
     float *const ws_ml = p.ws + uint64_t(total_partials) * kD;
+    // (The column's row and head are worked out again here, from a lane number the compiler
+    // cannot tie to the prologue's: kept from there they would hold registers across the loop.)
+    uint32_t jl_again = jl;
+    asm volatile("" : "+v"(jl_again));
 #pragma unroll
     for (int qt = 0; qt < kTiles; ++qt) {
         const float lt = l[qt][0];
-        const uint32_t j = qt * 16 + jl;
+        const uint32_t j = qt * 16 + jl_again;
         const uint32_t row = row_begin + j / gp, hq = j % gp, head = kv_head * group + hq;
         if (row >= item.rows || hq >= group) continue;
         if (final_out) {
