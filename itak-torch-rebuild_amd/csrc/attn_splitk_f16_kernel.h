@@ -315,7 +315,12 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
                 }
                 accumulate_by_row<RING>(st.o[qt], b, pbs[qt], qt, key_base, jl, kv_len, span);
             }
-            return;
+            if constexpr (FIRST) return;
+            // Later blocks fall through to the products every block runs, with the value operand
+            // cleared (they add zeros): the accumulators then have one definition at the end of
+            // the block, not two that the compiler must copy into one another.
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) b.v[dt] = half8{0, 0, 0, 0, 0, 0, 0, 0};
         }
 #pragma unroll
         for (int qt = 0; qt < NQ; ++qt)
