@@ -122,13 +122,11 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     constexpr int kFuseRows = fuse_rows(D);
     constexpr int kFusePieces = (kFuseRows + kRowsPerPass - 1) / kRowsPerPass;  // per thread
     constexpr int kVecPerWave = kTiles * 16;
-    // The row-by-row product for values that are not finite is compiled into every form but two.
-    // The one-tile form at head_dim 128, which also converts and stages a step's own rows, holds
-    // all 256 registers, and with the product in it the compiler keeps three to seven values of
-    // the product's own loop in scratch memory (the two-tile form stands at 190 to 210
-    // registers without it). At head_dim 96 the product's presence made a 512-row chunk 10 %
-    // slower (65 -> 71 us per layer), the other head dims 1 %.
-    constexpr bool kByRow = D == 128 ? kTiles == 2 : D != 96;
+    // The row-by-row product for values that are not finite is compiled into every form but
+    // those of head_dim 96: there the compiler, given the product, keeps the value operand as
+    // separate halves and puts it together again in every block (24 permutes; a 512-row chunk
+    // 65 -> 71 us per layer), the other head dims pay 0 to 2 %.
+    constexpr bool kByRow = D != 96;
     constexpr int kVecPerGroup = kWaves * kVecPerWave;  // query vectors per workgroup
     extern __shared__ __attribute__((aligned(16))) uint16_t lds_ring[];  // [kStages][K block | V block]
 
@@ -188,6 +186,7 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
             kb_begin + blocks_per_split);
     const uint32_t wave_row_end = min(item.rows, row_begin + rows_per_wave);
     [[maybe_unused]] const uint32_t wave_rows = wave_row_end - min(wave_row_end, row_begin);
+    [[maybe_unused]] const uint32_t gp_shift = __builtin_amdgcn_readfirstlane(__builtin_ctz(gp));
     const uint32_t wave_blocks =
         row_begin < item.rows
             ? (min(item.pos0 + wave_row_end, item.kv_len) + kBlockKeys - 1) / kBlockKeys
@@ -646,19 +645,38 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
 #pragma unroll
                     for (int qt = 0; qt < kTiles; ++qt) {
                         __builtin_amdgcn_sched_barrier(0);  // one tile after the other: registers
-                        const uint32_t my_row = row_begin + (uint32_t(qt) * 16 + jl) / gp;
+                        // (gp is a power of two; the shift is made here and not taken from the
+                        // prologue's division, whose result would otherwise be held through
+                        // every block for this path's sake.)
+                        uint32_t jl_here = jl;
+                        asm volatile("" : "+v"(jl_here));  // (nor moved out of the loop by the compiler)
+                        const uint32_t my_row = row_begin + ((uint32_t(qt) * 16 + jl_here) >> gp_shift);
 #pragma unroll 1
                         for (uint32_t r = row_begin; r < wave_row_end; ++r) {
                             const uint32_t pos = min(item.pos0 + r, item.kv_len - 1);
                             const uint32_t lo = RING ? lowest_visible(item.pos0 + r, window, kv_lo) : 0u;
                             const uint32_t end = min(pos + 1 - min(pos + 1, key_base), 8u);
-                            u32x4 keep = first_halves(end);
-                            if constexpr (RING) keep &= ~first_halves(min(lo - min(lo, key_base), 8u));
+                            const uint32_t first = RING ? min(lo - min(lo, key_base), 8u) : 0u;
                             const bool mine = my_row == r;
 #pragma unroll
                             for (int dt = 0; dt < kOut; ++dt) {
+                                // (The mask is made per product from the two counts: four registers
+                                // fewer to hold across the products, in a path no speed is asked of.)
+                                u32x4 keep = first_halves(end);
+                                if constexpr (RING) keep &= ~first_halves(first);
+                                asm volatile("" : "+v"(keep));
+                                // (The one-tile form, which holds all 256 registers, reads the
+                                // values from the stage again: the stage keeps them until the next
+                                // block's barrier, and the operand registers are then free for
+                                // this loop. The two-tile form has the registers, and with the
+                                // second read in it a windowed chunk ran 5 % slower.)
+                                half8 v;
+                                if constexpr (kTiles == 1)
+                                    v = *reinterpret_cast<const half8 *>(vl + dt * 64 * 8);
+                                else
+                                    v = va[dt];
                                 const floatx4 sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                    keep_halves(va[dt], keep), pb[qt], o[qt][dt], 0, 0, 0);
+                                    keep_halves(v, keep), pb[qt], o[qt][dt], 0, 0, 0);
                                 if (mine) o[qt][dt] = sum;
                                 __builtin_amdgcn_sched_barrier(0);
                             }
