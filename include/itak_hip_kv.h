@@ -100,10 +100,7 @@ enum {
    scale. ITAK_POOL_Q_TWO_HALVES lifts the limit for decode steps and blocks of up to 8 rows at
    head_dim 128 (4e-5 to 2.6e-4 observed at standard deviation 6).
    A value row that is not finite reaches the outputs of exactly the query rows that see its key
-   (the reference never reads the value row of a masked key) on f32 pools and on f16 pools, with
-   one exception: f16 pools at head_dim 96. There the rows of a step that one workgroup handles
-   (64 or 128 query vectors of a KV head) share a value operand, and those of them that do not
-   see the key come out NaN in the channels where the value is not finite.
+   (the reference never reads the value row of a masked key), on f32 pools and on f16 pools.
    Matrix-pipe kernels exist for f16 pools at head_dim 64, 96, 128 and 256 with up to 16 Q heads per
    KV head and for f32 pools at head_dim 64 and 128; every other shape (any head_dim up to 256)
    runs on a general kernel that is correct and one to two orders of magnitude slower. */

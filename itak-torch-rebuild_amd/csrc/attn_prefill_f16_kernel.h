@@ -122,11 +122,9 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     constexpr int kFuseRows = fuse_rows(D);
     constexpr int kFusePieces = (kFuseRows + kRowsPerPass - 1) / kRowsPerPass;  // per thread
     constexpr int kVecPerWave = kTiles * 16;
-    // The row-by-row product for values that are not finite is compiled into every form but
-    // those of head_dim 96: there the compiler, given the product, keeps the value operand as
-    // separate halves and puts it together again in every block (24 permutes; a 512-row chunk
-    // 65 -> 71 us per layer), the other head dims pay 0 to 2 %.
-    constexpr bool kByRow = D != 96;
+    // The row-by-row product for values that are not finite is compiled into every form (the
+    // switch is kept for measurements of what it costs: 0 to 2 %, head_dim 96 5 % on chunks).
+    constexpr bool kByRow = true;
     constexpr int kVecPerGroup = kWaves * kVecPerWave;  // query vectors per workgroup
     extern __shared__ __attribute__((aligned(16))) uint16_t lds_ring[];  // [kStages][K block | V block]
 
@@ -573,11 +571,25 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
                     // times a zero operand sum to zero unless one of them is an infinity or a NaN
                     // (eight MFMAs and a comparison, where looking at the 32 registers' exponent
                     // fields takes a hundred vector instructions).
+                    // At head_dim 96 the values are read from the stage again, here and in the
+                    // row-by-row loop below: given the operand registers in a second kind of
+                    // product and a cleared copy of them further down, the compiler keeps the
+                    // operand as separate halves there and puts it together again in every
+                    // block (24 permutes, a 512-row chunk 65 -> 71 us per layer; with the second
+                    // read 68). The stage's copy has not had the stale and unstored rows cleared:
+                    // at worst the row-by-row path is taken for a block that did not need it,
+                    // and its own masks, one row's at a time, leave those rows out as well.
                     floatx4 t = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
                     const half8 zero = half8{0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-                    for (int dt = 0; dt < kOut; ++dt)
-                        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[dt], zero, t, 0, 0, 0);
+                    for (int dt = 0; dt < kOut; ++dt) {
+                        half8 v;
+                        if constexpr (D == 96)
+                            v = *reinterpret_cast<const half8 *>(vl + dt * 64 * 8);
+                        else
+                            v = va[dt];
+                        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(v, zero, t, 0, 0, 0);
+                    }
                     const float any = (t[0] + t[1]) + (t[2] + t[3]);
                     by_row = __builtin_amdgcn_ballot_w64(any != any) != 0;
                 } else {
@@ -669,9 +681,10 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
                                 // values from the stage again: the stage keeps them until the next
                                 // block's barrier, and the operand registers are then free for
                                 // this loop. The two-tile form has the registers, and with the
-                                // second read in it a windowed chunk ran 5 % slower.)
+                                // second read in it a windowed chunk ran 5 % slower; head_dim 96
+                                // reads again in both forms, see the detection above.)
                                 half8 v;
-                                if constexpr (kTiles == 1)
+                                if constexpr (kTiles == 1 || D == 96)
                                     v = *reinterpret_cast<const half8 *>(vl + dt * 64 * 8);
                                 else
                                     v = va[dt];

@@ -8,13 +8,12 @@ sliding-window layer a ring row inside the first row's window lies outside the l
 matrix-pipe kernels multiply one shared value operand for all rows of a step, and a masked
 key's zero weight times such a value is NaN. The split-K kernels (f16 pools at head_dim 128,
 steps of up to 8 rows: decode batches and speculative blocks), the f32 kernel and the block
-kernel (longer blocks and prefill chunks; every step at head dims 64 and 256) take the
+kernel (longer blocks and prefill chunks; every step at head dims 64, 96 and 256) take the
 product row by row in the blocks where that can happen, and are compared with the oracle
 element for element: the same elements NaN, the same elements infinite with the same sign, the
-finite ones within the pool's bar. At head_dim 96 the block kernel keeps the shared product.
-There the rows that see the key are not finite where the oracle's are, rows
-that do not see it may be NaN in the same channels, and everything else is within the bar
-(`exact=False` below)."""
+finite ones within the pool's bar (`exact=True`; `exact=False` is the weaker check a kernel
+that keeps the shared product would be held to: rows that see the key not finite where the
+oracle's are, everything finite within the bar)."""
 import numpy as np
 import pytest
 import torch
@@ -99,7 +98,8 @@ SHAPES = [("f16", 128, 2, 700, True), ("f16", 128, 4, 700, True), ("f16", 128, 7
           ("f16", 128, 8, 2100, True), ("f32", 128, 2, 700, True), ("f32", 128, 6, 700, True),
           ("f16", 128, 24, 700, True), ("f16", 128, 64, 700, True), ("f16", 64, 4, 700, True),
           ("f16", 128, 96, 700, True), ("f16", 128, 200, 300, True), ("f16", 64, 40, 700, True),
-          ("f16", 96, 5, 700, False), ("f16", 256, 3, 700, True), ("f16", 64, 130, 300, True)]
+          ("f16", 96, 5, 700, True), ("f16", 96, 40, 700, True), ("f16", 96, 130, 300, True),
+          ("f16", 256, 3, 700, True), ("f16", 64, 130, 300, True)]
 ROWS_OF = {}
 
 
@@ -118,7 +118,8 @@ def test_a_later_row_of_the_step_holds_values_that_are_not_finite(elem, d, rows,
 
 @pytest.mark.parametrize("elem,d,rows,exact", [("f16", 128, 4, True), ("f16", 128, 7, True), ("f32", 128, 4, True),
                                                 ("f16", 128, 20, True), ("f16", 64, 4, True),
-                                                ("f16", 128, 80, True), ("f16", 96, 6, False)])
+                                                ("f16", 128, 80, True), ("f16", 96, 6, True),
+                                                ("f16", 96, 70, True)])
 def test_a_ring_row_inside_the_first_rows_window_and_outside_the_lasts(elem, d, rows, exact):
     window, ctx = 96, 333
     def plant(v_old):
