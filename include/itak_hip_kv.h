@@ -99,8 +99,12 @@ enum {
    about 4.5 on). Q and K normed per head, as the reference's model norms them, stay at unit
    scale. ITAK_POOL_Q_TWO_HALVES lifts the limit for decode steps and blocks of up to 8 rows at
    head_dim 128 (4e-5 to 2.6e-4 observed at standard deviation 6).
-   A value row that is not finite reaches the outputs of exactly the query rows that see its key
-   (the reference never reads the value row of a masked key), on f32 pools and on f16 pools.
+   Rows that are not finite reach the outputs of exactly the query rows that see their position
+   (the reference never reads the key or value row of a masked position), on f32 pools and on
+   f16 pools: an infinity or a NaN in a value row the channels it stands in, a key whose score
+   is NaN the whole output row. One difference is left on f16 pools: a softmax weight below about
+   2^-24 of its row's largest (a scaled score 17 below the row's maximum) is zero as an f16
+   operand, and zero times an infinite value is NaN where the reference has an infinity.
    Matrix-pipe kernels exist for f16 pools at head_dim 64, 96, 128 and 256 with up to 16 Q heads per
    KV head and for f32 pools at head_dim 64 and 128; every other shape (any head_dim up to 256)
    runs on a general kernel that is correct and one to two orders of magnitude slower. */

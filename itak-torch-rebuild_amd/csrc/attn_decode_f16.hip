@@ -265,11 +265,14 @@ __global__ __launch_bounds__(kWaves * 64) void attn_decode_f16_kernel(AttnParams
     for (int e = 1; e < 8; ++e) mx = fmaxf(mx, sc[e]);
     mx = column_max4(mx);
     const bool dead = mx == -INFINITY || !has_block;
+    // (A block with nothing finite in sight: -inf weighs zero against a reference of zero, and a
+    // NaN score, which the maximum passes over as the reference's comparison does, stays NaN.)
+    const float m_ref = mx == -INFINITY ? 0.0f : mx;
     float sum = 0.0f;
     half8 pb;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        const float pe = dead ? 0.0f : fast_exp2(sc[e] - mx);
+        const float pe = has_block ? fast_exp2(sc[e] - m_ref) : 0.0f;
         sum += pe;
         pb[e] = static_cast<_Float16>(pe);
     }

@@ -192,9 +192,13 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     const uint32_t first_masked = (min(item.pos0 + row_begin, item.kv_len - 1) + 1) / kBlockKeys;
     // Lower edge: blocks before wave_first hold nothing this wavefront's rows see; blocks
     // before low_masked_end hold positions too old for some of them.
-    const uint32_t item_lo = lowest_visible(item.pos0, window, kv_lo);
-    const uint32_t wave_first =
-        lowest_visible(item.pos0 + min(row_begin, item.rows - 1), window, kv_lo) / kBlockKeys;
+    // [wave_lo, wave_hi): the positions some row of this wavefront sees. Outside it the value
+    // operand is cleared (stale ring rows, rows past the stored length, and rows that only other
+    // wavefronts' rows see: a masked key's zero weight times a value that is not finite would
+    // be NaN); a wavefront with one row needs nothing else to be exact.
+    const uint32_t wave_lo = lowest_visible(item.pos0 + min(row_begin, item.rows - 1), window, kv_lo);
+    const uint32_t wave_hi = min(item.pos0 + max(wave_row_end, 1u), item.kv_len);
+    const uint32_t wave_first = wave_lo / kBlockKeys;
     const uint32_t low_masked_end =
         (lowest_visible(item.pos0 + wave_row_end - 1, window, kv_lo) + kBlockKeys - 1) / kBlockKeys;
 
@@ -539,9 +543,9 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
                         if (key_base + e < collo[qt]) x[qt][e >> 2][e & 3] = -INFINITY;
-                if (kb * kBlockKeys < item_lo) {
-                    // Ring rows older than anything the item's queries see may be stale.
-                    const uint32_t stale = min(item_lo - min(item_lo, key_base), 8u);
+                if (kb * kBlockKeys < wave_lo) {
+                    // Ring rows older than anything the wavefront's queries see may be stale.
+                    const uint32_t stale = min(wave_lo - min(wave_lo, key_base), 8u);
                     const u32x4 keep = ~first_halves(stale);
 #pragma unroll
                     for (int dt = 0; dt < kOut; ++dt)
@@ -555,9 +559,10 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
                         if (key_base + e > colpos[qt]) x[qt][e >> 2][e & 3] = -INFINITY;
-                if ((kb + 1) * kBlockKeys > item.kv_len) {
-                    // Rows past the stored length may hold stale data: keep them out of P.V.
-                    const uint32_t stored = min(item.kv_len - min(item.kv_len, key_base), 8u);
+                if ((kb + 1) * kBlockKeys > wave_hi) {
+                    // Rows past the stored length may hold stale data, rows past the wavefront's
+                    // last row values that are not finite: keep them out of P.V.
+                    const uint32_t stored = min(wave_hi - min(wave_hi, key_base), 8u);
                     const u32x4 keep = first_halves(stored);
 #pragma unroll
                     for (int dt = 0; dt < kOut; ++dt)

@@ -254,12 +254,17 @@ __device__ __forceinline__ void process_block(WaveState<NQ> &st, BlockOperands &
         // registers there and cost three instructions an element, then leaves the common path.
         constexpr float kSlack = NQ > 2 ? 8.0f : 0.0f;
         const float m_new = FIRST ? mx : (mx > st.m[qt] + kSlack ? mx : st.m[qt]);
-        const bool dead = m_new == -INFINITY;  // nothing visible to this column so far
+        // Nothing finite visible to this column so far: its scores are -inf (weight zero, taken
+        // against a reference of zero, since -inf - -inf is NaN) or NaN (a key that is not
+        // finite: the maximum passes over it, as the reference's comparison does
+        // (attention.rs:160-173), and its weight and with it the whole row must come out NaN).
+        const bool dead = m_new == -INFINITY;
+        const float m_ref = dead ? 0.0f : m_new;
         float p[8];
         float sum = 0.0f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            p[e] = dead ? 0.0f : fast_exp2(sc[e] - m_new);
+            p[e] = fast_exp2(sc[e] - m_ref);
             sum += p[e];
         }
         half8 pb;

@@ -134,7 +134,9 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
     const uint32_t row = j / group, head = kv_head * group + j % group;
     const uint32_t colpos = min(item.pos0 + row, item.kv_len - 1);
     const uint32_t collo = lowest_visible(item.pos0 + row, window, kv_lo);
-    const uint32_t lo_min = lowest_visible(item.pos0, window, kv_lo);
+    // [tile_lo, tile_hi): the positions some row of this tile sees.
+    const uint32_t tile_lo = lowest_visible(item.pos0 + row_first, window, kv_lo);
+    const uint32_t tile_hi = min(item.pos0 + row_last + 1, item.kv_len);
     const float softcap = p.softcap;
     const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
     const float qscale = softcap > 0.0f ? p.scale : p.scale * kLog2e;
@@ -209,9 +211,11 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
                 if (kp > colpos || (RING && kp < collo)) v = -INFINITY;
                 sc[t][r] = v;
                 mx = fmaxf(mx, v);
-                // A row no query of the item sees (past the stored length, or older than the
-                // oldest window on a ring) may hold anything: keep it out of P.V even as 0*x.
-                if (kp >= item.kv_len || (RING && kp < lo_min)) {
+                // A row no query of the tile sees (past the stored length or the tile's last
+                // row, or older than its oldest window on a ring) may hold anything, stale data
+                // or a value that is not finite: keep it out of P.V even as 0*x. A tile of one
+                // row needs nothing else to be exact.
+                if (kp >= tile_hi || (RING && kp < tile_lo)) {
 #pragma unroll
                     for (int h = 0; h < kH; ++h) vreg[t][r][h] = make_float4(0.f, 0.f, 0.f, 0.f);
                 }
@@ -225,7 +229,10 @@ __global__ __launch_bounds__(kWavesF32 * 64) void attn_splitk_f32_kernel(AttnPar
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float pe = dead ? 0.0f : fast_exp2(sc[t][r] - m_new);
+                // (Nothing finite in sight so far: -inf weighs zero against a reference of zero,
+                // and a NaN score, which the maximum passes over as the reference's comparison
+                // does, stays NaN and takes the row with it.)
+                const float pe = fast_exp2(sc[t][r] - (dead ? 0.0f : m_new));
                 sc[t][r] = pe;
                 sum += pe;
             }

@@ -192,9 +192,12 @@ struct ExchangeGroup {
                 const unsigned long long ml = rec[pr * kExchangeWords + 16];
                 const unsigned long long xv = rec[pr * kExchangeWords + k];
                 const float mp = __uint_as_float(uint32_t(ml)), lp = __uint_as_float(uint32_t(ml >> 32));
-                if (mp == -INFINITY) continue;
+                // (A producer that saw nothing finite has m = -inf: weight zero against a
+                // stand-in reference, and no branch around it, so that an l or a sum that is NaN
+                // there, from a key that is not finite, stays in the result.)
                 const float m_new = fmaxf(m_run, mp);
-                const float keep = fast_exp2(m_run - m_new), w = fast_exp2(mp - m_new);  // exp2(-inf) = 0
+                const float ref = m_new == -INFINITY ? 0.0f : m_new;
+                const float keep = fast_exp2(m_run - ref), w = fast_exp2(mp - ref);  // exp2(-inf) = 0
                 l_run = fmaf(lp, w, l_run * keep);
                 a0 = fmaf(__uint_as_float(uint32_t(xv)), w, a0 * keep);
                 a1 = fmaf(__uint_as_float(uint32_t(xv >> 32)), w, a1 * keep);
