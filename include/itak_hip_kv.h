@@ -149,7 +149,10 @@ enum {
        the rounding of the softmax weights to f16. These kernels wait for memory more than for
        the matrix pipe: the second product costs 1 % on a decode step or a ragged batch and 7 %
        on a speculative block of 64 query vectors per KV head. Longer blocks and prefill
-       chunks (the block kernel) are not affected by the flag. */
+       chunks (the block kernel) are not affected by the flag. One thing it changes for keys
+       that are not finite: an infinite channel of a visible key makes the score NaN when the
+       channel's two halves have opposite signs (inf - inf), and the output row with it, where
+       the single product and the reference have a score of plus or minus infinity. */
     ITAK_POOL_Q_TWO_HALVES = 8u
 };
 
