@@ -482,6 +482,27 @@ def probes(torch, pool, timed, dev):
     }
 
 
+def mfma_alone(torch, pool, timed, dev):
+    """What the matrix pipe sustains by itself on this device (itak_probe_mfma: 32 f16 MFMAs a
+    trip, operands in registers, two wavefronts a SIMD), on constant and on random operands, with
+    the clock it held: the prefill kernel's data is random, and the second figure is the most any
+    kernel built on this instruction could show for it here."""
+    out = {}
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    for name, random_operands in (("constant_operands", False), ("random_operands", True)):
+        trips = 20000
+        flops = pool.probe_mfma(random_operands, 2000)  # warm-up
+        best = None
+        for _ in range(3):
+            s, _ = timed(lambda: pool.probe_mfma(random_operands, trips, clocks.data_ptr()), 1)
+            best = s if best is None else min(best, s)
+        flops = flops // 2000 * trips
+        ticks = clocks.cpu().tolist()
+        out[name] = {"tflops": round(flops / best / 1e12, 1),
+                     "clock_ghz": round(ticks[0] / max(1, ticks[1]) * 0.1, 2)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -932,6 +953,11 @@ def run_workload(args, pkg, torch, np, dev, stream, timed):
             "timed": "the attention launch of a layer, event-timed in a graph of its own on a "
                      "cache that already holds the chunk",
         }
+        # Beside the published peak: the instruction alone on this device, in this run.
+        alone = mfma_alone(torch, pool, timed, dev)
+        roofline["mfma_alone"] = alone
+        roofline["frac_of_mfma_alone_on_random_operands"] = round(
+            flops_layer / attn_s / 1e12 / alone["random_operands"]["tflops"], 4)
     else:
         metric, unit = "decode-attn KV GB/s (all layers, ctx 4096)", "GB/s"
         if wl != "decode":

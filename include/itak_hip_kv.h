@@ -665,6 +665,18 @@ itak_status itak_probe_copy_device(itak_pool *pool, const void *src_dev, void *d
 /* One empty kernel on the pool's stream: timing a run of these gives the per-launch floor
    of dependent launches on this device. */
 itak_status itak_probe_empty_launch(itak_pool *pool);
+/* What the matrix pipe sustains by itself on this device, for the prefill roofline: `trips`
+   (1 ..= 2^22) trips of 32 v_mfma_f32_16x16x32_f16 per wavefront, operands held in registers,
+   two workgroups of four wavefronts on every compute unit, on the pool's stream. With
+   random_operands the operands are pseudo-random halves in (-1, 1), else one constant: the clock
+   the chip holds under the instruction, and with it the rate, depends on how many operand bits
+   change between products (on an MI355X 2.4 PFLOP/s at 2.39 GHz on constants, 1.85 PFLOP/s at
+   1.84 GHz on random halves). *flops_out (may be NULL) receives the launch's floating-point
+   operations; clocks_dev (device memory, two words, may be NULL) receives the ticks of the
+   shader clock and of the 100 MHz constant clock over the loop of one workgroup. The caller
+   times the launch. */
+itak_status itak_probe_mfma(itak_pool *pool, uint32_t random_operands, uint32_t trips,
+                            uint64_t *clocks_dev, uint64_t *flops_out);
 
 #ifdef __cplusplus
 }

@@ -189,6 +189,7 @@ PROTOTYPES = {
     "itak_convert_f32_to_f16_device": (_i32, [_P, _P, _P, _u64]),
     "itak_probe_copy_device": (_i32, [_P, _P, _P, _u64]),
     "itak_probe_empty_launch": (_i32, [_P]),
+    "itak_probe_mfma": (_i32, [_P, _u32, _u32, _P, _P]),
     "itak_set_debug_enabled": (None, [_i32]),
     "itak_debug_enabled": (_i32, []),
 }

@@ -174,6 +174,10 @@ hipError_t launch_stage_in(const void *pinned, void *dst, uint64_t bytes, hipStr
 hipError_t launch_signal_done(uint32_t *pinned_word, uint32_t value, hipStream_t stream);
 hipError_t launch_probe_copy(const void *src, void *dst, uint64_t bytes, hipStream_t stream);
 hipError_t launch_probe_empty(hipStream_t stream);
+// `iters` trips of 32 f16 MFMAs per wavefront, two workgroups of four wavefronts per compute unit
+// (*workgroups receives how many were launched); clocks: two device words or null.
+hipError_t launch_probe_mfma(bool random_operands, uint32_t iters, unsigned long long *clocks,
+                             uint32_t *workgroups, hipStream_t stream);
 
 // ---- attention preparation (per-head RMSNorm + RoPE of Q and K) and the output gate ------
 struct PrepArgs {

@@ -520,4 +520,67 @@ hipError_t launch_probe_empty(hipStream_t stream) {
     return hipGetLastError();
 }
 
+// What the matrix pipe sustains by itself: `iters` trips of 32 v_mfma_f32_16x16x32_f16 into 16
+// accumulators (two in a row per accumulator, the pattern of the block kernel's P.V), operands
+// held in registers, two wavefronts a SIMD on every compute unit. RANDOM fills the operands
+// with pseudo-random halves in (-1, 1), else with one constant: the clock the chip holds under
+// the instruction depends on how many operand bits change from one product to the next, and so
+// does what "the peak" is for data like a model's. clocks[0..1] receive the shader clock's and
+// the 100 MHz constant clock's ticks over the loop of workgroup 0 (their ratio is the clock).
+typedef _Float16 probe_half8 __attribute__((ext_vector_type(8)));
+typedef float probe_floatx4 __attribute__((ext_vector_type(4)));
+template <bool RANDOM>
+__global__ __launch_bounds__(256, 2) void probe_mfma_kernel(uint32_t iters, unsigned long long *clocks,
+                                                            float *sink) {
+    const uint32_t tid = threadIdx.x;
+    probe_half8 a[8], b[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t h = (tid * 131u + blockIdx.x * 977u + i * 17u + e) * 2654435761u;
+            a[i][e] = RANDOM ? (_Float16)(float((h >> 16) & 1023) / 512.0f - 1.0f) : (_Float16)0.0625f;
+            b[i][e] = RANDOM ? (_Float16)(0.2f * (float((h >> 6) & 1023) / 512.0f - 1.0f)) : (_Float16)0.0625f;
+        }
+    probe_floatx4 c[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) c[i] = probe_floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    const unsigned long long c0 = clock64(), w0 = wall_clock64();
+    for (uint32_t it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            c[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i & 7], b[(i + 1) & 7], c[i], 0, 0, 0);
+            c[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[(i + 3) & 7], b[i & 7], c[i], 0, 0, 0);
+        }
+        if ((it & 1023u) == 1023u) {  // the sums stay in range however long the loop
+#pragma unroll
+            for (int i = 0; i < 16; ++i) c[i] *= 0.001f;
+        }
+    }
+    if (clocks != nullptr && blockIdx.x == 0 && tid == 0) {
+        clocks[0] = clock64() - c0;
+        clocks[1] = wall_clock64() - w0;
+    }
+    probe_floatx4 acc = probe_floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc += c[i];
+    // (Never true; it keeps the products alive.)
+    if (sink != nullptr && acc[0] == 12345.678f) sink[blockIdx.x * 256 + tid] = acc[1] + acc[2] + acc[3];
+}
+
+hipError_t launch_probe_mfma(bool random_operands, uint32_t iters, unsigned long long *clocks,
+                             uint32_t *workgroups, hipStream_t stream) {
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        (void)hipGetLastError();
+    const uint32_t grid = 2u * uint32_t(cus > 0 ? cus : 256);
+    if (workgroups) *workgroups = grid;
+    if (random_operands)
+        probe_mfma_kernel<true><<<grid, 256, 0, stream>>>(iters, clocks, nullptr);
+    else
+        probe_mfma_kernel<false><<<grid, 256, 0, stream>>>(iters, clocks, nullptr);
+    return hipGetLastError();
+}
+
 }  // namespace itak

@@ -2785,4 +2785,18 @@ itak_status itak_probe_empty_launch(itak_pool *pool) {
     return ITAK_OK;
 }
 
+itak_status itak_probe_mfma(itak_pool *pool, uint32_t random_operands, uint32_t trips,
+                            uint64_t *clocks_dev, uint64_t *flops_out) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (trips == 0 || trips > (1u << 22)) return invalid_argument(pool->err, "trips is not in 1 ..= 2^22");
+    uint32_t workgroups = 0;
+    HIP_TRY(pool,
+            launch_probe_mfma(random_operands != 0, trips,
+                              reinterpret_cast<unsigned long long *>(clocks_dev), &workgroups, pool->stream),
+            "launch MFMA probe");
+    // 4 wavefronts a workgroup, 32 products a trip, 16 x 16 x 32 multiply-adds a product.
+    if (flops_out) *flops_out = uint64_t(workgroups) * 4u * uint64_t(trips) * 32u * 16384u;
+    return ITAK_OK;
+}
+
 }  // extern "C"

@@ -337,6 +337,14 @@ class KvPool:
         """Measurement aid: one empty kernel on the pool's stream."""
         _check(self._h, self._lib.itak_probe_empty_launch(self._h))
 
+    def probe_mfma(self, random_operands: bool, trips: int, clocks_ptr: int = 0) -> int:
+        """Measurement aid: a loop of f16 MFMAs alone on every compute unit, on the pool's
+        stream; returns the launch's floating-point operations (the caller times it)."""
+        flops = C.c_uint64(0)
+        _check(self._h, self._lib.itak_probe_mfma(self._h, 1 if random_operands else 0, trips,
+                                                  C.c_void_p(clocks_ptr or None), C.byref(flops)))
+        return int(flops.value)
+
     def convert_f32_to_f16_device(self, src_ptr: int, dst_ptr: int, count: int) -> None:
         _check(self._h, self._lib.itak_convert_f32_to_f16_device(self._h, src_ptr, dst_ptr, count))
 

@@ -525,3 +525,22 @@ def test_debug_channel_reports_cache_and_attention_events(capfd):
     cache.append(0, k_row(kv_heads, d, 3), v_row(kv_heads, d, 3), 3)
     assert "[itak_hip_kv::diag]" not in capfd.readouterr().err
     pool.close()
+
+
+def test_the_mfma_probe_reports_its_work_and_both_clocks():
+    # A measurement aid, not part of the path: the call launches, says how many floating-point
+    # operations the launch held, and leaves the ticks of the two clocks in device memory.
+    import torch
+    pool = P().KvPool(1, 1, 128, elem="f16", capacity_rows=64)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    clocks = torch.zeros(2, dtype=torch.int64, device="cuda")
+    flops = pool.probe_mfma(True, 64, clocks.data_ptr())
+    pool.synchronize()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    assert flops == 2 * cus * 4 * 64 * 32 * 16384
+    shader, constant = clocks.cpu().tolist()
+    assert shader > 0 and constant > 0 and 5 <= shader / constant <= 30   # 0.5 to 3 GHz against 100 MHz
+    assert pool.probe_mfma(False, 1) == 2 * cus * 4 * 32 * 16384
+    with pytest.raises(Exception, match="trips"):
+        pool.probe_mfma(True, 0)
+    pool.close()
