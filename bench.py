@@ -473,12 +473,15 @@ def probes(torch, pool, timed, dev):
     dst = torch.empty_like(src)
     pool.probe_copy_device(src.data_ptr(), dst.data_ptr(), n)
     copy_s, _ = timed(lambda: pool.probe_copy_device(src.data_ptr(), dst.data_ptr(), n), 5)
+    pool.probe_read_device(src.data_ptr(), n)
+    read_s, _ = timed(lambda: pool.probe_read_device(src.data_ptr(), n), 5)
     for _ in range(50):
         pool.probe_empty_launch()
     empty_s, _ = timed(pool.probe_empty_launch, 2000)
     return {
         "empty_kernel_us_per_launch": round(empty_s / 2000 * 1e6, 3),
         "copy_256MiB_GBps_read_plus_write": round(2 * n * 5 / copy_s / 1e9, 1),
+        "read_256MiB_GBps": round(n * 5 / read_s / 1e9, 1),
     }
 
 
@@ -694,8 +697,9 @@ def summary_of(result):
     out = {"metric": result["metric"], "value": result["value"], "unit": result["unit"],
            "ms_per_step": result["ms_per_step"], "bound": r["bound"], "frac": r["frac"],
            "us_per_launch": r.get("us_per_launch"), "kernel": r.get("kernel")}
-    if "step_frac" in r:
-        out["step_frac"] = r["step_frac"]
+    for key in ("step_frac", "frac_of_streaming_read", "mfma_alone", "frac_of_mfma_alone_on_random_operands"):
+        if key in r:
+            out[key] = r[key]
     return out
 
 
@@ -984,6 +988,9 @@ def run_workload(args, pkg, torch, np, dev, stream, timed):
             "traffic_source": PROFILE_TRAFFIC.get((wl, args.kv), (None, None))[1],
             "us_per_launch": round(layer_s * 1e6, 3),
             "bytes_per_launch": kv_bytes_layer,
+            # Beside the published peak: what a kernel that only reads gets from this device
+            # (itak_probe_read_device, 256 MiB), in this run.
+            "frac_of_streaming_read": round(kv_bytes_layer / layer_s / 1e9 / probe["read_256MiB_GBps"], 4),
             "timed": "one layer of the timed step (HIP graph replay of all layers), HIP events on "
                      "the stream the kernels run on",
             # The attention launches alone, on a cache that already holds the new rows.

@@ -267,6 +267,7 @@ extern "C" {
     pub fn itak_set_debug_enabled(enabled: i32);
     pub fn itak_debug_enabled() -> i32;
     pub fn itak_probe_copy_device(pool: *mut itak_pool, src_dev: *const c_void, dst_dev: *mut c_void, bytes: u64) -> itak_status;
+    pub fn itak_probe_read_device(pool: *mut itak_pool, src_dev: *const c_void, bytes: u64) -> itak_status;
     pub fn itak_probe_empty_launch(pool: *mut itak_pool) -> itak_status;
     pub fn itak_probe_mfma(pool: *mut itak_pool, random_operands: u32, trips: u32, clocks_dev: *mut u64, flops_out: *mut u64) -> itak_status;
 }

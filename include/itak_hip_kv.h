@@ -662,6 +662,10 @@ int32_t itak_debug_enabled(void);
    known size that hardware traffic counters are scaled by. */
 itak_status itak_probe_copy_device(itak_pool *pool, const void *src_dev, void *dst_dev,
                                    uint64_t bytes);
+/* A plain streaming read of `bytes` (a multiple of 16) on the pool's stream, nothing written:
+   what the device delivers to a kernel that only reads, which is what a decode step's
+   attention does with the cache. */
+itak_status itak_probe_read_device(itak_pool *pool, const void *src_dev, uint64_t bytes);
 /* One empty kernel on the pool's stream: timing a run of these gives the per-launch floor
    of dependent launches on this device. */
 itak_status itak_probe_empty_launch(itak_pool *pool);

@@ -188,6 +188,7 @@ PROTOTYPES = {
     "itak_store_capture_and_put": (_i32, [_P, _P, _u32, _P, _u64, C.c_char_p, _u64, _u32, _u64]),
     "itak_convert_f32_to_f16_device": (_i32, [_P, _P, _P, _u64]),
     "itak_probe_copy_device": (_i32, [_P, _P, _P, _u64]),
+    "itak_probe_read_device": (_i32, [_P, _P, _u64]),
     "itak_probe_empty_launch": (_i32, [_P]),
     "itak_probe_mfma": (_i32, [_P, _u32, _u32, _P, _P]),
     "itak_set_debug_enabled": (None, [_i32]),

@@ -173,6 +173,7 @@ hipError_t launch_widen_f16(const uint16_t *src, float *dst, uint64_t count, hip
 hipError_t launch_stage_in(const void *pinned, void *dst, uint64_t bytes, hipStream_t stream);
 hipError_t launch_signal_done(uint32_t *pinned_word, uint32_t value, hipStream_t stream);
 hipError_t launch_probe_copy(const void *src, void *dst, uint64_t bytes, hipStream_t stream);
+hipError_t launch_probe_read(const void *src, uint64_t bytes, hipStream_t stream);
 hipError_t launch_probe_empty(hipStream_t stream);
 // `iters` trips of 32 f16 MFMAs per wavefront, two workgroups of four wavefronts per compute unit
 // (*workgroups receives how many were launched); clocks: two device words or null.

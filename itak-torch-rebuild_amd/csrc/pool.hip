@@ -2774,6 +2774,14 @@ itak_status itak_probe_copy_device(itak_pool *pool, const void *src_dev, void *d
     return ITAK_OK;
 }
 
+itak_status itak_probe_read_device(itak_pool *pool, const void *src_dev, uint64_t bytes) {
+    if (!pool) return ITAK_INVALID_ARGUMENT;
+    if (bytes && !src_dev) return invalid_argument(pool->err, "src is null");
+    if (bytes % 16 != 0) return invalid_argument(pool->err, "bytes is not a multiple of 16");
+    HIP_TRY(pool, launch_probe_read(src_dev, bytes, pool->stream), "launch probe read");
+    return ITAK_OK;
+}
+
 void itak_set_debug_enabled(int32_t enabled) {
     g_debug_enabled.store(enabled != 0, std::memory_order_relaxed);
 }

@@ -333,6 +333,10 @@ class KvPool:
         """Measurement aid: a plain streaming copy of known size on the pool's stream."""
         _check(self._h, self._lib.itak_probe_copy_device(self._h, src_ptr, dst_ptr, nbytes))
 
+    def probe_read_device(self, src_ptr: int, nbytes: int) -> None:
+        """Measurement aid: a plain streaming read of known size on the pool's stream."""
+        _check(self._h, self._lib.itak_probe_read_device(self._h, src_ptr, nbytes))
+
     def probe_empty_launch(self) -> None:
         """Measurement aid: one empty kernel on the pool's stream."""
         _check(self._h, self._lib.itak_probe_empty_launch(self._h))

@@ -543,4 +543,9 @@ def test_the_mfma_probe_reports_its_work_and_both_clocks():
     assert pool.probe_mfma(False, 1) == 2 * cus * 4 * 32 * 16384
     with pytest.raises(Exception, match="trips"):
         pool.probe_mfma(True, 0)
+    src = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    pool.probe_read_device(src.data_ptr(), 1 << 20)   # launches and reads, nothing to compare
+    pool.synchronize()
+    with pytest.raises(Exception, match="multiple of 16"):
+        pool.probe_read_device(src.data_ptr(), 24)
     pool.close()
