@@ -91,8 +91,16 @@ __global__ __launch_bounds__(kPrepWaves * 64) void attn_prep_kernel(PrepArgs a) 
             const double angle = position * pow(double(a.rope_base), exponent);
             double s, c;
             sincos(angle, &s, &c);
-            dst[c0] = float(double(x) * c - double(y) * s);
-            dst[c1] = float(double(x) * s + double(y) * c);
+            // Two products and a sum, each rounded, as the reference's compiler emits them: a
+            // fused multiply-add here would differ from it in the last bit of the f64 result,
+            // which shows in the f32 row where the rotation cancels to something tiny.
+            {
+#pragma clang fp contract(off)
+                const double xc = double(x) * c, ys = double(y) * s;
+                const double xs = double(x) * s, yc = double(y) * c;
+                dst[c0] = float(xc - ys);
+                dst[c1] = float(xs + yc);
+            }
         } else {
             dst[c0] = x;
             dst[c1] = y;
