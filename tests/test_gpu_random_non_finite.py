@@ -18,7 +18,9 @@ cap from the others), so with a softcap the planted keys are NaN only.
 
 The seed lists hold the seeds that failed while the kernels were written (a wavefront or tile
 holding one row of a step of several; a NaN score as the only one a wavefront sees in its
-block) and some that never did."""
+block) and some that never did. The pools say `q_two_halves=False`: as two halves an infinite
+key channel scores NaN where one product scores an infinity (the flag's text in the header), and
+the planted keys include infinities."""
 import numpy as np
 import pytest
 import torch
@@ -84,7 +86,8 @@ def test_one_step_with_values_planted_near_the_edges_of_its_rows_masks(seed):
 
     okind = oracle.LayerKind.Global if window is None else oracle.LayerKind.windowed(window)
     pkind = P().LayerKind.Global if window is None else P().LayerKind.windowed(window)
-    pool = P().KvPool([pkind], kvh, d, elem=elem, capacity_rows=ctx + rows + 8, ring_headroom=max(64, rows))
+    pool = P().KvPool([pkind], kvh, d, elem=elem, capacity_rows=ctx + rows + 8, ring_headroom=max(64, rows),
+                      q_two_halves=False)
     pool.set_stream(torch.cuda.current_stream().cuda_stream)
     cache = pool.acquire()
     kd, vd, qd = dev(k), dev(v), dev(q)
@@ -133,7 +136,7 @@ def test_batched_steps_with_values_and_keys_planted(seed, keys):
     okind = oracle.LayerKind.Global if window is None else oracle.LayerKind.windowed(window)
     pkind = P().LayerKind.Global if window is None else P().LayerKind.windowed(window)
     pool = P().KvPool([pkind], kvh, d, elem=elem, max_slots=slots, ring_headroom=headroom,
-                      capacity_rows=max(prefixes) + sum(max(s) for s in steps) + 8)
+                      capacity_rows=max(prefixes) + sum(max(s) for s in steps) + 8, q_two_halves=False)
     pool.set_stream(torch.cuda.current_stream().cuda_stream)
     caches = [pool.acquire() for _ in range(slots)]
     refs = [oracle.KvCache.new([okind], kvh, d, store_f16=(elem == "f16")) for _ in range(slots)]
@@ -180,7 +183,7 @@ def test_a_nan_key_that_is_the_only_key_a_row_sees_in_its_block(elem, d):
     rng = np.random.default_rng(5)
     k, v, q = normal(rng, ctx + rows, width), normal(rng, ctx + rows, width), normal(rng, rows, q_heads * d)
     k[ctx + 2, d + 49] = np.nan
-    pool = P().KvPool([P().LayerKind.Global], kvh, d, elem=elem, capacity_rows=ctx + rows + 8)
+    pool = P().KvPool([P().LayerKind.Global], kvh, d, elem=elem, capacity_rows=ctx + rows + 8, q_two_halves=False)
     pool.set_stream(torch.cuda.current_stream().cuda_stream)
     cache = pool.acquire()
     kd, vd, qd = dev(k), dev(v), dev(q)
