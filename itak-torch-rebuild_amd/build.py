@@ -32,9 +32,15 @@ def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
+# Sources whose kernels the timeline run never reads stamps of: in the measurement build they are
+# compiled as in the ordinary one (the stamps cost registers, and the block kernel's forms at
+# head dims other than 128 have none to spare).
+NO_STAMPS = {"attn_prefill_f16_dims.hip"}
+
+
 def _compile(src: str, timeline: bool = False) -> str:
     obj = os.path.join(OBJ_DIR + ("_timeline" if timeline else ""), src.replace(".hip", ".o"))
-    cmd = [HIPCC, *FLAGS, *(["-DITAK_TIMELINE"] if timeline else []), "-c",
+    cmd = [HIPCC, *FLAGS, *(["-DITAK_TIMELINE"] if timeline and src not in NO_STAMPS else []), "-c",
            os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
