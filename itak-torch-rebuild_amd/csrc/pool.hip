@@ -1892,7 +1892,8 @@ itak_status itak_kv_read_rows(itak_pool *pool, uint32_t slot, uint64_t layer, ui
     if (layer >= pool->cfg.layer_count) return invalid_layer(pool->err, layer, pool->cfg.layer_count);
     const uint64_t stored = stored_of(pool, *s, layer);
     if (first > stored || rows > stored - first)
-        return shape_mismatch(pool->err, "visible rows", stored, first + rows);
+        return shape_mismatch(pool->err, "visible rows", stored,
+                              rows > UINT64_MAX - first ? UINT64_MAX : first + rows);  // (no wrapped sum in the text)
     const uint64_t oldest = first_visible(pool, *s, layer);
     if (positions_out)
         for (uint64_t i = 0; i < rows; ++i) positions_out[i] = oldest + first + i;  // cache.rs:878-883

@@ -549,3 +549,15 @@ def test_the_mfma_probe_reports_its_work_and_both_clocks():
     with pytest.raises(Exception, match="multiple of 16"):
         pool.probe_read_device(src.data_ptr(), 24)
     pool.close()
+
+
+def test_a_read_that_starts_past_the_end_is_refused_without_a_wrapped_sum():
+    pool = P().KvPool(1, 1, 16, elem="f32", capacity_rows=8)
+    cache = pool.acquire()
+    k = np.ones((3, 16), dtype=np.float32)
+    for i in range(3):
+        cache.append(0, k[i], k[i], i)
+    with pytest.raises(P().AttentionError) as e:
+        cache.read_rows(0, 2 ** 64 - 4, 64)      # a first row computed as 3 - 7 and the like
+    assert "18446744073709551615" in str(e.value) and "expected 3" in str(e.value)
+    pool.close()
