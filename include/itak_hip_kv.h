@@ -328,7 +328,11 @@ itak_status itak_kv_append(itak_pool *pool, uint32_t slot, uint64_t layer, const
    first_position.. into a fresh layer. keys/values may be pinned host memory
    (read in place by the gather kernel), ordinary host memory (staged) or device
    memory; *_len count elements of src_elem type. An f32 source into an f16 pool is
-   converted exactly as append converts; an f16 source needs an f16 pool. */
+   converted exactly as append converts; an f16 source needs an f16 pool. With host memory
+   of either kind the rows are in place when the call returns; rows that all lie in device
+   memory are gathered in the order of the pool's stream, like itak_kv_append_device, and the
+   call returns with the gather enqueued (the sources stay untouched until the stream has
+   passed it). The same holds for itak_kv_restore_snapshot. */
 itak_status itak_kv_restore_bulk(itak_pool *pool, uint32_t slot, uint64_t layer,
                                  uint64_t first_position, const void *keys, uint64_t keys_len,
                                  const void *values, uint64_t values_len, uint32_t src_elem);

@@ -1446,11 +1446,19 @@ static itak_status restore_layers(itak_pool *pool, uint32_t slot, Slot &s,
     // Sources the device cannot read in place are staged through one temporary buffer.
     uint64_t stage_need = 0;
     PtrClassifier kind_of;
+    // Rows that all lie in device memory are gathered in stream order, like a device append: the
+    // call returns with the gather enqueued. Host memory of either kind is the caller's to free
+    // when the call returns, so the call waits for the stream then.
+    bool all_device = true;
     for (uint64_t i = 0; i < count; ++i) {
         if (layers[i].rows == 0) continue;
         const uint64_t bytes = layers[i].rows * pool->row * src_bytes_per_elem;
         if (must_stage(kind_of, layers[i].keys, src_bytes_per_elem)) stage_need += align_up(bytes, 256);
         if (must_stage(kind_of, layers[i].values, src_bytes_per_elem)) stage_need += align_up(bytes, 256);
+        const void *usable;
+        if (kind_of(layers[i].keys, &usable) != PtrKind::Device ||
+            kind_of(layers[i].values, &usable) != PtrKind::Device)
+            all_device = false;
     }
     unsigned char *temp = nullptr;
     if (stage_need) HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&temp), stage_need), "allocate restore staging");
@@ -1532,8 +1540,10 @@ static itak_status restore_layers(itak_pool *pool, uint32_t slot, Slot &s,
         }
     }
     for (int w = 0; w < 2 && st == ITAK_OK; ++w) st = flush(w);
-    hipError_t he = hipStreamSynchronize(pool->stream);
-    if (st == ITAK_OK && he != hipSuccess) st = hip_error(pool->err, he, "synchronize after restore");
+    if (!all_device || stage_need || st != ITAK_OK) {
+        hipError_t he = hipStreamSynchronize(pool->stream);
+        if (st == ITAK_OK && he != hipSuccess) st = hip_error(pool->err, he, "synchronize after restore");
+    }
     if (temp) (void)hipFree(temp);
     if (st != ITAK_OK) return st;
     for (uint64_t i = 0; i < count; ++i) {

@@ -561,3 +561,28 @@ def test_a_read_that_starts_past_the_end_is_refused_without_a_wrapped_sum():
         cache.read_rows(0, 2 ** 64 - 4, 64)      # a first row computed as 3 - 7 and the like
     assert "18446744073709551615" in str(e.value) and "expected 3" in str(e.value)
     pool.close()
+
+
+def test_a_restore_from_device_memory_is_ordered_by_the_stream_and_one_from_host_memory_is_done_on_return():
+    import torch
+    kvh, d, n = 2, 64, 500
+    row = kvh * d
+    rng = np.random.default_rng(11)
+    k, v = normal(rng, n, row), normal(rng, n, row)
+    pool = P().KvPool(1, kvh, d, elem="f32", max_slots=2, capacity_rows=n + 8)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    a, b = pool.acquire(), pool.acquire()
+    # Device rows: the call returns with the gather enqueued; what reads the cache next on the
+    # same stream (here the read-back) comes after it.
+    kd, vd = torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda()
+    a.restore_bulk_ptr(0, 0, kd.data_ptr(), vd.data_ptr(), n * row, src_f16=False)
+    _, gk, gv = a.read_rows(0, 0, n)
+    assert np.array_equal(np.asarray(gk).reshape(n, row), k) and np.array_equal(np.asarray(gv).reshape(n, row), v)
+    # Pinned host rows are the caller's again when the call returns: overwritten at once, the
+    # cache still holds what they were.
+    kp, vp = torch.from_numpy(k.copy()).pin_memory(), torch.from_numpy(v.copy()).pin_memory()
+    b.restore_bulk_ptr(0, 0, kp.data_ptr(), vp.data_ptr(), n * row, src_f16=False)
+    kp.zero_(); vp.zero_()
+    _, gk, gv = b.read_rows(0, 0, n)
+    assert np.array_equal(np.asarray(gk).reshape(n, row), k) and np.array_equal(np.asarray(gv).reshape(n, row), v)
+    pool.close()
