@@ -546,11 +546,11 @@ itak_status itak_gqa_attention(itak_pool *pool, uint32_t slot, uint64_t layer, c
    leaves it ahead of the caller's position and the next call refuses until
    itak_slot_reset, as the reference does. The rotation uses f64 angles, sines and
    cosines like rope_interleaved.rs:103-114, on every shape: the K rows the call stores
-   are the reference's rotated rows, rounded once where the pool is f16. (The f64 pow, sine
-   and cosine are the device library's: where theirs and the host's differ in the last bit and
-   the f64 result lies that close to an f32 rounding boundary, or the rotation cancels to a
-   result many orders below its operands, a stored f32 element can differ from the host's by
-   a few units in the last place: seen in 2 elements of 3,000 random models.) */
+   are the reference's rotated rows, rounded once where the pool is f16. (The frequencies
+   rope_base^(-2i/d) are computed on the host, in the libm the reference's own host would use,
+   and kept on the device: the device library's pow may differ from it in the last bit, and a
+   last bit times the position is what reaches the row. Sine and cosine are the device
+   library's; no stored element has been seen to differ for it, up to position 10^6.) */
 itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t layer, const float *q,
                                    uint64_t q_len, const float *k, uint64_t k_len, const float *v,
                                    uint64_t v_len, uint64_t num_q_heads, uint64_t cache_position,

@@ -88,7 +88,8 @@ __global__ __launch_bounds__(kPrepWaves * 64) void attn_prep_kernel(PrepArgs a) 
         const float x = normed(c0), y = normed(c1);
         if (turn) {
             const double exponent = -double(2 * p) / double(rot);
-            const double angle = position * pow(double(a.rope_base), exponent);
+            const double freq = a.rope_freq ? a.rope_freq[p] : pow(double(a.rope_base), exponent);
+            const double angle = position * freq;
             double s, c;
             sincos(angle, &s, &c);
             // Two products and a sum, each rounded, as the reference's compiler emits them: a

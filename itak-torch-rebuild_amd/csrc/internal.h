@@ -190,6 +190,11 @@ struct PrepArgs {
     const float *k_weight;
     float eps;
     float rope_base;        // > 1 rotates, otherwise no rotation
+    // Pair i turns at position * rope_freq[i] radians: rope_base^(-2i/rotary_dim) as the host's
+    // libm gives it, which is what the reference's own host computes. Null: the kernel takes
+    // the power itself (the device library's may differ in the last bit, and a last bit times
+    // the position is what reaches the stored row).
+    const double *rope_freq;
     uint32_t interleaved;   // 1: pairs (2i, 2i+1); 0: pairs (i, i + rotary_dim/2)
     uint32_t rotary_dim;
     uint32_t head_dim;

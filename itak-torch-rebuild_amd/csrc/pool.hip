@@ -102,8 +102,16 @@ std::atomic<uint64_t> g_next_cache_id{1};  // cache.rs:32
 
 }  // namespace
 
+// rope_base^(-2i/rotary_dim), i < rotary_dim/2, computed on the host and kept on the device.
+struct RopeFreqTable {
+    float base;
+    uint32_t rotary;
+    double *dev;
+};
+
 struct itak_pool {
     itak_pool_config cfg{};
+    std::vector<RopeFreqTable> rope_tables;
     // Global layers and windowed layers are two groups of planes with their own row capacity:
     // `g` (capacity_rows per plane) and `gw` (the longest ring per plane). Within a group the
     // layers are consecutive, so the kernels that walk several layers take (group base,
@@ -342,6 +350,34 @@ itak_status ensure_stage(itak_pool *pool, uint64_t bytes) {
     HIP_TRY(pool, hipMalloc(reinterpret_cast<void **>(&pool->stage), want), "allocate staging");
     pool->stage_bytes = want;
     return ITAK_OK;
+}
+
+// The rotation frequencies of (base, rotary_dim) in device memory, made on first use: the same
+// expression, in the same f64 libm, as rope.rs:99-116 and rope_interleaved.rs:103-114 evaluate
+// on the host. Null when the table does not exist yet and cannot be made now (the stream is
+// being captured, or the allocation failed): the preparation kernel then takes the powers itself.
+const double *rope_freq_table(itak_pool *pool, float base, uint32_t rotary) {
+    if (!(base > 1.0f) || rotary < 2) return nullptr;
+    for (const RopeFreqTable &t : pool->rope_tables)
+        if (t.base == base && t.rotary == rotary) return t.dev;
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(pool->stream, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    if (status != hipStreamCaptureStatusNone || pool->rope_tables.size() >= 64) return nullptr;
+    std::vector<double> host(rotary / 2);
+    for (uint32_t i = 0; i < rotary / 2; ++i)
+        host[i] = std::pow(double(base), -double(2 * i) / double(rotary));
+    double *dev = nullptr;
+    if (hipMalloc(reinterpret_cast<void **>(&dev), host.size() * sizeof(double)) != hipSuccess ||
+        hipMemcpy(dev, host.data(), host.size() * sizeof(double), hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipGetLastError();
+        if (dev) (void)hipFree(dev);
+        return nullptr;
+    }
+    pool->rope_tables.push_back(RopeFreqTable{base, rotary, dev});
+    return dev;
 }
 
 itak_status ensure_workspace(itak_pool *pool, uint64_t floats) {
@@ -1207,6 +1243,8 @@ void itak_pool_destroy(itak_pool *pool) {
     if (pool->prep) (void)hipFree(pool->prep);
     if (pool->xws) (void)hipFree(pool->xws);
     if (pool->die_words) (void)hipFree(pool->die_words);
+    for (const RopeFreqTable &t : pool->rope_tables)
+        if (t.dev) (void)hipFree(t.dev);
     for (void *buf : pool->ring_saved)
         if (buf) (void)hipFree(buf);
     if (pool->hstage) (void)hipHostFree(pool->hstage);
@@ -2478,6 +2516,7 @@ itak_status itak_attention_prep_step_device(itak_pool *pool, uint64_t layer,
         a.k_weight = prep->k_norm_weight;
         a.eps = prep->eps;
         a.rope_base = rotate ? prep->rope_base : 0.0f;
+        a.rope_freq = rotate ? rope_freq_table(pool, prep->rope_base, rotary) : nullptr;
         a.interleaved = interleaved ? 1 : 0;
         a.rotary_dim = rotary;
         a.head_dim = D;
@@ -2652,6 +2691,7 @@ itak_status itak_compute_attention(itak_pool *pool, uint32_t slot, uint64_t laye
         a.q_in = a.q_out = qd + done * q_width;
         a.k_in = a.k_out = kd + done * pool->row;
         a.rope_base = rope_freq_base_swa;
+        a.rope_freq = rope_freq_table(pool, rope_freq_base_swa, pool->g.head_dim);
         a.interleaved = 1;
         a.rotary_dim = pool->g.head_dim;
         a.head_dim = pool->g.head_dim;

@@ -130,6 +130,34 @@ def test_long_positions_need_the_f64_angle_law():
     pool.close()
 
 
+@pytest.mark.parametrize("pos,base,interleaved,rotary", [(100_000, 1e4, True, 0), (1_000_000, 1e6, True, 0),
+                                                         (1_000_000, 1e4, False, 64)])
+def test_rotated_f32_keys_at_long_positions_are_the_oracles_bit_for_bit(pos, base, interleaved, rotary):
+    # The angle is position * base^(-2i/d): a last bit of the power is multiplied by the position,
+    # and at 10^6 it moved a dozen of 65,536 stored elements by up to 16 units in the last place
+    # while the kernel took the power from the device's library. The frequencies come from the
+    # host's libm, which is the reference's.
+    kvh, d, q_heads, window, rows = 2, 128, 4, 64, 64
+    width = kvh * d
+    rng = np.random.default_rng(pos + int(base))
+    pool = P().KvPool([P().LayerKind.windowed(window)], kvh, d, elem="f32", capacity_rows=pos + 2 * rows + 8)
+    pool.set_stream(torch.cuda.current_stream().cuda_stream)
+    cache = pool.acquire()
+    cache.restore_bulk(0, pos - window, normal(rng, window, width), normal(rng, window, width))
+    for rep in range(2):
+        q, k, v = normal(rng, rows, q_heads * d), normal(rng, rows, width), normal(rng, rows, width)
+        qd, kd, vd = dev(q), dev(k), dev(v)
+        out = torch.empty_like(qd)
+        pool.attention_prep_step_device(0, [(cache, rows)], qd.data_ptr(), kd.data_ptr(), vd.data_ptr(),
+                                        out.data_ptr(), q_heads, rope_base=base, interleaved=interleaved,
+                                        rotary_dim=rotary)
+        torch.cuda.synchronize()
+        want = oracle.attention_prep(k, kvh, d, pos + rep * rows, None, 1e-6, base, interleaved, rotary or None)
+        _, gk, _ = cache.read_rows(0, cache.stored_len(0) - rows, rows)
+        assert np.asarray(gk).reshape(rows, width).tobytes() == np.asarray(want, dtype=np.float32).tobytes()
+    pool.close()
+
+
 @pytest.mark.parametrize("rows,interleaved,rotary,norm,rope_base", [
     (7, True, 0, True, 1e6), (7, False, 0, True, 1e4), (5, False, 64, False, 1e4),
     (5, True, 32, True, 5e5), (1, True, 0, True, 0.0), (200, True, 0, True, 1e6),

@@ -16,7 +16,10 @@ pytestmark = pytest.mark.gpu
 # (Among them the seeds on which keys rotated inside the attention launch, with the hardware's
 # sine and cosine, once came out one f16 step from the oracle's; the call rotates by the
 # preparation launch since.)
-SEEDS = sorted({*range(24), 35, 44, 47, 100, 113, 146})
+# 5253 and 5604: a rotated f32 key one and three units in the last place off while the kernel took
+# the rotation frequencies from the device library's pow (a last bit that the position
+# multiplies); they come from the host's now.
+SEEDS = sorted({*range(24), 35, 44, 47, 100, 113, 146, 5253, 5604})
 
 
 def P():
