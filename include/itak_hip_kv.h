@@ -97,8 +97,8 @@ enum {
    of f32 arithmetic over the same rounded rows as long as the scaled scores q.k*scale have a
    standard deviation of at most about 3 (3e-5 at unit scale, 1.5e-3 at 3, above the bar from
    about 4.5 on). Q and K normed per head, as the reference's model norms them, stay at unit
-   scale. ITAK_POOL_Q_TWO_HALVES lifts the limit for decode steps and blocks of up to 8 rows at
-   head_dim 128 (4e-5 to 2.6e-4 observed at standard deviation 6).
+   scale. ITAK_POOL_Q_TWO_HALVES lifts the limit at head_dim 128 (4e-5 to 2.6e-4 observed at
+   standard deviation 6).
    Rows that are not finite reach the outputs of exactly the query rows that see their position
    (the reference never reads the key or value row of a masked position), on f32 pools and on
    f16 pools: an infinity or a NaN in a value row the channels it stands in, a key whose score
@@ -141,15 +141,17 @@ enum {
        level or slower below (the launch's own tail and a slower start cost what the second
        launch costs), so it is not the default. */
     ITAK_POOL_DIE_MERGE = 4u,
-    /* f16 pools at head_dim 128, decode steps and blocks of up to 8 rows (the split-K kernels):
+    /* f16 pools at head_dim 128, every step (decode rows, blocks, prefill chunks):
        the queries enter the score products as two f16 halves, q = hi + lo, and every score is
        K.hi + K.lo. Without the flag Q is rounded to f16 once, an error relative to each channel
        that grows with the scores: outputs meet the 2e-3 bar up to scaled scores of standard
        deviation 3 (see ITAK_ELEM_F16). With it the queries are good to 2^-22 and what is left is
-       the rounding of the softmax weights to f16. These kernels wait for memory more than for
-       the matrix pipe: the second product costs 1 % on a decode step or a ragged batch and 7 %
-       on a speculative block of 64 query vectors per KV head. Longer blocks and prefill
-       chunks (the block kernel) are not affected by the flag. One thing it changes for keys
+       the rounding of the softmax weights to f16. The decode and split-K kernels wait for
+       memory more than for the matrix pipe: the second product costs 1 % on a decode step or a
+       ragged batch and 7 % on a speculative block of 64 query vectors per KV head. Longer
+       blocks and prefill chunks (the block kernel, which the matrix pipe bounds) take 22 to
+       26 % longer, and blocks of 9 to 64 rows are appended by a launch of their own instead of
+       inside the attention launch. Other head dims ignore the flag. One thing it changes for keys
        that are not finite: an infinite channel of a visible key makes the score NaN when the
        channel's two halves have opposite signs (inf - inf), and the output row with it, where
        the single product and the reference have a score of plus or minus infinity. */

@@ -40,6 +40,7 @@ static int tiles_for(const AttnBatch &b, uint32_t group) {
         nvec = std::max(nvec, b.item[i].rows * padded_group(group));
         nblocks = std::max(nblocks, item_block_count(b.item[i]));
     }
+    if (b.two_halves) return kMaxTiles;  // the form with the registers for the second halves
     if (nvec <= uint32_t(kWaves * 16)) return 1;
     return nvec <= 512 && nblocks <= kOneTileBlocks ? 1 : kMaxTiles;
 }
@@ -162,6 +163,7 @@ hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, uint
     if (b.total_blocks == 0) return hipSuccess;
     const bool one = tiles_for(b, p.group) == 1;
     if (p.k_new && !one) return hipErrorInvalidValue;  // only the one-tile form appends
+    if (b.two_halves) return launch_attn_prefill_f16_qlo(p, b, total_partials, stream);
     if (p.g.head_dim == 128) return launch_prefill_head_dim<128, true>(p, b, total_partials, one, stream);
     return launch_attn_prefill_f16_dims(p, b, total_partials, one, stream);
 }

@@ -107,7 +107,11 @@ __device__ __forceinline__ void wait_vmcnt() {
 // lower edge); global layers run the instantiation without any of it.
 // D = head_dim. At 256 a stage of the ring is 32 KiB and a wavefront's accumulators alone are 64
 // to 128 registers: one workgroup per compute unit, up to 512 registers a lane.
-template <int N, bool SOFTCAP, int kTiles, bool RING, int STAGES, int D>
+// QLO (ITAK_POOL_Q_TWO_HALVES; head_dim 128, two tiles): the scaled queries are held as two
+// halves, q = hi + lo with hi = f16(q) and lo = f16(q - hi), and every score is K.hi + K.lo: the
+// queries' rounding to f16, which is relative to each channel and so grows with the scores,
+// leaves the scores. Half as many score products again on a kernel the matrix pipe bounds.
+template <int N, bool SOFTCAP, int kTiles, bool RING, int STAGES, int D, bool QLO = false>
 __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f16_kernel(
     AttnParams p, AttnBatchT<N> b, uint32_t total_partials) {
     constexpr int kD = D;
@@ -279,6 +283,8 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     const bool by_stage = stores_new && patches && item.rows >= 8 && (!RING || ring_blocks >= 3);
     [[maybe_unused]] uint2 npk[kCanFuse ? kFusePieces : 1];
     half8 qb[kTiles][kSteps];
+    static_assert(!QLO || (kTiles == 2 && D == 128), "the two-halves form exists for two tiles at head_dim 128");
+    [[maybe_unused]] half8 qb_lo[QLO ? kTiles : 1][kSteps];
     uint32_t colpos[kTiles], collo[kTiles];
     const float *qp[kTiles];
     float qsc[kTiles];
@@ -316,6 +322,12 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
                               static_cast<_Float16>(a[2] * sc), static_cast<_Float16>(a[3] * sc), \
                               static_cast<_Float16>(c[0] * sc), static_cast<_Float16>(c[1] * sc), \
                               static_cast<_Float16>(c[2] * sc), static_cast<_Float16>(c[3] * sc)}; \
+            if constexpr (QLO) {                                                                \
+                _Pragma("unroll") for (int e = 0; e < 8; ++e) {                                 \
+                    const float full = (e < 4 ? a[e & 3] : c[e & 3]) * sc;                      \
+                    qb_lo[qt][s][e] = static_cast<_Float16>(full - float(qb[qt][s][e]));        \
+                }                                                                               \
+            }                                                                                   \
         }
     bool took_new = false;
     if constexpr (kCanFuse) {
@@ -516,6 +528,11 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
 #pragma unroll
                         for (int k = 0; k < kSteps; ++k)
                             s = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[t][k], qb[qt][k], s, 0, 0, 0);
+                        if constexpr (QLO) {
+#pragma unroll
+                            for (int k = 0; k < kSteps; ++k)
+                                s = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[t][k], qb_lo[qt][k], s, 0, 0, 0);
+                        }
                         x[qt][t] = s;
                     }
             }
@@ -753,29 +770,29 @@ __global__ __launch_bounds__(kWaves * 64, D <= 128 ? 2 : 1) void attn_prefill_f1
     ITAK_MARK_END
 }
 
-template <int N, bool SOFTCAP, int TILES, bool RING, int STAGES, int D>
+template <int N, bool SOFTCAP, int TILES, bool RING, int STAGES, int D, bool QLO = false>
 hipError_t launch_prefill_ring(const AttnParams &p, const AttnBatch &b,
                                       uint32_t total_partials, hipStream_t stream) {
     constexpr size_t lds = size_t(STAGES) * stage_bytes(D);
     static const hipError_t granted = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(&attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING, STAGES, D>),
+        reinterpret_cast<const void *>(&attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING, STAGES, D, QLO>),
         hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
     if (granted != hipSuccess) return granted;
-    attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING, STAGES, D>
+    attn_prefill_f16_kernel<N, SOFTCAP, TILES, RING, STAGES, D, QLO>
         <<<b.total_blocks, kWaves * 64, lds, stream>>>(p, AttnBatchT<N>(b), total_partials);
     return hipGetLastError();
 }
 
-template <int N, bool SOFTCAP, int TILES, bool RING, int D>
+template <int N, bool SOFTCAP, int TILES, bool RING, int D, bool QLO = false>
 hipError_t launch_prefill(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                  hipStream_t stream) {
     if constexpr (D <= 128) {
         if (b.deep_ring)
-            return launch_prefill_ring<N, SOFTCAP, TILES, RING, kDeepStages, D>(p, b, total_partials, stream);
+            return launch_prefill_ring<N, SOFTCAP, TILES, RING, kDeepStages, D, QLO>(p, b, total_partials, stream);
     } else if (b.deep_ring) {
         return hipErrorInvalidValue;
     }
-    return launch_prefill_ring<N, SOFTCAP, TILES, RING, kStages, D>(p, b, total_partials, stream);
+    return launch_prefill_ring<N, SOFTCAP, TILES, RING, kStages, D, QLO>(p, b, total_partials, stream);
 }
 
 // Softcap, ring and tile count chosen for one head_dim. BY_CLASS: an instantiation per batch

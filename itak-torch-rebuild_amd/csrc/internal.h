@@ -244,6 +244,7 @@ struct AttnBatch {
     uint32_t rows_per_block;
     uint32_t deep_ring;  // host side only: the block kernel's plan asks for its deeper LDS ring
     uint32_t fold_units; // host side only: the block kernel's plan for AttnParams::fold_units
+    uint32_t two_halves; // host side only: the block kernel multiplies each query as two f16 halves
     AttnItem item[kMaxBatchItems];
 };
 // The kernel argument form of AttnBatch, sized to the batch: kernel arguments are
@@ -464,6 +465,9 @@ hipError_t launch_attn_prefill_f16(const AttnParams &p, const AttnBatch &b, uint
                                    hipStream_t stream);
 // The same at head dims 64, 96 and 256 (instantiated in a file of their own); `one` = the
 // one-tile form, as launch_attn_prefill_f16 decides it.
+// The two-halves form (head_dim 128, two tiles, no rows brought along).
+hipError_t launch_attn_prefill_f16_qlo(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
+                                       hipStream_t stream);
 hipError_t launch_attn_prefill_f16_dims(const AttnParams &p, const AttnBatch &b, uint32_t total_partials,
                                         bool one, hipStream_t stream);
 // Merge of split partials; total_rows = query rows of the batch. With `gate` the merged rows

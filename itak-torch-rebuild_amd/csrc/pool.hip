@@ -564,6 +564,7 @@ itak_status run_attention(itak_pool *pool, uint64_t layer, const PlanInput *in, 
         const uint32_t count = std::min<uint32_t>(kMaxBatchItems, n - first);
         AttnBatch b{};
         b.n = count;
+        b.two_halves = prefill && pool->q_two_halves && pool->g.head_dim == 128 ? 1 : 0;
         uint32_t total_rows = 0;
         for (uint32_t i = 0; i < count; ++i) {
             const PlanInput &pi = in[first + i];
@@ -2317,8 +2318,10 @@ static itak_status step_on_device(itak_pool *pool, uint64_t layer, const itak_ba
     for (const PlanInput &p : active)
         most_blocks = std::max(most_blocks, (p.kv_len + 31) / 32 - p.kv_lo / 32);
     const bool splitk = takes_splitk_f16(pool, active.data(), uint32_t(active.size()), num_q_heads, nullptr);
+    // (With the queries as two halves the block kernel runs its two-tile form, which brings no
+    // rows along: the append is a launch of its own.)
     const bool block_fuses =
-        !splitk && pool->elem_f16 && !active.empty() &&
+        !splitk && pool->elem_f16 && !active.empty() && !(pool->q_two_halves && pool->g.head_dim == 128) &&
         attn_prefill_f16_appends(pool->g, uint32_t(num_q_heads / pool->g.kv_heads), most_rows, most_blocks);
     const bool fuse =
         splitk || block_fuses ||

@@ -591,6 +591,19 @@ def test_queries_as_two_halves_hold_the_bar_at_scores_of_deviation_six(rows, slo
     print(f"rows {rows} slots {slots} q x{q_scale} k x{k_scale}: two halves {with_flag:.2e}")
 
 
+@pytest.mark.parametrize("rows,slots,ctx", [(32, 1, 4096), (300, 1, 3000), (20, 2, 1000), (9, 1, 40)])
+@pytest.mark.parametrize("q_scale,k_scale", [(3.0, 2.0), (1.0, 6.0)])
+def test_the_block_kernel_takes_the_queries_as_two_halves_too(rows, slots, ctx, q_scale, k_scale):
+    # Blocks of more than 8 rows and prefill chunks at head_dim 128: the block kernel's two-tile
+    # form with the second halves (blocks that would bring their rows along in the one-tile form
+    # are appended by a launch of their own). At these scores the single product is above the bar.
+    halves = _worst_error_at_scale(rows, q_scale, k_scale, ctx, slots, q_two_halves=True)
+    assert halves <= F16_ABS, halves
+    if (rows, slots) == (300, 1):
+        plain = _worst_error_at_scale(rows, q_scale, k_scale, ctx, slots)
+        assert halves * 2 < plain, (halves, plain)
+
+
 def test_queries_as_one_half_leave_the_bar_where_two_halves_hold_it():
     # The same step both ways at scores of deviation 6: the flag is what makes the difference.
     plain = _worst_error_at_scale(1, 3.0, 2.0, 4096)
