@@ -529,6 +529,9 @@ def main():
     ap.add_argument("--q-two-halves", action="store_true",
                     help="queries as two f16 halves in the split-K kernels' score products "
                          "(ITAK_POOL_Q_TWO_HALVES): the 2e-3 bar then holds off unit scale")
+    ap.add_argument("--prep-by-launch", action="store_true",
+                    help="with --prep: the preparation always as a launch of its own, the reference's "
+                         "f64 chain (ITAK_POOL_PREP_BY_LAUNCH)")
     ap.add_argument("--prep", action="store_true",
                     help="also time the step with the fused Q/K preparation (per-head RMSNorm + "
                          "RoPE) before it and the sigmoid gate after it, reported as 'with_prep'")
@@ -570,7 +573,7 @@ def main():
     result = run_workload(args, pkg, torch, np, dev, stream, timed)
     primary = (args.workload == "decode" and args.kv == "f16" and args.softcap == 0.0
                and not args.only and not args.merge_in_launch and not args.die_merge
-               and not args.q_two_halves)
+               and not args.q_two_halves and not args.prep_by_launch)
     if primary:
         # The other configurations in short runs of their own, so that one line carries every
         # kernel's figure; `metric`, `value` and `config` stay those of the decode step.
@@ -767,7 +770,8 @@ def run_workload(args, pkg, torch, np, dev, stream, timed):
                       ring_headroom=rows if wl == "prefill_windowed" else 0,
                       merge_in_launch=args.merge_in_launch,
                       die_merge=getattr(args, "die_merge", False),
-                      q_two_halves=getattr(args, "q_two_halves", False))
+                      q_two_halves=getattr(args, "q_two_halves", False),
+                      prep_by_launch=getattr(args, "prep_by_launch", False))
     pool.set_stream(stream.cuda_stream)
     caches = [pool.acquire() for _ in range(slots)]
 
@@ -903,7 +907,7 @@ def run_workload(args, pkg, torch, np, dev, stream, timed):
         for _ in range(max(args.warmup, 1)):
             g_prep.replay()
         prep_s = timed(g_prep.replay, args.steps)[0] / args.steps
-        folded = rows * (Q_HEADS // KV_HEADS) <= 64 and rows <= 8
+        folded = rows * (Q_HEADS // KV_HEADS) <= 64 and rows <= 8 and not args.prep_by_launch
         with_prep = {
             "us_per_layer": round(prep_s / layers * 1e6, 3),
             "added_us_per_layer": round((prep_s - step_s) / layers * 1e6, 3),

@@ -55,6 +55,7 @@ pub const ITAK_POOL_SCRUB_ON_TRUNCATE: u32 = 1;
 pub const ITAK_POOL_MERGE_IN_LAUNCH: u32 = 2;
 pub const ITAK_POOL_DIE_MERGE: u32 = 4;
 pub const ITAK_POOL_Q_TWO_HALVES: u32 = 8;
+pub const ITAK_POOL_PREP_BY_LAUNCH: u32 = 16;
 
 /// Opaque handle.
 #[repr(C)]

@@ -32,6 +32,7 @@ POOL_SCRUB_ON_TRUNCATE = 1
 POOL_MERGE_IN_LAUNCH = 2
 POOL_DIE_MERGE = 4
 POOL_Q_TWO_HALVES = 8
+POOL_PREP_BY_LAUNCH = 16
 
 
 class PoolConfig(C.Structure):

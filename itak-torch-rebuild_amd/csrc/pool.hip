@@ -159,6 +159,7 @@ struct itak_pool {
     bool die_merge = false;
     uint32_t *die_words = nullptr;
     bool q_two_halves = false;  // ITAK_POOL_Q_TWO_HALVES
+    bool prep_by_launch = false;  // ITAK_POOL_PREP_BY_LAUNCH
     // Per slot: the side buffer of a deep checkpoint's ring rows, kept for the next one
     // (cache.rs:620-625: allocated once per cache, not once per round).
     std::vector<void *> ring_saved;
@@ -1208,6 +1209,7 @@ itak_status itak_pool_create(const itak_pool_config *config, itak_pool **out) {
     pool->ring_saved_bytes.assign(config->max_slots, 0);
     pool->merge_in_launch = (config->flags & ITAK_POOL_MERGE_IN_LAUNCH) != 0;
     pool->q_two_halves = pool->elem_f16 && (config->flags & ITAK_POOL_Q_TWO_HALVES) != 0;
+    pool->prep_by_launch = (config->flags & ITAK_POOL_PREP_BY_LAUNCH) != 0;
     if (pool->elem_f16 && !pool->merge_in_launch && (config->flags & ITAK_POOL_DIE_MERGE) &&
         die_layout_ok(config->device)) {
         he = hipMalloc(reinterpret_cast<void **>(&pool->die_words), kDieTicketBytes + 256);
@@ -2489,7 +2491,7 @@ itak_status itak_attention_prep_step_device(itak_pool *pool, uint64_t layer,
     const bool splitk = takes_splitk_f16(pool, active.data(), uint32_t(active.size()), num_q_heads,
                                          nullptr);
     const bool interleaved = prep->rope_interleaved != 0;
-    const bool folds = splitk && (!rotate || interleaved || rotary % 8 == 0);
+    const bool folds = splitk && !pool->prep_by_launch && (!rotate || interleaved || rotary % 8 == 0);
     FoldedParams folded{};
     folded.gate = gate_dev;
     if (folds) {

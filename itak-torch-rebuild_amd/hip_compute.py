@@ -195,7 +195,7 @@ class KvPool:
                  *, elem: str = "f16", max_slots: int = 1, capacity_rows: int = 4096,
                  device: int = 0, scrub_on_truncate: bool = True, ring_headroom: int = 0,
                  merge_in_launch: bool = False, die_merge: Optional[bool] = None,
-                 q_two_halves: Optional[bool] = None):
+                 q_two_halves: Optional[bool] = None, prep_by_launch: bool = False):
         if isinstance(pattern, int):
             pattern = [LayerKind.Global] * pattern
         self.pattern = list(pattern)
@@ -229,6 +229,8 @@ class KvPool:
             q_two_halves = os.environ.get("ITAK_HIP_KV_Q_TWO_HALVES", "0") == "1"
         if q_two_halves:
             cfg.flags |= N.POOL_Q_TWO_HALVES
+        if prep_by_launch:  # attention_prep_step_device never prepares inside the attention launch
+            cfg.flags |= N.POOL_PREP_BY_LAUNCH
         cfg.ring_headroom = ring_headroom
         handle = C.c_void_p()
         self._h = None

@@ -130,6 +130,46 @@ def test_long_positions_need_the_f64_angle_law():
     pool.close()
 
 
+@pytest.mark.parametrize("rows,norm,pos0", [(1, True, 0), (2, False, 50_000), (7, True, 50_000)])
+def test_preparation_by_launch_stores_the_oracles_f16_keys_bit_for_bit(rows, norm, pos0):
+    # ITAK_POOL_PREP_BY_LAUNCH: decode rows and short blocks at head_dim 128, which otherwise
+    # prepare inside the attention launch in f32 (within one f16 step of the reference's chain:
+    # a few stored elements in ten thousand differ), go through the f64 preparation launch.
+    d, kvh, q_heads, window = 128, 4, 32, 128
+    width = kvh * d
+    rng = np.random.default_rng(rows + pos0)
+    differing = {}
+    for by_launch in (True, False):
+        data = np.random.default_rng(rows + pos0 + 1)
+        pool = P().KvPool([P().LayerKind.windowed(window)], kvh, d, elem="f16", ring_headroom=64,
+                          capacity_rows=pos0 + 60 * rows + 200, prep_by_launch=by_launch)
+        pool.set_stream(torch.cuda.current_stream().cuda_stream)
+        cache = pool.acquire()
+        if pos0:
+            cache.restore_bulk(0, pos0 - window, normal(data, window, width), normal(data, window, width))
+        w = 1.0 + 0.1 * normal(data, d)
+        wd = dev(w)
+        off = 0
+        for rep in range(60):
+            q, k, v = normal(data, rows, q_heads * d), normal(data, rows, width), normal(data, rows, width)
+            qd, kd, vd = dev(q), dev(k), dev(v)
+            out = torch.empty_like(qd)
+            pool.attention_prep_step_device(0, [(cache, rows)], qd.data_ptr(), kd.data_ptr(), vd.data_ptr(),
+                                            out.data_ptr(), q_heads, q_norm_ptr=wd.data_ptr() if norm else 0,
+                                            k_norm_ptr=wd.data_ptr() if norm else 0, eps=1e-6, rope_base=1e6,
+                                            interleaved=True)
+            torch.cuda.synchronize()
+            kp = oracle.attention_prep(k, kvh, d, pos0 + rep * rows, w if norm else None, 1e-6, 1e6, True, None)
+            _, gk, _ = cache.read_rows(0, cache.stored_len(0) - rows, rows)
+            want = oracle.f32_to_f16_array(np.asarray(kp, dtype=np.float32).reshape(rows, width))
+            off += int((np.asarray(gk).reshape(rows, width).view(np.int16) != want.view(np.int16)).sum())
+        differing[by_launch] = off
+        pool.close()
+    assert differing[True] == 0, differing
+    print(f"rows {rows}: stored f16 key elements that differ from the oracle's, folded form {differing[False]}, "
+          f"by launch {differing[True]}, of {60 * rows * width}")
+
+
 @pytest.mark.parametrize("pos,base,interleaved,rotary", [(100_000, 1e4, True, 0), (1_000_000, 1e6, True, 0),
                                                          (1_000_000, 1e4, False, 64)])
 def test_rotated_f32_keys_at_long_positions_are_the_oracles_bit_for_bit(pos, base, interleaved, rotary):
